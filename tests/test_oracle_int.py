@@ -1,0 +1,219 @@
+"""Pins for oracle/int_quant.py: hand-computed known answers (exact in fp32),
+numpy float32 recomputation of the IEEE chain, the zero-pad rule, invariants."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import int_quant as iq
+
+
+def T(*v, dtype=torch.float32):
+    return torch.tensor(v, dtype=dtype).reshape(-1, 1)
+
+
+# ---- scale / offset known answers -----------------------------------------
+def test_sym_scope_127_vs_128():
+    s, z = iq.scale_offset(T(1.27), T(-1.0), True, 'int8')
+    assert z is None and s.dtype == torch.float32
+    assert s.item() == np.float32(1.27) / np.float32(127)
+    s, _ = iq.scale_offset(T(1.0), T(-1.28), True, 'int8')
+    assert s.item() == np.float32(1.28) / np.float32(128)
+    # exact cases: power-of-two bounds
+    s, _ = iq.scale_offset(T(127.0), T(-1.0), True, 'int8')
+    assert s.item() == 1.0
+    s, _ = iq.scale_offset(T(1.0), T(-128.0), True, 'int8')
+    assert s.item() == 1.0
+    s, _ = iq.scale_offset(T(7.0), T(-8.0), True, 'int4')
+    assert s.item() == 1.0
+    s, _ = iq.scale_offset(T(8.0), T(-8.0), True, 'int4')      # equal magnitudes -> 7
+    assert s.item() == np.float32(8) / np.float32(7)
+
+
+def test_zero_range_guard():
+    s, z = iq.scale_offset(T(0.0), T(0.0), True, 'int8')
+    assert s.item() == 1.0 and z is None
+    s, z = iq.scale_offset(T(0.0), T(0.0), False, 'int8')
+    assert s.item() == 1.0 and z.item() == -128 and z.dtype == torch.int32
+    s, z = iq.scale_offset(T(0.0), T(0.0), False, 'int4')
+    assert s.item() == 1.0 and z.item() == -8
+    # below eps but not zero: guard still fires
+    s, z = iq.scale_offset(T(1e-6), T(0.0), False, 'int8')     # 1e-6/255 < eps
+    assert s.item() == 1.0 and z.item() == -128
+    s, z = iq.scale_offset(T(1e-6), T(-1e-6), True, 'int8')
+    assert s.item() == 1.0
+
+
+def test_asym_known_answers():
+    s, z = iq.scale_offset(T(1.5), T(0.0), False, 'int4')
+    assert s.item() == np.float32(1.5) / np.float32(15) and z.item() == -8
+    # min > 0 is clamped to 0, max < 0 is clamped to 0
+    s, z = iq.scale_offset(T(255.0), T(3.0), False, 'int8')
+    assert s.item() == 1.0 and z.item() == -128
+    s, z = iq.scale_offset(T(-3.0), T(-255.0), False, 'int8')
+    assert s.item() == 1.0 and z.item() == 127
+    # tie in the offset rounding goes to even: s = 0.5, z = -128 + 0.5 = -127.5 -> -128
+    s, z = iq.scale_offset(T(127.25), T(-0.25), False, 'int8')
+    assert s.item() == 0.5 and z.item() == -128
+    # -128 + 1.5 = -126.5 -> -126
+    s, z = iq.scale_offset(T(126.75), T(-0.75), False, 'int8')
+    assert s.item() == 0.5 and z.item() == -126
+
+
+def test_scale_offset_matches_numpy_f32_chain():
+    rng = np.random.default_rng(0)
+    n = 200000
+    mx = (rng.standard_normal(n) * 10 ** rng.uniform(-6, 6, n)).astype(np.float32)
+    mn = (rng.standard_normal(n) * 10 ** rng.uniform(-6, 6, n)).astype(np.float32)
+    mx, mn = np.maximum(mx, mn), np.minimum(mx, mn)
+    for kind, b in (('int8', 8), ('int4', 4)):
+        # symmetric
+        s, _ = iq.scale_offset(torch.from_numpy(mx), torch.from_numpy(mn), True, kind)
+        amx, amn = np.abs(mx), np.abs(mn)
+        scope = np.where(amx < amn, 2 ** (b - 1), 2 ** (b - 1) - 1).astype(np.float32)
+        ref = (np.where(amx > amn, amx, amn) / scope).astype(np.float32)
+        ref = np.where(ref < np.float32(1.192092896e-7), np.float32(1), ref)
+        assert np.array_equal(s.numpy(), ref)
+        # asymmetric
+        s, z = iq.scale_offset(torch.from_numpy(mx), torch.from_numpy(mn), False, kind)
+        cmx, cmn = np.maximum(mx, 0), np.minimum(mn, 0)
+        sc = ((cmx - cmn).astype(np.float32) / np.float32(2 ** b - 1)).astype(np.float32)
+        with np.errstate(all='ignore'):
+            off = (np.float32(-(2 ** (b - 1))) - (cmn / sc).astype(np.float32)).astype(np.float32)
+        off = np.where(cmx != cmn, off, np.float32(-(2 ** (b - 1))))
+        tiny = sc < np.float32(1.192092896e-7)
+        off = np.where(tiny, np.float32(-(2 ** (b - 1))), off)
+        sc = np.where(tiny, np.float32(1), sc)
+        assert np.array_equal(s.numpy(), sc)
+        assert np.array_equal(z.numpy(), np.rint(off).astype(np.int32))
+        assert z.min() >= -(2 ** (b - 1)) and z.max() <= 2 ** (b - 1) - 1
+
+
+def test_invalid_scale_raises():
+    with pytest.raises(RuntimeError, match="Param scale has invalid value"):
+        iq.scale_offset(T(float('inf')), T(0.0), True, 'int8')
+    with pytest.raises(RuntimeError, match="Param scale has invalid value"):
+        iq.scale_offset(T(float('nan')), T(0.0), False, 'int8')
+
+
+# ---- min/max ---------------------------------------------------------------
+def test_group_zero_pad_participates():
+    w = torch.full((2, 40), 3.0)                 # K=40, g=32 -> second group has 8 values + 24 zeros
+    mn, mx = iq.weight_min_max(w, 'group', 32)
+    assert mn.shape == (2, 2, 1) and mx.shape == (2, 2, 1)
+    assert mn[0, 0, 0] == 3.0 and mn[0, 1, 0] == 0.0 and mx[0, 1, 0] == 3.0
+    w = -w
+    mn, mx = iq.weight_min_max(w, 'group', 32)
+    assert mx[0, 1, 0] == 0.0 and mn[0, 1, 0] == -3.0
+
+
+def test_min_max_shapes():
+    w = torch.randn(8, 64)
+    mn, mx = iq.weight_min_max(w, 'channel')
+    assert mn.shape == (8, 1) and torch.equal(mx[:, 0], w.amax(1))
+    mn, mx = iq.weight_min_max(w, 'tensor')
+    assert mn.shape == (1, 1) and mx.item() == w.max().item()
+
+
+# ---- elementwise -----------------------------------------------------------
+def test_to_codes_ties_even_and_saturation():
+    t = torch.tensor([0.5, 1.5, 2.5, -0.5, -1.5, 126.5, 127.5, 300.0, -128.5, -129.5, -400.0])
+    assert iq.to_codes(t, 'int8').tolist() == [0, 2, 2, 0, -2, 126, 127, 127, -128, -128, -128]
+    c4 = iq.to_codes(torch.tensor([6.5, 7.5, 9.0, -7.5, -8.5, -20.0]), 'int4')
+    assert c4.dtype == torch.int32 and c4.tolist() == [6, 7, 7, -8, -8, -8]
+    with pytest.raises(ValueError, match="Not supported quant_dtype int2"):
+        iq.to_codes(t, 'int2')
+
+
+def test_variant_b_known_answer():
+    q, s = iq.absmax_quant(torch.tensor([[-127.0, 63.5, 62.5]]))
+    assert s.item() == 1.0 and q.tolist() == [[-127, 64, 62]]
+    q, s = iq.absmax_quant(torch.tensor([[-128.0, 127.0, 1.0]]))    # clamp at -qmax
+    assert q.min().item() >= -127
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("kind", ['int8', 'int4'])
+@pytest.mark.parametrize("sym", [True, False])
+def test_fake_quant_matches_numpy_chain(dtype, kind, sym):
+    g = torch.Generator().manual_seed(5)
+    w = (torch.randn(16, 96, generator=g) * 0.02).to(dtype)
+    s, z = iq.weight_scale_offset(w, 'channel', sym, kind)
+    dq = iq.fake_quant(w, kind, s, z)
+    assert dq.dtype == dtype
+    b = int(kind[3:])
+    wf = w.float().numpy()
+    t = (wf / s.numpy()).astype(np.float32)
+    if z is not None:
+        t = (t + z.numpy().astype(np.float32)).astype(np.float32)
+    q = np.clip(np.rint(t), -(2 ** (b - 1)), 2 ** (b - 1) - 1)
+    codes = iq.quant_codes(w, kind, s, z)
+    assert np.array_equal(codes.numpy().astype(np.float32), q)
+    if z is not None:
+        q = (q - z.numpy().astype(np.float32)).astype(np.float32)
+    ref = torch.from_numpy((q * s.numpy()).astype(np.float32)).to(dtype)
+    assert torch.equal(dq, ref)
+    # invariants
+    assert codes.min() >= -(2 ** (b - 1)) and codes.max() <= 2 ** (b - 1) - 1
+    if dtype == torch.float32:
+        # scope 128 rows can clip their largest positive value by one step
+        assert ((w - dq).abs() <= s * (1.0001 if sym else 0.50001)).all()
+        # idempotent given the same factors
+        assert torch.equal(iq.fake_quant(dq, kind, s, z), dq)
+
+
+def test_fake_quant_group_ragged():
+    g = torch.Generator().manual_seed(6)
+    w = torch.randn(4, 80, generator=g)
+    s, z = iq.weight_scale_offset(w, 'group', False, 'int4', 32)
+    assert s.shape == (4, 3, 1) and z.shape == (4, 3, 1)
+    dq = iq.fake_quant(w, 'int4', s, z, 32)
+    assert dq.shape == w.shape
+    # group 2 has 16 real columns: recompute by hand with zeros appended
+    blk = torch.cat([w[:, 64:], torch.zeros(4, 16)], 1)
+    s2, z2 = iq.scale_offset(blk.amax(1, keepdim=True), blk.amin(1, keepdim=True), False, 'int4')
+    assert torch.equal(s2, s[:, 2]) and torch.equal(z2, z[:, 2])
+
+
+def test_awq_path_differs_only_by_the_cast():
+    g = torch.Generator().manual_seed(7)
+    w = (torch.randn(8, 64, generator=g) * 0.05).to(torch.bfloat16)
+    s, z = iq.weight_scale_offset(w, 'group', False, 'int4', 32)
+    a = iq.awq_fake_quant(w, 'int4', s, z, 'group', 32)
+    b = iq.fake_quant(w, 'int4', s, z, 32)
+    assert a.dtype == b.dtype == torch.bfloat16 and a.shape == b.shape
+    # on fp32 weights the cast is the identity, so both paths agree exactly
+    wf = w.float()
+    s, z = iq.weight_scale_offset(wf, 'channel', True, 'int8')
+    assert torch.equal(iq.awq_fake_quant(wf, 'int8', s, z, 'channel'), iq.fake_quant(wf, 'int8', s, z))
+    # a bf16 value that the cast moves across a rounding boundary: t = 2.498 -> bf16(2.5) -> 2
+    # while the fp32 path rounds 2.498 -> 2 as well; 3.498 -> bf16 3.5 -> 4 vs fp32 -> 3
+    wv = torch.tensor([[3.498, 100.0]], dtype=torch.float32)
+    s1 = torch.tensor([[1.0]])
+    assert iq.fake_quant(wv, 'int8', s1)[0, 0].item() == 3.0
+    assert iq.awq_fake_quant(wv.to(torch.bfloat16), 'int8', s1, None, 'channel')[0, 0].item() == 4.0 or \
+        wv.to(torch.bfloat16)[0, 0].item() != 3.498
+
+
+def test_dynamic_token_quant():
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(12, 128, generator=g).to(torch.bfloat16)
+    x[3] = 0
+    q, s = iq.dynamic_token_quant(x)
+    assert q.dtype == torch.int8 and s.shape == (12,) and s[3].item() == 1.0 and q[3].abs().max() == 0
+    xf = x.float()
+    for m in range(12):
+        amx, amn = xf[m].max().abs().item(), xf[m].min().abs().item()
+        scope = 128 if amx < amn else 127
+        sm = np.float32(max(amx, amn)) / np.float32(scope) if max(amx, amn) > 0 else np.float32(1)
+        assert s[m].item() == sm
+    q2, s2 = iq.dynamic_token_quant_absmax(x)
+    assert s2[3].item() == 1.0 and q2.dtype == torch.int8
+
+
+def test_static_quantize_axes():
+    x = torch.tensor([[1.0, 2.5, -3.5], [100.0, -100.0, 0.25]], dtype=torch.bfloat16)
+    q = iq.static_quantize(x, torch.tensor([1.0], dtype=torch.bfloat16), torch.tensor([0.0], dtype=torch.bfloat16), -1)
+    assert q.tolist() == [[1, 2, -4], [100, -100, 0]]
+    q = iq.static_quantize(x, torch.tensor([2.0, 4.0], dtype=torch.bfloat16),
+                           torch.tensor([1.0, 0.0], dtype=torch.bfloat16), -2)
+    assert q.tolist() == [[3, 6, -6], [127, -128, 1]]
