@@ -1,0 +1,59 @@
+"""Builds amct_amd/lib/libamct_hip.so from csrc/*.hip with hipcc for gfx950.
+
+Run as `python -m amct_amd.build`.  hipcc cross-compiles without a GPU.
+"""
+import concurrent.futures
+import glob
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIBDIR = os.path.join(HERE, "lib")
+LIB = os.path.join(LIBDIR, "libamct_hip.so")
+OBJDIR = os.path.join(LIBDIR, "obj")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    "-ffp-contract=off",                 # every fp32 op rounds separately, as the eager reference does
+    "-fno-fast-math",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument", "-Wno-unknown-attributes",
+]
+
+
+def _compile(src):
+    obj = os.path.join(OBJDIR, os.path.basename(src)[:-4] + ".o")
+    cmd = [HIPCC] + FLAGS + ["-c", src, "-o", obj]
+    p = subprocess.run(cmd, capture_output=True, text=True)
+    return src, obj, p.returncode, p.stdout + p.stderr
+
+
+def build_library(verbose=True, jobs=8):
+    os.makedirs(OBJDIR, exist_ok=True)
+    srcs = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
+    objs = []
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
+        for src, obj, rc, out in ex.map(_compile, srcs):
+            msgs = "\n".join(l for l in out.splitlines() if "packed-fp32-ops" not in l)
+            if rc != 0:
+                raise RuntimeError("hipcc failed on {}:\n{}".format(src, out))
+            if verbose:
+                print("compiled", os.path.basename(src), flush=True)
+                if msgs.strip() and "warning" in msgs:
+                    print(msgs)
+            objs.append(obj)
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
+    p = subprocess.run(cmd, capture_output=True, text=True)
+    if p.returncode != 0:
+        raise RuntimeError("link failed:\n" + p.stdout + p.stderr)
+    if verbose:
+        print("linked", LIB, flush=True)
+    return LIB
+
+
+if __name__ == "__main__":
+    build_library()
+    sys.exit(0)

@@ -1,0 +1,199 @@
+// Shared device helpers for the gfx950 kernels: 16-byte vector I/O, dtype
+// conversion, wave64 DPP reductions, and the scale/offset closed form.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/amct_hip.h"
+
+namespace amct {
+
+constexpr int kWave = 64;
+constexpr int kBlock = 256;
+
+#define AMCT_DEV __device__ __forceinline__
+
+// ---------------------------------------------------------------------------
+// dtype traits: VEC = elements in one 16-byte load
+// ---------------------------------------------------------------------------
+template <int DT> struct Tr;
+template <> struct Tr<AMCT_F32> { static constexpr int VEC = 4; static constexpr int BYTES = 4; };
+template <> struct Tr<AMCT_F16> { static constexpr int VEC = 8; static constexpr int BYTES = 2; };
+template <> struct Tr<AMCT_BF16> { static constexpr int VEC = 8; static constexpr int BYTES = 2; };
+
+AMCT_DEV float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+AMCT_DEV uint32_t f32_to_bf16_bits(float f) {
+    // v_cvt_pk_bf16_f32: round-half-even
+    return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
+}
+AMCT_DEV float f16_bits_to_f32(uint32_t h) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+}
+AMCT_DEV uint32_t f32_to_f16_bits(float f) {
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+}
+
+// round a fp32 value to the precision of DT and back (identity for fp32)
+template <int DT> AMCT_DEV float round_to(float f) {
+    if constexpr (DT == AMCT_BF16) return bf16_bits_to_f32(f32_to_bf16_bits(f));
+    else if constexpr (DT == AMCT_F16) return f16_bits_to_f32(f32_to_f16_bits(f));
+    else return f;
+}
+
+template <int DT> AMCT_DEV void unpack16(const uint4& v, float* f) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    if constexpr (DT == AMCT_F32) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(w[i]);
+    } else if constexpr (DT == AMCT_BF16) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = __uint_as_float(w[i] << 16);
+            f[2 * i + 1] = __uint_as_float(w[i] & 0xFFFF0000u);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = f16_bits_to_f32(w[i] & 0xFFFFu);
+            f[2 * i + 1] = f16_bits_to_f32(w[i] >> 16);
+        }
+    }
+}
+
+template <int DT> AMCT_DEV uint4 pack16(const float* f) {
+    uint32_t w[4];
+    if constexpr (DT == AMCT_F32) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = __float_as_uint(f[i]);
+    } else if constexpr (DT == AMCT_BF16) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = f32_to_bf16_bits(f[2 * i]) | (f32_to_bf16_bits(f[2 * i + 1]) << 16);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = f32_to_f16_bits(f[2 * i]) | (f32_to_f16_bits(f[2 * i + 1]) << 16);
+    }
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+template <int DT> AMCT_DEV float load_scalar(const void* p, int64_t i) {
+    if constexpr (DT == AMCT_F32) return ((const float*)p)[i];
+    else if constexpr (DT == AMCT_BF16) return bf16_bits_to_f32(((const uint16_t*)p)[i]);
+    else return f16_bits_to_f32(((const uint16_t*)p)[i]);
+}
+template <int DT> AMCT_DEV void store_scalar(void* p, int64_t i, float f) {
+    if constexpr (DT == AMCT_F32) ((float*)p)[i] = f;
+    else if constexpr (DT == AMCT_BF16) ((uint16_t*)p)[i] = (uint16_t)f32_to_bf16_bits(f);
+    else ((uint16_t*)p)[i] = (uint16_t)f32_to_f16_bits(f);
+}
+
+AMCT_DEV uint4 ldg16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
+AMCT_DEV void stg16(void* p, const uint4& v) { *reinterpret_cast<uint4*>(p) = v; }
+
+// NaN-propagating max / min (v_maximum3_f32 / v_minimum3_f32), as torch.max does
+AMCT_DEV float fmax_nan(float a, float b) { return __builtin_elementwise_maximum(a, b); }
+AMCT_DEV float fmin_nan(float a, float b) { return __builtin_elementwise_minimum(a, b); }
+
+// ---------------------------------------------------------------------------
+// wave64 reductions.  DPP for distances 1,2 (quad_perm), 4 (row_half_mirror),
+// 8 (row_mirror); cross-row distances 16 and 32 go through ds_bpermute.
+// All lanes of a team of T consecutive lanes end up with the team's result.
+// ---------------------------------------------------------------------------
+template <int CTRL> AMCT_DEV float dpp_f(float v) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+template <int CTRL> AMCT_DEV uint32_t dpp_u(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, CTRL, 0xF, 0xF, true);
+}
+
+template <int T> AMCT_DEV void team_minmax(float& mn, float& mx) {
+    if constexpr (T >= 2) { mx = fmax_nan(mx, dpp_f<0xB1>(mx)); mn = fmin_nan(mn, dpp_f<0xB1>(mn)); }
+    if constexpr (T >= 4) { mx = fmax_nan(mx, dpp_f<0x4E>(mx)); mn = fmin_nan(mn, dpp_f<0x4E>(mn)); }
+    if constexpr (T >= 8) { mx = fmax_nan(mx, dpp_f<0x141>(mx)); mn = fmin_nan(mn, dpp_f<0x141>(mn)); }
+    if constexpr (T >= 16) { mx = fmax_nan(mx, dpp_f<0x140>(mx)); mn = fmin_nan(mn, dpp_f<0x140>(mn)); }
+    if constexpr (T >= 32) { mx = fmax_nan(mx, __shfl_xor(mx, 16)); mn = fmin_nan(mn, __shfl_xor(mn, 16)); }
+    if constexpr (T >= 64) { mx = fmax_nan(mx, __shfl_xor(mx, 32)); mn = fmin_nan(mn, __shfl_xor(mn, 32)); }
+}
+
+template <int T> AMCT_DEV uint32_t team_umax(uint32_t v) {
+    if constexpr (T >= 2) v = max(v, dpp_u<0xB1>(v));
+    if constexpr (T >= 4) v = max(v, dpp_u<0x4E>(v));
+    if constexpr (T >= 8) v = max(v, dpp_u<0x141>(v));
+    if constexpr (T >= 16) v = max(v, dpp_u<0x140>(v));
+    if constexpr (T >= 32) v = max(v, (uint32_t)__shfl_xor((int)v, 16));
+    if constexpr (T >= 64) v = max(v, (uint32_t)__shfl_xor((int)v, 32));
+    return v;
+}
+
+// ---------------------------------------------------------------------------
+// (max, min) -> (scale, offset): the closed form of
+// amct_pytorch/quantize_op/utils.py:75-108 with the eps guard of :26-51,
+// every operation a separately rounded fp32 op as in the eager reference.
+// `off` is returned as an integral float (after round-half-even).
+// ---------------------------------------------------------------------------
+constexpr float kEps = 1.1920928955078125e-7f;   // fp32(1.192092896e-7), utils.py:23
+
+struct Factors {
+    float s;
+    float z;
+    bool bad;     // scale, 1/scale or offset not finite (utils.py:54-72)
+};
+
+AMCT_DEV bool finite_f(float f) { return (__float_as_uint(f) & 0x7F800000u) != 0x7F800000u; }
+
+AMCT_DEV Factors make_factors(float vmax, float vmin, int bits, bool symmetric, int scope_rule) {
+    Factors r;
+    if (symmetric) {
+        const float amax = __builtin_fabsf(vmax), amin = __builtin_fabsf(vmin);
+        const float qpos = (float)((1 << (bits - 1)) - 1);
+        if (scope_rule == AMCT_SCOPE_ABSMAX) {
+            // deploy.py:128-137 -- torch.abs(t).max(): NaN propagates, no guard
+            r.s = fmax_nan(amax, amin) / qpos;
+            r.z = 0.f;
+            r.bad = !finite_f(r.s) || !finite_f(1.0f / r.s);
+            return r;
+        }
+        const float scope = (amax < amin) ? qpos + 1.0f : qpos;
+        const float bound = (amax > amin) ? amax : amin;
+        r.s = bound / scope;
+        r.z = 0.f;
+    } else {
+        // torch.clamp propagates NaN; (x < 0 ? 0 : x) keeps NaN as well
+        vmax = (vmax < 0.f) ? 0.f : vmax;
+        vmin = (vmin > 0.f) ? 0.f : vmin;
+        const float scope = (float)((1 << bits) - 1);
+        const float half = (float)(1 << (bits - 1));        // ceil(scope / 2)
+        r.s = (vmax - vmin) / scope;
+        r.z = (vmax != vmin) ? (-half - vmin / r.s) : -half;
+    }
+    const bool tiny = r.s < kEps;
+    if (!symmetric) r.z = tiny ? -(float)(1 << (bits - 1)) : r.z;
+    r.s = tiny ? 1.0f : r.s;
+    r.bad = !finite_f(r.s) || !finite_f(1.0f / r.s) || !finite_f(r.z);
+    r.z = __builtin_rintf(r.z);
+    return r;
+}
+
+// One element of the integer (fake-)quantiser.
+//   t = x / s (+ z); [narrow to the source dtype]; q = clamp(rne(t), qmin, qmax)
+// Returns q (integral float); *deq = (q - z) * s when requested.
+template <int DT, bool VIA_SRC>
+AMCT_DEV float quant_elem(float x, float s, float z, bool asym, float qmin, float qmax) {
+    float t = x / s;
+    if (asym) t = t + z;
+    if constexpr (VIA_SRC) t = round_to<DT>(t);
+    t = __builtin_rintf(t);
+    // v_med3_f32 clamps in one op; it differs from torch.clamp only for a NaN t, which can
+    // only come from NaN data or factors (reported through the bad-factor count)
+    t = __builtin_amdgcn_fmed3f(t, qmin, qmax);
+    return t;
+}
+AMCT_DEV float dequant_elem(float q, float s, float z, bool asym) {
+    if (asym) q = q - z;
+    return q * s;
+}
+
+inline int hip_status() { return hipGetLastError() == hipSuccess ? AMCT_OK : AMCT_E_HIP; }
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace amct

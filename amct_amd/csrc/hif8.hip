@@ -1,0 +1,172 @@
+// K5: HiFloat8 encode / decode by bit manipulation (gfx950 has no instruction for it; the
+// reference has no such code).  Layout, MSB first: S | dot | exponent (D bits, sign-magnitude
+// with a hidden leading one) | mantissa:
+//   dot 11 -> D=4, 1 mantissa bit (|E| 8..15)     dot 10 -> D=3, 2 bits (|E| 4..7)
+//   dot 01 -> D=2, 3 bits (|E| 2..3)              dot 001 -> D=1, 3 bits (|E| = 1)
+//   dot 0001 -> D=0, 3 bits (E = 0)               dot 0000 -> denormal 2^(M-23), M = 1..7
+// 0x00 zero, 0x80 NaN, 0x6F / 0xEF = +-Inf (E=15, M=1); largest finite 2^15.
+// Encode rounds to nearest, ties away from zero; |x| < 2^-23 -> 0; overflow -> Inf or +-2^15.
+#include "amct_common.h"
+
+namespace amct {
+
+AMCT_DEV uint32_t hif8_enc(float x, bool saturate) {
+    const uint32_t u = __float_as_uint(x);
+    const uint32_t sign = (u >> 24) & 0x80u;
+    const uint32_t a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return 0x80u;
+    const int E = (int)(a >> 23) - 127;
+    if (E < -23) return 0u;                                   // |x| < 2^-23 (fp32 denormals included)
+    const int absE = E < 0 ? -E : E;
+    // mantissa bits kept in this binade
+    int mb = (absE <= 3) ? 3 : (absE <= 7) ? 2 : (absE <= 15) ? 1 : 0;
+    if (E > 15) mb = 1;                                       // overflows below anyway
+    // ties away from zero: add half an ulp, truncate
+    uint32_t r = a + (1u << (22 - mb));
+    r &= ~((1u << (23 - mb)) - 1u);
+    const int E2 = (int)(r >> 23) - 127;
+    if (E2 < -23) return 0u;
+    if (E2 < -15) {                                           // denormal range: powers of two only
+        const int e = E2 < -22 ? -22 : E2;                    // [2^-23, 2^-22) rounds up to the smallest
+        return sign | (uint32_t)(e + 23);
+    }
+    const int a2 = E2 < 0 ? -E2 : E2;
+    if (E2 > 15 || (E2 == 15 && (r & 0x400000u))) return sign | (saturate ? 0x6Eu : 0x6Fu);
+    const uint32_t es = E2 < 0 ? 1u : 0u;
+    if (a2 == 0) return sign | 0x08u | ((r >> 20) & 7u);
+    if (a2 == 1) return sign | 0x10u | (es << 3) | ((r >> 20) & 7u);
+    if (a2 <= 3) return sign | 0x20u | (es << 4) | ((uint32_t)(a2 & 1) << 3) | ((r >> 20) & 7u);
+    if (a2 <= 7) return sign | 0x40u | (es << 4) | ((uint32_t)(a2 & 3) << 2) | ((r >> 21) & 3u);
+    return sign | 0x60u | (es << 4) | ((uint32_t)(a2 & 7) << 1) | ((r >> 22) & 1u);
+}
+
+AMCT_DEV float hif8_dec(uint32_t c) {
+    const uint32_t b = c & 0x7Fu;
+    float f;
+    int e;
+    uint32_t man;      // mantissa aligned to the top of the fp32 fraction
+    if (b >= 0x60u) { e = 8 + ((b >> 1) & 7); if (b & 0x10u) e = -e; man = (b & 1u) << 22; }
+    else if (b >= 0x40u) { e = 4 + ((b >> 2) & 3); if (b & 0x10u) e = -e; man = (b & 3u) << 21; }
+    else if (b >= 0x20u) { e = 2 + ((b >> 3) & 1); if (b & 0x10u) e = -e; man = (b & 7u) << 20; }
+    else if (b >= 0x10u) { e = (b & 0x08u) ? -1 : 1; man = (b & 7u) << 20; }
+    else if (b >= 0x08u) { e = 0; man = (b & 7u) << 20; }
+    else {
+        if (b == 0u) return (c & 0x80u) ? __uint_as_float(0x7FC00000u) : 0.f;
+        e = (int)b - 23;
+        man = 0;
+    }
+    if (b == 0x6Fu) f = __builtin_huge_valf();
+    else f = __uint_as_float(((uint32_t)(e + 127) << 23) | man);
+    return (c & 0x80u) ? -f : f;
+}
+
+template <int DT, int U>
+__global__ __launch_bounds__(kBlock) void hif8_encode_k(const void* x, uint8_t* y, int64_t nvec, int64_t n, int saturate) {
+    constexpr int VEC = Tr<DT>::VEC;
+    const int tid = threadIdx.x;
+    uint4 raw[U];
+    int64_t gv[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        gv[u] = ((int64_t)blockIdx.x * U + u) * kBlock + tid;
+        if (gv[u] < nvec) raw[u] = ldg16(reinterpret_cast<const char*>(x) + gv[u] * 16);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        if (gv[u] < nvec) {
+            float v[VEC];
+            unpack16<DT>(raw[u], v);
+            uint32_t w[VEC / 4];
+#pragma unroll
+            for (int j = 0; j < VEC / 4; ++j)
+                w[j] = hif8_enc(v[4 * j], saturate) | (hif8_enc(v[4 * j + 1], saturate) << 8) |
+                       (hif8_enc(v[4 * j + 2], saturate) << 16) | (hif8_enc(v[4 * j + 3], saturate) << 24);
+            uint32_t* p = reinterpret_cast<uint32_t*>(y + gv[u] * VEC);
+            if constexpr (VEC == 8) *reinterpret_cast<uint2*>(p) = make_uint2(w[0], w[1]);
+            else p[0] = w[0];
+        }
+    }
+    // tail (n % VEC elements), handled by block 0
+    if (blockIdx.x == 0) {
+        const int64_t e = nvec * VEC + tid;
+        if (e < n) y[e] = (uint8_t)hif8_enc(load_scalar<DT>(x, e), saturate);
+    }
+}
+
+// decode through a 256-entry table in LDS built by the block itself
+template <int DT>
+__global__ __launch_bounds__(kBlock) void hif8_decode_k(const uint8_t* x, void* y, int64_t nvec, int64_t n) {
+    constexpr int VEC = Tr<DT>::VEC;
+    __shared__ float tbl[256];
+    const int tid = threadIdx.x;
+    tbl[tid] = hif8_dec((uint32_t)tid);
+    __syncthreads();
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t gv = (int64_t)blockIdx.x * kBlock + tid; gv < nvec; gv += stride) {
+        uint32_t w[VEC / 4];
+        if constexpr (VEC == 8) {
+            const uint2 r = *reinterpret_cast<const uint2*>(x + gv * 8);
+            w[0] = r.x; w[1] = r.y;
+        } else {
+            w[0] = *reinterpret_cast<const uint32_t*>(x + gv * 4);
+        }
+        float out[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) out[j] = tbl[(w[j / 4] >> (8 * (j % 4))) & 0xFFu];
+        stg16(reinterpret_cast<char*>(y) + gv * 16, pack16<DT>(out));
+    }
+    if (blockIdx.x == 0) {
+        const int64_t e = nvec * VEC + tid;
+        if (e < n) store_scalar<DT>(y, e, tbl[x[e]]);
+    }
+}
+
+}  // namespace amct
+
+using namespace amct;
+
+extern "C" int amct_hif8_encode(const void* x, uint8_t* y, int64_t n, int dtype, int saturate, amct_stream_t stream) {
+    if (!x || !y || n < 0) return AMCT_E_BADARG;
+    if (!aligned16(x) || (reinterpret_cast<uintptr_t>(y) & 7u) != 0) return AMCT_E_ALIGN;
+    if (n == 0) return AMCT_OK;
+    constexpr int U = 4;
+    hipStream_t st = (hipStream_t)stream;
+#define AMCT_HE(DT)                                                                                              \
+    {                                                                                                            \
+        const int64_t nvec = n / Tr<DT>::VEC;                                                                    \
+        int64_t nb = (nvec + (int64_t)kBlock * U - 1) / ((int64_t)kBlock * U);                                   \
+        if (nb == 0) nb = 1;                                                                                     \
+        hipLaunchKernelGGL((hif8_encode_k<DT, U>), dim3((unsigned)nb), dim3(kBlock), 0, st, x, y, nvec, n, saturate); \
+    }
+    switch (dtype) {
+        case AMCT_F32: AMCT_HE(AMCT_F32) break;
+        case AMCT_F16: AMCT_HE(AMCT_F16) break;
+        case AMCT_BF16: AMCT_HE(AMCT_BF16) break;
+        default: return AMCT_E_BADARG;
+    }
+#undef AMCT_HE
+    return hip_status();
+}
+
+extern "C" int amct_hif8_decode(const uint8_t* x, void* y, int64_t n, int dtype, amct_stream_t stream) {
+    if (!x || !y || n < 0) return AMCT_E_BADARG;
+    if (!aligned16(y) || (reinterpret_cast<uintptr_t>(x) & 7u) != 0) return AMCT_E_ALIGN;
+    if (n == 0) return AMCT_OK;
+    hipStream_t st = (hipStream_t)stream;
+#define AMCT_HD(DT)                                                                                   \
+    {                                                                                                 \
+        const int64_t nvec = n / Tr<DT>::VEC;                                                         \
+        int64_t nb = (nvec + kBlock - 1) / kBlock;                                                    \
+        if (nb == 0) nb = 1;                                                                          \
+        if (nb > 8192) nb = 8192;                                                                     \
+        hipLaunchKernelGGL((hif8_decode_k<DT>), dim3((unsigned)nb), dim3(kBlock), 0, st, x, y, nvec, n); \
+    }
+    switch (dtype) {
+        case AMCT_F32: AMCT_HD(AMCT_F32) break;
+        case AMCT_F16: AMCT_HD(AMCT_F16) break;
+        case AMCT_BF16: AMCT_HD(AMCT_BF16) break;
+        default: return AMCT_E_BADARG;
+    }
+#undef AMCT_HD
+    return hip_status();
+}

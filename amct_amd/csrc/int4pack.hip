@@ -1,0 +1,283 @@
+// K2: int4 per-group quantise + nibble pack in one pass, and the int4 interchange layouts.
+// Reference behaviour: amct_pytorch/deploy_op/weight_npu_quant_module.py:38-66 (weight preparation),
+// amct_pytorch/utils/quant_util.py:76-93 (codes), amct_pytorch/quantize_op/utils.py:75-136 (factors).
+#include "amct_common.h"
+
+namespace amct {
+
+struct PackArgs {
+    const void* w;
+    uint8_t* packed;
+    void* scales16;
+    float* scales32;
+    uint8_t* zeros;
+    int32_t* bad;
+    const void* col;
+    int64_t nseg;
+    int seg_len;
+    int segs_per_row;
+    int scale_dtype;
+    int col_mode;
+    int symmetric;
+};
+
+// A team of T lanes owns one group; each lane holds NV 16-byte vectors; U groups in flight.
+template <int DT, int T, int NV, int U>
+__global__ __launch_bounds__(kBlock) void int4_group_pack(PackArgs a) {
+    constexpr int VEC = Tr<DT>::VEC;
+    constexpr int BYTES = Tr<DT>::BYTES;
+    constexpr int TEAMS = kBlock / T;
+    const int tid = threadIdx.x;
+    const int team = tid / T, lt = tid % T;
+    const int S = a.seg_len / VEC;
+    const bool asym = !a.symmetric;
+    const float inf = __builtin_huge_valf();
+
+    float x[U][NV][VEC];
+    int64_t seg[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        seg[u] = ((int64_t)blockIdx.x * U + u) * TEAMS + team;
+        const bool ok = seg[u] < a.nseg;
+        uint4 raw[NV];
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int v = i * T + lt;
+            raw[i] = make_uint4(0, 0, 0, 0);
+            if (ok && v < S)
+                raw[i] = ldg16(reinterpret_cast<const char*>(a.w) + (seg[u] * a.seg_len + (int64_t)v * VEC) * BYTES);
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i) unpack16<DT>(raw[i], x[u][i]);
+    }
+
+    if (a.col_mode != AMCT_COL_NONE) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t c0 = (seg[u] % a.segs_per_row) * (int64_t)a.seg_len;
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int v = i * T + lt;
+                if (seg[u] < a.nseg && v < S) {
+                    float c[VEC];
+                    unpack16<DT>(ldg16(reinterpret_cast<const char*>(a.col) + (c0 + (int64_t)v * VEC) * BYTES), c);
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j)
+                        x[u][i][j] = round_to<DT>(a.col_mode == AMCT_COL_DIV ? x[u][i][j] / c[j] : x[u][i][j] * c[j]);
+                }
+            }
+        }
+    }
+
+    float mx[U], mn[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        mx[u] = -inf;
+        mn[u] = inf;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int v = i * T + lt;
+            if (seg[u] < a.nseg && v < S) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    mx[u] = fmax_nan(mx[u], x[u][i][j]);
+                    mn[u] = fmin_nan(mn[u], x[u][i][j]);
+                }
+            }
+        }
+        team_minmax<T>(mn[u], mx[u]);
+    }
+
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const bool ok = seg[u] < a.nseg;
+        const Factors f = make_factors(mx[u], mn[u], 4, a.symmetric != 0, AMCT_SCOPE_AMCT);
+        if (ok && lt == 0) {
+            if (a.scales32) a.scales32[seg[u]] = f.s;
+            if (a.scales16) {
+                if (a.scale_dtype == AMCT_F16) reinterpret_cast<uint16_t*>(a.scales16)[seg[u]] = (uint16_t)f32_to_f16_bits(f.s);
+                else reinterpret_cast<uint16_t*>(a.scales16)[seg[u]] = (uint16_t)f32_to_bf16_bits(f.s);
+            }
+            if (a.zeros) a.zeros[seg[u]] = (uint8_t)((int)f.z + 8);
+            if (f.bad && a.bad) atomicAdd(a.bad, 1);
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int v = i * T + lt;
+            if (ok && v < S) {
+                uint32_t word = 0;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    const float q = quant_elem<DT, false>(x[u][i][j], f.s, f.z, asym, -8.f, 7.f);
+                    word |= (uint32_t)((int)q + 8) << (4 * j);
+                }
+                const int64_t b0 = (seg[u] * a.seg_len + (int64_t)v * VEC) / 2;
+                if constexpr (VEC == 8) *reinterpret_cast<uint32_t*>(a.packed + b0) = word;
+                else *reinterpret_cast<uint16_t*>(a.packed + b0) = (uint16_t)word;
+            }
+        }
+    }
+}
+
+// general kernel: one block per row, scalar loads; cols % group == 0 and cols even.
+template <int DT>
+__global__ __launch_bounds__(kBlock) void int4_group_pack_general(PackArgs a, int64_t cols) {
+    __shared__ float sm[2][kBlock / kWave];
+    const int tid = threadIdx.x;
+    const int64_t row = blockIdx.x;
+    const bool asym = !a.symmetric;
+    const float inf = __builtin_huge_valf();
+    for (int sg = 0; sg < a.segs_per_row; ++sg) {
+        const int64_t c_begin = (int64_t)sg * a.seg_len, c_end = c_begin + a.seg_len;
+        float mx = -inf, mn = inf;
+        for (int64_t c = c_begin + tid; c < c_end; c += kBlock) {
+            float x = load_scalar<DT>(a.w, row * cols + c);
+            if (a.col_mode != AMCT_COL_NONE) {
+                const float cs = load_scalar<DT>(a.col, c);
+                x = round_to<DT>(a.col_mode == AMCT_COL_DIV ? x / cs : x * cs);
+            }
+            mx = fmax_nan(mx, x);
+            mn = fmin_nan(mn, x);
+        }
+        team_minmax<kWave>(mn, mx);
+        __syncthreads();
+        if ((tid & (kWave - 1)) == 0) {
+            sm[0][tid / kWave] = mn;
+            sm[1][tid / kWave] = mx;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int wv = 0; wv < kBlock / kWave; ++wv) {
+            mn = fmin_nan(mn, sm[0][wv]);
+            mx = fmax_nan(mx, sm[1][wv]);
+        }
+        const Factors f = make_factors(mx, mn, 4, a.symmetric != 0, AMCT_SCOPE_AMCT);
+        const int64_t pi = row * a.segs_per_row + sg;
+        if (tid == 0) {
+            if (a.scales32) a.scales32[pi] = f.s;
+            if (a.scales16) {
+                if (a.scale_dtype == AMCT_F16) reinterpret_cast<uint16_t*>(a.scales16)[pi] = (uint16_t)f32_to_f16_bits(f.s);
+                else reinterpret_cast<uint16_t*>(a.scales16)[pi] = (uint16_t)f32_to_bf16_bits(f.s);
+            }
+            if (a.zeros) a.zeros[pi] = (uint8_t)((int)f.z + 8);
+            if (f.bad && a.bad) atomicAdd(a.bad, 1);
+        }
+        for (int64_t c = c_begin + 2 * tid; c < c_end; c += 2 * kBlock) {
+            uint32_t byte = 0;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                float x = load_scalar<DT>(a.w, row * cols + c + j);
+                if (a.col_mode != AMCT_COL_NONE) {
+                    const float cs = load_scalar<DT>(a.col, c + j);
+                    x = round_to<DT>(a.col_mode == AMCT_COL_DIV ? x / cs : x * cs);
+                }
+                const float q = quant_elem<DT, false>(x, f.s, f.z, asym, -8.f, 7.f);
+                byte |= (uint32_t)((int)q + 8) << (4 * j);
+            }
+            a.packed[(row * cols + c) / 2] = (uint8_t)byte;
+        }
+    }
+}
+
+template <int DT, int T, int NV, int U>
+static void launch_pack(const PackArgs& a, hipStream_t st) {
+    const int64_t per_block = (int64_t)(kBlock / T) * U;
+    const int64_t nb = (a.nseg + per_block - 1) / per_block;
+    hipLaunchKernelGGL((int4_group_pack<DT, T, NV, U>), dim3((unsigned)nb), dim3(kBlock), 0, st, a);
+}
+
+template <int DT>
+static int run_pack(const PackArgs& a, int64_t rows, int64_t cols, hipStream_t st) {
+    constexpr int VEC = Tr<DT>::VEC;
+    const int S = a.seg_len / VEC;
+    const bool vec_ok = aligned16(a.w) && (reinterpret_cast<uintptr_t>(a.packed) & 3u) == 0 &&
+                        (a.col_mode == AMCT_COL_NONE || aligned16(a.col));
+    if (vec_ok && S <= 512) {
+        if (S <= 4) launch_pack<DT, 4, 1, 4>(a, st);
+        else if (S <= 8) launch_pack<DT, 8, 1, 4>(a, st);
+        else if (S <= 16) launch_pack<DT, 16, 1, 4>(a, st);
+        else if (S <= 32) launch_pack<DT, 32, 1, 4>(a, st);
+        else if (S <= 64) launch_pack<DT, 64, 1, 4>(a, st);
+        else if (S <= 128) launch_pack<DT, 64, 2, 2>(a, st);
+        else if (S <= 256) launch_pack<DT, 64, 4, 1>(a, st);
+        else launch_pack<DT, 64, 8, 1>(a, st);
+        return hip_status();
+    }
+    if (rows > 0x7FFFFFFF) return AMCT_E_UNSUPPORTED;
+    hipLaunchKernelGGL((int4_group_pack_general<DT>), dim3((unsigned)rows), dim3(kBlock), 0, st, a, cols);
+    return hip_status();
+}
+
+// int32 [k, n] one signed int4 each -> int32 [k, n/8]
+__global__ __launch_bounds__(kBlock) void pack_words_k(const int32_t* codes, int32_t* words, int64_t nwords) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= nwords) return;
+    const int4 lo = *reinterpret_cast<const int4*>(codes + i * 8);
+    const int4 hi = *reinterpret_cast<const int4*>(codes + i * 8 + 4);
+    const uint32_t w = ((uint32_t)lo.x & 0xF) | (((uint32_t)lo.y & 0xF) << 4) | (((uint32_t)lo.z & 0xF) << 8) |
+                       (((uint32_t)lo.w & 0xF) << 12) | (((uint32_t)hi.x & 0xF) << 16) | (((uint32_t)hi.y & 0xF) << 20) |
+                       (((uint32_t)hi.z & 0xF) << 24) | (((uint32_t)hi.w & 0xF) << 28);
+    words[i] = (int32_t)w;
+}
+
+// int32 [k, n/8] (column 8i+j in nibble j, signed) -> uint8 [n, k/2] (code+8, even k low).
+// One thread per (word column i, k pair): reads two words, writes 8 bytes (strided by k/2).
+__global__ __launch_bounds__(kBlock) void words_to_nibbles_k(const int32_t* words, uint8_t* packed, int64_t k, int64_t n8) {
+    const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t kp = k / 2;
+    if (idx >= kp * n8) return;
+    const int64_t i = idx % n8, p = idx / n8;       // consecutive threads read consecutive words
+    const uint32_t w0 = (uint32_t)words[(2 * p) * n8 + i] ^ 0x88888888u;        // +8 mod 16 on every nibble
+    const uint32_t w1 = (uint32_t)words[(2 * p + 1) * n8 + i] ^ 0x88888888u;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t b = ((w0 >> (4 * j)) & 0xF) | (((w1 >> (4 * j)) & 0xF) << 4);
+        packed[(i * 8 + j) * kp + p] = (uint8_t)b;
+    }
+}
+
+}  // namespace amct
+
+using namespace amct;
+
+extern "C" int amct_quant_int4_group_pack(const void* w, uint8_t* packed, void* scales16, int scale_dtype,
+                                          float* scales32, uint8_t* zeros, int32_t* bad_count, const void* col_scale,
+                                          int col_mode, int64_t rows, int64_t cols, int group, int symmetric, int dtype,
+                                          amct_stream_t stream) {
+    if (!w || !packed || rows < 0 || cols <= 0 || group <= 0) return AMCT_E_BADARG;
+    if (scales16 && scale_dtype != AMCT_F16 && scale_dtype != AMCT_BF16) return AMCT_E_BADARG;
+    if (col_mode < 0 || col_mode > 2 || (col_mode != AMCT_COL_NONE && !col_scale)) return AMCT_E_BADARG;
+    if (cols % group != 0 || group % 32 != 0) return AMCT_E_ALIGN;
+    if (rows == 0) return AMCT_OK;
+    PackArgs a{};
+    a.w = w; a.packed = packed; a.scales16 = scales16; a.scales32 = scales32; a.zeros = zeros; a.bad = bad_count;
+    a.col = col_scale; a.col_mode = col_mode; a.seg_len = group; a.segs_per_row = (int)(cols / group);
+    a.nseg = rows * a.segs_per_row; a.scale_dtype = scale_dtype; a.symmetric = symmetric;
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case AMCT_F32: return run_pack<AMCT_F32>(a, rows, cols, st);
+        case AMCT_F16: return run_pack<AMCT_F16>(a, rows, cols, st);
+        case AMCT_BF16: return run_pack<AMCT_BF16>(a, rows, cols, st);
+        default: return AMCT_E_BADARG;
+    }
+}
+
+extern "C" int amct_pack_int4_words(const int32_t* codes, int32_t* words, int64_t k, int64_t n, amct_stream_t stream) {
+    if (!codes || !words || k < 0 || n < 0) return AMCT_E_BADARG;
+    if (n % 8 != 0 || !aligned16(codes)) return AMCT_E_ALIGN;
+    const int64_t nwords = k * (n / 8);
+    if (nwords == 0) return AMCT_OK;
+    hipLaunchKernelGGL(pack_words_k, dim3((unsigned)((nwords + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                       (hipStream_t)stream, codes, words, nwords);
+    return hip_status();
+}
+
+extern "C" int amct_words_to_nibbles_nk(const int32_t* words, uint8_t* packed, int64_t k, int64_t n, amct_stream_t stream) {
+    if (!words || !packed || k < 0 || n < 0) return AMCT_E_BADARG;
+    if (n % 8 != 0 || k % 2 != 0) return AMCT_E_ALIGN;
+    const int64_t total = (k / 2) * (n / 8);
+    if (total == 0) return AMCT_OK;
+    hipLaunchKernelGGL(words_to_nibbles_k, dim3((unsigned)((total + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                       (hipStream_t)stream, words, packed, k, n / 8);
+    return hip_status();
+}

@@ -1,0 +1,272 @@
+// K4: microscaling block-32 quantise / dequantise (FP8 E4M3 and FP4 E2M1 elements,
+// E8M0 shared exponents).  The reference has no such code; the format rules are:
+//   byte  = clamp(biased_exp(amax) - emax_elem, 0, 254)   (0xFF when the block holds a NaN)
+//   elem  = cast(x * 2^-(byte-127)), round-half-even, saturating to +-448 / +-6
+//   fp4   : two codes per byte, even column in the low nibble
+// Two element encoders are compiled: a bit-manipulation one and one using the gfx950
+// v_cvt_scalef32_pk_* instructions (pre-clamped so that the result saturates).
+#include "amct_common.h"
+
+namespace amct {
+
+typedef short v2i16 __attribute__((ext_vector_type(2)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+
+constexpr int kFmtE4M3 = 0, kFmtE2M1 = 1;
+
+// ---- software element casts -------------------------------------------------------------
+AMCT_DEV uint32_t sw_e4m3(float v) {
+    const uint32_t u = __float_as_uint(v);
+    const uint32_t sign = (u >> 24) & 0x80u;
+    uint32_t a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return sign | 0x7Fu;
+    a = min(a, 0x43E00000u);                                   // 448.0f
+    uint32_t code;
+    if (a >= 0x3C800000u) {                                    // >= 2^-6: normal
+        const uint32_t r = a + 0x7FFFFu + ((a >> 20) & 1u);
+        code = (r >> 20) - (120u << 3);
+    } else {                                                   // subnormal: units of 2^-9
+        const float f = __uint_as_float(a) + 16384.0f;
+        code = __float_as_uint(f) - 0x46800000u;
+    }
+    return sign | code;
+}
+
+AMCT_DEV uint32_t sw_e2m1(float v) {
+    const uint32_t u = __float_as_uint(v);
+    const uint32_t sign = (u >> 28) & 0x8u;
+    uint32_t a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return sign | 7u;
+    a = min(a, 0x40C00000u);                                   // 6.0f
+    uint32_t code;
+    if (a >= 0x3F800000u) {                                    // >= 1.0: normal, 1 mantissa bit
+        const uint32_t r = a + 0x1FFFFFu + ((a >> 22) & 1u);
+        code = (r >> 22) - (126u << 1);
+    } else {                                                   // units of 0.5
+        const float f = __uint_as_float(a) + 4194304.0f;       // 2^22: ulp 0.5
+        code = __float_as_uint(f) - 0x4A800000u;
+    }
+    return sign | code;
+}
+
+AMCT_DEV float sw_dec_e4m3(uint32_t c) {
+    const uint32_t a = c & 0x7Fu;
+    float f;
+    if (a == 0x7Fu) f = __uint_as_float(0x7FC00000u);
+    else if (a >= 8u) f = __uint_as_float((a << 20) + (120u << 23));
+    else f = (float)a * 0.001953125f;                          // 2^-9
+    return (c & 0x80u) ? -f : f;
+}
+
+AMCT_DEV float sw_dec_e2m1(uint32_t c) {
+    const uint32_t a = c & 7u;
+    float f;
+    if (a >= 2u) f = __uint_as_float((a << 22) + (126u << 23));
+    else f = (float)a * 0.5f;
+    return (c & 8u) ? -f : f;
+}
+
+// 2^(byte-127) as fp32; byte 0 is the denormal 2^-127, byte 255 a NaN
+AMCT_DEV float e8m0_to_f32(uint32_t byte) {
+    if (byte == 0u) return __uint_as_float(0x00400000u);
+    if (byte == 255u) return __uint_as_float(0x7FC00000u);
+    return __uint_as_float(byte << 23);
+}
+
+// ---- quantise -------------------------------------------------------------------------------
+// One 16-byte vector per lane and step; a block of 32 elements spans T = 32/VEC lanes.
+template <int DT, int FMT, bool HW, int U>
+__global__ __launch_bounds__(kBlock) void mx_quant_k(const void* x, uint8_t* el, uint8_t* e8, int64_t nvec, int scale_mode) {
+    constexpr int VEC = Tr<DT>::VEC;
+    constexpr int BYTES = Tr<DT>::BYTES;
+    constexpr int T = 32 / VEC;
+    constexpr int EMAX = (FMT == kFmtE4M3) ? 8 : 2;
+    constexpr uint32_t FMAX_MAN = (FMT == kFmtE4M3) ? 0x600000u : 0x400000u;
+    constexpr float FMAX = (FMT == kFmtE4M3) ? 448.0f : 6.0f;
+    const int tid = threadIdx.x;
+    float v[U][VEC];
+    int64_t gv[U];
+    uint4 raw[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        gv[u] = ((int64_t)blockIdx.x * U + u) * kBlock + tid;
+        raw[u] = make_uint4(0, 0, 0, 0);
+        if (gv[u] < nvec) raw[u] = ldg16(reinterpret_cast<const char*>(x) + gv[u] * 16);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        unpack16<DT>(raw[u], v[u]);
+        uint32_t amax = 0;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) amax = max(amax, __float_as_uint(v[u][j]) & 0x7FFFFFFFu);
+        amax = team_umax<T>(amax);
+        const bool has_nan = amax > 0x7F800000u;
+        int be = (int)(amax >> 23) - EMAX;
+        if (scale_mode == 1) be += ((amax & 0x7FFFFFu) > FMAX_MAN) ? 1 : 0;
+        be = has_nan ? 254 : min(max(be, 0), 254);             // a NaN block is cast at the largest scale
+        const uint32_t byte = has_nan ? 255u : (uint32_t)be;
+        // x * 2^-(be-127) as two exact power-of-two factors (a single one may not be representable)
+        const int e = be - 127;
+        const int h = e >> 1;                                  // floor(e / 2)
+        const float f1 = __uint_as_float((uint32_t)(127 - h) << 23);
+        const float f2 = __uint_as_float((uint32_t)(127 - (e - h)) << 23);
+        uint32_t codes[VEC];
+        if constexpr (HW) {
+            // hardware cast of (value / scale); pre-clamp so that overflow saturates
+            const float scale = 1.0f;
+            float t[VEC];
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                t[j] = v[u][j] * f1 * f2;
+                t[j] = __builtin_amdgcn_fmed3f(t[j], -FMAX, FMAX);     // NaN handled below
+            }
+            if constexpr (FMT == kFmtE4M3) {
+#pragma unroll
+                for (int j = 0; j < VEC; j += 4) {
+                    v2i16 o = {0, 0};
+                    o = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(o, t[j], t[j + 1], scale, false);
+                    o = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(o, t[j + 2], t[j + 3], scale, true);
+                    const uint32_t w = __builtin_bit_cast(uint32_t, o);
+                    codes[j] = w & 0xFFu; codes[j + 1] = (w >> 8) & 0xFFu; codes[j + 2] = (w >> 16) & 0xFFu; codes[j + 3] = w >> 24;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; j += 4) {
+                    uint32_t w = 0;
+                    w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, t[j], t[j + 1], scale, 0);
+                    w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, t[j + 2], t[j + 3], scale, 1);
+                    codes[j] = w & 0xFu; codes[j + 1] = (w >> 4) & 0xFu; codes[j + 2] = (w >> 8) & 0xFu; codes[j + 3] = (w >> 12) & 0xFu;
+                }
+            }
+            if (has_nan) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    const float tt = v[u][j] * f1 * f2;
+                    codes[j] = (FMT == kFmtE4M3) ? sw_e4m3(tt) : sw_e2m1(tt);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const float tt = v[u][j] * f1 * f2;
+                codes[j] = (FMT == kFmtE4M3) ? sw_e4m3(tt) : sw_e2m1(tt);
+            }
+        }
+        if (gv[u] < nvec) {
+            if constexpr (FMT == kFmtE4M3) {
+                uint32_t w[VEC / 4];
+#pragma unroll
+                for (int j = 0; j < VEC / 4; ++j)
+                    w[j] = codes[4 * j] | (codes[4 * j + 1] << 8) | (codes[4 * j + 2] << 16) | (codes[4 * j + 3] << 24);
+                uint32_t* p = reinterpret_cast<uint32_t*>(el + gv[u] * VEC);
+                if constexpr (VEC == 8) *reinterpret_cast<uint2*>(p) = make_uint2(w[0], w[1]);
+                else p[0] = w[0];
+            } else {
+                uint32_t w = 0;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) w |= codes[j] << (4 * j);
+                if constexpr (VEC == 8) *reinterpret_cast<uint32_t*>(el + gv[u] * 4) = w;
+                else *reinterpret_cast<uint16_t*>(el + gv[u] * 2) = (uint16_t)w;
+            }
+            if ((tid & (T - 1)) == 0) e8[gv[u] / T] = (uint8_t)byte;
+        }
+    }
+}
+
+// ---- dequantise -------------------------------------------------------------------------------
+// One lane produces one 16-byte output vector (VEC elements of the output dtype).
+template <int DT, int FMT>
+__global__ __launch_bounds__(kBlock) void mx_dequant_k(const uint8_t* el, const uint8_t* e8, void* y, int64_t nvec) {
+    constexpr int VEC = Tr<DT>::VEC;
+    constexpr int T = 32 / VEC;
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t gv = (int64_t)blockIdx.x * kBlock + threadIdx.x; gv < nvec; gv += stride) {
+        const uint32_t byte = e8[gv / T];
+        const float sc = e8m0_to_f32(byte);
+        float out[VEC];
+        if constexpr (FMT == kFmtE4M3) {
+            uint32_t w[VEC / 4];
+            if constexpr (VEC == 8) {
+                const uint2 r = *reinterpret_cast<const uint2*>(el + gv * 8);
+                w[0] = r.x; w[1] = r.y;
+            } else {
+                w[0] = *reinterpret_cast<const uint32_t*>(el + gv * 4);
+            }
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) out[j] = sw_dec_e4m3((w[j / 4] >> (8 * (j % 4))) & 0xFFu) * sc;
+        } else {
+            uint32_t w;
+            if constexpr (VEC == 8) w = *reinterpret_cast<const uint32_t*>(el + gv * 4);
+            else w = *reinterpret_cast<const uint16_t*>(el + gv * 2);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) out[j] = sw_dec_e2m1((w >> (4 * j)) & 0xFu) * sc;
+        }
+        stg16(reinterpret_cast<char*>(y) + gv * 16, pack16<DT>(out));
+    }
+}
+
+template <int DT, int FMT>
+static int launch_quant(const void* x, uint8_t* el, uint8_t* e8, int64_t nvec, int scale_mode, bool hw, hipStream_t st) {
+    constexpr int U = 4;
+    const int64_t nb = (nvec + (int64_t)kBlock * U - 1) / ((int64_t)kBlock * U);
+    if (hw) hipLaunchKernelGGL((mx_quant_k<DT, FMT, true, U>), dim3((unsigned)nb), dim3(kBlock), 0, st, x, el, e8, nvec, scale_mode);
+    else hipLaunchKernelGGL((mx_quant_k<DT, FMT, false, U>), dim3((unsigned)nb), dim3(kBlock), 0, st, x, el, e8, nvec, scale_mode);
+    return hip_status();
+}
+
+template <int DT, int FMT>
+static int launch_dequant(const uint8_t* el, const uint8_t* e8, void* y, int64_t nvec, hipStream_t st) {
+    int64_t nb = (nvec + kBlock - 1) / kBlock;
+    if (nb > 262144) nb = 262144;
+    hipLaunchKernelGGL((mx_dequant_k<DT, FMT>), dim3((unsigned)nb), dim3(kBlock), 0, st, el, e8, y, nvec);
+    return hip_status();
+}
+
+}  // namespace amct
+
+using namespace amct;
+
+// scale_mode: bit 0 = 0 floor / 1 round-up; bit 8 set selects the bit-manipulation element cast
+// instead of the hardware conversion instructions (both give identical codes).
+extern "C" int amct_mx_quant(const void* x, uint8_t* elems, uint8_t* e8m0, int64_t rows, int64_t cols, int fmt,
+                             int scale_mode, int dtype, amct_stream_t stream) {
+    if (!x || !elems || !e8m0 || rows < 0 || cols <= 0) return AMCT_E_BADARG;
+    if (fmt != kFmtE4M3 && fmt != kFmtE2M1) return AMCT_E_BADARG;
+    if ((scale_mode & ~0x101) != 0) return AMCT_E_BADARG;
+    if (cols % 32 != 0 || !aligned16(x) || (reinterpret_cast<uintptr_t>(elems) & 7u) != 0) return AMCT_E_ALIGN;
+    if (rows == 0) return AMCT_OK;
+    const bool hw = (scale_mode & 0x100) == 0;
+    const int mode = scale_mode & 1;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t n = rows * cols;
+#define AMCT_MXQ(DT)                                                                                   \
+    return fmt == kFmtE4M3 ? launch_quant<DT, kFmtE4M3>(x, elems, e8m0, n / Tr<DT>::VEC, mode, hw, st) \
+                           : launch_quant<DT, kFmtE2M1>(x, elems, e8m0, n / Tr<DT>::VEC, mode, hw, st);
+    switch (dtype) {
+        case AMCT_F32: AMCT_MXQ(AMCT_F32)
+        case AMCT_F16: AMCT_MXQ(AMCT_F16)
+        case AMCT_BF16: AMCT_MXQ(AMCT_BF16)
+        default: return AMCT_E_BADARG;
+    }
+#undef AMCT_MXQ
+}
+
+extern "C" int amct_mx_dequant(const uint8_t* elems, const uint8_t* e8m0, void* y, int64_t rows, int64_t cols, int fmt,
+                               int dtype, amct_stream_t stream) {
+    if (!elems || !e8m0 || !y || rows < 0 || cols <= 0) return AMCT_E_BADARG;
+    if (fmt != kFmtE4M3 && fmt != kFmtE2M1) return AMCT_E_BADARG;
+    if (cols % 32 != 0 || !aligned16(y) || (reinterpret_cast<uintptr_t>(elems) & 7u) != 0) return AMCT_E_ALIGN;
+    if (rows == 0) return AMCT_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t n = rows * cols;
+#define AMCT_MXD(DT)                                                                           \
+    return fmt == kFmtE4M3 ? launch_dequant<DT, kFmtE4M3>(elems, e8m0, y, n / Tr<DT>::VEC, st) \
+                           : launch_dequant<DT, kFmtE2M1>(elems, e8m0, y, n / Tr<DT>::VEC, st);
+    switch (dtype) {
+        case AMCT_F32: AMCT_MXD(AMCT_F32)
+        case AMCT_F16: AMCT_MXD(AMCT_F16)
+        case AMCT_BF16: AMCT_MXD(AMCT_BF16)
+        default: return AMCT_E_BADARG;
+    }
+#undef AMCT_MXD
+}

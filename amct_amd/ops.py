@@ -1,0 +1,340 @@
+"""Tensor-level wrappers around the C ABI: allocate outputs with torch, pass raw
+device pointers and the current HIP stream, raise on error codes.  All
+arithmetic happens in the HIP kernels; torch is used for memory only.
+"""
+import torch
+
+from . import _lib
+from ._lib import (BF16, CODES_I8, CODES_I32, CODES_NONE, COL_DIV, COL_MUL, COL_MUL_THEN_DIV, COL_NONE, F16, F32,
+                   MX_E2M1, MX_E4M3, MX_FLOOR, MX_RCEIL, SCOPE_ABSMAX, SCOPE_AMCT, STAGE_DEQUANT, STAGE_FULL,
+                   STAGE_SCALE)
+
+_DT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
+
+
+def dtype_code(dt):
+    try:
+        return _DT[dt]
+    except KeyError:
+        raise RuntimeError(
+            "dtype {} not support now, only support float32/float16/bfloat16.".format(dt)) from None
+
+
+def _dev(*tensors):
+    """All tensors must live on one HIP device; there is no CPU path."""
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError("amct_amd kernels run on the GPU only: got a tensor on '{}'".format(t.device))
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError("amct_amd: tensors on different devices ({} vs {})".format(dev, t.device))
+    return dev
+
+
+def _p(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(dev):
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _c(t):
+    return t if t.is_contiguous() else t.contiguous()
+
+
+# ---------------------------------------------------------------------------
+# A1 / A2
+# ---------------------------------------------------------------------------
+def minmax(w, group=0):
+    """w [rows, cols] -> (min, max) fp32, shape [rows] (group=0) or [rows, ceil(cols/group)]."""
+    dev = _dev(w)
+    w = _c(w)
+    rows, cols = w.shape
+    n = rows if group == 0 else rows * ((cols + group - 1) // group)
+    mn = torch.empty(n, dtype=torch.float32, device=dev)
+    mx = torch.empty(n, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().amct_minmax(_p(w), _p(mn), _p(mx), rows, cols, group, dtype_code(w.dtype), _stream(dev)))
+    if group:
+        return mn.reshape(rows, -1), mx.reshape(rows, -1)
+    return mn, mx
+
+
+def scale_offset(vmax, vmin, bits, symmetric, scope_rule=SCOPE_AMCT, bad=None):
+    """Elementwise (max, min) -> (scale fp32, offset int32 | None), same shape as the inputs."""
+    dev = _dev(vmax, vmin, bad)
+    if vmax.dtype != vmin.dtype or vmax.shape != vmin.shape:
+        raise RuntimeError("max and min must share dtype and shape")
+    vmax, vmin = _c(vmax), _c(vmin)
+    scale = torch.empty(vmax.shape, dtype=torch.float32, device=dev)
+    offset = None if symmetric else torch.empty(vmax.shape, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().amct_scale_offset(_p(vmax), _p(vmin), _p(scale), _p(offset), _p(bad), vmax.numel(), bits,
+                                                 int(symmetric), scope_rule, dtype_code(vmax.dtype), _stream(dev)))
+    return scale, offset
+
+
+# ---------------------------------------------------------------------------
+# A3..A6 with given factors
+# ---------------------------------------------------------------------------
+def quant_with_params(w, scale, offset, group, qmin, qmax, want_dq=True, codes_kind=CODES_NONE, col_scale=None,
+                      col_mode=COL_NONE, via_src=False, stage=STAGE_FULL):
+    """group: >0 per group, 0 per row, -1 per tensor.  Returns (dq | None, codes | None)."""
+    dev = _dev(w, scale, offset, col_scale)
+    w = _c(w)
+    rows, cols = w.shape
+    scale = _c(scale.to(torch.float32))
+    if offset is not None:
+        offset = _c(offset.to(torch.int32))
+    dq = torch.empty_like(w) if want_dq else None
+    codes = None
+    if codes_kind == CODES_I8:
+        codes = torch.empty(w.shape, dtype=torch.int8, device=dev)
+    elif codes_kind == CODES_I32:
+        codes = torch.empty(w.shape, dtype=torch.int32, device=dev)
+    if col_scale is not None:
+        col_scale = _c(col_scale.to(w.dtype))
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().amct_quant_with_params(
+            _p(w), _p(scale), _p(offset), _p(dq), _p(codes), codes_kind, _p(col_scale), col_mode, rows, cols, group,
+            qmin, qmax, int(via_src), stage, dtype_code(w.dtype), _stream(dev)))
+    return dq, codes
+
+
+# ---------------------------------------------------------------------------
+# K1 fused
+# ---------------------------------------------------------------------------
+def fakequant_int(w, bits, symmetric, group=0, want_dq=True, codes_kind=CODES_NONE, scope_rule=SCOPE_AMCT,
+                  qmin=None, qmax=None, col_scale=None, col_mode=COL_NONE, via_src=False, bad=None):
+    """One pass over w: min/max -> factors -> quantise.  Returns (dq, codes, scale, offset);
+    scale/offset are flat [rows] (group=0) or [rows, cols/group]."""
+    dev = _dev(w, col_scale, bad)
+    w = _c(w)
+    rows, cols = w.shape
+    nseg = rows if group == 0 else rows * ((cols + group - 1) // group)
+    if qmin is None:
+        qmin = -(1 << (bits - 1))
+    if qmax is None:
+        qmax = (1 << (bits - 1)) - 1
+    scale = torch.empty(nseg, dtype=torch.float32, device=dev)
+    offset = None if symmetric else torch.empty(nseg, dtype=torch.int32, device=dev)
+    dq = torch.empty_like(w) if want_dq else None
+    codes = None
+    if codes_kind == CODES_I8:
+        codes = torch.empty(w.shape, dtype=torch.int8, device=dev)
+    elif codes_kind == CODES_I32:
+        codes = torch.empty(w.shape, dtype=torch.int32, device=dev)
+    if col_scale is not None:
+        col_scale = _c(col_scale.to(w.dtype))
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().amct_fakequant_int(
+            _p(w), _p(dq), _p(codes), codes_kind, _p(scale), _p(offset), _p(bad), _p(col_scale), col_mode, rows, cols,
+            group, bits, int(symmetric), scope_rule, qmin, qmax, int(via_src), dtype_code(w.dtype), _stream(dev)))
+    if group:
+        scale = scale.reshape(rows, -1)
+        offset = offset.reshape(rows, -1) if offset is not None else None
+    return dq, codes, scale, offset
+
+
+# ---------------------------------------------------------------------------
+# K2
+# ---------------------------------------------------------------------------
+def quant_int4_group_pack(w, group, symmetric=False, scale_dtype=torch.float16, want_scales32=False, col_scale=None,
+                          col_mode=COL_NONE, bad=None):
+    """w [N,K] -> (packed uint8 [N,K/2], scales16 [N,K/g], zeros uint8 [N,K/g], scales32 | None)."""
+    dev = _dev(w, col_scale, bad)
+    w = _c(w)
+    rows, cols = w.shape
+    if cols % group or group % 32:
+        raise ValueError("int4 group pack needs cols % group == 0 and group % 32 == 0")
+    g = cols // group
+    packed = torch.empty(rows, cols // 2, dtype=torch.uint8, device=dev)
+    s16 = torch.empty(rows, g, dtype=scale_dtype, device=dev)
+    s32 = torch.empty(rows, g, dtype=torch.float32, device=dev) if want_scales32 else None
+    zeros = torch.empty(rows, g, dtype=torch.uint8, device=dev)
+    if col_scale is not None:
+        col_scale = _c(col_scale.to(w.dtype))
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().amct_quant_int4_group_pack(
+            _p(w), _p(packed), _p(s16), dtype_code(scale_dtype), _p(s32), _p(zeros), _p(bad), _p(col_scale), col_mode,
+            rows, cols, group, int(symmetric), dtype_code(w.dtype), _stream(dev)))
+    return packed, s16, zeros, s32
+
+
+def pack_int4_words(codes_i32):
+    """int32 [k,n] (one signed int4 each) -> int32 [k,n/8]."""
+    dev = _dev(codes_i32)
+    codes_i32 = _c(codes_i32)
+    if codes_i32.dtype != torch.int32 or codes_i32.dim() != 2:
+        raise RuntimeError("int4 packing expects a 2-D int32 tensor")
+    k, n = codes_i32.shape
+    if n % 8:
+        raise RuntimeError("int4 packing needs the last dim to be a multiple of 8")
+    words = torch.empty(k, n // 8, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().amct_pack_int4_words(_p(codes_i32), _p(words), k, n, _stream(dev)))
+    return words
+
+
+def words_to_nibbles_nk(words, k, n):
+    """int32 [k,n/8] -> uint8 [n,k/2] (code+8, even k in the low nibble)."""
+    dev = _dev(words)
+    words = _c(words)
+    packed = torch.empty(n, k // 2, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().amct_words_to_nibbles_nk(_p(words), _p(packed), k, n, _stream(dev)))
+    return packed
+
+
+# ---------------------------------------------------------------------------
+# K3
+# ---------------------------------------------------------------------------
+def act_quant_per_token_int8(x, smooth=None, mode=0):
+    """x [..., K] -> (int8 same shape, scale fp32 [rows])."""
+    dev = _dev(x, smooth)
+    x = _c(x)
+    K = x.shape[-1]
+    M = x.numel() // K
+    q = torch.empty(x.shape, dtype=torch.int8, device=dev)
+    s = torch.empty(M, dtype=torch.float32, device=dev)
+    if smooth is not None:
+        smooth = _c(smooth.reshape(-1).to(x.dtype))
+        if smooth.numel() != K:
+            raise RuntimeError("smooth factor must have K elements")
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().amct_act_quant_per_token_int8(_p(x), _p(smooth), _p(q), _p(s), M, K, mode,
+                                                             dtype_code(x.dtype), _stream(dev)))
+    return q, s
+
+
+def quantize_static(x, scales, zero_points, per_token, smooth=None):
+    """q = sat_int8(rne(x * scales + zero_points)); x [..., M, K]."""
+    dev = _dev(x, scales, zero_points, smooth)
+    x = _c(x)
+    K = x.shape[-1]
+    rows = x.numel() // K
+    scales = _c(scales.reshape(-1).to(x.dtype))
+    if zero_points is not None:
+        zero_points = _c(zero_points.reshape(-1).to(x.dtype))
+    if smooth is not None:
+        smooth = _c(smooth.reshape(-1).to(x.dtype))
+    n_scales = scales.numel()
+    if per_token:
+        # one scale per row of the last-but-one dim, shared by every leading batch index
+        m = x.shape[-2]
+        if n_scales != m:
+            raise RuntimeError("per-token quantize needs one scale per token ({} vs {})".format(n_scales, m))
+        reps = rows // m
+        if reps > 1:
+            scales = scales.repeat(reps)
+            zero_points = zero_points.repeat(reps) if zero_points is not None else None
+            n_scales = rows
+    q = torch.empty(x.shape, dtype=torch.int8, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().amct_quantize(_p(x), _p(smooth), _p(scales), _p(zero_points), _p(q), rows, K, n_scales,
+                                             int(per_token), dtype_code(x.dtype), _stream(dev)))
+    return q
+
+
+# ---------------------------------------------------------------------------
+# K4 / K5
+# ---------------------------------------------------------------------------
+def mx_quant(x, fmt, scale_mode=MX_FLOOR):
+    dev = _dev(x)
+    x = _c(x)
+    cols = x.shape[-1]
+    rows = x.numel() // cols
+    if cols % 32:
+        raise ValueError("MX quantisation needs the last dim to be a multiple of 32")
+    el = torch.empty(*x.shape[:-1], cols if fmt == MX_E4M3 else cols // 2, dtype=torch.uint8, device=dev)
+    e8 = torch.empty(*x.shape[:-1], cols // 32, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().amct_mx_quant(_p(x), _p(el), _p(e8), rows, cols, fmt, scale_mode, dtype_code(x.dtype),
+                                             _stream(dev)))
+    return el, e8
+
+
+def mx_dequant(el, e8, fmt, dtype=torch.bfloat16):
+    dev = _dev(el, e8)
+    el, e8 = _c(el), _c(e8)
+    cols = e8.shape[-1] * 32
+    rows = e8.numel() // e8.shape[-1]
+    y = torch.empty(*e8.shape[:-1], cols, dtype=dtype, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().amct_mx_dequant(_p(el), _p(e8), _p(y), rows, cols, fmt, dtype_code(dtype), _stream(dev)))
+    return y
+
+
+def hif8_encode(x, saturate=False):
+    dev = _dev(x)
+    x = _c(x)
+    y = torch.empty(x.shape, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().amct_hif8_encode(_p(x), _p(y), x.numel(), dtype_code(x.dtype), int(saturate), _stream(dev)))
+    return y
+
+
+def hif8_decode(c, dtype=torch.bfloat16):
+    dev = _dev(c)
+    c = _c(c)
+    y = torch.empty(c.shape, dtype=dtype, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().amct_hif8_decode(_p(c), _p(y), c.numel(), dtype_code(dtype), _stream(dev)))
+    return y
+
+
+# ---------------------------------------------------------------------------
+# K6 / K7
+# ---------------------------------------------------------------------------
+def gemm_w8a8(xq, wq_nk, s_ch, s_tok=None, bias=None, out_dtype=torch.bfloat16, want_acc=False):
+    """xq int8 [M,K], wq_nk int8 [N,K] (K contiguous) -> out [M,N] (and int32 accumulators)."""
+    dev = _dev(xq, wq_nk, s_ch, s_tok, bias)
+    xq, wq_nk = _c(xq), _c(wq_nk)
+    M, K = xq.shape
+    N = wq_nk.shape[0]
+    if wq_nk.shape[1] != K:
+        raise RuntimeError("int8 GEMM: K mismatch ({} vs {})".format(K, wq_nk.shape[1]))
+    s_ch = _c(s_ch.reshape(-1).to(torch.float32))
+    if s_ch.numel() == 1:
+        s_ch = s_ch.expand(N).contiguous()
+    if s_tok is not None:
+        s_tok = _c(s_tok.reshape(-1).to(torch.float32))
+    kind = 0
+    if bias is not None:
+        if bias.dtype == torch.int32:
+            kind = 1
+            bias = _c(bias)
+        else:
+            kind = 2
+            bias = _c(bias.to(torch.float32))
+    out = torch.empty(M, N, dtype=out_dtype, device=dev)
+    acc = torch.empty(M, N, dtype=torch.int32, device=dev) if want_acc else None
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().amct_gemm_w8a8(_p(xq), _p(wq_nk), _p(s_tok), _p(s_ch), _p(bias), kind, _p(out), _p(acc),
+                                              M, N, K, dtype_code(out_dtype), _stream(dev)))
+    return (out, acc) if want_acc else out
+
+
+def gemm_w4a16(x, wq_packed, scales, zeros, group, smooth=None, bias=None):
+    """x [M,K] bf16; wq_packed uint8 [N,K/2]; scales [N,K/g] f16|bf16; zeros uint8 [N,K/g]."""
+    dev = _dev(x, wq_packed, scales, zeros, smooth, bias)
+    x, wq_packed, scales, zeros = _c(x), _c(wq_packed), _c(scales), _c(zeros)
+    M, K = x.shape
+    N = wq_packed.shape[0]
+    if wq_packed.shape[1] * 2 != K:
+        raise RuntimeError("int4 GEMM: K mismatch ({} vs {})".format(K, wq_packed.shape[1] * 2))
+    if smooth is not None:
+        smooth = _c(smooth.reshape(-1).to(x.dtype))
+    if bias is not None:
+        bias = _c(bias.to(torch.float32))
+    out = torch.empty(M, N, dtype=x.dtype, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().amct_gemm_w4a16(_p(x), _p(smooth), _p(wq_packed), _p(scales), dtype_code(scales.dtype),
+                                               _p(zeros), _p(bias), _p(out), M, N, K, group, dtype_code(x.dtype),
+                                               _stream(dev)))
+    return out

@@ -1,0 +1,198 @@
+/*
+ * amct_hip.h -- C ABI of libamct_hip.so: the quantize / deploy hot path of AMCT
+ * as hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its name ends in _host;
+ *   - tensors are dense and row-major; 16-byte aligned bases take the fast
+ *     kernels, anything else a slower general kernel (same results);
+ *   - the library never allocates, frees or synchronises: the caller owns all
+ *     buffers (including workspaces) and supplies the stream; every call only
+ *     enqueues work on `stream` and returns;
+ *   - return value: 0 on success, a negative AMCT_E_* code otherwise
+ *     (amct_hip_strerror gives the text); no exception crosses the boundary;
+ *   - dtype arguments use AMCT_F32 / AMCT_F16 / AMCT_BF16, numbered like the
+ *     reference's DATA_MAP (amct_pytorch/utils/data_utils.py:19-23).
+ *
+ * Paths below are relative to the reference repository root.
+ */
+#ifndef AMCT_HIP_H
+#define AMCT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* amct_stream_t;            /* a hipStream_t */
+
+enum { AMCT_F32 = 0, AMCT_F16 = 1, AMCT_BF16 = 2 };
+
+enum {
+    AMCT_OK = 0,
+    AMCT_E_BADARG = -1,                 /* null pointer, negative size, unknown enum */
+    AMCT_E_UNSUPPORTED = -2,            /* shape / combination the kernels do not cover */
+    AMCT_E_ALIGN = -3,                  /* alignment or divisibility requirement violated */
+    AMCT_E_HIP = -4                     /* the HIP runtime reported a launch error */
+};
+
+/* symmetric scope rule */
+enum {
+    AMCT_SCOPE_AMCT = 0,                /* 2^(b-1)-1, +1 where |min| > |max|; eps guard
+                                           (amct_pytorch/quantize_op/utils.py:87-92,158-176,26-51) */
+    AMCT_SCOPE_ABSMAX = 1               /* absmax / qmax, no guard
+                                           (amct_pytorch/experimental/quantization/DeepSeekV3.2/deploy.py:128-137) */
+};
+
+/* per-column pre/post scaling fused into the weight kernels */
+enum {
+    AMCT_COL_NONE = 0,
+    AMCT_COL_MUL = 1,                   /* w * c[k], rounded to w's dtype (amct_pytorch/utils/quant_util.py:96-111) */
+    AMCT_COL_DIV = 2,                   /* w / c[k], rounded to w's dtype (amct_pytorch/utils/quant_util.py:143-159) */
+    AMCT_COL_MUL_THEN_DIV = 3           /* w * c[k] before, result / c[k] after: one AWQ grid point
+                                           (amct_pytorch/algorithm/awq.py:30-49) */
+};
+
+/* which part of the quantiser amct_quant_with_params runs */
+enum {
+    AMCT_STAGE_FULL = 0,                /* quantise (+ dequantise) */
+    AMCT_STAGE_SCALE = 1,               /* dq = w/s + z, no rounding: do_quant (amct_pytorch/algorithm/awq.py:129-149) */
+    AMCT_STAGE_DEQUANT = 2              /* dq = (w - z) * s: do_dequant (amct_pytorch/algorithm/awq.py:152-170) */
+};
+
+/* kind of integer code output */
+enum { AMCT_CODES_NONE = 0, AMCT_CODES_I8 = 1, AMCT_CODES_I32 = 2 };
+
+int amct_hip_version(void);
+const char* amct_hip_strerror(int code);
+
+/* ---- A1: min / max per row (group = 0) or per group of `group` columns ----------------
+ * Replaces get_weight_min_max_by_granularity (amct_pytorch/quantize_op/utils.py:111-136)
+ * and the per-token reductions of amct_pytorch/quantize_op/minmax_module.py:96-105.
+ * w [rows, cols]; mn, mx fp32 [rows * ceil(cols/group)] ([rows] when group = 0).
+ * A ragged last group is zero-padded and the zeros take part
+ * (amct_pytorch/utils/quant_util.py:23-36).  NaN propagates as in torch.max. */
+int amct_minmax(const void* w, float* mn, float* mx, int64_t rows, int64_t cols, int group,
+                int dtype, amct_stream_t stream);
+
+/* ---- A2: (max, min) -> (scale, offset) --------------------------------------------------
+ * Replaces calculate_scale_offset (amct_pytorch/quantize_op/utils.py:75-108).
+ * mx, mn: n values of `in_dtype`; scale fp32 [n]; offset int32 [n] (ignored / may be null
+ * when symmetric).  bad_count (int32[1], may be null) is incremented once per entry whose
+ * scale, 1/scale or offset is not finite (check_scale_offset, utils.py:54-72); the caller
+ * zeroes it beforehand and decides whether to read it. */
+int amct_scale_offset(const void* mx, const void* mn, float* scale, int32_t* offset, int32_t* bad_count,
+                      int64_t n, int bits, int symmetric, int scope_rule, int in_dtype,
+                      amct_stream_t stream);
+
+/* ---- A3 / A4 / A5 / A6: quantise with given factors -------------------------------------
+ * Replaces quant_dequant_weight (amct_pytorch/utils/quant_util.py:162-188), quant_weight +
+ * convert_dtype (:56-93), NpuQuantizationLinear.quant_wts
+ * (amct_pytorch/deploy_op/npu_quantization_linear.py:72-87) and, with
+ * round_via_src_dtype = 1, AWQ's do_quant -> convert_precision -> do_dequant
+ * (amct_pytorch/algorithm/awq.py:129-170, amct_pytorch/utils/data_utils.py:48-66).
+ * w [rows, cols]; scale fp32 and offset int32 (null = symmetric) indexed
+ *   group > 0 : [rows, ceil(cols/group)]   group = 0 : [rows]   group = -1 : [1]
+ * dq (same dtype as w, may be null) = ((clamp(rne(w/s + z), qmin, qmax)) - z) * s
+ * codes (may be null) = clamp(rne(w/s + z), qmin, qmax) as int8 or int32, [rows, cols].
+ * stage = AMCT_STAGE_SCALE / AMCT_STAGE_DEQUANT run only one half (dq required, codes null). */
+int amct_quant_with_params(const void* w, const float* scale, const int32_t* offset,
+                           void* dq, void* codes, int codes_kind,
+                           const void* col_scale, int col_mode,
+                           int64_t rows, int64_t cols, int group, int qmin, int qmax,
+                           int round_via_src_dtype, int stage, int dtype, amct_stream_t stream);
+
+/* ---- K1: A1 + A2 + A3/A4 fused, one read of w --------------------------------------------
+ * group >= 0 only (per-tensor factors are composed from amct_minmax / amct_scale_offset /
+ * amct_quant_with_params).  scale fp32 / offset int32 (null when symmetric) are OUTPUTS with
+ * the indexing above.  bad_count as in amct_scale_offset. */
+int amct_fakequant_int(const void* w, void* dq, void* codes, int codes_kind,
+                       float* scale, int32_t* offset, int32_t* bad_count,
+                       const void* col_scale, int col_mode,
+                       int64_t rows, int64_t cols, int group, int bits, int symmetric,
+                       int scope_rule, int qmin, int qmax, int round_via_src_dtype,
+                       int dtype, amct_stream_t stream);
+
+/* ---- K2: int4 per-group quantise + pack ---------------------------------------------------
+ * Replaces the weight preparation of NpuWeightQuantizedLinear.__init__
+ * (amct_pytorch/deploy_op/weight_npu_quant_module.py:38-66): min/max per group, factors,
+ * codes, packing, factor narrowing -- in one pass.
+ * w [rows, cols], cols % group == 0, group % 32 == 0.
+ * packed   uint8 [rows, cols/2]: code + 8 (unsigned 0..15), even column in the low nibble
+ * scales16 [rows, cols/group] of scale_dtype (AMCT_F16 / AMCT_BF16), may be null
+ * scales32 fp32 [rows, cols/group], may be null
+ * zeros    uint8 [rows, cols/group]: offset + 8 (8 everywhere when symmetric), may be null */
+int amct_quant_int4_group_pack(const void* w, uint8_t* packed, void* scales16, int scale_dtype,
+                               float* scales32, uint8_t* zeros, int32_t* bad_count,
+                               const void* col_scale, int col_mode,
+                               int64_t rows, int64_t cols, int group, int symmetric,
+                               int dtype, amct_stream_t stream);
+
+/* ---- int4 interchange layouts ---------------------------------------------------------------
+ * amct_pack_int4_words replaces torch_npu.npu_convert_weight_to_int4pack as called at
+ * amct_pytorch/deploy_op/weight_npu_quant_module.py:54-57: int32 [k, n] holding one signed
+ * int4 each -> int32 [k, n/8], column 8*i+j in bits 4j..4j+3 of word i.
+ * amct_words_to_nibbles_nk converts that [k, n/8] form to the GEMM layout
+ * uint8 [n, k/2] (code + 8, even k in the low nibble). */
+int amct_pack_int4_words(const int32_t* codes, int32_t* words, int64_t k, int64_t n, amct_stream_t stream);
+int amct_words_to_nibbles_nk(const int32_t* words, uint8_t* packed, int64_t k, int64_t n, amct_stream_t stream);
+
+/* ---- K3: activation quantise ------------------------------------------------------------------
+ * amct_act_quant_per_token_int8: dynamic symmetric int8 per row -- the per-token statistics of
+ * amct_pytorch/quantize_op/minmax_module.py:96-110 + calculate_scale_offset evaluated on the live
+ * batch, then convert_dtype.  mode 0: AMCT 127/128 scope rule with eps guard; mode 1: absmax/127,
+ * scale 1 for an all-zero row, clamp [-128,127]
+ * (amct_pytorch/experimental/quantization/DeepSeekV3.2/cores/quantization/node.py:39-43,181-204).
+ * smooth (dtype of x, [K], may be null) multiplies x first, rounded to x's dtype
+ * (amct_pytorch/deploy_op/npu_quantization_linear.py:96-97).
+ * amct_quantize: the static operator torch_npu.npu_quantize as called at
+ * npu_quantization_linear.py:98-99 (div_mode=False): q = sat_int8(rne(x * scales + zero_points)),
+ * scales / zero_points of x's dtype; per_token = 0: n_scales in {1, K} broadcast along the last
+ * dim; per_token = 1: one per row. */
+int amct_act_quant_per_token_int8(const void* x, const void* smooth, int8_t* q, float* scale,
+                                  int64_t M, int64_t K, int mode, int dtype, amct_stream_t stream);
+int amct_quantize(const void* x, const void* smooth, const void* scales, const void* zero_points,
+                  int8_t* q, int64_t M, int64_t K, int64_t n_scales, int per_token, int dtype,
+                  amct_stream_t stream);
+
+/* ---- K4: microscaling block-32 formats (no counterpart in the reference) ------------------------
+ * fmt: 0 = FP8 E4M3 (elements uint8 [rows, cols]), 1 = FP4 E2M1 (uint8 [rows, cols/2], even
+ * column in the low nibble).  e8m0 uint8 [rows, cols/32].  scale_mode 0 = floor, 1 = round-up.
+ * cols % 32 == 0. */
+int amct_mx_quant(const void* x, uint8_t* elems, uint8_t* e8m0, int64_t rows, int64_t cols,
+                  int fmt, int scale_mode, int dtype, amct_stream_t stream);
+int amct_mx_dequant(const uint8_t* elems, const uint8_t* e8m0, void* y, int64_t rows, int64_t cols,
+                    int fmt, int dtype, amct_stream_t stream);
+
+/* ---- K5: HiFloat8 (no counterpart in the reference) ------------------------------------------------ */
+int amct_hif8_encode(const void* x, uint8_t* y, int64_t n, int dtype, int saturate, amct_stream_t stream);
+int amct_hif8_decode(const uint8_t* x, void* y, int64_t n, int dtype, amct_stream_t stream);
+
+/* ---- K6: W8A8 Linear ----------------------------------------------------------------------------------
+ * Replaces torch_npu.npu_quant_matmul as called at
+ * amct_pytorch/deploy_op/npu_quantization_linear.py:100-102.
+ * xq int8 [M, K]; wq int8 [N, K] (K contiguous: the storage behind the reference's transposed
+ * [K, N] view, :53-55); s_ch fp32 [N]; s_tok fp32 [M] or null; bias: null, int32 [N]
+ * (bias_kind 1, joins the accumulator) or fp32 [N] (bias_kind 2, added after the rescale).
+ * out [M, N] of out_dtype = fp32(acc + ibias) * s_ch[n] * s_tok[m] + fbias, rounded once.
+ * acc_out (int32 [M, N], may be null) receives the raw accumulators. */
+int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s_tok, const float* s_ch,
+                   const void* bias, int bias_kind, void* out, int32_t* acc_out,
+                   int64_t M, int64_t N, int64_t K, int out_dtype, amct_stream_t stream);
+
+/* ---- K7: W4A16 Linear -------------------------------------------------------------------------------------
+ * Replaces torch_npu.npu_weight_quant_batchmatmul as called at
+ * amct_pytorch/deploy_op/weight_npu_quant_module.py:116-117 (with the x * scale_factor of :113-114
+ * fused in).  x [M, K] bf16; smooth [K] bf16 or null; wq uint8 [N, K/2] as written by
+ * amct_quant_int4_group_pack; scales [N, K/group] of scale_dtype; zeros uint8 [N, K/group];
+ * bias fp32 [N] or null.  out [M, N] bf16 = x' @ bf16((u - zero) * scale)^T + bias, fp32 accumulate. */
+int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t* wq, const void* scales,
+                    int scale_dtype, const uint8_t* zeros, const float* bias, void* out,
+                    int64_t M, int64_t N, int64_t K, int group, int dtype, amct_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AMCT_HIP_H */

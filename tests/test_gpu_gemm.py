@@ -1,0 +1,113 @@
+"""Parity of the two quantized Linear kernels with the CPU oracle."""
+import pytest
+import torch
+
+from amct_amd import ops, workloads
+from oracle import deploy as od
+from util import assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+
+
+def w8a8_case(M, N, K, seed, per_token=True, bias=None):
+    g = torch.Generator().manual_seed(seed)
+    xq = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int8)
+    wq = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8)
+    s_ch = 1e-3 + 9e-3 * torch.rand(N, generator=g)
+    s_tok = (0.01 + torch.rand(M, generator=g)) if per_token else None
+    b = None
+    if bias == 'int':
+        b = torch.randint(-100000, 100000, (N,), generator=g, dtype=torch.int32)
+    elif bias == 'float':
+        b = torch.randn(N, generator=g)
+    return xq, wq, s_ch, s_tok, b
+
+
+def brute_int_matmul(xq, wq):
+    M, K = xq.shape
+    N = wq.shape[0]
+    out = torch.zeros(M, N, dtype=torch.int64)
+    for m in range(M):
+        for n in range(N):
+            acc = 0
+            for k in range(K):
+                acc += int(xq[m, k]) * int(wq[n, k])
+            out[m, n] = acc
+    return out
+
+
+@pytest.mark.parametrize("M,N,K", [(5, 7, 9), (16, 16, 64), (33, 17, 100), (64, 64, 64)])
+def test_w8a8_tiny_bruteforce(dev, M, N, K):
+    xq, wq, s_ch, s_tok, b = w8a8_case(M, N, K, 89, True, 'int')
+    out, acc = ops.gemm_w8a8(xq.to(dev), wq.to(dev), s_ch.to(dev), s_tok.to(dev), b.to(dev), want_acc=True)
+    want_acc = brute_int_matmul(xq, wq) + b.to(torch.int64)
+    assert torch.equal(acc.cpu().to(torch.int64), want_acc)
+    assert torch.equal(od.int8_matmul_exact(xq, wq.t()) + b.to(torch.int64), want_acc)      # pins the fp64 oracle too
+    assert_bits_equal(out, od.quant_matmul(xq, wq.t(), s_ch, s_tok, b, torch.bfloat16), "out")
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 128, 64), (256, 384, 512), (130, 200, 192), (16, 512, 4096), (1, 256, 1024),
+                                   (300, 129, 320), (2048, 256, 4096)])
+@pytest.mark.parametrize("per_token,bias", [(True, None), (True, 'float'), (False, 'int'), (False, None)])
+def test_w8a8_vs_oracle(dev, M, N, K, per_token, bias):
+    xq, wq, s_ch, s_tok, b = w8a8_case(M, N, K, 97, per_token, bias)
+    for odt in (torch.bfloat16, torch.float16, torch.float32):
+        out, acc = ops.gemm_w8a8(xq.to(dev), wq.to(dev), s_ch.to(dev), None if s_tok is None else s_tok.to(dev),
+                                 None if b is None else b.to(dev), out_dtype=odt, want_acc=True)
+        want_acc = od.int8_matmul_exact(xq, wq.t())
+        if bias == 'int':
+            want_acc = want_acc + b.to(torch.int64)
+        assert torch.equal(acc.cpu().to(torch.int64), want_acc), "accumulators"
+        want = od.quant_matmul(xq, wq.t(), s_ch, s_tok, b, odt)
+        assert_bits_equal(out, want, "out %s" % odt)
+        # tolerance anchor: fp64 epilogue, 1e-3 of the largest magnitude
+        f64 = od.quant_matmul_f64(xq, wq.t(), s_ch, s_tok, b)
+        tol = 1e-3 if odt != torch.bfloat16 else 2.0 ** -8
+        assert ((out.cpu().double() - f64).abs() <= tol * f64.abs().clamp_min(f64.abs().max() * 1e-3)).all()
+
+
+def w4a16_case(M, N, K, group, seed, sdt=torch.float16):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    codes = torch.randint(0, 16, (N, K), generator=g, dtype=torch.uint8)
+    scales = (1e-3 + 9e-3 * torch.rand(N, K // group, generator=g)).to(sdt)
+    zeros = torch.randint(0, 16, (N, K // group), generator=g, dtype=torch.uint8)
+    smooth = (0.5 + torch.rand(K, generator=g)).to(torch.bfloat16)
+    bias = torch.randn(N, generator=g)
+    return x, codes, scales, zeros, smooth, bias
+
+
+def w4a16_oracle(x, codes, scales, zeros, group, smooth, bias):
+    signed = codes.to(torch.int32) - 8
+    anti = -(zeros.to(torch.float32) - 8)
+    return od.w4a16_forward_f64(x, signed, scales, anti, group, bias, None if smooth is None else smooth.reshape(1, -1))
+
+
+@pytest.mark.parametrize("M,N,K,group", [(1, 64, 256, 128), (16, 128, 512, 128), (7, 33, 128, 32), (64, 64, 256, 64),
+                                         (130, 200, 384, 128), (256, 256, 1024, 128), (2048, 128, 4096, 128)])
+@pytest.mark.parametrize("sdt", [torch.float16, torch.bfloat16])
+def test_w4a16_vs_oracle(dev, M, N, K, group, sdt):
+    x, codes, scales, zeros, smooth, bias = w4a16_case(M, N, K, group, 101, sdt)
+    packed = workloads.pack_nibbles(codes)
+    for sm, b in ((None, None), (smooth, bias)):
+        out = ops.gemm_w4a16(x.to(dev), packed.to(dev), scales.to(dev), zeros.to(dev), group,
+                             None if sm is None else sm.to(dev), None if b is None else b.to(dev))
+        want = w4a16_oracle(x, codes, scales, zeros, group, sm, b)
+        err = (out.cpu().double() - want).abs()
+        # 1e-3 relative to the row's largest output plus one bf16 ulp of the value itself
+        tol = 1e-3 * want.abs().amax(dim=1, keepdim=True) + want.abs() * 2.0 ** -8
+        assert (err <= tol).all(), (err.max().item(), tol.min().item())
+
+
+def test_w4a16_reduces_to_plain_matmul(dev):
+    """zero = 8 (code 0 in signed terms), scale = 1: the kernel is a bf16 GEMM against integer
+    weights, checked against torch.matmul."""
+    g = torch.Generator().manual_seed(103)
+    M, N, K = 64, 96, 256
+    x = torch.randint(-4, 5, (M, K), generator=g).to(torch.bfloat16)
+    codes = torch.randint(0, 16, (N, K), generator=g, dtype=torch.uint8)
+    scales = torch.ones(N, K // 128, dtype=torch.float16)
+    zeros = torch.full((N, K // 128), 8, dtype=torch.uint8)
+    out = ops.gemm_w4a16(x.to(dev), workloads.pack_nibbles(codes).to(dev), scales.to(dev), zeros.to(dev), 128)
+    want = torch.matmul(x.float(), (codes.float() - 8).t())          # small integers: exact in fp32
+    assert_bits_equal(out, want.to(torch.bfloat16), "plain matmul")
