@@ -70,7 +70,7 @@ __global__ __launch_bounds__(kBlock) void act_quant_token(const void* x, const v
     }
     float s;
     if (mode == 0) {
-        s = make_factors(mx, mn, 8, true, AMCT_SCOPE_AMCT).s;
+        s = make_factors<AMCT_F32>(mx, mn, 8, true, AMCT_SCOPE_AMCT).s;
     } else {
         // node.py:181-204: xmax = max(|min(amin,0)|, max(amax,0)); s = xmax / 127; s = 1 where xmax == 0
         const float hi = fmax_nan(mx, 0.f), lo = fmin_nan(mn, 0.f);
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(kBlock) void act_quant_token_general(const void* x,
     }
     float s;
     if (mode == 0) {
-        s = make_factors(mx, mn, 8, true, AMCT_SCOPE_AMCT).s;
+        s = make_factors<AMCT_F32>(mx, mn, 8, true, AMCT_SCOPE_AMCT).s;
     } else {
         const float hi = fmax_nan(mx, 0.f), lo = fmin_nan(mn, 0.f);
         const float amax = fmax_nan(__builtin_fabsf(lo), hi);

@@ -26,10 +26,16 @@ AMCT_DEV uint32_t f32_to_bf16_bits(float f) {
     // v_cvt_pk_bf16_f32: round-half-even
     return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
 }
+// The empty asm statements pin the fp16 conversions as separate instructions: without them the
+// compiler folds "convert, then multiply" into v_fma_mix* with a +0 addend, which turns a -0.0
+// product into +0.0.
 AMCT_DEV float f16_bits_to_f32(uint32_t h) {
-    return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+    float f = (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+    asm("" : "+v"(f));
+    return f;
 }
 AMCT_DEV uint32_t f32_to_f16_bits(float f) {
+    asm("" : "+v"(f));
     return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
 }
 
@@ -140,14 +146,16 @@ struct Factors {
 
 AMCT_DEV bool finite_f(float f) { return (__float_as_uint(f) & 0x7F800000u) != 0x7F800000u; }
 
+template <int DT>
 AMCT_DEV Factors make_factors(float vmax, float vmin, int bits, bool symmetric, int scope_rule) {
     Factors r;
     if (symmetric) {
         const float amax = __builtin_fabsf(vmax), amin = __builtin_fabsf(vmin);
         const float qpos = (float)((1 << (bits - 1)) - 1);
         if (scope_rule == AMCT_SCOPE_ABSMAX) {
-            // deploy.py:128-137 -- torch.abs(t).max(): NaN propagates, no guard
-            r.s = fmax_nan(amax, amin) / qpos;
+            // deploy.py:128-137 -- torch.abs(t).max() / qmax: NaN propagates, no guard, and the
+            // quotient of a tensor by a Python number keeps the tensor's dtype
+            r.s = round_to<DT>(fmax_nan(amax, amin) / qpos);
             r.z = 0.f;
             r.bad = !finite_f(r.s) || !finite_f(1.0f / r.s);
             return r;
@@ -169,7 +177,8 @@ AMCT_DEV Factors make_factors(float vmax, float vmin, int bits, bool symmetric, 
     if (!symmetric) r.z = tiny ? -(float)(1 << (bits - 1)) : r.z;
     r.s = tiny ? 1.0f : r.s;
     r.bad = !finite_f(r.s) || !finite_f(1.0f / r.s) || !finite_f(r.z);
-    r.z = __builtin_rintf(r.z);
+    // round-half-even, then through int32 as the reference does: a rounded -0.0 becomes +0.0
+    r.z = (float)(int)__builtin_rintf(r.z);
     return r;
 }
 

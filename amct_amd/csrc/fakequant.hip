@@ -182,7 +182,7 @@ __global__ __launch_bounds__(kBlock) void fq_fused(FqArgs a) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const bool ok = seg[u] < a.nseg;
-        const Factors f = make_factors(mx[u], mn[u], a.bits, a.symmetric != 0, a.scope_rule);
+        const Factors f = make_factors<DT>(mx[u], mn[u], a.bits, a.symmetric != 0, a.scope_rule);
         if (ok && lt == 0) {
             a.scale[seg[u]] = f.s;
             if (a.offset) a.offset[seg[u]] = (int32_t)f.z;
@@ -306,7 +306,7 @@ __global__ __launch_bounds__(kBlock) void fq_general(FqArgs a) {
                 mn = fmin_nan(mn, sm[0][wv]);
                 mx = fmax_nan(mx, sm[1][wv]);
             }
-            const Factors f = make_factors(mx, mn, a.bits, a.symmetric != 0, a.scope_rule);
+            const Factors f = make_factors<DT>(mx, mn, a.bits, a.symmetric != 0, a.scope_rule);
             s = f.s;
             z = f.z;
             if (tid == 0) {
@@ -406,7 +406,7 @@ __global__ __launch_bounds__(kBlock) void scale_offset_k(const void* mx, const v
                                                          int32_t* bad, int64_t n, int bits, int symmetric, int scope_rule) {
     const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     if (i >= n) return;
-    const Factors f = make_factors(load_scalar<DT>(mx, i), load_scalar<DT>(mn, i), bits, symmetric != 0, scope_rule);
+    const Factors f = make_factors<DT>(load_scalar<DT>(mx, i), load_scalar<DT>(mn, i), bits, symmetric != 0, scope_rule);
     scale[i] = f.s;
     if (offset && !symmetric) offset[i] = (int32_t)f.z;
     if (f.bad && bad) atomicAdd(bad, 1);

