@@ -11,7 +11,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libamct_hip.so")
 F32, F16, BF16 = 0, 1, 2
 SCOPE_AMCT, SCOPE_ABSMAX = 0, 1
 COL_NONE, COL_MUL, COL_DIV, COL_MUL_THEN_DIV = 0, 1, 2, 3
-STAGE_FULL, STAGE_SCALE, STAGE_DEQUANT = 0, 1, 2
+STAGE_FULL, STAGE_SCALE, STAGE_DEQUANT, STAGE_COL = 0, 1, 2, 3
 CODES_NONE, CODES_I8, CODES_I32 = 0, 1, 2
 MX_E4M3, MX_E2M1 = 0, 1
 MX_FLOOR, MX_RCEIL = 0, 1
@@ -31,6 +31,8 @@ SIGNATURES = {
     "amct_quant_int4_group_pack": (_I, [_P, _P, _P, _I, _P, _P, _P, _P, _I, _L, _L, _I, _I, _I, _P]),
     "amct_pack_int4_words": (_I, [_P, _P, _L, _L, _P]),
     "amct_words_to_nibbles_nk": (_I, [_P, _P, _L, _L, _P]),
+    "amct_pack_nibbles_nk": (_I, [_P, _P, _L, _L, _P]),
+    "amct_nibbles_nk_to_codes_kn": (_I, [_P, _P, _L, _L, _P]),
     "amct_act_quant_per_token_int8": (_I, [_P, _P, _P, _P, _L, _L, _I, _I, _P]),
     "amct_quantize": (_I, [_P, _P, _P, _P, _P, _L, _L, _L, _I, _I, _P]),
     "amct_mx_quant": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _P]),

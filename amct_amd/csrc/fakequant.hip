@@ -50,6 +50,7 @@ template <int DT> AMCT_DEV void apply_col_pre(float* x, const float* c, int mode
 //   FULL    : q = clamp(rne(x/s + z)); d = (q - z) * s
 //   SCALE   : d = x/s + z                      (do_quant, amct_pytorch/algorithm/awq.py:129-149)
 //   DEQUANT : d = (x - z [in x's dtype]) * s   (do_dequant, amct_pytorch/algorithm/awq.py:152-170)
+//   COL     : d = x after the column scaling   (amct_pytorch/utils/quant_util.py:96-111,143-159)
 template <int DT, bool VIA_SRC>
 AMCT_DEV void staged_elem(int stage, float x, float s, float z, bool asym, float qmin, float qmax, float& q, float& d) {
     if (stage == AMCT_STAGE_SCALE) {
@@ -61,6 +62,9 @@ AMCT_DEV void staged_elem(int stage, float x, float s, float z, bool asym, float
         const float t = asym ? round_to<DT>(x - z) : x;
         q = 0.f;
         d = t * s;
+    } else if (stage == AMCT_STAGE_COL) {
+        q = 0.f;
+        d = x;                                  // the column scaling has already been applied
     } else {
         q = quant_elem<DT, VIA_SRC>(x, s, z, asym, qmin, qmax);
         d = dequant_elem(q, s, z, asym);
@@ -552,7 +556,7 @@ extern "C" int amct_quant_with_params(const void* w, const float* scale, const i
                                       int group, int qmin, int qmax, int round_via_src_dtype, int stage, int dtype,
                                       amct_stream_t stream) {
     if (!w || !scale || rows < 0 || cols <= 0 || group < -1 || qmin > qmax) return AMCT_E_BADARG;
-    if (stage < AMCT_STAGE_FULL || stage > AMCT_STAGE_DEQUANT) return AMCT_E_BADARG;
+    if (stage < AMCT_STAGE_FULL || stage > AMCT_STAGE_COL) return AMCT_E_BADARG;
     if (stage != AMCT_STAGE_FULL && (codes || !dq)) return AMCT_E_BADARG;
     if (codes && codes_kind != AMCT_CODES_I8 && codes_kind != AMCT_CODES_I32) return AMCT_E_BADARG;
     if (col_mode < 0 || col_mode > 3 || (col_mode != AMCT_COL_NONE && !col_scale)) return AMCT_E_BADARG;

@@ -236,6 +236,24 @@ __global__ __launch_bounds__(kBlock) void words_to_nibbles_k(const int32_t* word
     }
 }
 
+// int8 codes [rows, cols] (signed int4 values) -> uint8 [rows, cols/2] (code+8, even column low)
+__global__ __launch_bounds__(kBlock) void pack_nibbles_k(const int8_t* codes, uint8_t* packed, int64_t nbytes) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= nbytes) return;
+    const uint32_t lo = ((uint32_t)codes[2 * i] + 8u) & 0xFu, hi = ((uint32_t)codes[2 * i + 1] + 8u) & 0xFu;
+    packed[i] = (uint8_t)(lo | (hi << 4));
+}
+
+// uint8 [n, k/2] -> int32 [k, n] signed codes (the operand of the word packer)
+__global__ __launch_bounds__(kBlock) void nibbles_to_codes_kn_k(const uint8_t* packed, int32_t* codes, int64_t k, int64_t n) {
+    const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (idx >= k * n) return;
+    const int64_t col = idx % n, row = idx / n;          // consecutive threads write consecutive n
+    const uint32_t b = packed[col * (k / 2) + row / 2];
+    const int32_t u = (row & 1) ? (int32_t)(b >> 4) : (int32_t)(b & 0xFu);
+    codes[idx] = u - 8;
+}
+
 }  // namespace amct
 
 using namespace amct;
@@ -279,5 +297,24 @@ extern "C" int amct_words_to_nibbles_nk(const int32_t* words, uint8_t* packed, i
     if (total == 0) return AMCT_OK;
     hipLaunchKernelGGL(words_to_nibbles_k, dim3((unsigned)((total + kBlock - 1) / kBlock)), dim3(kBlock), 0,
                        (hipStream_t)stream, words, packed, k, n / 8);
+    return hip_status();
+}
+
+extern "C" int amct_pack_nibbles_nk(const int8_t* codes, uint8_t* packed, int64_t rows, int64_t cols, amct_stream_t stream) {
+    if (!codes || !packed || rows < 0 || cols < 0) return AMCT_E_BADARG;
+    if (cols % 2 != 0) return AMCT_E_ALIGN;
+    const int64_t nbytes = rows * (cols / 2);
+    if (nbytes == 0) return AMCT_OK;
+    hipLaunchKernelGGL(pack_nibbles_k, dim3((unsigned)((nbytes + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                       (hipStream_t)stream, codes, packed, nbytes);
+    return hip_status();
+}
+
+extern "C" int amct_nibbles_nk_to_codes_kn(const uint8_t* packed, int32_t* codes, int64_t k, int64_t n, amct_stream_t stream) {
+    if (!packed || !codes || k < 0 || n < 0) return AMCT_E_BADARG;
+    if (k % 2 != 0) return AMCT_E_ALIGN;
+    if (k * n == 0) return AMCT_OK;
+    hipLaunchKernelGGL(nibbles_to_codes_kn_k, dim3((unsigned)((k * n + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                       (hipStream_t)stream, packed, codes, k, n);
     return hip_status();
 }

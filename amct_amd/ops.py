@@ -6,8 +6,8 @@ import torch
 
 from . import _lib
 from ._lib import (BF16, CODES_I8, CODES_I32, CODES_NONE, COL_DIV, COL_MUL, COL_MUL_THEN_DIV, COL_NONE, F16, F32,
-                   MX_E2M1, MX_E4M3, MX_FLOOR, MX_RCEIL, SCOPE_ABSMAX, SCOPE_AMCT, STAGE_DEQUANT, STAGE_FULL,
-                   STAGE_SCALE)
+                   MX_E2M1, MX_E4M3, MX_FLOOR, MX_RCEIL, SCOPE_ABSMAX, SCOPE_AMCT, STAGE_COL, STAGE_DEQUANT,
+                   STAGE_FULL, STAGE_SCALE)
 
 _DT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 
@@ -106,6 +106,15 @@ def quant_with_params(w, scale, offset, group, qmin, qmax, want_dq=True, codes_k
     return dq, codes
 
 
+def col_scale(w, c, divide):
+    """w * c[k] (or w / c[k]) rounded to w's dtype; c is [1,K] or [K]."""
+    dev = _dev(w, c)
+    one = torch.ones(1, dtype=torch.float32, device=dev)
+    out, _ = quant_with_params(w, one, None, -1, -128, 127, col_scale=c.reshape(-1),
+                               col_mode=COL_DIV if divide else COL_MUL, stage=STAGE_COL)
+    return out
+
+
 # ---------------------------------------------------------------------------
 # K1 fused
 # ---------------------------------------------------------------------------
@@ -189,6 +198,38 @@ def words_to_nibbles_nk(words, k, n):
     with torch.cuda.device(dev):
         _lib.check(_lib.load().amct_words_to_nibbles_nk(_p(words), _p(packed), k, n, _stream(dev)))
     return packed
+
+
+def pack_nibbles_nk(codes_i8):
+    """int8 [N,K] signed int4 codes -> uint8 [N,K/2] (code+8, even k in the low nibble)."""
+    dev = _dev(codes_i8)
+    codes_i8 = _c(codes_i8)
+    if codes_i8.dtype != torch.int8 or codes_i8.shape[1] % 2:
+        raise RuntimeError("nibble packing expects int8 codes with an even number of columns")
+    n, k = codes_i8.shape
+    packed = torch.empty(n, k // 2, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().amct_pack_nibbles_nk(_p(codes_i8), _p(packed), n, k, _stream(dev)))
+    return packed
+
+
+def unpack_nibbles_to_i32_kn(packed):
+    """uint8 [N,K/2] -> int32 [K,N] signed codes."""
+    dev = _dev(packed)
+    packed = _c(packed)
+    n, k = packed.shape[0], packed.shape[1] * 2
+    codes = torch.empty(k, n, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().amct_nibbles_nk_to_codes_kn(_p(packed), _p(codes), k, n, _stream(dev)))
+    return codes
+
+
+def bias_to_int32(bias, scale):
+    """round_half_even(bias / scale) as int32 (amct_pytorch/deploy_op/npu_quantization_linear.py:117-120)."""
+    scale = scale.reshape(-1)
+    _, codes = quant_with_params(bias.reshape(-1, 1), scale, None, 0 if scale.numel() > 1 else -1,
+                                 -2147483648, 2147483647, want_dq=False, codes_kind=CODES_I32)
+    return codes.reshape(-1)
 
 
 # ---------------------------------------------------------------------------

@@ -59,7 +59,8 @@ enum {
 enum {
     AMCT_STAGE_FULL = 0,                /* quantise (+ dequantise) */
     AMCT_STAGE_SCALE = 1,               /* dq = w/s + z, no rounding: do_quant (amct_pytorch/algorithm/awq.py:129-149) */
-    AMCT_STAGE_DEQUANT = 2              /* dq = (w - z) * s: do_dequant (amct_pytorch/algorithm/awq.py:152-170) */
+    AMCT_STAGE_DEQUANT = 2,             /* dq = (w - z) * s: do_dequant (amct_pytorch/algorithm/awq.py:152-170) */
+    AMCT_STAGE_COL = 3                  /* dq = w * c[k] or w / c[k] only (amct_pytorch/utils/quant_util.py:96-111,143-159) */
 };
 
 /* kind of integer code output */
@@ -97,7 +98,8 @@ int amct_scale_offset(const void* mx, const void* mn, float* scale, int32_t* off
  *   group > 0 : [rows, ceil(cols/group)]   group = 0 : [rows]   group = -1 : [1]
  * dq (same dtype as w, may be null) = ((clamp(rne(w/s + z), qmin, qmax)) - z) * s
  * codes (may be null) = clamp(rne(w/s + z), qmin, qmax) as int8 or int32, [rows, cols].
- * stage = AMCT_STAGE_SCALE / AMCT_STAGE_DEQUANT run only one half (dq required, codes null). */
+ * stage = AMCT_STAGE_SCALE / AMCT_STAGE_DEQUANT / AMCT_STAGE_COL run only one part (dq required,
+ * codes null). */
 int amct_quant_with_params(const void* w, const float* scale, const int32_t* offset,
                            void* dq, void* codes, int codes_kind,
                            const void* col_scale, int col_mode,
@@ -138,6 +140,12 @@ int amct_quant_int4_group_pack(const void* w, uint8_t* packed, void* scales16, i
  * uint8 [n, k/2] (code + 8, even k in the low nibble). */
 int amct_pack_int4_words(const int32_t* codes, int32_t* words, int64_t k, int64_t n, amct_stream_t stream);
 int amct_words_to_nibbles_nk(const int32_t* words, uint8_t* packed, int64_t k, int64_t n, amct_stream_t stream);
+/* amct_pack_nibbles_nk: int8 codes [rows, cols] (signed int4 values, as convert_dtype of
+ * amct_pytorch/utils/quant_util.py:56-73 yields them) -> uint8 [rows, cols/2] in the GEMM layout.
+ * amct_nibbles_nk_to_codes_kn: the way back to the reference's operand, int32 [k, n] signed codes
+ * (amct_pytorch/deploy_op/weight_npu_quant_module.py:52-53). */
+int amct_pack_nibbles_nk(const int8_t* codes, uint8_t* packed, int64_t rows, int64_t cols, amct_stream_t stream);
+int amct_nibbles_nk_to_codes_kn(const uint8_t* packed, int32_t* codes, int64_t k, int64_t n, amct_stream_t stream);
 
 /* ---- K3: activation quantise ------------------------------------------------------------------
  * amct_act_quant_per_token_int8: dynamic symmetric int8 per row -- the per-token statistics of

@@ -112,7 +112,9 @@ def quant_matmul(xq, wq_kn, scale, pertoken_scale=None, bias=None, output_dtype=
     f = acc.to(torch.int32).to(torch.float32)
     f = f * scale.reshape(1, -1).float()
     if pertoken_scale is not None:
-        f = f * pertoken_scale.reshape(-1, 1).float()
+        ps = pertoken_scale.reshape(-1).float()
+        ps = ps.repeat(f.shape[0] // ps.numel())          # one scale per token, shared by leading batch dims
+        f = f * ps.reshape(-1, 1)
     if fbias is not None:
         f = f + fbias
     return f.to(output_dtype).reshape(*xq.shape[:-1], -1)

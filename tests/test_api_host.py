@@ -1,0 +1,57 @@
+"""Host-side behaviour of the reference-shaped API that needs no GPU: argument checks raise the
+reference's exception types and messages before any kernel is launched."""
+import pytest
+import torch
+
+from amct_amd.quantize_op import utils as qutils
+from amct_amd.utils import data_utils, quant_util
+
+
+def test_shape_checks_and_messages():
+    w = torch.zeros(8, 64)
+    with pytest.raises(RuntimeError, match=r"smooth_factor shape should be \[1, 64\] current shape is \[64\]"):
+        quant_util.apply_smooth_weight(torch.ones(64), w)
+    with pytest.raises(RuntimeError, match=r"AWQ params scale.shape should be \[1, 64\] current shape is \[1, 32\]"):
+        quant_util.apply_awq_quantize_weight(w, torch.ones(1, 32), 32)
+    with pytest.raises(ValueError, match="Not supported quant_dtype int2"):
+        quant_util.convert_dtype(w, 'int2')
+    with pytest.raises(ValueError, match="Not supported quant_dtype int16"):
+        quant_util.quant_weight(w, 'int16', torch.ones(8, 1))
+    with pytest.raises(RuntimeError, match="Linear quant only support dim from 2 to 6"):
+        data_utils.check_linear_input_dim(torch.zeros(4))
+    with pytest.raises(RuntimeError, match="Linear quant only support dim from 2 to 6"):
+        data_utils.check_linear_input_dim(torch.zeros(1, 1, 1, 1, 1, 1, 4))
+    data_utils.check_linear_input_dim(torch.zeros(2, 3, 4))
+    with pytest.raises(RuntimeError, match="only support float32/float16/bfloat16"):
+        data_utils.convert_precision(torch.zeros(4, 4, dtype=torch.float64), 'int8')
+
+
+def test_check_scale_offset_shape():
+    w = torch.zeros(8, 70)
+    quant_util.check_scale_offset_shape(w, torch.ones(1))
+    quant_util.check_scale_offset_shape(w, torch.ones(8, 1))
+    with pytest.raises(RuntimeError, match="scale.shape should be equal to 1 or cout. current is 3"):
+        quant_util.check_scale_offset_shape(w, torch.ones(3, 1))
+    quant_util.check_scale_offset_shape(w, torch.ones(8, 3, 1), torch.ones(8, 3, 1), 32)
+    with pytest.raises(RuntimeError, match="scale.shape should be"):
+        quant_util.check_scale_offset_shape(w, torch.ones(8, 2, 1), None, 32)
+    with pytest.raises(RuntimeError, match="offset_w.shape should be equal to scale_w.shape"):
+        quant_util.check_scale_offset_shape(w, torch.ones(8, 3, 1), torch.ones(8, 3), 32)
+
+
+def test_layout_helpers_match_oracle():
+    from oracle import int_quant as iq
+    w = torch.arange(3 * 40, dtype=torch.float32).reshape(3, 40)
+    g = quant_util.convert_to_per_group_shape(w, 32)
+    assert torch.equal(g, iq.group_view(w, 32)) and g.shape == (3, 2, 32)
+    assert torch.equal(qutils.convert_to_dst_shape(g, w.shape), w)
+    assert quant_util.pad_zero_by_group(w, 32).shape == (3, 64)
+    assert qutils.get_int_quant_scope('int8', False) == 255
+    assert qutils.get_int_quant_scope('int4', True, torch.tensor([True, False])).tolist() == [8, 7]
+
+
+def test_check_scale_offset_messages():
+    with pytest.raises(RuntimeError, match="Param scale has invalid value inf, nan or zeros!"):
+        qutils.check_scale_offset(torch.tensor([0.0]), None)
+    with pytest.raises(RuntimeError, match="Param offset has invalid value inf or nan!"):
+        qutils.check_scale_offset(torch.tensor([1.0]), torch.tensor([float('inf')]))

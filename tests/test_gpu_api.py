@@ -1,0 +1,241 @@
+"""The reference-shaped Python API (function, module and operator level) on the GPU against the
+oracle's restatement of the reference."""
+import types
+
+import pytest
+import torch
+
+from amct_amd import torch_hip
+from amct_amd.algorithm import awq
+from amct_amd.deploy_op import HipQuantizationLinear, HipWeightQuantizedLinear
+from amct_amd.quantize_op import utils as qutils
+from amct_amd.utils import data_utils, quant_util
+from oracle import deploy as od
+from oracle import int_quant as iq
+from util import assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+
+
+def cfg(kind, sym, strategy, group=None):
+    w = {'quant_type': kind, 'symmetric': sym, 'strategy': strategy}
+    if group:
+        w['group_size'] = group
+    return {'weights_cfg': w}
+
+
+@pytest.mark.parametrize("kind", ['int8', 'int4'])
+@pytest.mark.parametrize("sym", [True, False])
+@pytest.mark.parametrize("strategy,group", [('tensor', None), ('channel', None), ('group', 32)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_weight_only_matrix(dev, kind, sym, strategy, group, dtype):
+    """The reference's weight-only test matrix (tests/amct_pytorch/test_minmax.py:56-381):
+    {int8,int4} x {tensor,channel,group32} x {sym,asym}, here with numeric checks."""
+    torch.manual_seed(0)
+    w = torch.randn(64, 80 if strategy == 'group' else 64).to(dtype)
+    c = cfg(kind, sym, strategy, group)
+    wd = w.to(dev)
+    mn, mx = qutils.get_weight_min_max_by_granularity(wd, c)
+    omn, omx = iq.weight_min_max(w, strategy, group)
+    assert mn.shape == omn.shape and mn.dtype == w.dtype
+    assert torch.equal(mn.cpu(), omn) and torch.equal(mx.cpu(), omx)
+    s, z = qutils.calculate_scale_offset(mx, mn, sym, kind)
+    os_, oz = iq.scale_offset(omx, omn, sym, kind)
+    assert s.shape == os_.shape and s.dtype == torch.float32
+    assert_bits_equal(s, os_, "scale")
+    assert (z is None) == sym                      # offset_w is None iff symmetric
+    if not sym:
+        assert z.dtype == torch.int32
+        assert_bits_equal(z, oz, "offset")
+    dq = quant_util.quant_dequant_weight(wd, c, s, z)
+    assert_bits_equal(dq, iq.fake_quant(w, kind, os_, oz, group), "quant_dequant_weight")
+    codes = quant_util.quant_weight(wd, kind, s, z, group)
+    oc = iq.quant_codes(w, kind, os_, oz, group)
+    assert codes.dtype == (torch.int8 if kind == 'int8' else torch.int32)      # test_quantize.py:84,101
+    assert_bits_equal(codes, oc, "quant_weight")
+
+
+def test_calculate_scale_offset_raises(dev):
+    with pytest.raises(RuntimeError, match="Param scale has invalid value inf, nan or zeros!"):
+        qutils.calculate_scale_offset(torch.tensor([[float('inf')]], device=dev), torch.tensor([[0.0]], device=dev), True, 'int8')
+
+
+def test_convert_helpers(dev):
+    t = (torch.randn(7, 33) * 100).to(torch.bfloat16)
+    assert_bits_equal(quant_util.convert_dtype(t.to(dev), 'int8'), iq.to_codes(t, 'int8'), "convert_dtype int8")
+    assert_bits_equal(quant_util.convert_dtype(t.to(dev), 'int4'), iq.to_codes(t, 'int4'), "convert_dtype int4")
+    want = torch.clamp(torch.round(t), -8, 7)
+    assert_bits_equal(data_utils.convert_precision(t.to(dev), 'int4'), want, "convert_precision")
+    cs = (0.5 + torch.rand(1, 33)).to(torch.bfloat16)
+    assert_bits_equal(quant_util.apply_smooth_weight(cs.to(dev), t.to(dev)), iq.smooth_weight(cs, t), "smooth")
+    assert_bits_equal(quant_util.apply_awq_quantize_weight(t.to(dev), cs.to(dev), 32), iq.awq_weight(t, cs), "awq div")
+
+
+def test_gptq_column_calls(dev):
+    """The call pattern of amct_pytorch/quantize_op/gptq_module.py:136-148: one [N,1] column at a time."""
+    torch.manual_seed(1)
+    w = torch.randn(48, 96)
+    for strategy, group in (('channel', None), ('group', 32), ('tensor', None)):
+        c = cfg('int4', False, strategy, group)
+        s, z = iq.weight_scale_offset(w, strategy, False, 'int4', group)
+        for col in (0, 37, 95):
+            x = w[:, col].reshape(-1, 1)
+            if group:
+                sc, zc = s[:, col // group], z[:, col // group]          # [N,1]
+                sc, zc = sc.unsqueeze(-1), zc.unsqueeze(-1)
+                sc, zc = s[:, col // group].unsqueeze(-1), z[:, col // group].unsqueeze(-1)
+            else:
+                sc, zc = s, z
+            want = iq.fake_quant(x, 'int4', sc, zc, group)
+            got = quant_util.quant_dequant_weight(x.to(dev), c, sc.to(dev), zc.to(dev))
+            assert_bits_equal(got, want, "%s col %d" % (strategy, col))
+
+
+@pytest.mark.parametrize("strategy,group,sym", [('group', 32, False), ('channel', None, True), ('tensor', None, False),
+                                                ('group', 48, False)])
+def test_awq_process_weights(dev, strategy, group, sym):
+    torch.manual_seed(2)
+    c = cfg('int4', sym, strategy, group)
+    layers = [torch.nn.Linear(96, 40, bias=False).to(torch.bfloat16) for _ in range(2)]
+    scale_awq = (0.5 + torch.rand(1, 96)).to(torch.bfloat16)
+    want = [iq.awq_grid_step(l.weight.data, scale_awq, 'int4', strategy, sym, group)[0] for l in layers]
+    dl = [torch.nn.Linear(96, 40, bias=False).to(torch.bfloat16).to(dev) for _ in range(2)]
+    for a, b in zip(dl, layers):
+        a.weight.data.copy_(b.weight.data)
+    awq.process_weights_for_layers(dl, scale_awq.to(dev), c)
+    for a, w_ in zip(dl, want):
+        assert_bits_equal(a.weight.data, w_, "awq grid step %s" % strategy)
+    # the staged functions on their own
+    w = layers[0].weight.data
+    s, z = iq.weight_scale_offset(w, strategy, sym, 'int4', group)
+    if group is None or 96 % group == 0:
+        t = iq.group_view(w, group) / s if group else w / s
+        if z is not None:
+            t = t + z
+        want_q = iq.ungroup(t, w.shape).to(w.dtype)
+        got = awq.do_quant(w.to(dev), s.to(dev), None if z is None else z.to(dev), strategy, group)
+        assert_bits_equal(got, want_q, "do_quant")
+
+
+def quant_module(weight, bias, **kw):
+    m = types.SimpleNamespace(weight=torch.nn.Parameter(weight, requires_grad=False), bias=bias, act_type='int8',
+                              wts_type='int8', scale_w=None, offset_w=None, scale_d=None, offset_d=None, scale=None,
+                              group_size=None)
+    for k, v in kw.items():
+        setattr(m, k, v)
+    return m
+
+
+@pytest.mark.parametrize("mode", ['tensor_sym', 'tensor_asym', 'token_sym', 'tensor_sym_smooth'])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_w8a8_module(dev, mode, with_bias):
+    torch.manual_seed(3)
+    N, K, M = 96, 128, 24
+    w = (torch.randn(N, K) * 0.05).to(torch.bfloat16)
+    b = torch.randn(N).to(torch.bfloat16) if with_bias else None
+    x = torch.randn(2, M, K).to(torch.bfloat16)
+    smooth = (0.5 + torch.rand(1, K)).to(torch.bfloat16) if mode.endswith('smooth') else None
+    ws = iq.smooth_weight(smooth, w) if smooth is not None else w
+    scale_w, _ = iq.weight_scale_offset(ws, 'channel', True, 'int8')
+    xs = x / smooth if smooth is not None else x
+    if mode.startswith('tensor'):
+        sym = 'asym' not in mode
+        scale_d, offset_d = iq.scale_offset(xs.max().reshape(-1), xs.min().reshape(-1), sym, 'int8')
+    else:
+        mn, mx = iq.token_min_max(xs)
+        scale_d, offset_d = iq.scale_offset(mx, mn, True, 'int8')
+        scale_d = scale_d.reshape(M, 1)
+    buf = od.w8a8_buffers(w, b, scale_w, scale_d, offset_d, smooth)
+    want = od.w8a8_forward(buf, x)
+    qm = quant_module(w.to(dev), None if b is None else torch.nn.Parameter(b.to(dev), requires_grad=False),
+                      scale_w=scale_w.to(dev), scale_d=scale_d.to(dev),
+                      offset_d=None if offset_d is None else offset_d.to(dev),
+                      scale=None if smooth is None else smooth.to(dev))
+    mod = HipQuantizationLinear(qm)
+    assert_bits_equal(mod.quantized_weight, buf['quantized_weight'], "quantized_weight")
+    assert mod.quantized_weight.shape == (K, N) and mod.quantized_weight.dtype == torch.int8
+    assert_bits_equal(mod.act_scale, buf['act_scale'], "act_scale")
+    assert_bits_equal(mod.deq_scale, buf['deq_scale'], "deq_scale")
+    if buf['bias'] is None:
+        assert mod.bias is None
+    else:
+        assert_bits_equal(mod.bias, buf['bias'], "bias")
+    got = mod(x.to(dev))
+    assert got.shape == (2, M, N) and got.dtype == torch.bfloat16
+    assert_bits_equal(got, want, "forward")
+    keys = set(mod.state_dict().keys())
+    assert {'act_scale', 'act_offset', 'quantized_weight', 'deq_scale'} <= keys
+
+
+def test_w8a8_module_dynamic(dev):
+    torch.manual_seed(4)
+    N, K, M = 64, 256, 40
+    w = (torch.randn(N, K) * 0.05).to(torch.bfloat16)
+    x = torch.randn(M, K).to(torch.bfloat16)
+    scale_w, _ = iq.weight_scale_offset(w, 'channel', True, 'int8')
+    qm = quant_module(w.to(dev), None, scale_w=scale_w.to(dev), scale_d=torch.ones(1, device=dev))
+    mod = HipQuantizationLinear(qm, dynamic_act=True)
+    got = mod(x.to(dev))
+    xq, s_tok = iq.dynamic_token_quant(x)
+    wq = iq.to_codes(w / scale_w, 'int8')
+    want = od.quant_matmul(xq, wq.t(), scale_w.reshape(-1), s_tok, None, torch.bfloat16)
+    assert_bits_equal(got, want, "dynamic forward")
+
+
+@pytest.mark.parametrize("group,sym,with_awq", [(32, False, True), (128, False, False), (None, True, False), (64, True, True)])
+def test_w4a16_module(dev, group, sym, with_awq):
+    torch.manual_seed(5)
+    N, K, M = 64, 256, 9
+    w = (torch.randn(N, K) * 0.05).to(torch.bfloat16)
+    b = torch.randn(N).to(torch.bfloat16)
+    x = torch.randn(3, M, K).to(torch.bfloat16)
+    awq_scale = (0.5 + torch.rand(1, K)).to(torch.bfloat16) if with_awq else None
+    wa = iq.awq_weight(w, awq_scale) if with_awq else w
+    strategy = 'group' if group else 'channel'
+    scale_w, offset_w = iq.weight_scale_offset(wa, strategy, sym, 'int4', group)
+    buf = od.w4a16_buffers(w, b, scale_w, offset_w, 'int4', group, awq_scale)
+    qm = quant_module(w.to(dev), torch.nn.Parameter(b.to(dev), requires_grad=False), wts_type='int4',
+                      scale_w=scale_w.to(dev), offset_w=None if offset_w is None else offset_w.to(dev),
+                      scale=None if awq_scale is None else awq_scale.to(dev), group_size=group)
+    mod = HipWeightQuantizedLinear(qm)
+    # codes and factors agree with the reference's buffers after conversion to its layout
+    words, sw, ow = mod.reference_layout()
+    assert_bits_equal(words, buf['quantized_weight'], "int4 words [K,N/8]")
+    assert words.dtype == torch.int32 and words.shape == (K, N // 8)
+    assert_bits_equal(sw, buf['scale_w'], "scale_w [K/g,N]")
+    if buf['offset_w'] is not None:
+        assert_bits_equal(ow, buf['offset_w'], "offset_w [K/g,N]")
+    assert mod.bias.dtype == torch.float32
+    got = mod(x.to(dev))
+    g = group or K
+    want = od.w4a16_forward_f64(x, buf['codes_nk'].reshape(N, K), buf['scale_w'].t(),
+                                None if buf['offset_w'] is None else buf['offset_w'].t().float(), g, buf['bias'],
+                                awq_scale)
+    assert got.shape == (3, M, N)
+    err = (got.cpu().double() - want).abs()
+    tol = 1e-3 * want.abs().amax(dim=-1, keepdim=True) + want.abs() * 2.0 ** -8
+    assert (err <= tol).all()
+    # operator-level drop-in with the reference's operand layouts gives the same result
+    xs = x.to(dev) if awq_scale is None else torch.mul(x.to(dev), awq_scale.to(dev))
+    out2 = torch_hip.npu_weight_quant_batchmatmul(xs.reshape(-1, K), words, sw, antiquant_offset=ow if not sym else None,
+                                                  bias=mod.bias, antiquant_group_size=group or 0)
+    assert_bits_equal(out2.reshape(3, M, N), got.cpu(), "operator vs module")
+
+
+def test_operator_level_w8a8(dev):
+    torch.manual_seed(6)
+    M, K, N = 20, 192, 72
+    x = torch.randn(M, K).to(torch.bfloat16)
+    sc = torch.tensor([31.0], dtype=torch.bfloat16)
+    zp = torch.tensor([3.0], dtype=torch.bfloat16)
+    xq = torch_hip.npu_quantize(x.to(dev), sc.to(dev), zp.to(dev), dtype=torch.int8, axis=-1, div_mode=False)
+    assert_bits_equal(xq, iq.static_quantize(x, sc, zp), "npu_quantize")
+    wq = torch.randint(-128, 128, (N, K), dtype=torch.int8)
+    scale = torch.rand(N) * 0.01
+    out = torch_hip.npu_quant_matmul(xq, wq.to(dev).t(), scale=scale.to(dev), pertoken_scale=None, bias=None,
+                                     output_dtype=torch.bfloat16)
+    assert_bits_equal(out, od.quant_matmul(xq.cpu(), wq.t(), scale, None, None, torch.bfloat16), "npu_quant_matmul")
+    codes = torch.randint(-8, 8, (K, N), dtype=torch.int32)
+    words = torch_hip.npu_convert_weight_to_int4pack(codes.to(dev))
+    assert_bits_equal(words, od.pack_int4_words(codes), "int4pack")
+    assert torch_hip.npu.is_available()
