@@ -1,8 +1,19 @@
 // K6: W8A8 Linear.  out[m,n] = cast(fp32(sum_k xq[m,k]*wq[n,k] + ibias[n]) * s_ch[n] * s_tok[m] + fbias[n])
 // Reference call site: amct_pytorch/deploy_op/npu_quantization_linear.py:100-102.
+//
+// Both operands are K-contiguous, which is the natural operand order of the gfx950 int8 MFMA
+// (v_mfma_i32_32x32x32_i8: lane l supplies 16 consecutive k-bytes of row l%32, k-half l/32).
+//   tile kernel   : 128x128 block tile, 4 waves of 64x64, BK = 128 bytes, LDS double buffered,
+//                   global loads of step k+1 in flight while step k feeds the MFMAs.
+//   skinny kernel : M <= 64 (decode): the weight is streamed once straight from HBM into MFMA
+//                   operands (v_mfma_i32_16x16x64_i8), split-K across the 4 waves of a block.
+//   general kernel: any shape, one output per thread.
 #include "amct_common.h"
 
 namespace amct {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
 
 struct W8A8Args {
     const int8_t* xq;
@@ -30,8 +41,167 @@ AMCT_DEV void w8a8_epilogue(const W8A8Args& a, int64_t m, int64_t n, int32_t acc
     else store_scalar<AMCT_F32>(a.out, o, f);
 }
 
-// general kernel: any M, N, K; one output per thread.  Used for shapes the tiled kernel
-// does not cover.
+// ---------------------------------------------------------------------------
+// tile kernel
+// ---------------------------------------------------------------------------
+constexpr int kBM = 128, kBN = 128, kBK = 128;      // BK in bytes (= int8 elements)
+constexpr int kRow = kBK + 16;                      // padded LDS row: conflict-free ds_read_b128
+constexpr int kLoads = (kBM * kBK / 16) / kBlock;   // 16-byte chunks per thread and operand: 4
+
+AMCT_DEV uint4 ld_chunk_or_zero(const int8_t* base, int64_t row, int64_t rows, int64_t K, int64_t k) {
+    // rows beyond the matrix are clamped (their results are never stored); k beyond K reads zero
+    const int64_t r = row < rows ? row : rows - 1;
+    if (k < K) return ldg16(base + r * K + k);
+    return make_uint4(0, 0, 0, 0);
+}
+
+__global__ __launch_bounds__(kBlock) void w8a8_tile(W8A8Args a) {
+    __shared__ __attribute__((aligned(16))) int8_t As[2][kBM * kRow];
+    __shared__ __attribute__((aligned(16))) int8_t Bs[2][kBN * kRow];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int64_t m0 = (int64_t)blockIdx.y * kBM, n0 = (int64_t)blockIdx.x * kBN;
+    const int ld_row = tid >> 3, ld_chunk = tid & 7;            // 8 chunks of 16 B per row
+    const int nsteps = (int)((a.K + kBK - 1) / kBK);
+
+    uint4 ra[kLoads], rb[kLoads];
+    auto load_global = [&](int step) {
+        const int64_t k = (int64_t)step * kBK + ld_chunk * 16;
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) {
+            ra[i] = ld_chunk_or_zero(a.xq, m0 + ld_row + 32 * i, a.M, a.K, k);
+            rb[i] = ld_chunk_or_zero(a.wq, n0 + ld_row + 32 * i, a.N, a.K, k);
+        }
+    };
+    auto store_lds = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) {
+            *reinterpret_cast<uint4*>(&As[buf][(ld_row + 32 * i) * kRow + ld_chunk * 16]) = ra[i];
+            *reinterpret_cast<uint4*>(&Bs[buf][(ld_row + 32 * i) * kRow + ld_chunk * 16]) = rb[i];
+        }
+    };
+
+    v16i acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+    const int frag_row = lane & 31, frag_k = (lane >> 5) * 16;
+    for (int step = 0; step < nsteps; ++step) {
+        const int cur = step & 1;
+        if (step + 1 < nsteps) load_global(step + 1);
+#pragma unroll
+        for (int ks = 0; ks < kBK / 32; ++ks) {
+            v4i fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                fa[i] = *reinterpret_cast<const v4i*>(&As[cur][(wm * 64 + i * 32 + frag_row) * kRow + ks * 32 + frag_k]);
+                fb[i] = *reinterpret_cast<const v4i*>(&Bs[cur][(wn * 64 + i * 32 + frag_row) * kRow + ks * 32 + frag_k]);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+        if (step + 1 < nsteps) store_lds(cur ^ 1);
+        __syncthreads();
+    }
+
+    // epilogue: register r of a 32x32 tile holds row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int64_t n = n0 + wn * 64 + j * 32 + (lane & 31);
+        if (n >= a.N) continue;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int64_t m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (m < a.M) w8a8_epilogue(a, m, n, acc[i][j][r]);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// skinny kernel: M <= 16 * MT.  One block = 16 output columns; its 4 waves split K.
+// Lane l of a wave streams row n0 + l%16 of the weight, 16 bytes per MFMA, k-slot l/16.
+// ---------------------------------------------------------------------------
+template <int MT>
+__global__ __launch_bounds__(kBlock) void w8a8_skinny(W8A8Args a) {
+    __shared__ int32_t red[3][MT][64][4];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int64_t n0 = (int64_t)blockIdx.x * 16;
+    const int64_t nrow = (n0 + (lane & 15) < a.N) ? n0 + (lane & 15) : a.N - 1;
+    const int8_t* wrow = a.wq + nrow * a.K;
+    const int kslot = (lane >> 4) * 16;
+    // K is split into 4 contiguous spans, one per wave, each a multiple of 64 bytes
+    const int64_t steps_total = (a.K + 63) / 64;
+    const int64_t steps_per_wave = (steps_total + 3) / 4;
+    const int64_t s_begin = wave * steps_per_wave;
+    const int64_t s_end = (s_begin + steps_per_wave < steps_total) ? s_begin + steps_per_wave : steps_total;
+
+    v4i acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[t] = v4i{0, 0, 0, 0};
+    const int8_t* xrow[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        const int64_t m = t * 16 + (lane & 15);
+        xrow[t] = a.xq + (m < a.M ? m : a.M - 1) * a.K;
+    }
+    constexpr int UN = 4;
+    for (int64_t s = s_begin; s < s_end; s += UN) {
+        uint4 wv[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int64_t k = (s + u) * 64 + kslot;
+            wv[u] = (s + u < s_end && k < a.K) ? ldg16(wrow + k) : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int64_t k = (s + u) * 64 + kslot;
+            const bool ok = (s + u < s_end) && k < a.K;
+            const v4i fb = v4i{(int)wv[u].x, (int)wv[u].y, (int)wv[u].z, (int)wv[u].w};
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                const uint4 xv = ok ? ldg16(xrow[t] + k) : make_uint4(0, 0, 0, 0);
+                const v4i fa = v4i{(int)xv.x, (int)xv.y, (int)xv.z, (int)xv.w};
+                acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa, fb, acc[t], 0, 0, 0);
+            }
+        }
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) red[wave - 1][t][lane][r] = acc[t][r];
+    }
+    __syncthreads();
+    if (wave == 0) {
+        // register r of a 16x16 tile holds row 4*(lane/16) + r, column lane%16
+        const int64_t n = n0 + (lane & 15);
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int32_t v = acc[t][r] + red[0][t][lane][r] + red[1][t][lane][r] + red[2][t][lane][r];
+                const int64_t m = t * 16 + 4 * (lane >> 4) + r;
+                if (n < a.N && m < a.M) w8a8_epilogue(a, m, n, v);
+            }
+        }
+    }
+}
+
+// general kernel: any M, N, K; one output per thread.
 __global__ __launch_bounds__(kBlock) void w8a8_general(W8A8Args a) {
     const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     if (idx >= a.M * a.N) return;
@@ -56,6 +226,21 @@ extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s
     if (M == 0) return AMCT_OK;
     W8A8Args a{xq, wq, s_tok, s_ch, bias_kind ? bias : nullptr, out, acc_out, M, N, K, bias_kind, out_dtype};
     hipStream_t st = (hipStream_t)stream;
+    const bool vec_ok = (K % 16 == 0) && aligned16(xq) && aligned16(wq);
+    if (vec_ok && M <= 64) {
+        const dim3 grid((unsigned)((N + 15) / 16));
+        if (M <= 16) hipLaunchKernelGGL((w8a8_skinny<1>), grid, dim3(kBlock), 0, st, a);
+        else if (M <= 32) hipLaunchKernelGGL((w8a8_skinny<2>), grid, dim3(kBlock), 0, st, a);
+        else if (M <= 48) hipLaunchKernelGGL((w8a8_skinny<3>), grid, dim3(kBlock), 0, st, a);
+        else hipLaunchKernelGGL((w8a8_skinny<4>), grid, dim3(kBlock), 0, st, a);
+        return hip_status();
+    }
+    if (vec_ok) {
+        const dim3 grid((unsigned)((N + kBN - 1) / kBN), (unsigned)((M + kBM - 1) / kBM));
+        if (grid.y > 65535) return AMCT_E_UNSUPPORTED;
+        hipLaunchKernelGGL(w8a8_tile, grid, dim3(kBlock), 0, st, a);
+        return hip_status();
+    }
     const int64_t nb = (M * N + kBlock - 1) / kBlock;
     if (nb > 0x7FFFFFFF) return AMCT_E_UNSUPPORTED;
     hipLaunchKernelGGL(w8a8_general, dim3((unsigned)nb), dim3(kBlock), 0, st, a);

@@ -168,6 +168,31 @@ def build_cases(dev, only):
         ns = ns4
         cases.append(Case("act_quant_per_token", "hbm", work, "B", launch, ns, "f32",
                           "dynamic per-token INT8 quantize, X[2048,4096] bf16 (config 4)"))
+
+    # ---- K6: W8A8 Linear, W[14336,4096] int8 ----------------------------------------------------------
+    if want("w8a8_m2048") or want("w8a8_m16"):
+        x6, wq6, sw6 = workloads.c4_w8a8()
+        N6, K6 = wq6.shape
+        nw = 6                                           # 6 x 58.7 MB of weights rotate through HBM
+        wqs = dev_copies(wq6, nw)
+        swd = sw6.to(dev)
+        for name, M6 in (("w8a8_m2048", 2048), ("w8a8_m16", 16)):
+            if not want(name):
+                continue
+            xq6, st6 = ops.act_quant_per_token_int8(x6[:M6].to(dev))
+            outs = [torch.empty(M6, N6, dtype=torch.bfloat16, device=dev) for _ in range(nw)]
+
+            def launch(i, xq6=xq6, st6=st6, outs=outs, M6=M6, wqs=wqs, swd=swd, N6=N6, K6=K6):
+                j = i % len(wqs)
+                rc = lib.amct_gemm_w8a8(xq6.data_ptr(), wqs[j].data_ptr(), st6.data_ptr(), swd.data_ptr(), None, 0,
+                                        outs[j].data_ptr(), None, M6, N6, K6, _lib.BF16, st)
+                assert rc == 0, rc
+            if M6 >= 256:
+                cases.append(Case(name, "mfma_i8", 2 * M6 * N6 * K6, "op", launch, nw, "int8",
+                                  "W8A8 Linear M=%d N=14336 K=4096, per-token x per-channel rescale, bf16 out (config 4)" % M6))
+            else:
+                cases.append(Case(name, "hbm", N6 * K6 + M6 * K6 + M6 * N6 * 2 + N6 * 4 + M6 * 4, "B", launch, nw, "int8",
+                                  "W8A8 Linear M=%d (decode): weight streaming (config 4)" % M6))
     return cases
 
 
