@@ -2,9 +2,22 @@
 //   x'  = bf16(x * smooth[k])                         (weight_npu_quant_module.py:113-114)
 //   wdq = bf16((u[n,k] - zero[n,k/g]) * scale[n,k/g]) (the operator called at :116-117)
 // wq holds u = code + 8 as nibbles, even k in the low nibble.
+//
+//   tile kernel   : 128x128 block tile, BK = 64, bf16 MFMA 32x32x16.  The weight tile is
+//                   dequantised on its way from global memory to LDS: byte-wise nibble split,
+//                   v_cvt_f32_ubyteN, one fma per element ((u - z) * s == fma(u, s, -z*s) exactly),
+//                   v_cvt_pk_bf16_f32.  The smooth multiply is applied to the activation tile on the
+//                   same path.
+//   skinny kernel : M <= 64 (decode): weights streamed once from HBM, dequantised in registers,
+//                   bf16 MFMA 16x16x32, split-K over the 4 waves of a block.
+//   general kernel: any shape, one output per thread.
 #include "amct_common.h"
 
 namespace amct {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
 struct W4A16Args {
     const uint16_t* x;
@@ -22,6 +35,222 @@ struct W4A16Args {
 AMCT_DEV float load_scale(const W4A16Args& a, int64_t i) {
     const uint16_t h = reinterpret_cast<const uint16_t*>(a.scales)[i];
     return a.scale_dtype == AMCT_F16 ? f16_bits_to_f32(h) : bf16_bits_to_f32(h);
+}
+
+AMCT_DEV uint32_t pack_bf16x2(float lo, float hi) { return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16); }
+
+// 8 nibbles of `w` (element j in bits 4j..4j+3) -> 8 bf16 of (u - z) * s, as 4 packed dwords
+AMCT_DEV uint4 dequant8(uint32_t w, float s, float nzs) {
+    const uint32_t lo = w & 0x0F0F0F0Fu;            // elements 0,2,4,6 in bytes 0..3
+    const uint32_t hi = (w >> 4) & 0x0F0F0F0Fu;     // elements 1,3,5,7
+    uint32_t o[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        const float e0 = (float)((lo >> (8 * b)) & 0xFFu);
+        const float e1 = (float)((hi >> (8 * b)) & 0xFFu);
+        o[b] = pack_bf16x2(__builtin_fmaf(e0, s, nzs), __builtin_fmaf(e1, s, nzs));
+    }
+    return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+// 8 bf16 activations times 8 bf16 smooth factors, each product rounded to bf16
+AMCT_DEV uint4 smooth8(const uint4& x, const uint4& c) {
+    const uint32_t xs[4] = {x.x, x.y, x.z, x.w}, cs[4] = {c.x, c.y, c.z, c.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float lo = __uint_as_float(xs[i] << 16) * __uint_as_float(cs[i] << 16);
+        const float hi = __uint_as_float(xs[i] & 0xFFFF0000u) * __uint_as_float(cs[i] & 0xFFFF0000u);
+        o[i] = pack_bf16x2(lo, hi);
+    }
+    return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+// ---------------------------------------------------------------------------
+// tile kernel
+// ---------------------------------------------------------------------------
+constexpr int kTM = 128, kTN = 128, kTK = 64;       // BK in elements
+constexpr int kTRow = kTK * 2 + 16;                 // bytes per padded LDS row of bf16
+
+__global__ __launch_bounds__(kBlock) void w4a16_tile(W4A16Args a) {
+    __shared__ __attribute__((aligned(16))) uint8_t As[2][kTM * kTRow];
+    __shared__ __attribute__((aligned(16))) uint8_t Bs[2][kTN * kTRow];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int64_t m0 = (int64_t)blockIdx.y * kTM, n0 = (int64_t)blockIdx.x * kTN;
+    const int a_row = tid >> 3, a_chunk = tid & 7;              // activation tile: 8 chunks of 8 bf16 per row
+    const int b_row = tid >> 1, b_half = tid & 1;               // weight tile: 2 chunks of 32 nibbles per row
+    const int nsteps = (int)(a.K / kTK);
+    const int64_t G = a.K / a.group;
+    const int64_t wrow = (n0 + b_row < a.N) ? n0 + b_row : a.N - 1;
+
+    uint4 ra[4], rw, rc;
+    float s_cur = 0.f, nzs_cur = 0.f;
+    auto load_global = [&](int step) {
+        const int64_t k = (int64_t)step * kTK;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int64_t m = m0 + a_row + 32 * i;
+            ra[i] = ldg16(a.x + (m < a.M ? m : a.M - 1) * a.K + k + a_chunk * 8);
+        }
+        if (a.smooth) rc = ldg16(a.smooth + k + a_chunk * 8);
+        const int64_t kw = k + b_half * 32;
+        rw = ldg16(a.wq + wrow * (a.K / 2) + kw / 2);
+        const int64_t gi = wrow * G + kw / a.group;
+        s_cur = load_scale(a, gi);
+        nzs_cur = -((float)a.zeros[gi] * s_cur);
+    };
+    auto store_lds = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint4 v = a.smooth ? smooth8(ra[i], rc) : ra[i];
+            *reinterpret_cast<uint4*>(&As[buf][(a_row + 32 * i) * kTRow + a_chunk * 16]) = v;
+        }
+        const uint32_t ws[4] = {rw.x, rw.y, rw.z, rw.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            *reinterpret_cast<uint4*>(&Bs[buf][b_row * kTRow + b_half * 64 + j * 16]) = dequant8(ws[j], s_cur, nzs_cur);
+    };
+
+    v16f acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+    const int frag_row = lane & 31, frag_k = (lane >> 5) * 16;
+    for (int step = 0; step < nsteps; ++step) {
+        const int cur = step & 1;
+        if (step + 1 < nsteps) load_global(step + 1);
+#pragma unroll
+        for (int ks = 0; ks < kTK / 16; ++ks) {
+            v8bf fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                fa[i] = *reinterpret_cast<const v8bf*>(&As[cur][(wm * 64 + i * 32 + frag_row) * kTRow + ks * 32 + frag_k]);
+                fb[i] = *reinterpret_cast<const v8bf*>(&Bs[cur][(wn * 64 + i * 32 + frag_row) * kTRow + ks * 32 + frag_k]);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+        if (step + 1 < nsteps) store_lds(cur ^ 1);
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int64_t n = n0 + wn * 64 + j * 32 + (lane & 31);
+        if (n >= a.N) continue;
+        const float b = a.bias ? a.bias[n] : 0.f;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int64_t m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (m < a.M) {
+                    float v = acc[i][j][r];
+                    if (a.bias) v = v + b;
+                    a.out[m * a.N + n] = (uint16_t)f32_to_bf16_bits(v);
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// skinny kernel: M <= 16 * MT.  One block = 16 output columns, its 4 waves split K.
+// Per iteration a wave covers 128 k: lane (r = l%16, g = l/16) loads the 32 nibbles
+// k = kb + 32g .. +32 of weight row n0 + r; MFMA s (0..3) consumes nibbles 8s..8s+7 of every lane,
+// and the activation fragment of that MFMA is x[m][kb + 32g + 8s .. +8]: the k order inside an MFMA
+// is permuted identically for both operands, which leaves the dot product unchanged.
+// ---------------------------------------------------------------------------
+template <int MT>
+__global__ __launch_bounds__(kBlock) void w4a16_skinny(W4A16Args a) {
+    __shared__ float red[3][MT][64][4];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int64_t n0 = (int64_t)blockIdx.x * 16;
+    const int64_t nrow = (n0 + r16 < a.N) ? n0 + r16 : a.N - 1;
+    const int64_t G = a.K / a.group;
+    const uint8_t* wrow = a.wq + nrow * (a.K / 2);
+    const int64_t iters_total = a.K / 128;
+    const int64_t per_wave = (iters_total + 3) / 4;
+    const int64_t it_begin = wave * per_wave;
+    const int64_t it_end = (it_begin + per_wave < iters_total) ? it_begin + per_wave : iters_total;
+
+    const uint16_t* xrow[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        const int64_t m = t * 16 + r16;
+        xrow[t] = a.x + (m < a.M ? m : a.M - 1) * a.K;
+    }
+    v4f acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[t] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    constexpr int UN = 2;
+    for (int64_t it = it_begin; it < it_end; it += UN) {
+        uint4 wv[UN];
+        float sc[UN], nzs[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const bool ok = it + u < it_end;
+            const int64_t k = (it + u) * 128 + g * 32;
+            wv[u] = ok ? ldg16(wrow + k / 2) : make_uint4(0, 0, 0, 0);
+            const int64_t gi = nrow * G + (ok ? k / a.group : 0);
+            sc[u] = load_scale(a, gi);
+            nzs[u] = -((float)a.zeros[gi] * sc[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const bool ok = it + u < it_end;
+            const int64_t k = (it + u) * 128 + g * 32;
+            const uint32_t ws[4] = {wv[u].x, wv[u].y, wv[u].z, wv[u].w};
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const uint4 bq = ok ? dequant8(ws[s], sc[u], nzs[u]) : make_uint4(0, 0, 0, 0);
+                const v8bf fb = __builtin_bit_cast(v8bf, bq);
+                uint4 cs = make_uint4(0, 0, 0, 0);
+                if (a.smooth && ok) cs = ldg16(a.smooth + k + s * 8);
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    uint4 xv = ok ? ldg16(xrow[t] + k + s * 8) : make_uint4(0, 0, 0, 0);
+                    if (a.smooth) xv = smooth8(xv, cs);
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, xv), fb, acc[t], 0, 0, 0);
+                }
+            }
+        }
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) red[wave - 1][t][lane][r] = acc[t][r];
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const int64_t n = n0 + r16;
+        const float b = (a.bias && n < a.N) ? a.bias[n] : 0.f;
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float v = ((acc[t][r] + red[0][t][lane][r]) + red[1][t][lane][r]) + red[2][t][lane][r];
+                if (a.bias) v = v + b;
+                const int64_t m = t * 16 + 4 * g + r;
+                if (n < a.N && m < a.M) a.out[m * a.N + n] = (uint16_t)f32_to_bf16_bits(v);
+            }
+        }
+    }
 }
 
 // general kernel: one output per thread, sequential fp32 accumulation over k
@@ -58,6 +287,21 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
     if (M == 0) return AMCT_OK;
     W4A16Args a{(const uint16_t*)x, (const uint16_t*)smooth, wq, scales, zeros, bias, (uint16_t*)out, M, N, K, group, scale_dtype};
     hipStream_t st = (hipStream_t)stream;
+    const bool vec_ok = aligned16(x) && aligned16(wq) && (!smooth || aligned16(smooth)) && group % 32 == 0;
+    if (vec_ok && M <= 64 && K % 128 == 0) {
+        const dim3 grid((unsigned)((N + 15) / 16));
+        if (M <= 16) hipLaunchKernelGGL((w4a16_skinny<1>), grid, dim3(kBlock), 0, st, a);
+        else if (M <= 32) hipLaunchKernelGGL((w4a16_skinny<2>), grid, dim3(kBlock), 0, st, a);
+        else if (M <= 48) hipLaunchKernelGGL((w4a16_skinny<3>), grid, dim3(kBlock), 0, st, a);
+        else hipLaunchKernelGGL((w4a16_skinny<4>), grid, dim3(kBlock), 0, st, a);
+        return hip_status();
+    }
+    if (vec_ok && K % kTK == 0) {
+        const dim3 grid((unsigned)((N + kTN - 1) / kTN), (unsigned)((M + kTM - 1) / kTM));
+        if (grid.y > 65535) return AMCT_E_UNSUPPORTED;
+        hipLaunchKernelGGL(w4a16_tile, grid, dim3(kBlock), 0, st, a);
+        return hip_status();
+    }
     const int64_t nb = (M * N + kBlock - 1) / kBlock;
     if (nb > 0x7FFFFFFF) return AMCT_E_UNSUPPORTED;
     hipLaunchKernelGGL(w4a16_general, dim3((unsigned)nb), dim3(kBlock), 0, st, a);

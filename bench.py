@@ -193,6 +193,33 @@ def build_cases(dev, only):
             else:
                 cases.append(Case(name, "hbm", N6 * K6 + M6 * K6 + M6 * N6 * 2 + N6 * 4 + M6 * 4, "B", launch, nw, "int8",
                                   "W8A8 Linear M=%d (decode): weight streaming (config 4)" % M6))
+
+    # ---- K7: W4A16 Linear, W[14336,4096] int4 g128 ------------------------------------------------------
+    if want("w4a16_m2048") or want("w4a16_m16") or want("w4a16_m1"):
+        x7, codes7, sc7, z7, smr7 = workloads.c5_w4a16(2048)
+        N7, K7 = codes7.shape
+        g7 = 128
+        nw7 = 12                                         # 12 x 29.4 MB of packed weights rotate
+        pk7 = dev_copies(workloads.pack_nibbles(codes7), nw7)
+        scd, zd, smd = sc7.to(dev), z7.to(dev), smr7.to(dev)
+        for name, M7 in (("w4a16_m2048", 2048), ("w4a16_m16", 16), ("w4a16_m1", 1)):
+            if not want(name):
+                continue
+            xd = x7[:M7].contiguous().to(dev)
+            outs7 = [torch.empty(M7, N7, dtype=torch.bfloat16, device=dev) for _ in range(nw7)]
+
+            def launch(i, xd=xd, outs7=outs7, M7=M7, pk7=pk7, scd=scd, zd=zd, smd=smd, N7=N7, K7=K7, g7=g7):
+                j = i % len(pk7)
+                rc = lib.amct_gemm_w4a16(xd.data_ptr(), smd.data_ptr(), pk7[j].data_ptr(), scd.data_ptr(), _lib.F16,
+                                         zd.data_ptr(), None, outs7[j].data_ptr(), M7, N7, K7, g7, _lib.BF16, st)
+                assert rc == 0, rc
+            wbytes = N7 * K7 // 2 + N7 * (K7 // g7) * 3
+            if M7 >= 256:
+                cases.append(Case(name, "mfma_bf16", 2 * M7 * N7 * K7, "flop", launch, nw7, "bf16",
+                                  "W4A16 Linear M=%d N=14336 K=4096, group-128 dequant fused, smoothing fused (config 5)" % M7))
+            else:
+                cases.append(Case(name, "hbm", wbytes + M7 * K7 * 2 + M7 * N7 * 2, "B", launch, nw7, "bf16",
+                                  "W4A16 Linear M=%d (decode): weight streaming (config 5)" % M7))
     return cases
 
 
@@ -279,7 +306,7 @@ def run(args, dev, only):
         rate = c.work / (ms * 1e-3) / 1e9 if c.bound == "hbm" else c.work / (ms * 1e-3) / 1e12
         peak = HBM_PEAK_GBS if c.bound == "hbm" else (PEAK_INT8_TOPS if c.bound == "mfma_i8" else PEAK_BF16_TFLOPS)
         results[c.name] = {"desc": c.desc, "us_per_launch": round(ms * 1e3, 2), "achieved": round(rate, 1),
-                           "unit": "GB/s" if c.bound == "hbm" else "TOP/s", "peak": peak,
+                           "unit": "GB/s" if c.bound == "hbm" else ("TOP/s" if c.bound == "mfma_i8" else "TFLOP/s"), "peak": peak,
                            "frac": round(rate / peak, 4), "work_per_launch": c.work, "sets": c.nsets}
         if c.name == "int4_group_pack":
             head = (c, wall, ms)
