@@ -4,6 +4,8 @@
 //      amct_pytorch/quantize_op/utils.py:75-108, codes as amct_pytorch/utils/quant_util.py:56-73)
 //   static: q = sat(rne(x * scale + zero_point)), the operator called at
 //     amct_pytorch/deploy_op/npu_quantization_linear.py:98-99.
+#include <type_traits>
+
 #include "amct_common.h"
 
 namespace amct {
@@ -28,33 +30,28 @@ __global__ __launch_bounds__(kBlock) void act_quant_token(const void* x, const v
     uint4 raw[NV];
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-        const int vi = i * kBlock + tid;
-        raw[i] = make_uint4(0, 0, 0, 0);
-        if (vi < S) raw[i] = ldg16(reinterpret_cast<const char*>(x) + (row * K + (int64_t)vi * VEC) * BYTES);
+        const int vi = (i * kBlock + tid < S) ? i * kBlock + tid : S - 1;       // clamped: unconditional load
+        raw[i] = ldg16_nt(reinterpret_cast<const char*>(x) + (row * K + (int64_t)vi * VEC) * BYTES);
     }
 #pragma unroll
     for (int i = 0; i < NV; ++i) unpack16<DT>(raw[i], v[i]);
     if (smooth) {
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            const int vi = i * kBlock + tid;
-            if (vi < S) {
-                float c[VEC];
-                unpack16<DT>(ldg16(reinterpret_cast<const char*>(smooth) + (int64_t)vi * VEC * BYTES), c);
+            const int vi = (i * kBlock + tid < S) ? i * kBlock + tid : S - 1;
+            float c[VEC];
+            unpack16<DT>(ldg16(reinterpret_cast<const char*>(smooth) + (int64_t)vi * VEC * BYTES), c);
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) v[i][j] = round_to<DT>(v[i][j] * c[j]);
-            }
+            for (int j = 0; j < VEC; ++j) v[i][j] = round_to<DT>(v[i][j] * c[j]);
         }
     }
     float mx = -inf, mn = inf;
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-        if (i * kBlock + tid < S) {
+    for (int i = 0; i < NV; ++i) {                       // clamped duplicates cannot change a min/max
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) {
-                mx = fmax_nan(mx, v[i][j]);
-                mn = fmin_nan(mn, v[i][j]);
-            }
+        for (int j = 0; j < VEC; ++j) {
+            mx = fmax_nan(mx, v[i][j]);
+            mn = fmin_nan(mn, v[i][j]);
         }
     }
     team_minmax<kWave>(mn, mx);
@@ -79,18 +76,26 @@ __global__ __launch_bounds__(kBlock) void act_quant_token(const void* x, const v
         s = (amax == 0.f) ? 1.0f : s;
     }
     if (tid == 0) scale[row] = s;
+    const Divisor dv = make_divisor(s);
+    const uint32_t big = max(__float_as_uint(mx) & 0x7FFFFFFFu, __float_as_uint(mn) & 0x7FFFFFFFu);
+    const bool fast = dv.fast && big < 0x5D800000u;      // uniform over the block
+    auto emit = [&](auto fast_tag) {
+        constexpr bool FAST = decltype(fast_tag)::value;
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-        const int vi = i * kBlock + tid;
-        if (vi < S) {
+        for (int i = 0; i < NV; ++i) {
+            const int vi = i * kBlock + tid;
             float c[VEC];
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) c[j] = quant_elem<DT, false>(v[i][j], s, 0.f, false, -128.f, 127.f);
-            uint32_t* p = reinterpret_cast<uint32_t*>(q + row * K + (int64_t)vi * VEC);
-            if constexpr (VEC == 4) p[0] = pack4_i8(c);
-            else *reinterpret_cast<uint2*>(p) = make_uint2(pack4_i8(c), pack4_i8(c + 4));
+            for (int j = 0; j < VEC; ++j) c[j] = quant_elem<DT, false, FAST>(v[i][j], dv, 0.f, false, -128.f, 127.f);
+            if (vi < S) {
+                uint32_t* p = reinterpret_cast<uint32_t*>(q + row * K + (int64_t)vi * VEC);
+                if constexpr (VEC == 4) stg4_nt(p, pack4_i8(c));
+                else stg8_nt(p, pack4_i8(c), pack4_i8(c + 4));
+            }
         }
-    }
+    };
+    if (fast) emit(std::true_type{});
+    else emit(std::false_type{});
 }
 
 // general: any K, scalar accesses, two passes over the row

@@ -95,6 +95,20 @@ template <int DT> AMCT_DEV void store_scalar(void* p, int64_t i, float f) {
 AMCT_DEV uint4 ldg16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
 AMCT_DEV void stg16(void* p, const uint4& v) { *reinterpret_cast<uint4*>(p) = v; }
 
+// streaming (non-temporal) variants for data that is read or written exactly once: they bypass
+// cache retention and measurably raise copy bandwidth on MI355X
+typedef unsigned int u4v __attribute__((ext_vector_type(4)));
+typedef unsigned int u2v __attribute__((ext_vector_type(2)));
+AMCT_DEV uint4 ldg16_nt(const void* p) {
+    const u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+AMCT_DEV void stg16_nt(void* p, const uint4& v) {
+    __builtin_nontemporal_store(u4v{v.x, v.y, v.z, v.w}, reinterpret_cast<u4v*>(p));
+}
+AMCT_DEV void stg8_nt(void* p, uint32_t a, uint32_t b) { __builtin_nontemporal_store(u2v{a, b}, reinterpret_cast<u2v*>(p)); }
+AMCT_DEV void stg4_nt(void* p, uint32_t a) { __builtin_nontemporal_store(a, reinterpret_cast<uint32_t*>(p)); }
+
 // NaN-propagating max / min (v_maximum3_f32 / v_minimum3_f32), as torch.max does
 AMCT_DEV float fmax_nan(float a, float b) { return __builtin_elementwise_maximum(a, b); }
 AMCT_DEV float fmin_nan(float a, float b) { return __builtin_elementwise_minimum(a, b); }
@@ -110,6 +124,12 @@ template <int CTRL> AMCT_DEV float dpp_f(float v) {
 template <int CTRL> AMCT_DEV uint32_t dpp_u(uint32_t v) {
     return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, CTRL, 0xF, 0xF, true);
 }
+
+// value held by lane (lane & ~3) + Q of every quad
+template <int Q> AMCT_DEV float quad_bcast(float v) { return dpp_f<Q * 0x55>(v); }
+
+// all lanes of the wave agree that `p` holds
+AMCT_DEV bool wave_all(bool p) { return __builtin_amdgcn_ballot_w64(p) == __builtin_amdgcn_ballot_w64(true); }
 
 template <int T> AMCT_DEV void team_minmax(float& mn, float& mx) {
     if constexpr (T >= 2) { mx = fmax_nan(mx, dpp_f<0xB1>(mx)); mn = fmin_nan(mn, dpp_f<0xB1>(mn)); }
@@ -182,12 +202,45 @@ AMCT_DEV Factors make_factors(float vmax, float vmin, int bits, bool symmetric, 
     return r;
 }
 
+// Correctly rounded x / s from a precomputed y = RN(1/s) (Markstein): q0 = RN(x*y); two rounds of
+// "exact remainder by fma, correct by remainder*y".  After the first round q1 is within half an ulp
+// (plus 2^-45 relative) of x/s; the second round's error, <= 2^-25 ulp, is below the smallest
+// distance a quotient of two fp32 numbers can have from a rounding boundary (2^-47 relative), so q2
+// equals the IEEE quotient.  Valid while no intermediate over/underflows: the callers use it only
+// for |s| in [2^-60, 2^60], finite x, and results that are zero or at least 2^-60 in magnitude
+// matter only through round(q + z) (smaller quotients round to the same integer whatever their ulp).
+struct Divisor {
+    float s;      // divisor
+    float y;      // RN(1/s)
+    bool fast;    // the fma sequence may be used
+};
+AMCT_DEV Divisor make_divisor(float s) {
+    Divisor d;
+    d.s = s;
+    d.y = 1.0f / s;
+    const uint32_t e = (__float_as_uint(s) >> 23) & 0xFFu;
+    d.fast = (e >= 67u) && (e <= 187u) && s > 0.f;
+    return d;
+}
+AMCT_DEV float div_fast(float x, const Divisor& d) {
+    const float q0 = x * d.y;
+    const float r0 = __builtin_fmaf(-q0, d.s, x);
+    const float q1 = __builtin_fmaf(r0, d.y, q0);
+    const float r1 = __builtin_fmaf(-q1, d.s, x);
+    const float q2 = __builtin_fmaf(r1, d.y, q1);
+    // the divisor is positive, so the quotient carries the sign of x; the fma chain loses it only
+    // when the quotient is a zero (-0.0 + 0.0 = +0.0): put it back
+    return __uint_as_float(__float_as_uint(q2) | (__float_as_uint(x) & 0x80000000u));
+}
+
 // One element of the integer (fake-)quantiser.
 //   t = x / s (+ z); [narrow to the source dtype]; q = clamp(rne(t), qmin, qmax)
 // Returns q (integral float); *deq = (q - z) * s when requested.
-template <int DT, bool VIA_SRC>
-AMCT_DEV float quant_elem(float x, float s, float z, bool asym, float qmin, float qmax) {
-    float t = x / s;
+template <int DT, bool VIA_SRC, bool FAST = false>
+AMCT_DEV float quant_elem(float x, const Divisor& d, float z, bool asym, float qmin, float qmax) {
+    float t;
+    if constexpr (FAST) t = div_fast(x, d);
+    else t = x / d.s;
     if (asym) t = t + z;
     if constexpr (VIA_SRC) t = round_to<DT>(t);
     t = __builtin_rintf(t);
@@ -195,6 +248,14 @@ AMCT_DEV float quant_elem(float x, float s, float z, bool asym, float qmin, floa
     // only come from NaN data or factors (reported through the bad-factor count)
     t = __builtin_amdgcn_fmed3f(t, qmin, qmax);
     return t;
+}
+template <int DT, bool VIA_SRC>
+AMCT_DEV float quant_elem(float x, float s, float z, bool asym, float qmin, float qmax) {
+    Divisor d;
+    d.s = s;
+    d.y = 0.f;
+    d.fast = false;
+    return quant_elem<DT, VIA_SRC, false>(x, d, z, asym, qmin, qmax);
 }
 AMCT_DEV float dequant_elem(float q, float s, float z, bool asym) {
     if (asym) q = q - z;

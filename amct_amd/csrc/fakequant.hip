@@ -5,6 +5,8 @@
 //   general path : scalar kernel for ragged / unaligned shapes (zero-pad semantics).
 // Reference behaviour: amct_pytorch/quantize_op/utils.py:75-136,
 // amct_pytorch/utils/quant_util.py:56-93,162-188, amct_pytorch/algorithm/awq.py:129-170.
+#include <type_traits>
+
 #include "amct_common.h"
 
 namespace amct {
@@ -92,10 +94,12 @@ template <int DT> AMCT_DEV void store_codes(void* codes, int kind, int64_t e0, c
 }
 
 // ---------------------------------------------------------------------------
-// fused kernel.  A team of T lanes owns a segment; every lane caches NV 16-byte
-// vectors of it; U independent segments per team are in flight at once.
+// fused kernel.  A team of T lanes owns U consecutive segments; every lane caches NV 16-byte
+// vectors of each, all loaded up front (unconditional, streaming; indices are clamped and a
+// duplicated vector cannot change a min/max).  With U == 4 the factors of segment u are computed by
+// the lanes with lt % 4 == u and shared by DPP inside each quad.
 // ---------------------------------------------------------------------------
-template <int DT, int T, int NV, int U, bool VIA_SRC>
+template <int DT, int T, int NV, int U, bool VIA_SRC, bool COL>
 __global__ __launch_bounds__(kBlock) void fq_fused(FqArgs a) {
     constexpr int VEC = Tr<DT>::VEC;
     constexpr int BYTES = Tr<DT>::BYTES;
@@ -104,61 +108,53 @@ __global__ __launch_bounds__(kBlock) void fq_fused(FqArgs a) {
     const int team = tid / T, lt = tid % T;
     const int S = a.seg_len / VEC;
     const bool asym = !a.symmetric;
+    const int64_t seg0 = ((int64_t)blockIdx.x * TEAMS + team) * U;
 
     float x[U][NV][VEC];
-    int64_t seg[U];
-    float mx[U], mn[U];
-    const float inf = __builtin_huge_valf();
-
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-        seg[u] = ((int64_t)blockIdx.x * U + u) * TEAMS + team;
-        const bool ok = seg[u] < a.nseg;
-        uint4 raw[NV];
-#pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            const int v = i * T + lt;
-            raw[i] = make_uint4(0, 0, 0, 0);
-            if (ok && v < S)
-                raw[i] = ldg16(reinterpret_cast<const char*>(a.w) + (seg[u] * a.seg_len + (int64_t)v * VEC) * BYTES);
-        }
-#pragma unroll
-        for (int i = 0; i < NV; ++i) unpack16<DT>(raw[i], x[u][i]);
-    }
-
-    if (a.col_mode != AMCT_COL_NONE) {
+    int64_t segc[U];
+    {
+        uint4 raw[U][NV];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int64_t c0 = (seg[u] % a.segs_per_row) * (int64_t)a.seg_len;
+            segc[u] = (seg0 + u < a.nseg) ? seg0 + u : a.nseg - 1;
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
-                const int v = i * T + lt;
-                if (seg[u] < a.nseg && v < S) {
-                    float c[VEC];
-                    unpack16<DT>(ldg16(reinterpret_cast<const char*>(a.col) + (c0 + (int64_t)v * VEC) * BYTES), c);
-                    apply_col_pre<DT>(x[u][i], c, a.col_mode);
-                }
+                const int v = (i * T + lt < S) ? i * T + lt : S - 1;
+                raw[u][i] = ldg16_nt(reinterpret_cast<const char*>(a.w) + (segc[u] * a.seg_len + (int64_t)v * VEC) * BYTES);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int i = 0; i < NV; ++i) unpack16<DT>(raw[u][i], x[u][i]);
+    }
+    if constexpr (COL) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t c0 = (segc[u] % a.segs_per_row) * (int64_t)a.seg_len;
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int v = (i * T + lt < S) ? i * T + lt : S - 1;
+                float c[VEC];
+                unpack16<DT>(ldg16(reinterpret_cast<const char*>(a.col) + (c0 + (int64_t)v * VEC) * BYTES), c);
+                apply_col_pre<DT>(x[u][i], c, a.col_mode);
             }
         }
     }
 
+    float mx[U], mn[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-        mx[u] = -inf;
-        mn[u] = inf;
+        mx[u] = x[u][0][0];
+        mn[u] = x[u][0][0];
 #pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            const int v = i * T + lt;
-            if (seg[u] < a.nseg && v < S) {
+        for (int i = 0; i < NV; ++i)
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) {
-                    mx[u] = fmax_nan(mx[u], x[u][i][j]);
-                    mn[u] = fmin_nan(mn[u], x[u][i][j]);
-                }
+            for (int j = 0; j < VEC; ++j) {
+                mx[u] = fmax_nan(mx[u], x[u][i][j]);
+                mn[u] = fmin_nan(mn[u], x[u][i][j]);
             }
-        }
     }
-
     if constexpr (T <= kWave) {
 #pragma unroll
         for (int u = 0; u < U; ++u) team_minmax<T>(mn[u], mx[u]);
@@ -183,41 +179,79 @@ __global__ __launch_bounds__(kBlock) void fq_fused(FqArgs a) {
         }
     }
 
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-        const bool ok = seg[u] < a.nseg;
-        const Factors f = make_factors<DT>(mx[u], mn[u], a.bits, a.symmetric != 0, a.scope_rule);
-        if (ok && lt == 0) {
-            a.scale[seg[u]] = f.s;
-            if (a.offset) a.offset[seg[u]] = (int32_t)f.z;
+    Divisor dv[U];
+    float z[U];
+    bool fast;
+    if constexpr (U == 4) {
+        const int my = lt & 3;
+        const float mx_my = my == 0 ? mx[0] : my == 1 ? mx[1] : my == 2 ? mx[2] : mx[3];
+        const float mn_my = my == 0 ? mn[0] : my == 1 ? mn[1] : my == 2 ? mn[2] : mn[3];
+        const Factors f = make_factors<DT>(mx_my, mn_my, a.bits, a.symmetric != 0, a.scope_rule);
+        const Divisor dmy = make_divisor(f.s);
+        const uint32_t big = max(__float_as_uint(mx_my) & 0x7FFFFFFFu, __float_as_uint(mn_my) & 0x7FFFFFFFu);
+        fast = wave_all(dmy.fast && big < 0x5D800000u);
+        if (lt < 4 && seg0 + lt < a.nseg) {
+            a.scale[seg0 + lt] = f.s;
+            if (a.offset) a.offset[seg0 + lt] = (int32_t)f.z;
             if (f.bad && a.bad) atomicAdd(a.bad, 1);
         }
-        const int64_t c0 =
-            (a.col_mode == AMCT_COL_MUL_THEN_DIV) ? (seg[u] % a.segs_per_row) * (int64_t)a.seg_len : 0;
+        dv[0].s = quad_bcast<0>(f.s); dv[0].y = quad_bcast<0>(dmy.y); z[0] = quad_bcast<0>(f.z);
+        dv[1].s = quad_bcast<1>(f.s); dv[1].y = quad_bcast<1>(dmy.y); z[1] = quad_bcast<1>(f.z);
+        dv[2].s = quad_bcast<2>(f.s); dv[2].y = quad_bcast<2>(dmy.y); z[2] = quad_bcast<2>(f.z);
+        dv[3].s = quad_bcast<3>(f.s); dv[3].y = quad_bcast<3>(dmy.y); z[3] = quad_bcast<3>(f.z);
+    } else {
+        bool ok = true;
 #pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            const int v = i * T + lt;
-            if (ok && v < S) {
-                const int64_t e0 = seg[u] * a.seg_len + (int64_t)v * VEC;
+        for (int u = 0; u < U; ++u) {
+            const Factors f = make_factors<DT>(mx[u], mn[u], a.bits, a.symmetric != 0, a.scope_rule);
+            dv[u] = make_divisor(f.s);
+            z[u] = f.z;
+            const uint32_t big = max(__float_as_uint(mx[u]) & 0x7FFFFFFFu, __float_as_uint(mn[u]) & 0x7FFFFFFFu);
+            ok = ok && dv[u].fast && big < 0x5D800000u;
+            if (lt == 0 && seg0 + u < a.nseg) {
+                a.scale[seg0 + u] = f.s;
+                if (a.offset) a.offset[seg0 + u] = (int32_t)f.z;
+                if (f.bad && a.bad) atomicAdd(a.bad, 1);
+            }
+        }
+        fast = wave_all(ok);
+    }
+
+    auto emit = [&](auto fast_tag) {
+        constexpr bool FAST = decltype(fast_tag)::value;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const bool ok = seg0 + u < a.nseg;
+            const int64_t c0 = (COL && a.col_mode == AMCT_COL_MUL_THEN_DIV) ? (segc[u] % a.segs_per_row) * (int64_t)a.seg_len : 0;
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int v = i * T + lt;
                 float q[VEC], d[VEC];
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) {
-                    q[j] = quant_elem<DT, VIA_SRC>(x[u][i][j], f.s, f.z, asym, a.qmin, a.qmax);
-                    d[j] = dequant_elem(q[j], f.s, f.z, asym);
+                    q[j] = quant_elem<DT, VIA_SRC, FAST>(x[u][i][j], dv[u], z[u], asym, a.qmin, a.qmax);
+                    d[j] = dequant_elem(q[j], dv[u].s, z[u], asym);
                 }
-                if (a.codes) store_codes<DT>(a.codes, a.codes_kind, e0, q);
-                if (a.dq) {
-                    if (a.col_mode == AMCT_COL_MUL_THEN_DIV) {
-                        float c[VEC];
-                        unpack16<DT>(ldg16(reinterpret_cast<const char*>(a.col) + (c0 + (int64_t)v * VEC) * BYTES), c);
+                if (ok && v < S) {
+                    const int64_t e0 = (seg0 + u) * a.seg_len + (int64_t)v * VEC;
+                    if (a.codes) store_codes<DT>(a.codes, a.codes_kind, e0, q);
+                    if (a.dq) {
+                        if constexpr (COL) {
+                            if (a.col_mode == AMCT_COL_MUL_THEN_DIV) {
+                                float c[VEC];
+                                unpack16<DT>(ldg16(reinterpret_cast<const char*>(a.col) + (c0 + (int64_t)v * VEC) * BYTES), c);
 #pragma unroll
-                        for (int j = 0; j < VEC; ++j) d[j] = round_to<DT>(d[j]) / c[j];
+                                for (int j = 0; j < VEC; ++j) d[j] = round_to<DT>(d[j]) / c[j];
+                            }
+                        }
+                        stg16_nt(reinterpret_cast<char*>(a.dq) + e0 * BYTES, pack16<DT>(d));
                     }
-                    stg16(reinterpret_cast<char*>(a.dq) + e0 * BYTES, pack16<DT>(d));
                 }
             }
         }
-    }
+    };
+    if (fast) emit(std::true_type{});
+    else emit(std::false_type{});
 }
 
 // ---------------------------------------------------------------------------
@@ -424,10 +458,13 @@ static void launch_fused(const FqArgs& a, hipStream_t st) {
     constexpr int TEAMS = kBlock / T;
     const int64_t per_block = (int64_t)TEAMS * U;
     const int64_t nb = (a.nseg + per_block - 1) / per_block;
-    if (a.via_src && DT != AMCT_F32)
-        hipLaunchKernelGGL((fq_fused<DT, T, NV, U, true>), dim3((unsigned)nb), dim3(kBlock), 0, st, a);
-    else
-        hipLaunchKernelGGL((fq_fused<DT, T, NV, U, false>), dim3((unsigned)nb), dim3(kBlock), 0, st, a);
+    const dim3 grid((unsigned)nb), block(kBlock);
+    const bool via = a.via_src && DT != AMCT_F32;
+    const bool col = a.col_mode != AMCT_COL_NONE;
+    if (via && col) hipLaunchKernelGGL((fq_fused<DT, T, NV, U, true, true>), grid, block, 0, st, a);
+    else if (via) hipLaunchKernelGGL((fq_fused<DT, T, NV, U, true, false>), grid, block, 0, st, a);
+    else if (col) hipLaunchKernelGGL((fq_fused<DT, T, NV, U, false, true>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((fq_fused<DT, T, NV, U, false, false>), grid, block, 0, st, a);
 }
 
 template <int DT>

@@ -66,10 +66,11 @@ __global__ __launch_bounds__(kBlock) void hif8_encode_k(const void* x, uint8_t* 
     const int tid = threadIdx.x;
     uint4 raw[U];
     int64_t gv[U];
+    if (nvec > 0) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         gv[u] = ((int64_t)blockIdx.x * U + u) * kBlock + tid;
-        if (gv[u] < nvec) raw[u] = ldg16(reinterpret_cast<const char*>(x) + gv[u] * 16);
+        raw[u] = ldg16_nt(reinterpret_cast<const char*>(x) + ((gv[u] < nvec ? gv[u] : nvec - 1) * 16));
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -82,9 +83,10 @@ __global__ __launch_bounds__(kBlock) void hif8_encode_k(const void* x, uint8_t* 
                 w[j] = hif8_enc(v[4 * j], saturate) | (hif8_enc(v[4 * j + 1], saturate) << 8) |
                        (hif8_enc(v[4 * j + 2], saturate) << 16) | (hif8_enc(v[4 * j + 3], saturate) << 24);
             uint32_t* p = reinterpret_cast<uint32_t*>(y + gv[u] * VEC);
-            if constexpr (VEC == 8) *reinterpret_cast<uint2*>(p) = make_uint2(w[0], w[1]);
-            else p[0] = w[0];
+            if constexpr (VEC == 8) stg8_nt(p, w[0], w[1]);
+            else stg4_nt(p, w[0]);
         }
+    }
     }
     // tail (n % VEC elements), handled by block 0
     if (blockIdx.x == 0) {

@@ -1,6 +1,8 @@
 // K2: int4 per-group quantise + nibble pack in one pass, and the int4 interchange layouts.
 // Reference behaviour: amct_pytorch/deploy_op/weight_npu_quant_module.py:38-66 (weight preparation),
 // amct_pytorch/utils/quant_util.py:76-93 (codes), amct_pytorch/quantize_op/utils.py:75-136 (factors).
+#include <type_traits>
+
 #include "amct_common.h"
 
 namespace amct {
@@ -119,6 +121,120 @@ __global__ __launch_bounds__(kBlock) void int4_group_pack(PackArgs a) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// main kernel (groups of at most 64 vectors).  A team of T lanes owns 4 consecutive groups; lane lt
+// holds vector lt of each, so 4 x 16 bytes per lane are in flight.  Loads are unconditional (indices
+// are clamped, duplicates do not change a min/max), streaming, and issued before any use.
+// The factors of group u are computed by the lanes with lt % 4 == u and shared inside each quad by
+// DPP; the per-element division is the exact fma sequence when every group of the wave allows it.
+// ---------------------------------------------------------------------------
+template <int DT, int T, bool COL>
+__global__ __launch_bounds__(kBlock) void int4_group_pack4(PackArgs a) {
+    constexpr int U = 4;
+    constexpr int VEC = Tr<DT>::VEC;
+    constexpr int BYTES = Tr<DT>::BYTES;
+    constexpr int TEAMS = kBlock / T;
+    const int tid = threadIdx.x;
+    const int team = tid / T, lt = tid % T;
+    const int S = a.seg_len / VEC;
+    const int vl = lt < S ? lt : S - 1;
+    const bool asym = !a.symmetric;
+    const int64_t seg0 = ((int64_t)blockIdx.x * TEAMS + team) * U;
+
+    uint4 raw[U];
+    int64_t segc[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        segc[u] = (seg0 + u < a.nseg) ? seg0 + u : a.nseg - 1;
+        raw[u] = ldg16_nt(reinterpret_cast<const char*>(a.w) + (segc[u] * a.seg_len + (int64_t)vl * VEC) * BYTES);
+    }
+    float x[U][VEC];
+#pragma unroll
+    for (int u = 0; u < U; ++u) unpack16<DT>(raw[u], x[u]);
+    if constexpr (COL) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t c0 = (segc[u] % a.segs_per_row) * (int64_t)a.seg_len;
+            float c[VEC];
+            unpack16<DT>(ldg16(reinterpret_cast<const char*>(a.col) + (c0 + (int64_t)vl * VEC) * BYTES), c);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+                x[u][j] = round_to<DT>(a.col_mode == AMCT_COL_DIV ? x[u][j] / c[j] : x[u][j] * c[j]);
+        }
+    }
+    float mx[U], mn[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        mx[u] = x[u][0];
+        mn[u] = x[u][0];
+#pragma unroll
+        for (int j = 1; j < VEC; ++j) {
+            mx[u] = fmax_nan(mx[u], x[u][j]);
+            mn[u] = fmin_nan(mn[u], x[u][j]);
+        }
+        team_minmax<T>(mn[u], mx[u]);
+    }
+    // lane lt computes the factors of group lt % 4
+    const int my = lt & 3;
+    const float mx_my = my == 0 ? mx[0] : my == 1 ? mx[1] : my == 2 ? mx[2] : mx[3];
+    const float mn_my = my == 0 ? mn[0] : my == 1 ? mn[1] : my == 2 ? mn[2] : mn[3];
+    const Factors f = make_factors<AMCT_F32>(mx_my, mn_my, 4, a.symmetric != 0, AMCT_SCOPE_AMCT);
+    const Divisor dmy = make_divisor(f.s);
+    const uint32_t big = max(__float_as_uint(mx_my) & 0x7FFFFFFFu, __float_as_uint(mn_my) & 0x7FFFFFFFu);
+    const bool fast = wave_all(dmy.fast && big < 0x5D800000u);       // |x| < 2^60, finite
+    if (lt < 4 && seg0 + lt < a.nseg) {
+        const int64_t sg = seg0 + lt;
+        if (a.scales32) a.scales32[sg] = f.s;
+        if (a.scales16) {
+            reinterpret_cast<uint16_t*>(a.scales16)[sg] =
+                (uint16_t)(a.scale_dtype == AMCT_F16 ? f32_to_f16_bits(f.s) : f32_to_bf16_bits(f.s));
+        }
+        if (a.zeros) a.zeros[sg] = (uint8_t)((int)f.z + 8);
+        if (f.bad && a.bad) atomicAdd(a.bad, 1);
+    }
+    Divisor dv[U];
+    float z[U];
+    dv[0].s = quad_bcast<0>(f.s); dv[0].y = quad_bcast<0>(dmy.y); z[0] = quad_bcast<0>(f.z);
+    dv[1].s = quad_bcast<1>(f.s); dv[1].y = quad_bcast<1>(dmy.y); z[1] = quad_bcast<1>(f.z);
+    dv[2].s = quad_bcast<2>(f.s); dv[2].y = quad_bcast<2>(dmy.y); z[2] = quad_bcast<2>(f.z);
+    dv[3].s = quad_bcast<3>(f.s); dv[3].y = quad_bcast<3>(dmy.y); z[3] = quad_bcast<3>(f.z);
+
+    // codes u = q + 8 are gathered by exact fp32 arithmetic: sum (q_j + 8) * 16^j over 4 nibbles
+    uint32_t word[U];
+    auto encode = [&](auto fast_tag) {
+        constexpr bool FAST = decltype(fast_tag)::value;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            float lo = 34952.0f, hi = 34952.0f;                  // 8 * (1 + 16 + 256 + 4096)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float q = quant_elem<DT, false, FAST>(x[u][j], dv[u], z[u], asym, -8.f, 7.f);
+                lo = __builtin_fmaf(q, (float)(1 << (4 * j)), lo);
+            }
+            if constexpr (VEC == 8) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float q = quant_elem<DT, false, FAST>(x[u][4 + j], dv[u], z[u], asym, -8.f, 7.f);
+                    hi = __builtin_fmaf(q, (float)(1 << (4 * j)), hi);
+                }
+                word[u] = (uint32_t)lo | ((uint32_t)hi << 16);
+            } else {
+                word[u] = (uint32_t)lo;
+            }
+        }
+    };
+    if (fast) encode(std::true_type{});
+    else encode(std::false_type{});
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        if (lt < S && seg0 + u < a.nseg) {
+            const int64_t b0 = ((seg0 + u) * a.seg_len + (int64_t)lt * VEC) / 2;
+            if constexpr (VEC == 8) stg4_nt(a.packed + b0, word[u]);
+            else *reinterpret_cast<uint16_t*>(a.packed + b0) = (uint16_t)word[u];
+        }
+    }
+}
+
 // general kernel: one block per row, scalar loads; cols % group == 0 and cols even.
 template <int DT>
 __global__ __launch_bounds__(kBlock) void int4_group_pack_general(PackArgs a, int64_t cols) {
@@ -186,19 +302,30 @@ static void launch_pack(const PackArgs& a, hipStream_t st) {
     hipLaunchKernelGGL((int4_group_pack<DT, T, NV, U>), dim3((unsigned)nb), dim3(kBlock), 0, st, a);
 }
 
+template <int DT, int T>
+static void launch_pack4(const PackArgs& a, hipStream_t st) {
+    const int64_t per_block = (int64_t)(kBlock / T) * 4;
+    const int64_t nb = (a.nseg + per_block - 1) / per_block;
+    if (a.col_mode != AMCT_COL_NONE) hipLaunchKernelGGL((int4_group_pack4<DT, T, true>), dim3((unsigned)nb), dim3(kBlock), 0, st, a);
+    else hipLaunchKernelGGL((int4_group_pack4<DT, T, false>), dim3((unsigned)nb), dim3(kBlock), 0, st, a);
+}
+
 template <int DT>
 static int run_pack(const PackArgs& a, int64_t rows, int64_t cols, hipStream_t st) {
     constexpr int VEC = Tr<DT>::VEC;
     const int S = a.seg_len / VEC;
     const bool vec_ok = aligned16(a.w) && (reinterpret_cast<uintptr_t>(a.packed) & 3u) == 0 &&
                         (a.col_mode == AMCT_COL_NONE || aligned16(a.col));
+    if (vec_ok && S <= 64) {
+        if (S <= 4) launch_pack4<DT, 4>(a, st);
+        else if (S <= 8) launch_pack4<DT, 8>(a, st);
+        else if (S <= 16) launch_pack4<DT, 16>(a, st);
+        else if (S <= 32) launch_pack4<DT, 32>(a, st);
+        else launch_pack4<DT, 64>(a, st);
+        return hip_status();
+    }
     if (vec_ok && S <= 512) {
-        if (S <= 4) launch_pack<DT, 4, 1, 4>(a, st);
-        else if (S <= 8) launch_pack<DT, 8, 1, 4>(a, st);
-        else if (S <= 16) launch_pack<DT, 16, 1, 4>(a, st);
-        else if (S <= 32) launch_pack<DT, 32, 1, 4>(a, st);
-        else if (S <= 64) launch_pack<DT, 64, 1, 4>(a, st);
-        else if (S <= 128) launch_pack<DT, 64, 2, 2>(a, st);
+        if (S <= 128) launch_pack<DT, 64, 2, 2>(a, st);
         else if (S <= 256) launch_pack<DT, 64, 4, 1>(a, st);
         else launch_pack<DT, 64, 8, 1>(a, st);
         return hip_status();

@@ -90,8 +90,8 @@ __global__ __launch_bounds__(kBlock) void mx_quant_k(const void* x, uint8_t* el,
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         gv[u] = ((int64_t)blockIdx.x * U + u) * kBlock + tid;
-        raw[u] = make_uint4(0, 0, 0, 0);
-        if (gv[u] < nvec) raw[u] = ldg16(reinterpret_cast<const char*>(x) + gv[u] * 16);
+        // unconditional streaming load (index clamped; whole blocks of 32 are valid or not together)
+        raw[u] = ldg16_nt(reinterpret_cast<const char*>(x) + (gv[u] < nvec ? gv[u] : nvec - 1) * 16);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -159,13 +159,13 @@ __global__ __launch_bounds__(kBlock) void mx_quant_k(const void* x, uint8_t* el,
                 for (int j = 0; j < VEC / 4; ++j)
                     w[j] = codes[4 * j] | (codes[4 * j + 1] << 8) | (codes[4 * j + 2] << 16) | (codes[4 * j + 3] << 24);
                 uint32_t* p = reinterpret_cast<uint32_t*>(el + gv[u] * VEC);
-                if constexpr (VEC == 8) *reinterpret_cast<uint2*>(p) = make_uint2(w[0], w[1]);
-                else p[0] = w[0];
+                if constexpr (VEC == 8) stg8_nt(p, w[0], w[1]);
+                else stg4_nt(p, w[0]);
             } else {
                 uint32_t w = 0;
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) w |= codes[j] << (4 * j);
-                if constexpr (VEC == 8) *reinterpret_cast<uint32_t*>(el + gv[u] * 4) = w;
+                if constexpr (VEC == 8) stg4_nt(el + gv[u] * 4, w);
                 else *reinterpret_cast<uint16_t*>(el + gv[u] * 2) = (uint16_t)w;
             }
             if ((tid & (T - 1)) == 0) e8[gv[u] / T] = (uint8_t)byte;

@@ -61,6 +61,19 @@ def build_cases(dev, only):
         base = t.to(dev)
         return [base] + [base.clone() for _ in range(n - 1)]
 
+    # ---- streaming copy yardstick: 128 MiB read + 128 MiB write ------------------------------------------
+    if want("copy"):
+        nbytes = 128 << 20
+        nsc = 6
+        src = [torch.empty(nbytes, dtype=torch.uint8, device=dev).fill_(1) for _ in range(nsc)]
+        dst = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(nsc)]
+
+        def launch(i, src=src, dst=dst, nbytes=nbytes):
+            j = i % len(src)
+            rc = lib.amct_copy_bytes(src[j].data_ptr(), dst[j].data_ptr(), nbytes, st)
+            assert rc == 0, rc
+        cases.append(Case("copy", "hbm", 2 * nbytes, "B", launch, nsc, "u8", "plain copy of 128 MiB (yardstick)"))
+
     # ---- K2 (headline): int4 asym g128 quant + pack, W[14336,4096] bf16 -------------------------
     if want("int4_group_pack"):
         w = workloads.c2_weight()

@@ -69,6 +69,10 @@ enum { AMCT_CODES_NONE = 0, AMCT_CODES_I8 = 1, AMCT_CODES_I32 = 2 };
 int amct_hip_version(void);
 const char* amct_hip_strerror(int code);
 
+/* Plain device-to-device streaming copy (nbytes % 16 == 0).  No counterpart in the reference: it is
+ * the yardstick for the bandwidth figures and for scaling hardware traffic counters. */
+int amct_copy_bytes(const void* src, void* dst, int64_t nbytes, amct_stream_t stream);
+
 /* ---- A1: min / max per row (group = 0) or per group of `group` columns ----------------
  * Replaces get_weight_min_max_by_granularity (amct_pytorch/quantize_op/utils.py:111-136)
  * and the per-token reductions of amct_pytorch/quantize_op/minmax_module.py:96-105.
