@@ -140,6 +140,38 @@ template <int T> AMCT_DEV void team_minmax(float& mn, float& mx) {
     if constexpr (T >= 64) { mx = fmax_nan(mx, __shfl_xor(mx, 32)); mn = fmin_nan(mn, __shfl_xor(mn, 32)); }
 }
 
+// Reduce 4 (min, max) pairs over a team of T lanes (T >= 4, a power of two) so that lane lt ends up
+// with the pair of segment seg4_of_lane(lt), reduced over the whole team: two exchange steps that
+// halve the data a lane carries, then plain butterflies.  About half the instructions of four
+// independent all-reduces.
+AMCT_DEV int seg4_of_lane(int lt) { return ((lt & 1) << 1) | ((lt >> 1) & 1); }
+
+template <int T> AMCT_DEV void team_minmax_scatter4(const float* mn, const float* mx, int lt, float& mn_my, float& mx_my) {
+    const bool b0 = lt & 1, b1 = lt & 2;
+    // step 1 (partner lt^1): lanes with b0 = 0 keep segments {0,1}, the others {2,3}
+    float kn0 = b0 ? mn[2] : mn[0], kn1 = b0 ? mn[3] : mn[1];
+    float kx0 = b0 ? mx[2] : mx[0], kx1 = b0 ? mx[3] : mx[1];
+    const float gn0 = b0 ? mn[0] : mn[2], gn1 = b0 ? mn[1] : mn[3];          // what the partner keeps
+    const float gx0 = b0 ? mx[0] : mx[2], gx1 = b0 ? mx[1] : mx[3];
+    kn0 = fmin_nan(kn0, dpp_f<0xB1>(gn0)); kn1 = fmin_nan(kn1, dpp_f<0xB1>(gn1));
+    kx0 = fmax_nan(kx0, dpp_f<0xB1>(gx0)); kx1 = fmax_nan(kx1, dpp_f<0xB1>(gx1));
+    // step 2 (partner lt^2): lanes with b1 = 0 keep the first of their two, the others the second
+    float n = b1 ? kn1 : kn0, x = b1 ? kx1 : kx0;
+    const float gn = b1 ? kn0 : kn1, gx = b1 ? kx0 : kx1;
+    n = fmin_nan(n, dpp_f<0x4E>(gn));
+    x = fmax_nan(x, dpp_f<0x4E>(gx));
+    // remaining steps keep lt % 4: rotations by 4 and 8 inside a row of 16, then cross-row shuffles
+    if constexpr (T == 8) { n = fmin_nan(n, __shfl_xor(n, 4)); x = fmax_nan(x, __shfl_xor(x, 4)); }
+    if constexpr (T >= 16) {
+        n = fmin_nan(n, dpp_f<0x124>(n)); x = fmax_nan(x, dpp_f<0x124>(x));      // row_ror:4
+        n = fmin_nan(n, dpp_f<0x128>(n)); x = fmax_nan(x, dpp_f<0x128>(x));      // row_ror:8
+    }
+    if constexpr (T >= 32) { n = fmin_nan(n, __shfl_xor(n, 16)); x = fmax_nan(x, __shfl_xor(x, 16)); }
+    if constexpr (T >= 64) { n = fmin_nan(n, __shfl_xor(n, 32)); x = fmax_nan(x, __shfl_xor(x, 32)); }
+    mn_my = n;
+    mx_my = x;
+}
+
 template <int T> AMCT_DEV uint32_t team_umax(uint32_t v) {
     if constexpr (T >= 2) v = max(v, dpp_u<0xB1>(v));
     if constexpr (T >= 4) v = max(v, dpp_u<0x4E>(v));
@@ -148,6 +180,48 @@ template <int T> AMCT_DEV uint32_t team_umax(uint32_t v) {
     if constexpr (T >= 32) v = max(v, (uint32_t)__shfl_xor((int)v, 16));
     if constexpr (T >= 64) v = max(v, (uint32_t)__shfl_xor((int)v, 32));
     return v;
+}
+
+// Correctly rounded x / s from a precomputed y = RN(1/s) (Markstein): q0 = RN(x*y); two rounds of
+// "exact remainder by fma, correct by remainder*y".  After the first round q1 is within half an ulp
+// (plus 2^-45 relative) of x/s; the second round's error, <= 2^-25 ulp, is below the smallest
+// distance a quotient of two fp32 numbers can have from a rounding boundary (2^-47 relative), so q2
+// equals the IEEE quotient.  Valid while no intermediate over/underflows: the callers use it only
+// for |s| in [2^-60, 2^60], finite x, and results that are zero or at least 2^-60 in magnitude
+// matter only through round(q + z) (smaller quotients round to the same integer whatever their ulp).
+struct Divisor {
+    float s;      // divisor
+    float y;      // RN(1/s)
+    bool fast;    // the fma sequence may be used
+};
+AMCT_DEV Divisor make_divisor(float s) {
+    Divisor d;
+    d.s = s;
+    d.y = 1.0f / s;
+    const uint32_t e = (__float_as_uint(s) >> 23) & 0xFFu;
+    d.fast = (e >= 67u) && (e <= 187u) && s > 0.f;
+    return d;
+}
+template <bool KEEP_ZERO_SIGN = true>
+AMCT_DEV float div_fast(float x, const Divisor& d) {
+    const float q0 = x * d.y;
+    const float r0 = __builtin_fmaf(-q0, d.s, x);
+    const float q1 = __builtin_fmaf(r0, d.y, q0);
+    const float r1 = __builtin_fmaf(-q1, d.s, x);
+    const float q2 = __builtin_fmaf(r1, d.y, q1);
+    // the divisor is positive, so the quotient carries the sign of x; the fma chain loses it only
+    // when the quotient is a zero (-0.0 + 0.0 = +0.0): put it back where a caller can see it
+    if constexpr (KEEP_ZERO_SIGN) return __uint_as_float(__float_as_uint(q2) | (__float_as_uint(x) & 0x80000000u));
+    else return q2;
+}
+
+// x / c for a compile-time-known positive constant through the same sequence
+AMCT_DEV float div_const(float x, float c, float rc) {
+    Divisor d;
+    d.s = c;
+    d.y = rc;
+    d.fast = true;
+    return div_fast<true>(x, d);
 }
 
 // ---------------------------------------------------------------------------
@@ -190,8 +264,17 @@ AMCT_DEV Factors make_factors(float vmax, float vmin, int bits, bool symmetric, 
         vmin = (vmin > 0.f) ? 0.f : vmin;
         const float scope = (float)((1 << bits) - 1);
         const float half = (float)(1 << (bits - 1));        // ceil(scope / 2)
-        r.s = (vmax - vmin) / scope;
-        r.z = (vmax != vmin) ? (-half - vmin / r.s) : -half;
+        const float diff = vmax - vmin;
+        const uint32_t ed = (__float_as_uint(diff) >> 23) & 0xFFu;
+        if (ed >= 67u && ed <= 187u) {
+            // diff in [2^-60, 2^61): both quotients by the exact fma sequence (same results as '/')
+            r.s = div_const(diff, scope, bits == 8 ? (1.0f / 255.0f) : (1.0f / 15.0f));
+            const Divisor ds = make_divisor(r.s);
+            r.z = (vmax != vmin) ? (-half - div_fast<true>(vmin, ds)) : -half;
+        } else {
+            r.s = diff / scope;
+            r.z = (vmax != vmin) ? (-half - vmin / r.s) : -half;
+        }
     }
     const bool tiny = r.s < kEps;
     if (!symmetric) r.z = tiny ? -(float)(1 << (bits - 1)) : r.z;
@@ -202,44 +285,13 @@ AMCT_DEV Factors make_factors(float vmax, float vmin, int bits, bool symmetric, 
     return r;
 }
 
-// Correctly rounded x / s from a precomputed y = RN(1/s) (Markstein): q0 = RN(x*y); two rounds of
-// "exact remainder by fma, correct by remainder*y".  After the first round q1 is within half an ulp
-// (plus 2^-45 relative) of x/s; the second round's error, <= 2^-25 ulp, is below the smallest
-// distance a quotient of two fp32 numbers can have from a rounding boundary (2^-47 relative), so q2
-// equals the IEEE quotient.  Valid while no intermediate over/underflows: the callers use it only
-// for |s| in [2^-60, 2^60], finite x, and results that are zero or at least 2^-60 in magnitude
-// matter only through round(q + z) (smaller quotients round to the same integer whatever their ulp).
-struct Divisor {
-    float s;      // divisor
-    float y;      // RN(1/s)
-    bool fast;    // the fma sequence may be used
-};
-AMCT_DEV Divisor make_divisor(float s) {
-    Divisor d;
-    d.s = s;
-    d.y = 1.0f / s;
-    const uint32_t e = (__float_as_uint(s) >> 23) & 0xFFu;
-    d.fast = (e >= 67u) && (e <= 187u) && s > 0.f;
-    return d;
-}
-AMCT_DEV float div_fast(float x, const Divisor& d) {
-    const float q0 = x * d.y;
-    const float r0 = __builtin_fmaf(-q0, d.s, x);
-    const float q1 = __builtin_fmaf(r0, d.y, q0);
-    const float r1 = __builtin_fmaf(-q1, d.s, x);
-    const float q2 = __builtin_fmaf(r1, d.y, q1);
-    // the divisor is positive, so the quotient carries the sign of x; the fma chain loses it only
-    // when the quotient is a zero (-0.0 + 0.0 = +0.0): put it back
-    return __uint_as_float(__float_as_uint(q2) | (__float_as_uint(x) & 0x80000000u));
-}
-
 // One element of the integer (fake-)quantiser.
 //   t = x / s (+ z); [narrow to the source dtype]; q = clamp(rne(t), qmin, qmax)
 // Returns q (integral float); *deq = (q - z) * s when requested.
-template <int DT, bool VIA_SRC, bool FAST = false>
+template <int DT, bool VIA_SRC, bool FAST = false, bool KEEP_ZERO_SIGN = true>
 AMCT_DEV float quant_elem(float x, const Divisor& d, float z, bool asym, float qmin, float qmax) {
     float t;
-    if constexpr (FAST) t = div_fast(x, d);
+    if constexpr (FAST) t = div_fast<KEEP_ZERO_SIGN>(x, d);
     else t = x / d.s;
     if (asym) t = t + z;
     if constexpr (VIA_SRC) t = round_to<DT>(t);

@@ -155,7 +155,9 @@ __global__ __launch_bounds__(kBlock) void fq_fused(FqArgs a) {
                 mn[u] = fmin_nan(mn[u], x[u][i][j]);
             }
     }
-    if constexpr (T <= kWave) {
+    if constexpr (U == 4) {
+        // reduced further below by a scatter-reduction
+    } else if constexpr (T <= kWave) {
 #pragma unroll
         for (int u = 0; u < U; ++u) team_minmax<T>(mn[u], mx[u]);
     } else {
@@ -183,21 +185,21 @@ __global__ __launch_bounds__(kBlock) void fq_fused(FqArgs a) {
     float z[U];
     bool fast;
     if constexpr (U == 4) {
-        const int my = lt & 3;
-        const float mx_my = my == 0 ? mx[0] : my == 1 ? mx[1] : my == 2 ? mx[2] : mx[3];
-        const float mn_my = my == 0 ? mn[0] : my == 1 ? mn[1] : my == 2 ? mn[2] : mn[3];
+        const int my = seg4_of_lane(lt);
+        float mx_my, mn_my;
+        team_minmax_scatter4<T>(mn, mx, lt, mn_my, mx_my);
         const Factors f = make_factors<DT>(mx_my, mn_my, a.bits, a.symmetric != 0, a.scope_rule);
         const Divisor dmy = make_divisor(f.s);
         const uint32_t big = max(__float_as_uint(mx_my) & 0x7FFFFFFFu, __float_as_uint(mn_my) & 0x7FFFFFFFu);
         fast = wave_all(dmy.fast && big < 0x5D800000u);
-        if (lt < 4 && seg0 + lt < a.nseg) {
-            a.scale[seg0 + lt] = f.s;
-            if (a.offset) a.offset[seg0 + lt] = (int32_t)f.z;
+        if (lt < 4 && seg0 + my < a.nseg) {
+            a.scale[seg0 + my] = f.s;
+            if (a.offset) a.offset[seg0 + my] = (int32_t)f.z;
             if (f.bad && a.bad) atomicAdd(a.bad, 1);
         }
         dv[0].s = quad_bcast<0>(f.s); dv[0].y = quad_bcast<0>(dmy.y); z[0] = quad_bcast<0>(f.z);
-        dv[1].s = quad_bcast<1>(f.s); dv[1].y = quad_bcast<1>(dmy.y); z[1] = quad_bcast<1>(f.z);
-        dv[2].s = quad_bcast<2>(f.s); dv[2].y = quad_bcast<2>(dmy.y); z[2] = quad_bcast<2>(f.z);
+        dv[1].s = quad_bcast<2>(f.s); dv[1].y = quad_bcast<2>(dmy.y); z[1] = quad_bcast<2>(f.z);
+        dv[2].s = quad_bcast<1>(f.s); dv[2].y = quad_bcast<1>(dmy.y); z[2] = quad_bcast<1>(f.z);
         dv[3].s = quad_bcast<3>(f.s); dv[3].y = quad_bcast<3>(dmy.y); z[3] = quad_bcast<3>(f.z);
     } else {
         bool ok = true;

@@ -172,18 +172,17 @@ __global__ __launch_bounds__(kBlock) void int4_group_pack4(PackArgs a) {
             mx[u] = fmax_nan(mx[u], x[u][j]);
             mn[u] = fmin_nan(mn[u], x[u][j]);
         }
-        team_minmax<T>(mn[u], mx[u]);
     }
-    // lane lt computes the factors of group lt % 4
-    const int my = lt & 3;
-    const float mx_my = my == 0 ? mx[0] : my == 1 ? mx[1] : my == 2 ? mx[2] : mx[3];
-    const float mn_my = my == 0 ? mn[0] : my == 1 ? mn[1] : my == 2 ? mn[2] : mn[3];
+    // lane lt ends up with the extrema of group seg4_of_lane(lt) and computes its factors
+    const int my = seg4_of_lane(lt);
+    float mx_my, mn_my;
+    team_minmax_scatter4<T>(mn, mx, lt, mn_my, mx_my);
     const Factors f = make_factors<AMCT_F32>(mx_my, mn_my, 4, a.symmetric != 0, AMCT_SCOPE_AMCT);
     const Divisor dmy = make_divisor(f.s);
     const uint32_t big = max(__float_as_uint(mx_my) & 0x7FFFFFFFu, __float_as_uint(mn_my) & 0x7FFFFFFFu);
     const bool fast = wave_all(dmy.fast && big < 0x5D800000u);       // |x| < 2^60, finite
-    if (lt < 4 && seg0 + lt < a.nseg) {
-        const int64_t sg = seg0 + lt;
+    if (lt < 4 && seg0 + my < a.nseg) {
+        const int64_t sg = seg0 + my;
         if (a.scales32) a.scales32[sg] = f.s;
         if (a.scales16) {
             reinterpret_cast<uint16_t*>(a.scales16)[sg] =
@@ -192,29 +191,31 @@ __global__ __launch_bounds__(kBlock) void int4_group_pack4(PackArgs a) {
         if (a.zeros) a.zeros[sg] = (uint8_t)((int)f.z + 8);
         if (f.bad && a.bad) atomicAdd(a.bad, 1);
     }
+    // quad lane holding segment u: u = 0 -> lane 0, 1 -> lane 2, 2 -> lane 1, 3 -> lane 3
     Divisor dv[U];
     float z[U];
     dv[0].s = quad_bcast<0>(f.s); dv[0].y = quad_bcast<0>(dmy.y); z[0] = quad_bcast<0>(f.z);
-    dv[1].s = quad_bcast<1>(f.s); dv[1].y = quad_bcast<1>(dmy.y); z[1] = quad_bcast<1>(f.z);
-    dv[2].s = quad_bcast<2>(f.s); dv[2].y = quad_bcast<2>(dmy.y); z[2] = quad_bcast<2>(f.z);
+    dv[1].s = quad_bcast<2>(f.s); dv[1].y = quad_bcast<2>(dmy.y); z[1] = quad_bcast<2>(f.z);
+    dv[2].s = quad_bcast<1>(f.s); dv[2].y = quad_bcast<1>(dmy.y); z[2] = quad_bcast<1>(f.z);
     dv[3].s = quad_bcast<3>(f.s); dv[3].y = quad_bcast<3>(dmy.y); z[3] = quad_bcast<3>(f.z);
 
     // codes u = q + 8 are gathered by exact fp32 arithmetic: sum (q_j + 8) * 16^j over 4 nibbles
     uint32_t word[U];
-    auto encode = [&](auto fast_tag) {
+    auto encode = [&](auto fast_tag, auto asym_tag) {
         constexpr bool FAST = decltype(fast_tag)::value;
+        constexpr bool ASYM = decltype(asym_tag)::value;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             float lo = 34952.0f, hi = 34952.0f;                  // 8 * (1 + 16 + 256 + 4096)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const float q = quant_elem<DT, false, FAST>(x[u][j], dv[u], z[u], asym, -8.f, 7.f);
+                const float q = quant_elem<DT, false, FAST, false>(x[u][j], dv[u], z[u], ASYM, -8.f, 7.f);
                 lo = __builtin_fmaf(q, (float)(1 << (4 * j)), lo);
             }
             if constexpr (VEC == 8) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const float q = quant_elem<DT, false, FAST>(x[u][4 + j], dv[u], z[u], asym, -8.f, 7.f);
+                    const float q = quant_elem<DT, false, FAST, false>(x[u][4 + j], dv[u], z[u], ASYM, -8.f, 7.f);
                     hi = __builtin_fmaf(q, (float)(1 << (4 * j)), hi);
                 }
                 word[u] = (uint32_t)lo | ((uint32_t)hi << 16);
@@ -223,8 +224,10 @@ __global__ __launch_bounds__(kBlock) void int4_group_pack4(PackArgs a) {
             }
         }
     };
-    if (fast) encode(std::true_type{});
-    else encode(std::false_type{});
+    if (fast && asym) encode(std::true_type{}, std::true_type{});
+    else if (fast) encode(std::true_type{}, std::false_type{});
+    else if (asym) encode(std::false_type{}, std::true_type{});
+    else encode(std::false_type{}, std::false_type{});
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         if (lt < S && seg0 + u < a.nseg) {
