@@ -50,12 +50,16 @@ constexpr int kLoads = (kBM * kBK / 16) / kBlock;   // 16-byte chunks per thread
 
 AMCT_DEV uint4 ld_chunk_or_zero(const int8_t* base, int64_t row, int64_t rows, int64_t K, int64_t k) {
     // rows beyond the matrix are clamped (their results are never stored); k beyond K reads zero
+    // (the load itself is unconditional: a predicated load would force a wait on every load)
     const int64_t r = row < rows ? row : rows - 1;
-    if (k < K) return ldg16(base + r * K + k);
-    return make_uint4(0, 0, 0, 0);
+    const int64_t kk = k < K ? k : K - 16;
+    uint4 v = ldg16(base + r * K + kk);
+    if (k >= K) v = make_uint4(0, 0, 0, 0);
+    return v;
 }
 
-__global__ __launch_bounds__(kBlock) void w8a8_tile(W8A8Args a) {
+template <int ODT>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2, 2))) void w8a8_tile(W8A8Args a) {
     __shared__ __attribute__((aligned(16))) int8_t As[2][kBM * kRow];
     __shared__ __attribute__((aligned(16))) int8_t Bs[2][kBN * kRow];
     const int tid = threadIdx.x;
@@ -65,20 +69,23 @@ __global__ __launch_bounds__(kBlock) void w8a8_tile(W8A8Args a) {
     const int ld_row = tid >> 3, ld_chunk = tid & 7;            // 8 chunks of 16 B per row
     const int nsteps = (int)((a.K + kBK - 1) / kBK);
 
-    uint4 ra[kLoads], rb[kLoads];
-    auto load_global = [&](int step) {
+    // two register stages: the loads of step s+2 are issued while step s is computed and the
+    // registers of step s+1 (loaded one iteration earlier) are moved to the free LDS buffer, so two
+    // K-steps of global traffic are in flight behind the MFMAs
+    uint4 ra[2][kLoads], rb[2][kLoads];
+    auto load_global = [&](int step, uint4* pa, uint4* pb) {
         const int64_t k = (int64_t)step * kBK + ld_chunk * 16;
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
-            ra[i] = ld_chunk_or_zero(a.xq, m0 + ld_row + 32 * i, a.M, a.K, k);
-            rb[i] = ld_chunk_or_zero(a.wq, n0 + ld_row + 32 * i, a.N, a.K, k);
+            pa[i] = ld_chunk_or_zero(a.xq, m0 + ld_row + 32 * i, a.M, a.K, k);
+            pb[i] = ld_chunk_or_zero(a.wq, n0 + ld_row + 32 * i, a.N, a.K, k);
         }
     };
-    auto store_lds = [&](int buf) {
+    auto store_lds = [&](int buf, const uint4* pa, const uint4* pb) {
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
-            *reinterpret_cast<uint4*>(&As[buf][(ld_row + 32 * i) * kRow + ld_chunk * 16]) = ra[i];
-            *reinterpret_cast<uint4*>(&Bs[buf][(ld_row + 32 * i) * kRow + ld_chunk * 16]) = rb[i];
+            *reinterpret_cast<uint4*>(&As[buf][(ld_row + 32 * i) * kRow + ld_chunk * 16]) = pa[i];
+            *reinterpret_cast<uint4*>(&Bs[buf][(ld_row + 32 * i) * kRow + ld_chunk * 16]) = pb[i];
         }
     };
 
@@ -90,13 +97,8 @@ __global__ __launch_bounds__(kBlock) void w8a8_tile(W8A8Args a) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-    load_global(0);
-    store_lds(0);
-    __syncthreads();
     const int frag_row = lane & 31, frag_k = (lane >> 5) * 16;
-    for (int step = 0; step < nsteps; ++step) {
-        const int cur = step & 1;
-        if (step + 1 < nsteps) load_global(step + 1);
+    auto compute = [&](int cur) {
 #pragma unroll
         for (int ks = 0; ks < kBK / 32; ++ks) {
             v4i fa[2], fb[2];
@@ -110,21 +112,58 @@ __global__ __launch_bounds__(kBlock) void w8a8_tile(W8A8Args a) {
 #pragma unroll
                 for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
         }
-        if (step + 1 < nsteps) store_lds(cur ^ 1);
+    };
+
+    // loads past the last step re-read the last step (never used) instead of branching around the load
+    const int last = nsteps - 1;
+    load_global(0, ra[0], rb[0]);
+    load_global(1 < last ? 1 : last, ra[1], rb[1]);
+    store_lds(0, ra[0], rb[0]);
+    __syncthreads();
+    for (int step = 0; step < nsteps; step += 2) {
+        // even step: LDS buffer 0 holds step, registers 1 hold step+1, registers 0 are free
+        load_global(step + 2 < last ? step + 2 : last, ra[0], rb[0]);
+        compute(0);
+        store_lds(1, ra[1], rb[1]);
+        __syncthreads();
+        if (step + 1 >= nsteps) break;
+        // odd step: LDS buffer 1 holds step+1, registers 0 hold step+2, registers 1 are free
+        load_global(step + 3 < last ? step + 3 : last, ra[1], rb[1]);
+        compute(1);
+        store_lds(0, ra[0], rb[0]);
         __syncthreads();
     }
 
-    // epilogue: register r of a 32x32 tile holds row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
+    // epilogue: register r of a 32x32 tile holds row 8*(r/4) + 4*(lane/32) + r%4, column lane%32.
+    // Per-column and per-row factors are fetched once; fp32(acc + ibias) * s_ch * s_tok + fbias.
+    float sc[2], fb[2];
+    int32_t ib[2];
+    int64_t ncol[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        const int64_t n = n0 + wn * 64 + j * 32 + (lane & 31);
-        if (n >= a.N) continue;
+        ncol[j] = n0 + wn * 64 + j * 32 + (lane & 31);
+        const int64_t nc = ncol[j] < a.N ? ncol[j] : a.N - 1;
+        sc[j] = a.s_ch[nc];
+        ib[j] = a.bias_kind == 1 ? reinterpret_cast<const int32_t*>(a.bias)[nc] : 0;
+        fb[j] = a.bias_kind == 2 ? reinterpret_cast<const float*>(a.bias)[nc] : 0.f;
+    }
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < 2; ++i) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int64_t m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (m < a.M) w8a8_epilogue(a, m, n, acc[i][j][r]);
+        for (int r = 0; r < 16; ++r) {
+            const int64_t m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            if (m >= a.M) continue;
+            const float tk = a.s_tok ? a.s_tok[m] : 1.0f;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                if (ncol[j] >= a.N) continue;
+                const int32_t v = acc[i][j][r] + ib[j];
+                const int64_t o = m * a.N + ncol[j];
+                if (a.acc_out) a.acc_out[o] = v;
+                float f = (float)v * sc[j];
+                if (a.s_tok) f = f * tk;
+                if (a.bias_kind == 2) f = f + fb[j];
+                store_scalar<ODT>(a.out, o, f);
             }
         }
     }
@@ -238,7 +277,9 @@ extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s
     if (vec_ok) {
         const dim3 grid((unsigned)((N + kBN - 1) / kBN), (unsigned)((M + kBM - 1) / kBM));
         if (grid.y > 65535) return AMCT_E_UNSUPPORTED;
-        hipLaunchKernelGGL(w8a8_tile, grid, dim3(kBlock), 0, st, a);
+        if (out_dtype == AMCT_BF16) hipLaunchKernelGGL((w8a8_tile<AMCT_BF16>), grid, dim3(kBlock), 0, st, a);
+        else if (out_dtype == AMCT_F16) hipLaunchKernelGGL((w8a8_tile<AMCT_F16>), grid, dim3(kBlock), 0, st, a);
+        else hipLaunchKernelGGL((w8a8_tile<AMCT_F32>), grid, dim3(kBlock), 0, st, a);
         return hip_status();
     }
     const int64_t nb = (M * N + kBlock - 1) / kBlock;
