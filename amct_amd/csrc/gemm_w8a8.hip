@@ -170,6 +170,169 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2, 2))) 
 }
 
 // ---------------------------------------------------------------------------
+// large-tile kernel: 256x256 block tile, 8 waves (2 x 4) of 128x64, BK = 64 bytes, four LDS stages
+// filled by direct global->LDS loads (global_load_lds_dwordx4: no VGPR staging, no ds_write), three
+// K-steps of loads in flight behind the MFMAs, one barrier per K-step, epilogue transposed through LDS
+// so that every lane stores 16 contiguous bytes.
+//
+// A direct-to-LDS load writes the 64 lanes' 16-byte pieces to 1024 contiguous LDS bytes, so the LDS
+// layout is unpadded [row][64 B]; bank conflicts are avoided by a swizzle instead: 16-byte chunk c of
+// row r lives at chunk position c ^ ((r >> 1) & 3), applied by choosing which global chunk a lane
+// fetches.  The loads and their s_waitcnt are inline asm: the compiler would otherwise wait for ALL
+// outstanding direct-to-LDS loads before every LDS read.
+// ---------------------------------------------------------------------------
+constexpr int kLM = 256, kLN = 256, kLK = 64, kLStages = 4, kLThreads = 512;
+constexpr int kLStageBytes = (kLM + kLN) * kLK;                // 32 KiB
+
+AMCT_DEV void dma16(uint32_t lds_addr, const void* gptr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(gptr) : "memory");
+}
+
+template <int ODT>
+__global__ __launch_bounds__(kLThreads) void w8a8_tile256(W8A8Args a) {
+    __shared__ __attribute__((aligned(1024))) int8_t smem[kLStages * kLStageBytes];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 2, wn = wave & 3;
+    const int64_t m0 = (int64_t)blockIdx.y * kLM, n0 = (int64_t)blockIdx.x * kLN;
+    const int nsteps = (int)(a.K / kLK);
+    const int last = nsteps - 1;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t*)smem;
+
+    // this wave's four 1 KiB pieces of a stage: waves 0..3 fetch A rows, waves 4..7 fetch B rows
+    const int8_t* gp[4];
+    {
+        const int rin = lane >> 2;                                  // row inside the 16-row piece
+        const int lc = (lane & 3) ^ ((rin >> 1) & 3);               // logical chunk this lane fetches
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int piece = wave * 4 + j;                         // 0..31
+            if (piece < 16) {
+                const int64_t r = m0 + piece * 16 + rin;
+                gp[j] = a.xq + (r < a.M ? r : a.M - 1) * a.K + lc * 16;
+            } else {
+                const int64_t r = n0 + (piece - 16) * 16 + rin;
+                gp[j] = a.wq + (r < a.N ? r : a.N - 1) * a.K + lc * 16;
+            }
+        }
+    }
+    auto dma_stage = [&](int stage, int step) {
+        const uint32_t base = __builtin_amdgcn_readfirstlane(lds0 + stage * kLStageBytes + wave * 4096);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dma16(base + j * 1024, gp[j] + (int64_t)step * kLK);
+    };
+
+    // fragment offsets: lane reads row (tile base + lane%32), logical chunk 2*ks + lane/32
+    int offA[2], offB[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+        const int r = lane & 31;
+        const int phys = (ks * 2 + (lane >> 5)) ^ ((r >> 1) & 3);
+        offA[ks] = (wm * 128 + r) * kLK + phys * 16;
+        offB[ks] = kLM * kLK + (wn * 64 + r) * kLK + phys * 16;
+    }
+
+    v16i acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+#pragma unroll
+    for (int s = 0; s < kLStages - 1; ++s) dma_stage(s, s < last ? s : last);
+
+    for (int step = 0; step < nsteps; ++step) {
+        // the four loads of `step` are the oldest: allow the 8 of the next two steps to stay in flight
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        // the stage consumed in the previous iteration is free now (every wave passed the barrier)
+        dma_stage((step + 3) & 3, step + 3 < last ? step + 3 : last);
+        const int8_t* st = smem + (step & 3) * kLStageBytes;
+        v4i fa[2][4], fb[2][2];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) fa[ks][i] = *reinterpret_cast<const v4i*>(st + offA[ks] + i * 32 * kLK);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) fb[ks][j] = *reinterpret_cast<const v4i*>(st + offB[ks] + j * 32 * kLK);
+        }
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[ks][i], fb[ks][j], acc[i][j], 0, 0, 0);
+    }
+    // all loads landed and every wave is done with the stages before LDS is reused
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+
+    // epilogue: fp32(acc + ibias) * s_ch * s_tok + fbias, narrowed, transposed through a per-wave LDS
+    // patch of 32 rows x 64 columns, stored as 16-byte pieces of full rows
+    constexpr int ES = (ODT == AMCT_F32) ? 4 : 2;                   // bytes per output element
+    constexpr int kPatchRow = 64 * ES + 16;                        // padded patch row
+    constexpr int CPR = 64 * ES / 16;                              // 16-byte chunks per patch row
+    constexpr int RPI = 64 / CPR;                                  // patch rows covered by one wave-wide read
+    int8_t* patch = smem + wave * 16384;
+    float sc[2], fb2[2];
+    int32_t ib[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int64_t n = n0 + wn * 64 + j * 32 + (lane & 31);
+        const int64_t nc = n < a.N ? n : a.N - 1;
+        sc[j] = a.s_ch[nc];
+        ib[j] = a.bias_kind == 1 ? reinterpret_cast<const int32_t*>(a.bias)[nc] : 0;
+        fb2[j] = a.bias_kind == 2 ? reinterpret_cast<const float*>(a.bias)[nc] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int64_t mbase = m0 + wm * 128 + i * 32;
+        float tks[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {                              // all 16 row factors in flight together
+            const int64_t m = mbase + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            tks[r] = a.s_tok ? a.s_tok[m < a.M ? m : a.M - 1] : 1.0f;
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int prow = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            const int64_t m = mbase + prow;
+            const float tk = tks[r];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int32_t v = acc[i][j][r] + ib[j];
+                if (a.acc_out) {
+                    const int64_t n = n0 + wn * 64 + j * 32 + (lane & 31);
+                    if (m < a.M && n < a.N) a.acc_out[m * a.N + n] = v;
+                }
+                float f = (float)v * sc[j];
+                if (a.s_tok) f = f * tk;
+                if (a.bias_kind == 2) f = f + fb2[j];
+                int8_t* dst = patch + prow * kPatchRow + (j * 32 + (lane & 31)) * ES;
+                if constexpr (ODT == AMCT_F32) *reinterpret_cast<float*>(dst) = f;
+                else if constexpr (ODT == AMCT_BF16) *reinterpret_cast<uint16_t*>(dst) = (uint16_t)f32_to_bf16_bits(f);
+                else *reinterpret_cast<uint16_t*>(dst) = (uint16_t)f32_to_f16_bits(f);
+            }
+        }
+        // LDS operations of one wave complete in order: the reads below see the writes above
+#pragma unroll
+        for (int it = 0; it < 32 / RPI; ++it) {
+            const int prow = it * RPI + lane / CPR;
+            const int chunk = lane % CPR;
+            const uint4 v = *reinterpret_cast<const uint4*>(patch + prow * kPatchRow + chunk * 16);
+            const int64_t m = mbase + prow;
+            const int64_t n = n0 + wn * 64 + chunk * (16 / ES);
+            if (m < a.M && n < a.N) stg16(reinterpret_cast<char*>(a.out) + (m * a.N + n) * ES, v);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // skinny kernel: M <= 16 * MT.  One block = 16 output columns; its 4 waves split K.
 // Lane l of a wave streams row n0 + l%16 of the weight, 16 bytes per MFMA, k-slot l/16.
 // ---------------------------------------------------------------------------
@@ -272,6 +435,14 @@ extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s
         else if (M <= 32) hipLaunchKernelGGL((w8a8_skinny<2>), grid, dim3(kBlock), 0, st, a);
         else if (M <= 48) hipLaunchKernelGGL((w8a8_skinny<3>), grid, dim3(kBlock), 0, st, a);
         else hipLaunchKernelGGL((w8a8_skinny<4>), grid, dim3(kBlock), 0, st, a);
+        return hip_status();
+    }
+    if (vec_ok && M >= 256 && K % kLK == 0 && K >= kLK && N % 8 == 0 && aligned16(out)) {
+        const dim3 grid((unsigned)((N + kLN - 1) / kLN), (unsigned)((M + kLM - 1) / kLM));
+        if (grid.y > 65535) return AMCT_E_UNSUPPORTED;
+        if (out_dtype == AMCT_BF16) hipLaunchKernelGGL((w8a8_tile256<AMCT_BF16>), grid, dim3(kLThreads), 0, st, a);
+        else if (out_dtype == AMCT_F16) hipLaunchKernelGGL((w8a8_tile256<AMCT_F16>), grid, dim3(kLThreads), 0, st, a);
+        else hipLaunchKernelGGL((w8a8_tile256<AMCT_F32>), grid, dim3(kLThreads), 0, st, a);
         return hip_status();
     }
     if (vec_ok) {
