@@ -3,8 +3,10 @@
 //
 // Both operands are K-contiguous, which is the natural operand order of the gfx950 int8 MFMA
 // (v_mfma_i32_32x32x32_i8: lane l supplies 16 consecutive k-bytes of row l%32, k-half l/32).
-//   tile kernel   : 128x128 block tile, 4 waves of 64x64, BK = 128 bytes, LDS double buffered,
-//                   global loads of step k+1 in flight while step k feeds the MFMAs.
+//   large tiles   : 256x256 block tile, 8 waves of 128x64, BK = 64 bytes, 4 LDS stages filled by
+//                   direct global->LDS loads, fragment reads software-pipelined against the MFMAs.
+//   tile kernel   : 128x128 block tile, 4 waves of 64x64, BK = 128 bytes, two register stages of
+//                   prefetch (shapes the large-tile kernel does not take).
 //   skinny kernel : M <= 64 (decode): the weight is streamed once straight from HBM into MFMA
 //                   operands (v_mfma_i32_16x16x64_i8), split-K across the 4 waves of a block.
 //   general kernel: any shape, one output per thread.
@@ -177,49 +179,57 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2, 2))) 
 //
 // A direct-to-LDS load writes the 64 lanes' 16-byte pieces to 1024 contiguous LDS bytes, so the LDS
 // layout is unpadded [row][64 B]; bank conflicts are avoided by a swizzle instead: 16-byte chunk c of
-// row r lives at chunk position c ^ ((r >> 1) & 3), applied by choosing which global chunk a lane
+// row r lives at chunk position c ^ ((r >> 2) & 3) (measured conflict-free with SQ_LDS_BANK_CONFLICT), applied by choosing which global chunk a lane
 // fetches.  The loads and their s_waitcnt are inline asm: the compiler would otherwise wait for ALL
 // outstanding direct-to-LDS loads before every LDS read.
 // ---------------------------------------------------------------------------
-constexpr int kLM = 256, kLN = 256, kLK = 64, kLStages = 4, kLThreads = 512;
-constexpr int kLStageBytes = (kLM + kLN) * kLK;                // 32 KiB
+constexpr int kLK = 64;
 
 AMCT_DEV void dma16(uint32_t lds_addr, const void* gptr) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(gptr) : "memory");
 }
+template <int N> AMCT_DEV void wait_dma_lds() { asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"(N) : "memory"); }
 
-template <int ODT>
-__global__ __launch_bounds__(kLThreads) void w8a8_tile256(W8A8Args a) {
-    __shared__ __attribute__((aligned(1024))) int8_t smem[kLStages * kLStageBytes];
+// WM x WN waves of 128x64 each: block tile (128*WM) x (64*WN); STAGES LDS stages of BK = 64 bytes
+template <int ODT, int WM, int WN, int STAGES>
+__global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void w8a8_tile_dma(W8A8Args a) {
+    constexpr int kLM = 128 * WM, kLN = 64 * WN, kWaves = WM * WN;
+    constexpr int kLStageBytes = (kLM + kLN) * kLK;
+    constexpr int kPieces = (kLM + kLN) / 16;                      // 1 KiB pieces per stage
+    constexpr int kPPW = kPieces / kWaves;                         // pieces per wave
+    static_assert(kPieces % kWaves == 0, "pieces must divide evenly among the waves");
+    constexpr int kEpiBytes = kWaves * 16384;
+    constexpr int kSmem = STAGES * kLStageBytes > kEpiBytes ? STAGES * kLStageBytes : kEpiBytes;
+    __shared__ __attribute__((aligned(1024))) int8_t smem[kSmem];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 2, wn = wave & 3;
+    const int wm = wave / WN, wn = wave % WN;
     const int64_t m0 = (int64_t)blockIdx.y * kLM, n0 = (int64_t)blockIdx.x * kLN;
     const int nsteps = (int)(a.K / kLK);
     const int last = nsteps - 1;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t*)smem;
 
-    // this wave's four 1 KiB pieces of a stage: waves 0..3 fetch A rows, waves 4..7 fetch B rows
-    const int8_t* gp[4];
+    // this wave's 1 KiB pieces of a stage: pieces 0 .. kLM/16-1 are A rows, the rest B rows
+    const int8_t* gp[kPPW];
     {
         const int rin = lane >> 2;                                  // row inside the 16-row piece
-        const int lc = (lane & 3) ^ ((rin >> 1) & 3);               // logical chunk this lane fetches
+        const int lc = (lane & 3) ^ ((rin >> 2) & 3);               // logical chunk this lane fetches
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int piece = wave * 4 + j;                         // 0..31
-            if (piece < 16) {
+        for (int j = 0; j < kPPW; ++j) {
+            const int piece = wave * kPPW + j;
+            if (piece < kLM / 16) {
                 const int64_t r = m0 + piece * 16 + rin;
                 gp[j] = a.xq + (r < a.M ? r : a.M - 1) * a.K + lc * 16;
             } else {
-                const int64_t r = n0 + (piece - 16) * 16 + rin;
+                const int64_t r = n0 + (piece - kLM / 16) * 16 + rin;
                 gp[j] = a.wq + (r < a.N ? r : a.N - 1) * a.K + lc * 16;
             }
         }
     }
     auto dma_stage = [&](int stage, int step) {
-        const uint32_t base = __builtin_amdgcn_readfirstlane(lds0 + stage * kLStageBytes + wave * 4096);
+        const uint32_t base = __builtin_amdgcn_readfirstlane(lds0 + stage * kLStageBytes + wave * kPPW * 1024);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) dma16(base + j * 1024, gp[j] + (int64_t)step * kLK);
+        for (int j = 0; j < kPPW; ++j) dma16(base + j * 1024, gp[j] + (int64_t)step * kLK);
     };
 
     // fragment offsets: lane reads row (tile base + lane%32), logical chunk 2*ks + lane/32
@@ -227,7 +237,7 @@ __global__ __launch_bounds__(kLThreads) void w8a8_tile256(W8A8Args a) {
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
         const int r = lane & 31;
-        const int phys = (ks * 2 + (lane >> 5)) ^ ((r >> 1) & 3);
+        const int phys = (ks * 2 + (lane >> 5)) ^ ((r >> 2) & 3);
         offA[ks] = (wm * 128 + r) * kLK + phys * 16;
         offB[ks] = kLM * kLK + (wn * 64 + r) * kLK + phys * 16;
     }
@@ -241,31 +251,44 @@ __global__ __launch_bounds__(kLThreads) void w8a8_tile256(W8A8Args a) {
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
 #pragma unroll
-    for (int s = 0; s < kLStages - 1; ++s) dma_stage(s, s < last ? s : last);
+    for (int s = 0; s < STAGES - 1; ++s) dma_stage(s, s < last ? s : last);
 
+    auto read_frags = [&](int stage, int ks, v4i (&fa)[4], v4i (&fb)[2]) {
+        const int8_t* st = smem + stage * kLStageBytes;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) fa[i] = *reinterpret_cast<const v4i*>(st + offA[ks] + i * 32 * kLK);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) fb[j] = *reinterpret_cast<const v4i*>(st + offB[ks] + j * 32 * kLK);
+    };
+    auto mfma_half = [&](const v4i (&fa)[4], const v4i (&fb)[2]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    };
+
+    // software pipeline over half K-steps: while the 8 MFMAs of one half run, the fragments of the
+    // next half are read from LDS.  At the barrier of iteration s every wave holds the last fragments
+    // of stage s % STAGES in registers (lgkmcnt(0)), so that stage is free for the loads of step
+    // s + STAGES; the loads of the STAGES-2 steps after s+1 stay in flight.
+    v4i fa0[4], fb0[2], fa1[4], fb1[2];
+    wait_dma_lds<(STAGES - 2) * kPPW>();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    dma_stage(STAGES - 1, STAGES - 1 < last ? STAGES - 1 : last);
+    read_frags(0, 0, fa0, fb0);
+    int stage = 0;
     for (int step = 0; step < nsteps; ++step) {
-        // the four loads of `step` are the oldest: allow the 8 of the next two steps to stay in flight
-        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        const int next = stage + 1 == STAGES ? 0 : stage + 1;
+        read_frags(stage, 1, fa1, fb1);
+        mfma_half(fa0, fb0);
+        wait_dma_lds<(STAGES - 2) * kPPW>();
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        // the stage consumed in the previous iteration is free now (every wave passed the barrier)
-        dma_stage((step + 3) & 3, step + 3 < last ? step + 3 : last);
-        const int8_t* st = smem + (step & 3) * kLStageBytes;
-        v4i fa[2][4], fb[2][2];
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) fa[ks][i] = *reinterpret_cast<const v4i*>(st + offA[ks] + i * 32 * kLK);
-#pragma unroll
-            for (int j = 0; j < 2; ++j) fb[ks][j] = *reinterpret_cast<const v4i*>(st + offB[ks] + j * 32 * kLK);
-        }
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[ks][i], fb[ks][j], acc[i][j], 0, 0, 0);
+        dma_stage(stage, step + STAGES < last ? step + STAGES : last);
+        if (step + 1 < nsteps) read_frags(next, 0, fa0, fb0);
+        mfma_half(fa1, fb1);
+        stage = next;
     }
     // all loads landed and every wave is done with the stages before LDS is reused
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -438,11 +461,13 @@ extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s
         return hip_status();
     }
     if (vec_ok && M >= 256 && K % kLK == 0 && K >= kLK && N % 8 == 0 && aligned16(out)) {
-        const dim3 grid((unsigned)((N + kLN - 1) / kLN), (unsigned)((M + kLM - 1) / kLM));
+        // 256x256 tiles, 8 waves, 4 stages (measured faster than 256x128 with two blocks per CU:
+        // the traffic from L2 into LDS matters more than decoupling the barriers)
+        const dim3 grid((unsigned)((N + 255) / 256), (unsigned)((M + 255) / 256));
         if (grid.y > 65535) return AMCT_E_UNSUPPORTED;
-        if (out_dtype == AMCT_BF16) hipLaunchKernelGGL((w8a8_tile256<AMCT_BF16>), grid, dim3(kLThreads), 0, st, a);
-        else if (out_dtype == AMCT_F16) hipLaunchKernelGGL((w8a8_tile256<AMCT_F16>), grid, dim3(kLThreads), 0, st, a);
-        else hipLaunchKernelGGL((w8a8_tile256<AMCT_F32>), grid, dim3(kLThreads), 0, st, a);
+        if (out_dtype == AMCT_BF16) hipLaunchKernelGGL((w8a8_tile_dma<AMCT_BF16, 2, 4, 4>), grid, dim3(512), 0, st, a);
+        else if (out_dtype == AMCT_F16) hipLaunchKernelGGL((w8a8_tile_dma<AMCT_F16, 2, 4, 4>), grid, dim3(512), 0, st, a);
+        else hipLaunchKernelGGL((w8a8_tile_dma<AMCT_F32, 2, 4, 4>), grid, dim3(512), 0, st, a);
         return hip_status();
     }
     if (vec_ok) {
