@@ -11,6 +11,8 @@
 //   skinny kernel : M <= 64 (decode): weights streamed once from HBM, dequantised in registers,
 //                   bf16 MFMA 16x16x32, split-K over the 4 waves of a block.
 //   general kernel: any shape, one output per thread.
+#include <type_traits>
+
 #include "amct_common.h"
 
 namespace amct {
@@ -166,6 +168,190 @@ __global__ __launch_bounds__(kBlock) void w4a16_tile(W4A16Args a) {
 }
 
 // ---------------------------------------------------------------------------
+// large-tile kernel: 256x256 block tile, 8 waves (2 x 4) of 128x64, BK = 32 elements (64-byte rows of
+// bf16), four LDS stages.  The activation tile arrives by direct global->LDS loads; the weight tile is
+// fetched as packed nibbles into registers four K-steps ahead (8 bytes = 16 weights per thread and
+// step), dequantised and written to its LDS stage one step before use.  All global loads and their
+// s_waitcnt are inline asm so that the compiler never drains the queue of direct-to-LDS loads; a load
+// issued in iteration t is guaranteed complete at the wait of iteration t+3 because the counter
+// retires in order and every iteration issues the same number of operations.
+// LDS layout as in the int8 kernel: unpadded [row][64 B], 16-byte chunk c of row r at c ^ ((r >> 2) & 3).
+// ---------------------------------------------------------------------------
+constexpr int kQK = 32;                                            // elements per K-step
+constexpr int kQRow = 64;                                          // bytes per LDS row
+constexpr int kQM = 256, kQN = 256, kQStages = 4, kQThreads = 512;
+constexpr int kQStageBytes = (kQM + kQN) * kQRow;                  // 32 KiB
+constexpr int kQPPW = (kQM / 16) / 8;                              // activation pieces per wave: 2
+constexpr int kQOps = kQPPW + 3;                                   // vm operations per thread and iteration
+
+AMCT_DEV void dma16(uint32_t lds_addr, const void* gptr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(gptr) : "memory");
+}
+AMCT_DEV void gload8(uint64_t& dst, const void* p) { asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(dst) : "v"(p) : "memory"); }
+AMCT_DEV void gload_u16(uint32_t& dst, const void* p) { asm volatile("global_load_ushort %0, %1, off" : "=v"(dst) : "v"(p) : "memory"); }
+AMCT_DEV void gload_u8(uint32_t& dst, const void* p) { asm volatile("global_load_ubyte %0, %1, off" : "=v"(dst) : "v"(p) : "memory"); }
+
+__global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void w4a16_tile_dma(W4A16Args a) {
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[kQStages * kQStageBytes];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 2, wn = wave & 3;
+    const int64_t m0 = (int64_t)blockIdx.y * kQM, n0 = (int64_t)blockIdx.x * kQN;
+    const int nsteps = (int)(a.K / kQK);
+    const int last = nsteps - 1;
+    const int64_t G = a.K / a.group;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
+
+    // activation pieces of this wave (16 rows x 64 B each)
+    const uint16_t* gp[kQPPW];
+    {
+        const int rin = lane >> 2;
+        const int lc = (lane & 3) ^ ((rin >> 2) & 3);
+#pragma unroll
+        for (int j = 0; j < kQPPW; ++j) {
+            const int64_t r = m0 + (wave * kQPPW + j) * 16 + rin;
+            gp[j] = a.x + (r < a.M ? r : a.M - 1) * a.K + lc * 8;
+        }
+    }
+    // weight row of this thread: row tid/2, 16 weights (8 bytes) per step, which half from tid%2
+    const int brow = tid >> 1, bhalf = tid & 1;
+    const int64_t wrow = (n0 + brow < a.N) ? n0 + brow : a.N - 1;
+    const uint8_t* wp = a.wq + wrow * (a.K / 2) + bhalf * 8;
+    const int bphys0 = (bhalf * 2) ^ ((brow >> 2) & 3), bphys1 = (bhalf * 2 + 1) ^ ((brow >> 2) & 3);
+    const int boff0 = kQM * kQRow + brow * kQRow + bphys0 * 16, boff1 = kQM * kQRow + brow * kQRow + bphys1 * 16;
+    const int sbytes = 2;
+    const uint8_t* sp = reinterpret_cast<const uint8_t*>(a.scales) + wrow * G * sbytes;
+    const uint8_t* zp = a.zeros + wrow * G;
+
+    uint64_t wreg[4];
+    uint32_t sreg[4], zreg[4];
+    auto issue = [&](int slot, int stage, int step) {              // the loads of K-step `step`
+        const int st = step < last ? step : last;
+        const int64_t k = (int64_t)st * kQK;
+        const int64_t gi = (k + bhalf * 16) / a.group;
+        gload8(wreg[slot], wp + k / 2);
+        gload_u16(sreg[slot], sp + gi * sbytes);
+        gload_u8(zreg[slot], zp + gi);
+        const uint32_t base = __builtin_amdgcn_readfirstlane(lds0 + stage * kQStageBytes + wave * kQPPW * 1024);
+#pragma unroll
+        for (int j = 0; j < kQPPW; ++j) dma16(base + j * 1024, gp[j] + k);
+    };
+    auto write_b = [&](int slot, int stage) {                      // dequantise 16 weights into LDS
+        const float sc = a.scale_dtype == AMCT_F16 ? f16_bits_to_f32(sreg[slot]) : bf16_bits_to_f32(sreg[slot]);
+        const float nzs = -((float)zreg[slot] * sc);
+        uint8_t* st = smem + stage * kQStageBytes;
+        *reinterpret_cast<uint4*>(st + boff0) = dequant8((uint32_t)wreg[slot], sc, nzs);
+        *reinterpret_cast<uint4*>(st + boff1) = dequant8((uint32_t)(wreg[slot] >> 32), sc, nzs);
+    };
+    // wait until at most N vm operations are outstanding and all LDS operations are done; the slot's
+    // registers are tied to the statement so that their uses stay behind it
+#define AMCT_WAIT_SLOT(N, slot) \
+    asm volatile("s_waitcnt vmcnt(%3) lgkmcnt(0)" : "+v"(wreg[slot]), "+v"(sreg[slot]), "+v"(zreg[slot]) : "n"(N) : "memory")
+
+    int offA[2], offB[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+        const int r = lane & 31;
+        const int phys = (ks * 2 + (lane >> 5)) ^ ((r >> 2) & 3);
+        offA[ks] = (wm * 128 + r) * kQRow + phys * 16;
+        offB[ks] = kQM * kQRow + (wn * 64 + r) * kQRow + phys * 16;
+    }
+    v16f acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    auto read_frags = [&](int stage, int ks, v8bf (&fa)[4], v8bf (&fb)[2]) {
+        const uint8_t* st = smem + stage * kQStageBytes;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) fa[i] = *reinterpret_cast<const v8bf*>(st + offA[ks] + i * 32 * kQRow);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) fb[j] = *reinterpret_cast<const v8bf*>(st + offB[ks] + j * 32 * kQRow);
+    };
+    auto mfma_half = [&](const v8bf (&fa)[4], const v8bf (&fb)[2]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    };
+
+    // prologue: the loads of steps 0..3; step 0 must have landed before its weights are dequantised
+#pragma unroll
+    for (int s = 0; s < 4; ++s) issue(s, s, s);
+    AMCT_WAIT_SLOT(3 * kQOps, 0);
+    write_b(0, 0);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    v8bf fa0[4], fb0[2], fa1[4], fb1[2];
+    read_frags(0, 0, fa0, fb0);
+
+    // iteration t (stage/slot U = t % 4): second half of the fragments of step t, MFMAs of the first
+    // half; wait for the loads of step t+1; dequantise the weights of step t+1 into their stage;
+    // barrier; issue the loads of step t+4 into stage/slot U (both free now); first half of step t+1.
+#define AMCT_ITER(U, NX, step)                           \
+    {                                                    \
+        read_frags(U, 1, fa1, fb1);                      \
+        mfma_half(fa0, fb0);                             \
+        AMCT_WAIT_SLOT(2 * kQOps, NX);                   \
+        write_b(NX, NX);                                 \
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); \
+        __builtin_amdgcn_s_barrier();                    \
+        asm volatile("" ::: "memory");                   \
+        issue(U, U, (step) + 4);                         \
+        read_frags(NX, 0, fa0, fb0);                     \
+        mfma_half(fa1, fb1);                             \
+    }
+    for (int step = 0; step < nsteps; step += 4) {
+        AMCT_ITER(0, 1, step)
+        AMCT_ITER(1, 2, step + 1)
+        AMCT_ITER(2, 3, step + 2)
+        AMCT_ITER(3, 0, step + 3)
+    }
+#undef AMCT_ITER
+#undef AMCT_WAIT_SLOT
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+
+    // epilogue: + bias, narrow to bf16, transpose through a per-wave LDS patch, 16-byte stores
+    constexpr int kPatchRow = 64 * 2 + 16;
+    uint8_t* patch = smem + wave * 16384;
+    float bs[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int64_t n = n0 + wn * 64 + j * 32 + (lane & 31);
+        bs[j] = a.bias ? a.bias[n < a.N ? n : a.N - 1] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int64_t mbase = m0 + wm * 128 + i * 32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int prow = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                float v = acc[i][j][r];
+                if (a.bias) v = v + bs[j];
+                *reinterpret_cast<uint16_t*>(patch + prow * kPatchRow + (j * 32 + (lane & 31)) * 2) = (uint16_t)f32_to_bf16_bits(v);
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int prow = it * 8 + (lane >> 3);
+            const int chunk = lane & 7;
+            const uint4 v = *reinterpret_cast<const uint4*>(patch + prow * kPatchRow + chunk * 16);
+            const int64_t m = mbase + prow;
+            const int64_t n = n0 + wn * 64 + chunk * 8;
+            if (m < a.M && n < a.N) stg16(reinterpret_cast<char*>(a.out) + (m * a.N + n) * 2, v);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // skinny kernel: M <= 16 * MT.  One block = 16 output columns, its 4 waves split K.
 // Per iteration a wave covers 128 k: lane (r = l%16, g = l/16) loads the 32 nibbles
 // k = kb + 32g .. +32 of weight row n0 + r; MFMA s (0..3) consumes nibbles 8s..8s+7 of every lane,
@@ -294,6 +480,12 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
         else if (M <= 32) hipLaunchKernelGGL((w4a16_skinny<2>), grid, dim3(kBlock), 0, st, a);
         else if (M <= 48) hipLaunchKernelGGL((w4a16_skinny<3>), grid, dim3(kBlock), 0, st, a);
         else hipLaunchKernelGGL((w4a16_skinny<4>), grid, dim3(kBlock), 0, st, a);
+        return hip_status();
+    }
+    if (vec_ok && !smooth && M >= 256 && K % 128 == 0 && N % 8 == 0 && group % 16 == 0 && aligned16(out)) {
+        const dim3 grid((unsigned)((N + kQN - 1) / kQN), (unsigned)((M + kQM - 1) / kQM));
+        if (grid.y > 65535) return AMCT_E_UNSUPPORTED;
+        hipLaunchKernelGGL(w4a16_tile_dma, grid, dim3(kQThreads), 0, st, a);
         return hip_status();
     }
     if (vec_ok && K % kTK == 0) {
