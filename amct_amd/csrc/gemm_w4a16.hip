@@ -182,16 +182,19 @@ constexpr int kQRow = 64;                                          // bytes per 
 constexpr int kQM = 256, kQN = 256, kQStages = 4, kQThreads = 512;
 constexpr int kQStageBytes = (kQM + kQN) * kQRow;                  // 32 KiB
 constexpr int kQPPW = (kQM / 16) / 8;                              // activation pieces per wave: 2
-constexpr int kQOps = kQPPW + 3;                                   // vm operations per thread and iteration
+template <bool SMOOTH> constexpr int kQOps = kQPPW + 3 + (SMOOTH ? 1 : 0);   // vm operations per thread and iteration
 
 AMCT_DEV void dma16(uint32_t lds_addr, const void* gptr) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(gptr) : "memory");
 }
+AMCT_DEV void gload16(u4v& dst, const void* p) { asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(p) : "memory"); }
 AMCT_DEV void gload8(uint64_t& dst, const void* p) { asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(dst) : "v"(p) : "memory"); }
 AMCT_DEV void gload_u16(uint32_t& dst, const void* p) { asm volatile("global_load_ushort %0, %1, off" : "=v"(dst) : "v"(p) : "memory"); }
 AMCT_DEV void gload_u8(uint32_t& dst, const void* p) { asm volatile("global_load_ubyte %0, %1, off" : "=v"(dst) : "v"(p) : "memory"); }
 
+template <bool SMOOTH>
 __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void w4a16_tile_dma(W4A16Args a) {
+    constexpr int OPS = kQOps<SMOOTH>;
     __shared__ __attribute__((aligned(1024))) uint8_t smem[kQStages * kQStageBytes];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -204,9 +207,11 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
 
     // activation pieces of this wave (16 rows x 64 B each)
     const uint16_t* gp[kQPPW];
+    const uint16_t* smp = nullptr;                                 // smooth factors of this lane's chunk
     {
         const int rin = lane >> 2;
         const int lc = (lane & 3) ^ ((rin >> 2) & 3);
+        if constexpr (SMOOTH) smp = a.smooth + lc * 8;
 #pragma unroll
         for (int j = 0; j < kQPPW; ++j) {
             const int64_t r = m0 + (wave * kQPPW + j) * 16 + rin;
@@ -225,6 +230,7 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
 
     uint64_t wreg[4];
     uint32_t sreg[4], zreg[4];
+    u4v mreg[4];
     auto issue = [&](int slot, int stage, int step) {              // the loads of K-step `step`
         const int st = step < last ? step : last;
         const int64_t k = (int64_t)st * kQK;
@@ -232,6 +238,7 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
         gload8(wreg[slot], wp + k / 2);
         gload_u16(sreg[slot], sp + gi * sbytes);
         gload_u8(zreg[slot], zp + gi);
+        if constexpr (SMOOTH) gload16(mreg[slot], smp + k);
         const uint32_t base = __builtin_amdgcn_readfirstlane(lds0 + stage * kQStageBytes + wave * kQPPW * 1024);
 #pragma unroll
         for (int j = 0; j < kQPPW; ++j) dma16(base + j * 1024, gp[j] + k);
@@ -243,10 +250,22 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
         *reinterpret_cast<uint4*>(st + boff0) = dequant8((uint32_t)wreg[slot], sc, nzs);
         *reinterpret_cast<uint4*>(st + boff1) = dequant8((uint32_t)(wreg[slot] >> 32), sc, nzs);
     };
+    // x' = bf16(x * smooth) in place on the pieces this wave fetched itself (lane l owns bytes
+    // 16 l .. 16 l + 15 of each piece), one K-step before the stage is consumed
+    auto smooth_a = [&](int slot, int stage) {
+        uint8_t* st = smem + stage * kQStageBytes + wave * kQPPW * 1024 + lane * 16;
+        const uint4 c = make_uint4(mreg[slot].x, mreg[slot].y, mreg[slot].z, mreg[slot].w);
+#pragma unroll
+        for (int j = 0; j < kQPPW; ++j) {
+            uint4* p = reinterpret_cast<uint4*>(st + j * 1024);
+            *p = smooth8(*p, c);
+        }
+    };
     // wait until at most N vm operations are outstanding and all LDS operations are done; the slot's
     // registers are tied to the statement so that their uses stay behind it
 #define AMCT_WAIT_SLOT(N, slot) \
     asm volatile("s_waitcnt vmcnt(%3) lgkmcnt(0)" : "+v"(wreg[slot]), "+v"(sreg[slot]), "+v"(zreg[slot]) : "n"(N) : "memory")
+#define AMCT_TIE_SMOOTH(slot) asm volatile("" : "+v"(mreg[slot]) : : "memory")
 
     int offA[2], offB[2];
 #pragma unroll
@@ -281,7 +300,15 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
     // prologue: the loads of steps 0..3; step 0 must have landed before its weights are dequantised
 #pragma unroll
     for (int s = 0; s < 4; ++s) issue(s, s, s);
-    AMCT_WAIT_SLOT(3 * kQOps, 0);
+    if constexpr (SMOOTH) {
+        AMCT_WAIT_SLOT(2 * OPS, 0);                                 // steps 0 and 1 have landed
+        AMCT_TIE_SMOOTH(0);
+        AMCT_TIE_SMOOTH(1);
+        smooth_a(0, 0);
+        smooth_a(1, 1);
+    } else {
+        AMCT_WAIT_SLOT(3 * OPS, 0);
+    }
     write_b(0, 0);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
@@ -292,11 +319,18 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
     // iteration t (stage/slot U = t % 4): second half of the fragments of step t, MFMAs of the first
     // half; wait for the loads of step t+1; dequantise the weights of step t+1 into their stage;
     // barrier; issue the loads of step t+4 into stage/slot U (both free now); first half of step t+1.
-#define AMCT_ITER(U, NX, step)                           \
+    // With smoothing the loads of step t+2 must have landed too (they are multiplied in place now).
+#define AMCT_ITER(U, NX, NX2, step)                      \
     {                                                    \
         read_frags(U, 1, fa1, fb1);                      \
         mfma_half(fa0, fb0);                             \
-        AMCT_WAIT_SLOT(2 * kQOps, NX);                   \
+        if constexpr (SMOOTH) {                          \
+            AMCT_WAIT_SLOT(OPS, NX);                     \
+            AMCT_TIE_SMOOTH(NX2);                        \
+            smooth_a(NX2, NX2);                          \
+        } else {                                         \
+            AMCT_WAIT_SLOT(2 * OPS, NX);                 \
+        }                                                \
         write_b(NX, NX);                                 \
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); \
         __builtin_amdgcn_s_barrier();                    \
@@ -306,13 +340,14 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
         mfma_half(fa1, fb1);                             \
     }
     for (int step = 0; step < nsteps; step += 4) {
-        AMCT_ITER(0, 1, step)
-        AMCT_ITER(1, 2, step + 1)
-        AMCT_ITER(2, 3, step + 2)
-        AMCT_ITER(3, 0, step + 3)
+        AMCT_ITER(0, 1, 2, step)
+        AMCT_ITER(1, 2, 3, step + 1)
+        AMCT_ITER(2, 3, 0, step + 2)
+        AMCT_ITER(3, 0, 1, step + 3)
     }
 #undef AMCT_ITER
 #undef AMCT_WAIT_SLOT
+#undef AMCT_TIE_SMOOTH
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
@@ -482,10 +517,11 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
         else hipLaunchKernelGGL((w4a16_skinny<4>), grid, dim3(kBlock), 0, st, a);
         return hip_status();
     }
-    if (vec_ok && !smooth && M >= 256 && K % 128 == 0 && N % 8 == 0 && group % 16 == 0 && aligned16(out)) {
+    if (vec_ok && M >= 256 && K % 128 == 0 && N % 8 == 0 && group % 16 == 0 && aligned16(out)) {
         const dim3 grid((unsigned)((N + kQN - 1) / kQN), (unsigned)((M + kQM - 1) / kQM));
         if (grid.y > 65535) return AMCT_E_UNSUPPORTED;
-        hipLaunchKernelGGL(w4a16_tile_dma, grid, dim3(kQThreads), 0, st, a);
+        if (smooth) hipLaunchKernelGGL((w4a16_tile_dma<true>), grid, dim3(kQThreads), 0, st, a);
+        else hipLaunchKernelGGL((w4a16_tile_dma<false>), grid, dim3(kQThreads), 0, st, a);
         return hip_status();
     }
     if (vec_ok && K % kTK == 0) {
