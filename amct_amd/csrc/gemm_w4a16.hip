@@ -251,15 +251,20 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
         *reinterpret_cast<uint4*>(st + boff1) = dequant8((uint32_t)(wreg[slot] >> 32), sc, nzs);
     };
     // x' = bf16(x * smooth) in place on the pieces this wave fetched itself (lane l owns bytes
-    // 16 l .. 16 l + 15 of each piece), one K-step before the stage is consumed
-    auto smooth_a = [&](int slot, int stage) {
+    // 16 l .. 16 l + 15 of each piece).  Split in two so that the LDS read latency is not exposed: the
+    // raw chunks are read in the second half of iteration t, multiplied and written back in the first
+    // half of iteration t+1, one barrier before the stage is consumed.
+    uint4 araw[kQPPW];
+    auto smooth_read = [&](int stage) {
+        const uint8_t* st = smem + stage * kQStageBytes + wave * kQPPW * 1024 + lane * 16;
+#pragma unroll
+        for (int j = 0; j < kQPPW; ++j) araw[j] = *reinterpret_cast<const uint4*>(st + j * 1024);
+    };
+    auto smooth_write = [&](int slot, int stage) {
         uint8_t* st = smem + stage * kQStageBytes + wave * kQPPW * 1024 + lane * 16;
         const uint4 c = make_uint4(mreg[slot].x, mreg[slot].y, mreg[slot].z, mreg[slot].w);
 #pragma unroll
-        for (int j = 0; j < kQPPW; ++j) {
-            uint4* p = reinterpret_cast<uint4*>(st + j * 1024);
-            *p = smooth8(*p, c);
-        }
+        for (int j = 0; j < kQPPW; ++j) *reinterpret_cast<uint4*>(st + j * 1024) = smooth8(araw[j], c);
     };
     // wait until at most N vm operations are outstanding and all LDS operations are done; the slot's
     // registers are tied to the statement so that their uses stay behind it
@@ -304,8 +309,9 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
         AMCT_WAIT_SLOT(2 * OPS, 0);                                 // steps 0 and 1 have landed
         AMCT_TIE_SMOOTH(0);
         AMCT_TIE_SMOOTH(1);
-        smooth_a(0, 0);
-        smooth_a(1, 1);
+        smooth_read(0);
+        smooth_write(0, 0);
+        smooth_read(1);                                             // written back in iteration 0
     } else {
         AMCT_WAIT_SLOT(3 * OPS, 0);
     }
@@ -319,25 +325,33 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
     // iteration t (stage/slot U = t % 4): second half of the fragments of step t, MFMAs of the first
     // half; wait for the loads of step t+1; dequantise the weights of step t+1 into their stage;
     // barrier; issue the loads of step t+4 into stage/slot U (both free now); first half of step t+1.
-    // With smoothing the loads of step t+2 must have landed too (they are multiplied in place now).
+    // The dequantisation (and, with smoothing, the in-place multiply of the activations of step t+2)
+    // sits in the same scheduling region as 8 MFMAs and is interleaved with them instruction by
+    // instruction: a wave issues in order, so VALU work placed after a run of MFMAs would only start
+    // once the matrix pipe has accepted all of them.
+#define AMCT_INTERLEAVE()                                                   \
+    _Pragma("unroll") for (int q_ = 0; q_ < 8; ++q_) {                      \
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* 1 MFMA  */     \
+        __builtin_amdgcn_sched_group_barrier(0x002, 8, 0); /* 8 VALU  */     \
+        __builtin_amdgcn_sched_group_barrier(0x080, 1, 0); /* 1 DS    */     \
+    }
 #define AMCT_ITER(U, NX, NX2, step)                      \
     {                                                    \
+        AMCT_WAIT_SLOT(2 * OPS, NX);                     \
         read_frags(U, 1, fa1, fb1);                      \
-        mfma_half(fa0, fb0);                             \
-        if constexpr (SMOOTH) {                          \
-            AMCT_WAIT_SLOT(OPS, NX);                     \
-            AMCT_TIE_SMOOTH(NX2);                        \
-            smooth_a(NX2, NX2);                          \
-        } else {                                         \
-            AMCT_WAIT_SLOT(2 * OPS, NX);                 \
-        }                                                \
         write_b(NX, NX);                                 \
+        if constexpr (SMOOTH) smooth_write(NX, NX);      \
+        mfma_half(fa0, fb0);                             \
+        AMCT_INTERLEAVE()                                \
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); \
         __builtin_amdgcn_s_barrier();                    \
         asm volatile("" ::: "memory");                   \
         issue(U, U, (step) + 4);                         \
+        if constexpr (SMOOTH) asm volatile("s_waitcnt vmcnt(%1)" : "+v"(mreg[NX2]) : "n"(2 * OPS) : "memory"); \
         read_frags(NX, 0, fa0, fb0);                     \
+        if constexpr (SMOOTH) smooth_read(NX2);          \
         mfma_half(fa1, fb1);                             \
+        AMCT_INTERLEAVE()                                \
     }
     for (int step = 0; step < nsteps; step += 4) {
         AMCT_ITER(0, 1, 2, step)
@@ -346,6 +360,7 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
         AMCT_ITER(3, 0, 1, step + 3)
     }
 #undef AMCT_ITER
+#undef AMCT_INTERLEAVE
 #undef AMCT_WAIT_SLOT
 #undef AMCT_TIE_SMOOTH
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -474,6 +489,16 @@ __global__ __launch_bounds__(kBlock) void w4a16_skinny(W4A16Args a) {
     }
 }
 
+// x' = bf16(x * smooth[k]) over the whole activation matrix (K % 8 == 0): used when the caller lends a
+// workspace, so that the multiply is done once instead of once per column tile
+__global__ __launch_bounds__(kBlock) void smooth_rows(const uint16_t* x, const uint16_t* smooth, uint16_t* y, int64_t nvec, int kvec) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += stride) {
+        const uint4 c = ldg16(smooth + (v % kvec) * 8);
+        stg16(y + v * 8, smooth8(ldg16_nt(x + v * 8), c));
+    }
+}
+
 // general kernel: one output per thread, sequential fp32 accumulation over k
 __global__ __launch_bounds__(kBlock) void w4a16_general(W4A16Args a) {
     const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -500,7 +525,8 @@ using namespace amct;
 
 extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t* wq, const void* scales,
                                int scale_dtype, const uint8_t* zeros, const float* bias, void* out, int64_t M,
-                               int64_t N, int64_t K, int group, int dtype, amct_stream_t stream) {
+                               int64_t N, int64_t K, int group, int dtype, void* workspace, size_t workspace_bytes,
+                               amct_stream_t stream) {
     if (!x || !wq || !scales || !zeros || !out || M < 0 || N <= 0 || K <= 0 || group <= 0) return AMCT_E_BADARG;
     if (scale_dtype != AMCT_F16 && scale_dtype != AMCT_BF16) return AMCT_E_BADARG;
     if (dtype != AMCT_BF16) return AMCT_E_UNSUPPORTED;
@@ -520,6 +546,16 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
     if (vec_ok && M >= 256 && K % 128 == 0 && N % 8 == 0 && group % 16 == 0 && aligned16(out)) {
         const dim3 grid((unsigned)((N + kQN - 1) / kQN), (unsigned)((M + kQM - 1) / kQM));
         if (grid.y > 65535) return AMCT_E_UNSUPPORTED;
+        if (smooth && workspace && workspace_bytes >= (size_t)(M * K * 2) && aligned16(workspace)) {
+            // smoothing once into the lent workspace, then the kernel without the in-tile multiply
+            const int64_t nvec = M * K / 8;
+            int64_t nb = (nvec + kBlock - 1) / kBlock;
+            if (nb > 16384) nb = 16384;
+            hipLaunchKernelGGL(smooth_rows, dim3((unsigned)nb), dim3(kBlock), 0, st, a.x, a.smooth, (uint16_t*)workspace, nvec, (int)(K / 8));
+            a.x = (const uint16_t*)workspace;
+            a.smooth = nullptr;
+            smooth = nullptr;
+        }
         if (smooth) hipLaunchKernelGGL((w4a16_tile_dma<true>), grid, dim3(kQThreads), 0, st, a);
         else hipLaunchKernelGGL((w4a16_tile_dma<false>), grid, dim3(kQThreads), 0, st, a);
         return hip_status();

@@ -220,11 +220,13 @@ def build_cases(dev, only):
                 continue
             xd = x7[:M7].contiguous().to(dev)
             outs7 = [torch.empty(M7, N7, dtype=torch.bfloat16, device=dev) for _ in range(nw7)]
+            ws7 = torch.empty(M7, K7, dtype=torch.bfloat16, device=dev)       # lent workspace (smoothed x)
 
-            def launch(i, xd=xd, outs7=outs7, M7=M7, pk7=pk7, scd=scd, zd=zd, smd=smd, N7=N7, K7=K7, g7=g7):
+            def launch(i, xd=xd, outs7=outs7, M7=M7, pk7=pk7, scd=scd, zd=zd, smd=smd, N7=N7, K7=K7, g7=g7, ws7=ws7):
                 j = i % len(pk7)
                 rc = lib.amct_gemm_w4a16(xd.data_ptr(), smd.data_ptr(), pk7[j].data_ptr(), scd.data_ptr(), _lib.F16,
-                                         zd.data_ptr(), None, outs7[j].data_ptr(), M7, N7, K7, g7, _lib.BF16, st)
+                                         zd.data_ptr(), None, outs7[j].data_ptr(), M7, N7, K7, g7, _lib.BF16,
+                                         ws7.data_ptr(), ws7.numel() * 2, st)
                 assert rc == 0, rc
             wbytes = N7 * K7 // 2 + N7 * (K7 // g7) * 3
             if M7 >= 256:
