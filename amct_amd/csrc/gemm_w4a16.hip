@@ -32,6 +32,7 @@ struct W4A16Args {
     int64_t M, N, K;
     int group;
     int scale_dtype;
+    uint32_t group_magic;                            // floor(2^32 / group) + 1: k / group == mulhi(k, magic) for k, group < 2^16
 };
 
 AMCT_DEV float load_scale(const W4A16Args& a, int64_t i) {
@@ -39,12 +40,23 @@ AMCT_DEV float load_scale(const W4A16Args& a, int64_t i) {
     return a.scale_dtype == AMCT_F16 ? f16_bits_to_f32(h) : bf16_bits_to_f32(h);
 }
 
-AMCT_DEV uint32_t pack_bf16x2(float lo, float hi) { return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16); }
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+// one v_cvt_pk_bf16_f32 for the pair (round-half-even); converting the halves separately costs four
+// instructions instead
+AMCT_DEV uint32_t pack_bf16x2(float lo, float hi) {
+    const v2f f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, v2bf));
+}
 
 // 8 nibbles of `w` (element j in bits 4j..4j+3) -> 8 bf16 of (u - z) * s, as 4 packed dwords
 AMCT_DEV uint4 dequant8(uint32_t w, float s, float nzs) {
-    const uint32_t lo = w & 0x0F0F0F0Fu;            // elements 0,2,4,6 in bytes 0..3
-    const uint32_t hi = (w >> 4) & 0x0F0F0F0Fu;     // elements 1,3,5,7
+    uint32_t lo = w & 0x0F0F0F0Fu;                  // elements 0,2,4,6 in bytes 0..3
+    uint32_t hi = (w >> 4) & 0x0F0F0F0Fu;           // elements 1,3,5,7
+    // opaque to the optimiser: otherwise it rewrites the byte extraction below as one bit-field extract
+    // per nibble followed by a conversion, two instructions per element instead of v_cvt_f32_ubyteN alone
+    asm("" : "+v"(lo));
+    asm("" : "+v"(hi));
     uint32_t o[4];
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
@@ -499,6 +511,368 @@ __global__ __launch_bounds__(kBlock) void smooth_rows(const uint16_t* x, const u
     }
 }
 
+// ---------------------------------------------------------------------------
+// decode kernel (M <= 16 * MT, K % 128 == 0, group % 32 == 0): weight streaming.
+// A block owns 64 output columns; its waves split K in runs of 128 (one iteration = 4 MFMA k-slots of
+// 32).  Per iteration a lane fetches 16 bytes of each of its 4 weight rows (row 16 t + lane % 16,
+// k-slot lane / 16): 64 bytes per lane, twice that in flight with the prefetch of the next iteration.
+// All loads are unconditional (indices clamped), so none forces a full wait.  The activation fragments
+// of an iteration (smoothed once) are shared by the 4 column tiles; the weights are dequantised to bf16
+// exactly as in the large-tile kernel, so both produce the same operand bits.
+// ---------------------------------------------------------------------------
+constexpr int kDN = 64;                                           // output columns per block
+
+template <int MT, int WAVES, bool SMOOTH>
+__global__ __launch_bounds__(WAVES * 64) void w4a16_decode(W4A16Args a) {
+    __shared__ float red[WAVES - 1 > 0 ? WAVES - 1 : 1][MT][4][64][4];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int64_t n0 = (int64_t)blockIdx.x * kDN;
+    const int64_t G = a.K / a.group;
+    const int iters_total = (int)(a.K / 128);
+    const int per_wave = iters_total / WAVES;                      // host guarantees divisibility
+    const int it0 = wave * per_wave;
+    const bool scale_is_f16 = a.scale_dtype == AMCT_F16;
+
+    const uint8_t* wrow[4];
+    const uint8_t* srow[4];
+    const uint8_t* zrow[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const int64_t n = n0 + t * 16 + r16;
+        const int64_t nc = n < a.N ? n : a.N - 1;
+        wrow[t] = a.wq + nc * (a.K / 2) + g * 16;
+        srow[t] = reinterpret_cast<const uint8_t*>(a.scales) + nc * G * 2;
+        zrow[t] = a.zeros + nc * G;
+    }
+    const uint16_t* xrow[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int64_t m = mt * 16 + r16;
+        xrow[mt] = a.x + (m < a.M ? m : a.M - 1) * a.K + g * 32;
+    }
+
+    v4f y[MT][4];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) y[mt][t] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    // one iteration's loads, all issued together and all consumed one iteration later: the waits the
+    // compiler derives (in issue order) then never cover the batch that was just issued
+    uint4 wv[2][4], xv[2][MT][4], cv[2][4];
+    uint32_t sb[2][4], zb[2][4];
+    auto load_w = [&](int buf, int it) {
+        const int itc = it < it0 + per_wave ? it : it0 + per_wave - 1;      // clamped: loads are unconditional
+        const uint32_t kb = (uint32_t)itc * 128u;
+        const uint32_t gi = __umulhi(kb + (uint32_t)g * 32u, a.group_magic);   // (kb + 32 g) / group
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4) {
+            if constexpr (SMOOTH) cv[buf][s4] = ldg16(a.smooth + kb + g * 32 + s4 * 8);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) xv[buf][mt][s4] = ldg16(xrow[mt] + kb + s4 * 8);
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            sb[buf][t] = *reinterpret_cast<const uint16_t*>(srow[t] + gi * 2);
+            zb[buf][t] = zrow[t][gi];
+            wv[buf][t] = ldg16_nt(wrow[t] + kb / 2);
+        }
+    };
+    auto compute = [&](int buf) {
+        v8bf fa[MT][4];
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                fa[mt][s4] = __builtin_bit_cast(v8bf, SMOOTH ? smooth8(xv[buf][mt][s4], cv[buf][s4]) : xv[buf][mt][s4]);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const float sc_h = f16_bits_to_f32(sb[buf][t]), sc_b = bf16_bits_to_f32(sb[buf][t]);
+            const float sc = scale_is_f16 ? sc_h : sc_b;
+            const float nzs = -((float)zb[buf][t] * sc);
+            const uint32_t ws[4] = {wv[buf][t].x, wv[buf][t].y, wv[buf][t].z, wv[buf][t].w};
+#pragma unroll
+            for (int s4 = 0; s4 < 4; ++s4) {
+                const v8bf fb = __builtin_bit_cast(v8bf, dequant8(ws[s4], sc, nzs));
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    y[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[mt][s4], fb, y[mt][t], 0, 0, 0);
+            }
+        }
+    };
+
+    load_w(0, it0);
+    for (int i = 0; i < per_wave; i += 2) {
+        load_w(1, it0 + i + 1);
+        __builtin_amdgcn_sched_barrier(0);                        // keep the prefetch ahead of the arithmetic
+        compute(0);
+        if (i + 1 >= per_wave) break;
+        __builtin_amdgcn_sched_barrier(0);
+        load_w(0, it0 + i + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(1);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    if constexpr (WAVES > 1) {
+        if (wave > 0) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) red[wave - 1][mt][t][lane][r] = y[mt][t][r];
+        }
+        __syncthreads();
+    }
+    if (wave == 0) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int64_t n = n0 + t * 16 + r16;
+            const float b = (a.bias && n < a.N) ? a.bias[n] : 0.f;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    float v = y[mt][t][r];
+                    if constexpr (WAVES > 1) {
+#pragma unroll
+                        for (int w = 0; w < WAVES - 1; ++w) v = v + red[w][mt][t][lane][r];
+                    }
+                    if (a.bias) v = v + b;
+                    const int64_t m = mt * 16 + 4 * g + r;
+                    if (n < a.N && m < a.M) a.out[m * a.N + n] = (uint16_t)f32_to_bf16_bits(v);
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// decode kernel with the block's activations in LDS (M <= 16, K % 256 == 0, M * K small enough).
+// Everything that is not the weight stream is fetched once per block with coalesced loads: the
+// activations (smoothed on the way, rows padded by 16 bytes so that the 16 rows of a fragment read fall
+// into different banks) and the block's 64 x G scales and zero-points.  The weight stream is the only
+// per-lane traffic left; a lane's loads come in pairs that cover both 64-byte halves of a 128-byte
+// line back to back (k-slots h = 0, 1 of a 256-wide iteration), two iterations are in flight.
+// ---------------------------------------------------------------------------
+template <int WAVES, bool SMOOTH, int XJ, int TN>
+__global__ __launch_bounds__(WAVES * 64) void w4a16_decode_lds(W4A16Args a) {
+    extern __shared__ __align__(16) uint8_t lds_raw[];
+    constexpr int NT = WAVES * 64;
+    constexpr int DN = 16 * TN;                                   // output columns per block
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int64_t n0 = (int64_t)blockIdx.x * DN;
+    const uint32_t K = (uint32_t)a.K, M = (uint32_t)a.M;
+    const uint32_t G = K / (uint32_t)a.group;
+    const uint32_t xstride = K * 2 + 16;                          // bytes per staged activation row
+    const uint32_t xbytes = M * xstride;
+    const uint32_t red_bytes = (WAVES - 1) * TN * 64 * 16;
+    uint8_t* xs = lds_raw;
+    uint16_t* sc_lds = reinterpret_cast<uint16_t*>(lds_raw + (xbytes > red_bytes ? xbytes : red_bytes));
+    uint8_t* z_lds = reinterpret_cast<uint8_t*>(sc_lds + DN * G);
+    const bool scale_is_f16 = a.scale_dtype == AMCT_F16;
+    const int per_wave = (int)(K / 256) / WAVES;
+    const int it0 = wave * per_wave;
+
+    // ---- staging loads first, the weight stream after them: waits are in issue order, so the staged data
+    // can be consumed (and the block barrier passed) while the weights are still arriving
+    // scales: DN rows x G u16 = 2 TN G vectors of 16 bytes; zero-points: TN G vectors.  Rows past N read the last
+    // vectors of the tensors (in bounds, never used for a stored output).
+    constexpr int SJ = (2 * TN * 128 + NT - 1) / NT;              // G <= 128
+    constexpr int ZJ = (TN * 128 + NT - 1) / NT;
+    const int64_t sv_total = a.N * (int64_t)G / 8, zv_total = a.N * (int64_t)G / 16;
+    const int64_t sv0 = n0 * (int64_t)G / 8, zv0 = n0 * (int64_t)G / 16;
+    uint4 sv[SJ], zv[ZJ];
+#pragma unroll
+    for (int j = 0; j < SJ; ++j) {
+        const int64_t i = sv0 + tid + NT * j;
+        sv[j] = ldg16(reinterpret_cast<const uint8_t*>(a.scales) + (i < sv_total ? i : sv_total - 1) * 16);
+    }
+#pragma unroll
+    for (int j = 0; j < ZJ; ++j) {
+        const int64_t i = zv0 + tid + NT * j;
+        zv[j] = ldg16(a.zeros + (i < zv_total ? i : zv_total - 1) * 16);
+    }
+    const uint32_t KV = K / 8, n_xv = M * KV;
+    uint4 xv[XJ], cv[XJ];
+    uint32_t xdst[XJ];
+    const bool cv_same = NT % KV == 0;                            // a thread's vectors then share their k position
+#pragma unroll
+    for (int j = 0; j < XJ; ++j) {
+        const uint32_t v = tid + NT * j;
+        const uint32_t vc = v < n_xv ? v : n_xv - 1;
+        const uint32_t row = vc / KV, kv = vc - row * KV;
+        xv[j] = ldg16(a.x + (int64_t)row * K + kv * 8);
+        if constexpr (SMOOTH) {
+            if (j == 0 || !cv_same) cv[j] = ldg16(a.smooth + kv * 8);
+        }
+        xdst[j] = row * xstride + kv * 16;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    const uint8_t* wrow[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t) {
+        const int64_t n = n0 + t * 16 + r16;
+        wrow[t] = a.wq + (n < a.N ? n : a.N - 1) * (int64_t)(K / 2) + g * 16;
+    }
+    uint4 wv[2][TN * 2];
+    auto load_w = [&](int buf, int it) {
+        const int itc = it < it0 + per_wave ? it : it0 + per_wave - 1;      // clamped: loads are unconditional
+        const uint32_t kb2 = (uint32_t)itc * 128u;                          // byte offset of the iteration
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) wv[buf][t * 2 + h] = ldg16(wrow[t] + kb2 + h * 64);
+    };
+    load_w(0, it0);
+    load_w(1, it0 + 1);
+    __builtin_amdgcn_sched_barrier(0);
+
+#pragma unroll
+    for (int j = 0; j < SJ; ++j) {
+        const uint32_t i = tid + NT * j;
+        if (i < 2 * TN * G) *reinterpret_cast<uint4*>(reinterpret_cast<uint8_t*>(sc_lds) + i * 16) = sv[j];
+    }
+#pragma unroll
+    for (int j = 0; j < ZJ; ++j) {
+        const uint32_t i = tid + NT * j;
+        if (i < TN * G) *reinterpret_cast<uint4*>(z_lds + i * 16) = zv[j];
+    }
+#pragma unroll
+    for (int j = 0; j < XJ; ++j) {
+        const uint32_t v = tid + NT * j;
+        if constexpr (SMOOTH) xv[j] = smooth8(xv[j], cv_same ? cv[0] : cv[j]);
+        if (v < n_xv) *reinterpret_cast<uint4*>(xs + xdst[j]) = xv[j];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+
+    v4f y[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t) y[t] = v4f{0.f, 0.f, 0.f, 0.f};
+    const uint8_t* xlane = xs + (r16 < (int)M ? r16 : (int)M - 1) * xstride + g * 64;
+
+    auto compute = [&](int buf, int it) {
+        const uint32_t kb = (uint32_t)it * 256u;
+        v8bf fa[2][4];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int s4 = 0; s4 < 4; ++s4)
+                fa[h][s4] = *reinterpret_cast<const v8bf*>(xlane + (kb + h * 128) * 2 + s4 * 16);
+#pragma unroll
+        for (int t = 0; t < TN; ++t) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint32_t k0 = kb + h * 128 + g * 32;
+                const uint32_t gi = __umulhi(k0, a.group_magic);  // k0 / group
+                const uint32_t sbits = sc_lds[(t * 16 + r16) * G + gi];
+                const float sc_h = f16_bits_to_f32(sbits), sc_b = bf16_bits_to_f32(sbits);
+                const float sc = scale_is_f16 ? sc_h : sc_b;
+                const float nzs = -((float)z_lds[(t * 16 + r16) * G + gi] * sc);
+                const uint4 w4 = wv[buf][t * 2 + h];
+                const uint32_t ws[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+                for (int s4 = 0; s4 < 4; ++s4) {
+                    const v8bf fb = __builtin_bit_cast(v8bf, dequant8(ws[s4], sc, nzs));
+                    y[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[h][s4], fb, y[t], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    for (int i = 0; i < per_wave; i += 2) {
+        compute(0, it0 + i);
+        __builtin_amdgcn_sched_barrier(0);
+        if (i + 1 >= per_wave) break;
+        load_w(0, it0 + i + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(1, it0 + i + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        load_w(1, it0 + i + 3);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    float* red = reinterpret_cast<float*>(lds_raw);               // reuses the activation rows
+    if constexpr (WAVES > 1) {
+        __syncthreads();                                          // every wave is done reading activations
+        if (wave > 0) {
+#pragma unroll
+            for (int t = 0; t < TN; ++t)
+                *reinterpret_cast<v4f*>(red + (((wave - 1) * TN + t) * 64 + lane) * 4) = y[t];
+        }
+        __syncthreads();
+    }
+    if (wave == 0) {
+#pragma unroll
+        for (int t = 0; t < TN; ++t) {
+            const int64_t n = n0 + t * 16 + r16;
+            const float b = (a.bias && n < a.N) ? a.bias[n] : 0.f;
+            v4f acc = y[t];
+            if constexpr (WAVES > 1) {
+#pragma unroll
+                for (int w = 0; w < WAVES - 1; ++w) {
+                    const v4f o = *reinterpret_cast<const v4f*>(red + ((w * TN + t) * 64 + lane) * 4);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[r] = acc[r] + o[r];
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float v = acc[r];
+                if (a.bias) v = v + b;
+                const int64_t m = 4 * g + r;
+                if (n < a.N && m < a.M) a.out[m * a.N + n] = (uint16_t)f32_to_bf16_bits(v);
+            }
+        }
+    }
+}
+
+// LDS bytes of w4a16_decode_lds, 0 if the shape does not fit
+static size_t decode_lds_bytes(int64_t M, int64_t K, int group, int waves, int tn) {
+    const size_t xbytes = (size_t)M * ((size_t)K * 2 + 16);
+    const size_t red = (size_t)(waves - 1) * tn * 64 * 16;
+    const size_t G = (size_t)(K / group);
+    const size_t total = (xbytes > red ? xbytes : red) + (size_t)tn * 16 * G * 3;
+    return total <= 150 * 1024 ? total : 0;
+}
+
+template <int WAVES, bool SMOOTH, int XJ, int TN>
+static int launch_decode_lds(const W4A16Args& a, size_t lds, hipStream_t st) {
+    // per device and cheap; no state is kept in the library
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w4a16_decode_lds<WAVES, SMOOTH, XJ, TN>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess) {
+        (void)hipGetLastError();
+        return AMCT_E_HIP;
+    }
+    const dim3 grid((unsigned)((a.N + 16 * TN - 1) / (16 * TN)));
+    hipLaunchKernelGGL((w4a16_decode_lds<WAVES, SMOOTH, XJ, TN>), grid, dim3(WAVES * 64), lds, st, a);
+    return hip_status();
+}
+
+template <int WAVES, bool SMOOTH, int TN>
+static int launch_decode_lds_xj(const W4A16Args& a, size_t lds, hipStream_t st) {
+    const int64_t per_thread = (a.M * (a.K / 8) + WAVES * 64 - 1) / (WAVES * 64);
+    if (per_thread <= 1) return launch_decode_lds<WAVES, SMOOTH, 1, TN>(a, lds, st);
+    if (per_thread <= 4) return launch_decode_lds<WAVES, SMOOTH, 4, TN>(a, lds, st);
+    if (per_thread <= 16) return launch_decode_lds<WAVES, SMOOTH, 16, TN>(a, lds, st);
+    return AMCT_E_UNSUPPORTED;                                    // caller falls through to the register kernel
+}
+
+template <bool SMOOTH, int TN>
+static int launch_decode_lds_w(const W4A16Args& a, int waves, size_t lds, hipStream_t st) {
+    if constexpr (TN == 4) {
+        if (waves == 8) return launch_decode_lds_xj<8, SMOOTH, TN>(a, lds, st);
+    }
+    return waves == 4 ? launch_decode_lds_xj<4, SMOOTH, TN>(a, lds, st) : launch_decode_lds_xj<1, SMOOTH, TN>(a, lds, st);
+}
+
 // general kernel: one output per thread, sequential fp32 accumulation over k
 __global__ __launch_bounds__(kBlock) void w4a16_general(W4A16Args a) {
     const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -532,9 +906,49 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
     if (dtype != AMCT_BF16) return AMCT_E_UNSUPPORTED;
     if (K % group != 0 || K % 2 != 0) return AMCT_E_ALIGN;
     if (M == 0) return AMCT_OK;
-    W4A16Args a{(const uint16_t*)x, (const uint16_t*)smooth, wq, scales, zeros, bias, (uint16_t*)out, M, N, K, group, scale_dtype};
+    W4A16Args a{(const uint16_t*)x, (const uint16_t*)smooth, wq, scales, zeros, bias, (uint16_t*)out, M, N, K, group, scale_dtype,
+                (uint32_t)(0x100000000ull / (uint64_t)group) + 1u};
     hipStream_t st = (hipStream_t)stream;
     const bool vec_ok = aligned16(x) && aligned16(wq) && (!smooth || aligned16(smooth)) && group % 32 == 0;
+    if (vec_ok && M <= 16 && K % 256 == 0 && K < 65536 && group % 32 == 0 && K / group <= 128 && (N * (K / group)) % 16 == 0 &&
+        aligned16(scales) && aligned16(zeros)) {
+        // Few activations (M * K small): narrow blocks of 4 waves, several per CU, so that one block's start-up
+        // and reduction overlap with another's streaming.  More activations: wide blocks, which stage the
+        // activations fewer times.
+        const int iters = (int)(K / 256);
+        const bool few = M * K <= 32768;
+        const int waves = (!few && iters % 8 == 0) ? 8 : iters % 4 == 0 ? 4 : 1;
+        const int tn = M * K <= 8192 ? 1 : few ? 2 : 4;
+        const size_t lds = decode_lds_bytes(M, K, group, waves, tn);
+        int rc = AMCT_E_UNSUPPORTED;
+        if (lds) {
+            if (tn == 1) rc = smooth ? launch_decode_lds_w<true, 1>(a, waves, lds, st) : launch_decode_lds_w<false, 1>(a, waves, lds, st);
+            else if (tn == 2) rc = smooth ? launch_decode_lds_w<true, 2>(a, waves, lds, st) : launch_decode_lds_w<false, 2>(a, waves, lds, st);
+            else rc = smooth ? launch_decode_lds_w<true, 4>(a, waves, lds, st) : launch_decode_lds_w<false, 4>(a, waves, lds, st);
+        }
+        if (rc != AMCT_E_UNSUPPORTED) return rc;
+    }
+    if (vec_ok && M <= 64 && K % 128 == 0 && K < 65536 && group % 32 == 0) {
+        const dim3 grid((unsigned)((N + kDN - 1) / kDN));
+        const int iters = (int)(K / 128);
+#define AMCT_DEC2(MT, SM)                                                                                    \
+    {                                                                                                        \
+        if (iters % 8 == 0 && MT < 4) hipLaunchKernelGGL((w4a16_decode<MT, (MT < 4 ? 8 : 4), SM>), grid, dim3(512), 0, st, a); \
+        else if (iters % 4 == 0) hipLaunchKernelGGL((w4a16_decode<MT, 4, SM>), grid, dim3(256), 0, st, a);   \
+        else if (iters % 2 == 0) hipLaunchKernelGGL((w4a16_decode<MT, 2, SM>), grid, dim3(128), 0, st, a);   \
+        else hipLaunchKernelGGL((w4a16_decode<MT, 1, SM>), grid, dim3(64), 0, st, a);                        \
+    }
+#define AMCT_DEC(MT)                                                                                         \
+    {                                                                                                        \
+        if (smooth) AMCT_DEC2(MT, true) else AMCT_DEC2(MT, false)                                            \
+    }
+        if (M <= 16) AMCT_DEC(1)
+        else if (M <= 32) AMCT_DEC(2)
+        else AMCT_DEC(4)
+#undef AMCT_DEC2
+#undef AMCT_DEC
+        return hip_status();
+    }
     if (vec_ok && M <= 64 && K % 128 == 0) {
         const dim3 grid((unsigned)((N + 15) / 16));
         if (M <= 16) hipLaunchKernelGGL((w4a16_skinny<1>), grid, dim3(kBlock), 0, st, a);

@@ -84,7 +84,10 @@ def w4a16_oracle(x, codes, scales, zeros, group, smooth, bias):
 
 
 @pytest.mark.parametrize("M,N,K,group", [(1, 64, 256, 128), (16, 128, 512, 128), (7, 33, 128, 32), (64, 64, 256, 64),
-                                         (130, 200, 384, 128), (256, 256, 1024, 128), (2048, 128, 4096, 128)])
+                                         (130, 200, 384, 128), (256, 256, 1024, 128), (2048, 128, 4096, 128),
+                                         (16, 136, 4096, 128), (3, 72, 1024, 256), (20, 64, 768, 128),
+                                         (40, 96, 1024, 128), (64, 200, 2048, 128), (33, 64, 384, 128),
+                                         (8, 96, 4096, 128), (5, 80, 2048, 64), (12, 64, 4096, 128), (2, 48, 8192, 128)])
 @pytest.mark.parametrize("sdt", [torch.float16, torch.bfloat16])
 def test_w4a16_vs_oracle(dev, M, N, K, group, sdt):
     x, codes, scales, zeros, smooth, bias = w4a16_case(M, N, K, group, 101, sdt)
