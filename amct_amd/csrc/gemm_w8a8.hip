@@ -426,6 +426,168 @@ __global__ __launch_bounds__(kBlock) void w8a8_skinny(W8A8Args a) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// decode kernel (M <= 16, K % 256 == 0): the weight matrix is streamed once, nothing else is expensive.
+// A block owns 16 * TN output columns, its waves split K in runs of 256.  The block's activations are
+// staged in LDS once (rows padded by 16 bytes: the 16 rows of a fragment read fall into different
+// banks).  The staging loads are issued before the weight loads: waits follow issue order, so the staged
+// data is consumed, and the block barrier passed, while the weights are still arriving.  A lane's weight
+// loads cover the 64-byte quarters of a row's 256-byte run back to back; two iterations are in flight.
+// All loads are unconditional (indices clamped).
+// ---------------------------------------------------------------------------
+template <int WAVES, int XJ, int TN>
+__global__ __launch_bounds__(WAVES * 64) void w8a8_decode_lds(W8A8Args a) {
+    extern __shared__ __align__(16) uint8_t lds_raw[];
+    constexpr int NT = WAVES * 64;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int64_t n0 = (int64_t)blockIdx.x * (16 * TN);
+    const uint32_t K = (uint32_t)a.K, M = (uint32_t)a.M;
+    const uint32_t xstride = K + 16;
+    const int per_wave = (int)(K / 256) / WAVES;
+    const int it0 = wave * per_wave;
+
+    const uint32_t KV = K / 16, n_xv = M * KV;
+    uint4 xv[XJ];
+    uint32_t xdst[XJ];
+#pragma unroll
+    for (int j = 0; j < XJ; ++j) {
+        const uint32_t v = tid + NT * j;
+        const uint32_t vc = v < n_xv ? v : n_xv - 1;
+        const uint32_t row = vc / KV, kv = vc - row * KV;
+        xv[j] = ldg16(a.xq + (int64_t)row * K + kv * 16);
+        xdst[j] = row * xstride + kv * 16;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    const int8_t* wrow[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t) {
+        const int64_t n = n0 + t * 16 + r16;
+        wrow[t] = a.wq + (n < a.N ? n : a.N - 1) * (int64_t)K + g * 16;
+    }
+    uint4 wv[2][TN * 4];
+    auto load_w = [&](int buf, int it) {
+        const int itc = it < it0 + per_wave ? it : it0 + per_wave - 1;
+        const uint32_t kb = (uint32_t)itc * 256u;
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) wv[buf][t * 4 + q] = ldg16(wrow[t] + kb + q * 64);
+    };
+    load_w(0, it0);
+    load_w(1, it0 + 1);
+    __builtin_amdgcn_sched_barrier(0);
+
+#pragma unroll
+    for (int j = 0; j < XJ; ++j) {
+        const uint32_t v = tid + NT * j;
+        if (v < n_xv) *reinterpret_cast<uint4*>(lds_raw + xdst[j]) = xv[j];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+
+    v4i acc[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t) acc[t] = v4i{0, 0, 0, 0};
+    const uint8_t* xlane = lds_raw + (r16 < (int)M ? r16 : (int)M - 1) * xstride + g * 16;
+
+    auto compute = [&](int buf, int it) {
+        const uint32_t kb = (uint32_t)it * 256u;
+        v4i fa[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) fa[q] = *reinterpret_cast<const v4i*>(xlane + kb + q * 64);
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint4 w4 = wv[buf][t * 4 + q];
+                const v4i fb = v4i{(int)w4.x, (int)w4.y, (int)w4.z, (int)w4.w};
+                acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[q], fb, acc[t], 0, 0, 0);
+            }
+    };
+    for (int i = 0; i < per_wave; i += 2) {
+        compute(0, it0 + i);
+        __builtin_amdgcn_sched_barrier(0);
+        if (i + 1 >= per_wave) break;
+        load_w(0, it0 + i + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(1, it0 + i + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        load_w(1, it0 + i + 3);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    int32_t* red = reinterpret_cast<int32_t*>(lds_raw);           // reuses the activation rows
+    if constexpr (WAVES > 1) {
+        __syncthreads();                                          // every wave is done reading activations
+        if (wave > 0) {
+#pragma unroll
+            for (int t = 0; t < TN; ++t)
+                *reinterpret_cast<v4i*>(red + (((wave - 1) * TN + t) * 64 + lane) * 4) = acc[t];
+        }
+        __syncthreads();
+    }
+    if (wave == 0) {
+#pragma unroll
+        for (int t = 0; t < TN; ++t) {
+            const int64_t n = n0 + t * 16 + r16;
+            v4i v = acc[t];
+            if constexpr (WAVES > 1) {
+#pragma unroll
+                for (int w = 0; w < WAVES - 1; ++w) {
+                    const v4i o = *reinterpret_cast<const v4i*>(red + ((w * TN + t) * 64 + lane) * 4);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) v[r] += o[r];
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int64_t m = 4 * g + r;                      // register r of a 16x16 tile: row 4*(lane/16) + r
+                if (n < a.N && m < a.M) w8a8_epilogue(a, m, n, v[r]);
+            }
+        }
+    }
+}
+
+// LDS bytes of w8a8_decode_lds, 0 if the shape does not fit
+static size_t w8a8_decode_lds_bytes(int64_t M, int64_t K, int waves, int tn) {
+    const size_t xbytes = (size_t)M * ((size_t)K + 16);
+    const size_t red = (size_t)(waves - 1) * tn * 64 * 16;
+    const size_t total = xbytes > red ? xbytes : red;
+    return total <= 150 * 1024 ? total : 0;
+}
+
+template <int WAVES, int XJ, int TN>
+static int launch_w8a8_decode(const W8A8Args& a, size_t lds, hipStream_t st) {
+    // per device and cheap; no state is kept in the library
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_decode_lds<WAVES, XJ, TN>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess) {
+        (void)hipGetLastError();
+        return AMCT_E_HIP;
+    }
+    const dim3 grid((unsigned)((a.N + 16 * TN - 1) / (16 * TN)));
+    hipLaunchKernelGGL((w8a8_decode_lds<WAVES, XJ, TN>), grid, dim3(WAVES * 64), lds, st, a);
+    return hip_status();
+}
+
+template <int WAVES, int TN>
+static int launch_w8a8_decode_xj(const W8A8Args& a, size_t lds, hipStream_t st) {
+    const int64_t per_thread = (a.M * (a.K / 16) + WAVES * 64 - 1) / (WAVES * 64);
+    if (per_thread <= 1) return launch_w8a8_decode<WAVES, 1, TN>(a, lds, st);
+    if (per_thread <= 4) return launch_w8a8_decode<WAVES, 4, TN>(a, lds, st);
+    if (per_thread <= 16) return launch_w8a8_decode<WAVES, 16, TN>(a, lds, st);
+    return AMCT_E_UNSUPPORTED;
+}
+
+template <int TN>
+static int launch_w8a8_decode_w(const W8A8Args& a, int waves, size_t lds, hipStream_t st) {
+    return waves == 4   ? launch_w8a8_decode_xj<4, TN>(a, lds, st)
+           : waves == 2 ? launch_w8a8_decode_xj<2, TN>(a, lds, st)
+                        : launch_w8a8_decode_xj<1, TN>(a, lds, st);
+}
+
 // general kernel: any M, N, K; one output per thread.
 __global__ __launch_bounds__(kBlock) void w8a8_general(W8A8Args a) {
     const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -452,6 +614,19 @@ extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s
     W8A8Args a{xq, wq, s_tok, s_ch, bias_kind ? bias : nullptr, out, acc_out, M, N, K, bias_kind, out_dtype};
     hipStream_t st = (hipStream_t)stream;
     const bool vec_ok = (K % 16 == 0) && aligned16(xq) && aligned16(wq);
+    if (vec_ok && M <= 16 && K % 256 == 0) {
+        const int iters = (int)(K / 256);
+        // measured: blocks of 2 or 4 waves, several per CU, stream best (one block's start-up and reduction
+        // overlap with another's loads); wider blocks only pay when the activations are large
+        const int64_t mk = M * K;
+        int waves = mk <= 8192 ? 2 : 4;
+        while (iters % waves != 0) waves >>= 1;
+        const int tn = (mk <= 8192 || mk > 32768) ? 2 : 1;
+        const size_t lds = w8a8_decode_lds_bytes(M, K, waves, tn);
+        int rc = AMCT_E_UNSUPPORTED;
+        if (lds) rc = tn == 1 ? launch_w8a8_decode_w<1>(a, waves, lds, st) : launch_w8a8_decode_w<2>(a, waves, lds, st);
+        if (rc != AMCT_E_UNSUPPORTED) return rc;
+    }
     if (vec_ok && M <= 64) {
         const dim3 grid((unsigned)((N + 15) / 16));
         if (M <= 16) hipLaunchKernelGGL((w8a8_skinny<1>), grid, dim3(kBlock), 0, st, a);

@@ -47,7 +47,8 @@ def test_w8a8_tiny_bruteforce(dev, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(128, 128, 64), (256, 384, 512), (130, 200, 192), (16, 512, 4096), (1, 256, 1024),
-                                   (300, 129, 320), (2048, 256, 4096)])
+                                   (300, 129, 320), (2048, 256, 4096), (2, 72, 4096), (8, 40, 2048), (7, 33, 768), (12, 100, 1280),
+                                   (3, 48, 256)])
 @pytest.mark.parametrize("per_token,bias", [(True, None), (True, 'float'), (False, 'int'), (False, None)])
 def test_w8a8_vs_oracle(dev, M, N, K, per_token, bias):
     xq, wq, s_ch, s_tok, b = w8a8_case(M, N, K, 97, per_token, bias)
