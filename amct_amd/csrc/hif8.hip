@@ -60,33 +60,89 @@ AMCT_DEV float hif8_dec(uint32_t c) {
     return (c & 0x80u) ? -f : f;
 }
 
+// Encode through two small tables in LDS, indexed by sign and biased exponent (9 bits), which the block
+// builds once and then uses for many elements:
+//   rnd[se]  half an ulp of the HiF8 precision of that binade (0 where the result is 0 or the input is
+//            Inf/NaN): r = bits + rnd is the magnitude rounded to nearest, ties away, before truncation;
+//   par[se]  for the binade of r: {shift, width, base}; the code is base | bitfield(r, shift, width).  base
+//            carries the sign, the dot field and the exponent field; zero results have base 0 (no sign:
+//            0x80 is NaN), denormal and overflow results width 0.  Exponent 15 has base 0x6E and width 1,
+//            so that mantissa bit 1 yields 0x6F, the Inf code (width 0 when saturating).
+// A carry out of the mantissa moves r into the next binade with its top mantissa bits zero, which is why no
+// truncation mask is needed before the lookup.  NaN is patched afterwards (one compare, one select).
+struct Hif8Tables {
+    uint32_t rnd[512];
+    uint4 par[512];
+};
+
+AMCT_DEV void hif8_build_tables(Hif8Tables& t, int tid, int nthreads, bool saturate) {
+    for (int i = tid; i < 512; i += nthreads) {
+        const uint32_t sign = (uint32_t)(i >> 8) << 7;
+        const int eb = i & 255, E = eb - 127;
+        const int absE = E < 0 ? -E : E;
+        const int mb = (absE <= 3) ? 3 : (absE <= 7) ? 2 : (absE <= 15 || E > 15) ? 1 : 0;
+        t.rnd[i] = (E < -23 || eb == 255) ? 0u : (1u << (22 - mb));
+        uint32_t shift = 0, width = 0, base = 0;
+        if (E < -23) {
+            base = 0;
+        } else if (E < -15) {
+            base = sign | (uint32_t)((E < -22 ? -22 : E) + 23);   // [2^-23, 2^-22) rounds up to the smallest
+        } else if (E > 15) {
+            base = sign | (saturate ? 0x6Eu : 0x6Fu);
+        } else {
+            const uint32_t es = E < 0 ? 1u : 0u;
+            if (absE == 0) { base = 0x08u; shift = 20; width = 3; }
+            else if (absE == 1) { base = 0x10u | (es << 3); shift = 20; width = 3; }
+            else if (absE <= 3) { base = 0x20u | (es << 4) | ((uint32_t)(absE & 1) << 3); shift = 20; width = 3; }
+            else if (absE <= 7) { base = 0x40u | (es << 4) | ((uint32_t)(absE & 3) << 2); shift = 21; width = 2; }
+            else { base = 0x60u | (es << 4) | ((uint32_t)(absE & 7) << 1); shift = 22; width = 1; }
+            if (E == 15 && saturate) width = 0;
+            base |= sign;
+        }
+        t.par[i] = make_uint4(shift, width, base, 0u);
+    }
+}
+
+AMCT_DEV uint32_t hif8_enc_lut(const Hif8Tables& t, float x) {
+    const uint32_t u = __float_as_uint(x);
+    const uint32_t r = u + t.rnd[u >> 23];
+    const uint4 p = t.par[r >> 23];
+    const uint32_t code = p.z | __builtin_amdgcn_ubfe(r, p.x, p.y);
+    return __builtin_isnan(x) ? 0x80u : code;
+}
+
 template <int DT, int U>
 __global__ __launch_bounds__(kBlock) void hif8_encode_k(const void* x, uint8_t* y, int64_t nvec, int64_t n, int saturate) {
     constexpr int VEC = Tr<DT>::VEC;
+    __shared__ Hif8Tables tbl;
     const int tid = threadIdx.x;
-    uint4 raw[U];
-    int64_t gv[U];
-    if (nvec > 0) {
+    hif8_build_tables(tbl, tid, kBlock, saturate != 0);
+    __syncthreads();
+    const int64_t chunk = (int64_t)kBlock * U;
+    const int64_t nchunks = (nvec + chunk - 1) / chunk;
+    for (int64_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
+        uint4 raw[U];
+        int64_t gv[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-        gv[u] = ((int64_t)blockIdx.x * U + u) * kBlock + tid;
-        raw[u] = ldg16_nt(reinterpret_cast<const char*>(x) + ((gv[u] < nvec ? gv[u] : nvec - 1) * 16));
-    }
+        for (int u = 0; u < U; ++u) {
+            gv[u] = c * chunk + u * kBlock + tid;
+            raw[u] = ldg16_nt(reinterpret_cast<const char*>(x) + ((gv[u] < nvec ? gv[u] : nvec - 1) * 16));
+        }
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-        if (gv[u] < nvec) {
+        for (int u = 0; u < U; ++u) {
             float v[VEC];
             unpack16<DT>(raw[u], v);
             uint32_t w[VEC / 4];
 #pragma unroll
             for (int j = 0; j < VEC / 4; ++j)
-                w[j] = hif8_enc(v[4 * j], saturate) | (hif8_enc(v[4 * j + 1], saturate) << 8) |
-                       (hif8_enc(v[4 * j + 2], saturate) << 16) | (hif8_enc(v[4 * j + 3], saturate) << 24);
-            uint32_t* p = reinterpret_cast<uint32_t*>(y + gv[u] * VEC);
-            if constexpr (VEC == 8) stg8_nt(p, w[0], w[1]);
-            else stg4_nt(p, w[0]);
+                w[j] = hif8_enc_lut(tbl, v[4 * j]) | (hif8_enc_lut(tbl, v[4 * j + 1]) << 8) |
+                       (hif8_enc_lut(tbl, v[4 * j + 2]) << 16) | (hif8_enc_lut(tbl, v[4 * j + 3]) << 24);
+            if (gv[u] < nvec) {
+                uint32_t* p = reinterpret_cast<uint32_t*>(y + gv[u] * VEC);
+                if constexpr (VEC == 8) stg8_nt(p, w[0], w[1]);
+                else stg4_nt(p, w[0]);
+            }
         }
-    }
     }
     // tail (n % VEC elements), handled by block 0
     if (blockIdx.x == 0) {
@@ -138,6 +194,7 @@ extern "C" int amct_hif8_encode(const void* x, uint8_t* y, int64_t n, int dtype,
         const int64_t nvec = n / Tr<DT>::VEC;                                                                    \
         int64_t nb = (nvec + (int64_t)kBlock * U - 1) / ((int64_t)kBlock * U);                                   \
         if (nb == 0) nb = 1;                                                                                     \
+        if (nb > 2048) nb = 2048; /* blocks loop over chunks: the table build is paid 8 times per CU at most */ \
         hipLaunchKernelGGL((hif8_encode_k<DT, U>), dim3((unsigned)nb), dim3(kBlock), 0, st, x, y, nvec, n, saturate); \
     }
     switch (dtype) {
