@@ -151,27 +151,38 @@ __global__ __launch_bounds__(kBlock) void hif8_encode_k(const void* x, uint8_t* 
     }
 }
 
-// decode through a 256-entry table in LDS built by the block itself
-template <int DT>
+// decode through a 256-entry table in LDS built by the block itself; U vectors per lane in flight
+template <int DT, int U>
 __global__ __launch_bounds__(kBlock) void hif8_decode_k(const uint8_t* x, void* y, int64_t nvec, int64_t n) {
     constexpr int VEC = Tr<DT>::VEC;
     __shared__ float tbl[256];
     const int tid = threadIdx.x;
     tbl[tid] = hif8_dec((uint32_t)tid);
     __syncthreads();
-    const int64_t stride = (int64_t)gridDim.x * kBlock;
-    for (int64_t gv = (int64_t)blockIdx.x * kBlock + tid; gv < nvec; gv += stride) {
-        uint32_t w[VEC / 4];
-        if constexpr (VEC == 8) {
-            const uint2 r = *reinterpret_cast<const uint2*>(x + gv * 8);
-            w[0] = r.x; w[1] = r.y;
-        } else {
-            w[0] = *reinterpret_cast<const uint32_t*>(x + gv * 4);
-        }
-        float out[VEC];
+    const int64_t chunk = (int64_t)kBlock * U;
+    const int64_t nchunks = (nvec + chunk - 1) / chunk;
+    for (int64_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
+        uint32_t w[U][2];
+        int64_t gv[U];
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) out[j] = tbl[(w[j / 4] >> (8 * (j % 4))) & 0xFFu];
-        stg16(reinterpret_cast<char*>(y) + gv * 16, pack16<DT>(out));
+        for (int u = 0; u < U; ++u) {
+            gv[u] = c * chunk + u * kBlock + tid;
+            const int64_t g = gv[u] < nvec ? gv[u] : nvec - 1;      // clamped: loads are unconditional
+            w[u][1] = 0;
+            if constexpr (VEC == 8) {
+                const u2v r = __builtin_nontemporal_load(reinterpret_cast<const u2v*>(x + g * 8));
+                w[u][0] = r.x; w[u][1] = r.y;
+            } else {
+                w[u][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(x + g * 4));
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            float out[VEC];
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) out[j] = tbl[(w[u][j / 4] >> (8 * (j % 4))) & 0xFFu];
+            if (gv[u] < nvec) stg16_nt(reinterpret_cast<char*>(y) + gv[u] * 16, pack16<DT>(out));
+        }
     }
     if (blockIdx.x == 0) {
         const int64_t e = nvec * VEC + tid;
@@ -215,10 +226,10 @@ extern "C" int amct_hif8_decode(const uint8_t* x, void* y, int64_t n, int dtype,
 #define AMCT_HD(DT)                                                                                   \
     {                                                                                                 \
         const int64_t nvec = n / Tr<DT>::VEC;                                                         \
-        int64_t nb = (nvec + kBlock - 1) / kBlock;                                                    \
+        int64_t nb = (nvec + (int64_t)kBlock * 4 - 1) / ((int64_t)kBlock * 4);                        \
         if (nb == 0) nb = 1;                                                                          \
-        if (nb > 8192) nb = 8192;                                                                     \
-        hipLaunchKernelGGL((hif8_decode_k<DT>), dim3((unsigned)nb), dim3(kBlock), 0, st, x, y, nvec, n); \
+        if (nb > 4096) nb = 4096;                                                                     \
+        hipLaunchKernelGGL((hif8_decode_k<DT, 4>), dim3((unsigned)nb), dim3(kBlock), 0, st, x, y, nvec, n); \
     }
     switch (dtype) {
         case AMCT_F32: AMCT_HD(AMCT_F32) break;

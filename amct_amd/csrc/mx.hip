@@ -174,34 +174,58 @@ __global__ __launch_bounds__(kBlock) void mx_quant_k(const void* x, uint8_t* el,
 }
 
 // ---- dequantise -------------------------------------------------------------------------------
-// One lane produces one 16-byte output vector (VEC elements of the output dtype).
-template <int DT, int FMT>
+// One lane produces one 16-byte output vector (VEC elements of the output dtype) per step, U steps in
+// flight.  Element codes are decoded through a table in LDS that the block builds once: 256 floats for
+// E4M3, 256 pairs of floats (both nibbles of a byte) for E2M1; the product with the block scale is the
+// same fp32 multiplication as in the element-wise form.
+template <int DT, int FMT, int U>
 __global__ __launch_bounds__(kBlock) void mx_dequant_k(const uint8_t* el, const uint8_t* e8, void* y, int64_t nvec) {
     constexpr int VEC = Tr<DT>::VEC;
     constexpr int T = 32 / VEC;
-    const int64_t stride = (int64_t)gridDim.x * kBlock;
-    for (int64_t gv = (int64_t)blockIdx.x * kBlock + threadIdx.x; gv < nvec; gv += stride) {
-        const uint32_t byte = e8[gv / T];
-        const float sc = e8m0_to_f32(byte);
-        float out[VEC];
-        if constexpr (FMT == kFmtE4M3) {
-            uint32_t w[VEC / 4];
-            if constexpr (VEC == 8) {
-                const uint2 r = *reinterpret_cast<const uint2*>(el + gv * 8);
-                w[0] = r.x; w[1] = r.y;
+    constexpr int EB = FMT == kFmtE4M3 ? VEC : VEC / 2;         // element bytes per output vector
+    __shared__ float2 tbl[256];
+    const int tid = threadIdx.x;
+    if constexpr (FMT == kFmtE4M3) tbl[tid] = make_float2(sw_dec_e4m3((uint32_t)tid), 0.f);
+    else tbl[tid] = make_float2(sw_dec_e2m1((uint32_t)tid & 0xFu), sw_dec_e2m1((uint32_t)tid >> 4));
+    __syncthreads();
+    const int64_t chunk = (int64_t)kBlock * U;
+    const int64_t nchunks = (nvec + chunk - 1) / chunk;
+    for (int64_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
+        uint32_t w[U][2];
+        uint32_t sb[U];
+        int64_t gv[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            gv[u] = c * chunk + u * kBlock + tid;
+            const int64_t g = gv[u] < nvec ? gv[u] : nvec - 1;  // clamped: loads are unconditional
+            sb[u] = e8[g / T];
+            w[u][1] = 0;
+            if constexpr (EB == 8) {
+                const u2v r = __builtin_nontemporal_load(reinterpret_cast<const u2v*>(el + g * 8));
+                w[u][0] = r.x; w[u][1] = r.y;
+            } else if constexpr (EB == 4) {
+                w[u][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(el + g * 4));
             } else {
-                w[0] = *reinterpret_cast<const uint32_t*>(el + gv * 4);
+                w[u][0] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(el + g * 2));
             }
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) out[j] = sw_dec_e4m3((w[j / 4] >> (8 * (j % 4))) & 0xFFu) * sc;
-        } else {
-            uint32_t w;
-            if constexpr (VEC == 8) w = *reinterpret_cast<const uint32_t*>(el + gv * 4);
-            else w = *reinterpret_cast<const uint16_t*>(el + gv * 2);
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) out[j] = sw_dec_e2m1((w >> (4 * j)) & 0xFu) * sc;
         }
-        stg16(reinterpret_cast<char*>(y) + gv * 16, pack16<DT>(out));
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const float sc = e8m0_to_f32(sb[u]);
+            float out[VEC];
+            if constexpr (FMT == kFmtE4M3) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) out[j] = tbl[(w[u][j / 4] >> (8 * (j % 4))) & 0xFFu].x * sc;
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC / 2; ++j) {
+                    const float2 p = tbl[(w[u][0] >> (8 * j)) & 0xFFu];
+                    out[2 * j] = p.x * sc;
+                    out[2 * j + 1] = p.y * sc;
+                }
+            }
+            if (gv[u] < nvec) stg16_nt(reinterpret_cast<char*>(y) + gv[u] * 16, pack16<DT>(out));
+        }
     }
 }
 
@@ -216,9 +240,10 @@ static int launch_quant(const void* x, uint8_t* el, uint8_t* e8, int64_t nvec, i
 
 template <int DT, int FMT>
 static int launch_dequant(const uint8_t* el, const uint8_t* e8, void* y, int64_t nvec, hipStream_t st) {
-    int64_t nb = (nvec + kBlock - 1) / kBlock;
-    if (nb > 262144) nb = 262144;
-    hipLaunchKernelGGL((mx_dequant_k<DT, FMT>), dim3((unsigned)nb), dim3(kBlock), 0, st, el, e8, y, nvec);
+    constexpr int U = 4;
+    int64_t nb = (nvec + (int64_t)kBlock * U - 1) / ((int64_t)kBlock * U);
+    if (nb > 4096) nb = 4096;                                     // blocks loop over chunks; the table is built once per block
+    hipLaunchKernelGGL((mx_dequant_k<DT, FMT, U>), dim3((unsigned)nb), dim3(kBlock), 0, st, el, e8, y, nvec);
     return hip_status();
 }
 
