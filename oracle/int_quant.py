@@ -29,7 +29,11 @@ Reference lines followed (paths relative to the reference root):
 Pin status: every function here is pinned by tests/test_oracle_int.py --
 hand-computed known answers that are exact in fp32 (power-of-two scales, ties
 to even), numpy float32 cross-computation of the IEEE division chain, the
-zero-padding rule for ragged groups, and range/idempotence invariants.
+zero-padding rule for ragged groups, and range/idempotence invariants -- and
+by tests/golden/int_quant_kat.json, the whole chain computed with exact
+fractions and an explicit round-to-nearest-even after every operation (no
+floating-point library involved), which both this oracle and the HIP path must
+reproduce bit for bit.
 """
 import math
 

@@ -256,3 +256,16 @@ def test_config1_full_size(dev):
     # idempotence at full size
     dq2, _ = ops.quant_with_params(dq, s, None, 0, -128, 127)
     assert_bits_equal(dq2, dq.cpu(), "idempotent")
+
+
+def test_fakequant_matches_exact_arithmetic_fixture(dev):
+    """The committed known answers (exact fractions, one explicit rounding to binary32 per operation) through
+    the C ABI: scale, offset, codes and dequantised values bit for bit, for int8 / int4, symmetric / asymmetric."""
+    from util import load_int_quant_kat
+    for bits, sym, w, scale, offset, codes, dq in load_int_quant_kat():
+        got_dq, got_codes, got_s, got_z = ops.fakequant_int(w.to(dev), bits, sym, group=0, codes_kind=ops.CODES_I32)
+        assert_bits_equal(got_s.cpu().reshape(()), scale, "scale int%d sym=%s" % (bits, sym))
+        if not sym:
+            assert int(got_z.cpu().reshape(())) == offset
+        assert torch.equal(got_codes.cpu(), codes)
+        assert_bits_equal(got_dq.cpu(), dq, "dq int%d sym=%s" % (bits, sym))

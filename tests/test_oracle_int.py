@@ -5,6 +5,7 @@ import pytest
 import torch
 
 from oracle import int_quant as iq
+from util import assert_bits_equal
 
 
 def T(*v, dtype=torch.float32):
@@ -217,3 +218,23 @@ def test_static_quantize_axes():
     q = iq.static_quantize(x, torch.tensor([2.0, 4.0], dtype=torch.bfloat16),
                            torch.tensor([1.0, 0.0], dtype=torch.bfloat16), -2)
     assert q.tolist() == [[3, 6, -6], [127, -128, 1]]
+
+
+def test_oracle_matches_exact_arithmetic_fixture():
+    """tests/golden/int_quant_kat.json holds the whole chain computed with exact fractions and an explicit
+    round-to-nearest-even to binary32 after every operation (no floating-point library involved): scale,
+    offset, codes and dequantised values must agree bit for bit."""
+    from util import load_int_quant_kat
+    cases = load_int_quant_kat()
+    assert len(cases) >= 70
+    for bits, sym, w, scale, offset, codes, dq in cases:
+        kind = 'int%d' % bits
+        s, z = iq.weight_scale_offset(w, 'channel', sym, kind)
+        assert_bits_equal(s.reshape(()), scale, "scale")
+        if sym:
+            assert z is None
+        else:
+            assert int(z.reshape(())) == offset
+        got_codes = iq.quant_codes(w, kind, s, z)
+        assert torch.equal(got_codes.to(torch.int32), codes)
+        assert_bits_equal(iq.fake_quant(w, kind, s, z), dq, "dq")
