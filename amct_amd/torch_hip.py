@@ -109,3 +109,38 @@ def factors_to_native(antiquant_scale, antiquant_offset, N, G):
             raise RuntimeError("antiquant_offset outside the int4 range")
         zeros = z.to(torch.uint8).contiguous()
     return sc, zeros
+
+
+# ---------------------------------------------------------------------------
+# The same four operators in the dispatcher, as torch.ops.amct_hip.*, for callers that go through
+# torch.ops (scripted or exported graphs).  Device implementations only: a CPU tensor finds no kernel.
+# ---------------------------------------------------------------------------
+_torch_lib = torch.library.Library("amct_hip", "DEF")
+_torch_lib.define("quantize(Tensor input, Tensor scales, Tensor? zero_points=None, int axis=-1, "
+                  "bool div_mode=False) -> Tensor")
+_torch_lib.define("quant_matmul(Tensor x1, Tensor x2, Tensor scale, Tensor? pertoken_scale=None, "
+                  "Tensor? bias=None, ScalarType? output_dtype=None) -> Tensor")
+_torch_lib.define("weight_quant_batchmatmul(Tensor x, Tensor weight, Tensor antiquant_scale, "
+                  "Tensor? antiquant_offset=None, Tensor? bias=None, int antiquant_group_size=0) -> Tensor")
+_torch_lib.define("convert_weight_to_int4pack(Tensor weight) -> Tensor")
+
+
+def _op_quantize(input, scales, zero_points=None, axis=-1, div_mode=False):
+    return npu_quantize(input, scales, zero_points, torch.int8, axis, div_mode)
+
+
+def _op_quant_matmul(x1, x2, scale, pertoken_scale=None, bias=None, output_dtype=None):
+    return npu_quant_matmul(x1, x2, scale, bias=bias, pertoken_scale=pertoken_scale,
+                            output_dtype=output_dtype if output_dtype is not None else torch.bfloat16)
+
+
+def _op_weight_quant_batchmatmul(x, weight, antiquant_scale, antiquant_offset=None, bias=None,
+                                 antiquant_group_size=0):
+    return npu_weight_quant_batchmatmul(x, weight, antiquant_scale, antiquant_offset, bias=bias,
+                                        antiquant_group_size=antiquant_group_size)
+
+
+_torch_lib.impl("quantize", _op_quantize, "CUDA")
+_torch_lib.impl("quant_matmul", _op_quant_matmul, "CUDA")
+_torch_lib.impl("weight_quant_batchmatmul", _op_weight_quant_batchmatmul, "CUDA")
+_torch_lib.impl("convert_weight_to_int4pack", npu_convert_weight_to_int4pack, "CUDA")

@@ -239,3 +239,30 @@ def test_operator_level_w8a8(dev):
     words = torch_hip.npu_convert_weight_to_int4pack(codes.to(dev))
     assert_bits_equal(words, od.pack_int4_words(codes), "int4pack")
     assert torch_hip.npu.is_available()
+
+
+def test_dispatcher_operators(dev):
+    """The same operators through torch.ops.amct_hip.*: identical results to the function-level entry points;
+    a CPU tensor finds no kernel (there is no host implementation)."""
+    torch.manual_seed(8)
+    M, K, N, g = 12, 256, 64, 128
+    x = torch.randn(M, K).to(torch.bfloat16)
+    sc = torch.tensor([25.0], dtype=torch.bfloat16)
+    xq = torch.ops.amct_hip.quantize(x.to(dev), sc.to(dev), None, -1, False)
+    assert_bits_equal(xq, torch_hip.npu_quantize(x.to(dev), sc.to(dev)), "quantize")
+    wq = torch.randint(-128, 128, (N, K), dtype=torch.int8)
+    scale = (torch.rand(N) * 0.01).to(dev)
+    tok = (torch.rand(M) * 0.1 + 0.01).to(dev)
+    a = torch.ops.amct_hip.quant_matmul(xq, wq.to(dev).t(), scale, tok, None, torch.float16)
+    b = torch_hip.npu_quant_matmul(xq, wq.to(dev).t(), scale=scale, pertoken_scale=tok, output_dtype=torch.float16)
+    assert_bits_equal(a, b, "quant_matmul")
+    codes = torch.randint(-8, 8, (K, N), dtype=torch.int32)
+    words = torch.ops.amct_hip.convert_weight_to_int4pack(codes.to(dev))
+    assert_bits_equal(words, od.pack_int4_words(codes), "int4pack")
+    sw = (torch.rand(K // g, N) * 0.01 + 0.001).to(torch.bfloat16).to(dev)
+    ow = torch.randint(-7, 8, (K // g, N)).to(torch.bfloat16).to(dev)
+    c = torch.ops.amct_hip.weight_quant_batchmatmul(x.to(dev), words, sw, ow, None, g)
+    d = torch_hip.npu_weight_quant_batchmatmul(x.to(dev), words, sw, antiquant_offset=ow, antiquant_group_size=g)
+    assert_bits_equal(c, d, "weight_quant_batchmatmul")
+    with pytest.raises(NotImplementedError):
+        torch.ops.amct_hip.convert_weight_to_int4pack(codes)
