@@ -845,8 +845,10 @@ static size_t decode_lds_bytes(int64_t M, int64_t K, int group, int waves, int t
 
 template <int WAVES, bool SMOOTH, int XJ, int TN>
 static int launch_decode_lds(const W4A16Args& a, size_t lds, hipStream_t st) {
-    // per device and cheap; no state is kept in the library
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w4a16_decode_lds<WAVES, SMOOTH, XJ, TN>),
+    // only launches above the default 64 KiB of dynamic LDS need the attribute; it is per device and cheap,
+    // so it is simply set on every such launch and no state is kept in the library
+    if (lds > 64 * 1024 &&
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&w4a16_decode_lds<WAVES, SMOOTH, XJ, TN>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess) {
         (void)hipGetLastError();
         return AMCT_E_HIP;

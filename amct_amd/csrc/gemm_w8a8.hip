@@ -385,21 +385,26 @@ __global__ __launch_bounds__(kBlock) void w8a8_skinny(W8A8Args a) {
     }
     constexpr int UN = 4;
     for (int64_t s = s_begin; s < s_end; s += UN) {
-        uint4 wv[UN];
+        // every load is unconditional (a predicated load forces a full wait): out-of-range positions read
+        // the last 16 bytes of the row instead and the weight fragment is zeroed afterwards
+        uint4 wv[UN], xv[UN][MT];
+        bool ok[UN];
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
             const int64_t k = (s + u) * 64 + kslot;
-            wv[u] = (s + u < s_end && k < a.K) ? ldg16(wrow + k) : make_uint4(0, 0, 0, 0);
+            ok[u] = (s + u < s_end) && k < a.K;
+            const int64_t kc = ok[u] ? k : a.K - 16;
+            wv[u] = ldg16(wrow + kc);
+#pragma unroll
+            for (int t = 0; t < MT; ++t) xv[u][t] = ldg16(xrow[t] + kc);
         }
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
-            const int64_t k = (s + u) * 64 + kslot;
-            const bool ok = (s + u < s_end) && k < a.K;
-            const v4i fb = v4i{(int)wv[u].x, (int)wv[u].y, (int)wv[u].z, (int)wv[u].w};
+            const uint4 w4 = ok[u] ? wv[u] : make_uint4(0, 0, 0, 0);
+            const v4i fb = v4i{(int)w4.x, (int)w4.y, (int)w4.z, (int)w4.w};
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
-                const uint4 xv = ok ? ldg16(xrow[t] + k) : make_uint4(0, 0, 0, 0);
-                const v4i fa = v4i{(int)xv.x, (int)xv.y, (int)xv.z, (int)xv.w};
+                const v4i fa = v4i{(int)xv[u][t].x, (int)xv[u][t].y, (int)xv[u][t].z, (int)xv[u][t].w};
                 acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa, fb, acc[t], 0, 0, 0);
             }
         }
@@ -561,8 +566,10 @@ static size_t w8a8_decode_lds_bytes(int64_t M, int64_t K, int waves, int tn) {
 
 template <int WAVES, int XJ, int TN>
 static int launch_w8a8_decode(const W8A8Args& a, size_t lds, hipStream_t st) {
-    // per device and cheap; no state is kept in the library
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_decode_lds<WAVES, XJ, TN>),
+    // only launches above the default 64 KiB of dynamic LDS need the attribute; it is per device and cheap,
+    // so it is simply set on every such launch and no state is kept in the library
+    if (lds > 64 * 1024 &&
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_decode_lds<WAVES, XJ, TN>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess) {
         (void)hipGetLastError();
         return AMCT_E_HIP;
