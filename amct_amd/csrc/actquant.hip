@@ -182,8 +182,9 @@ using namespace amct;
 
 extern "C" int amct_act_quant_per_token_int8(const void* x, const void* smooth, int8_t* q, float* scale, int64_t M,
                                              int64_t K, int mode, int dtype, amct_stream_t stream) {
-    if (!x || !q || !scale || M < 0 || K <= 0 || (mode != 0 && mode != 1)) return AMCT_E_BADARG;
-    if (M == 0) return AMCT_OK;
+    if (M < 0 || K <= 0 || (mode != 0 && mode != 1)) return AMCT_E_BADARG;
+    if (M == 0) return AMCT_OK;                                   // nothing is read: null pointers are fine
+    if (!x || !q || !scale) return AMCT_E_BADARG;
     if (M > 0x7FFFFFFF) return AMCT_E_UNSUPPORTED;
     hipStream_t st = (hipStream_t)stream;
     switch (dtype) {
@@ -196,9 +197,10 @@ extern "C" int amct_act_quant_per_token_int8(const void* x, const void* smooth, 
 
 extern "C" int amct_quantize(const void* x, const void* smooth, const void* scales, const void* zero_points, int8_t* q,
                              int64_t M, int64_t K, int64_t n_scales, int per_token, int dtype, amct_stream_t stream) {
-    if (!x || !scales || !q || M < 0 || K <= 0) return AMCT_E_BADARG;
+    if (M < 0 || K <= 0) return AMCT_E_BADARG;
     if (per_token ? (n_scales != M) : (n_scales != 1 && n_scales != K)) return AMCT_E_BADARG;
     if (M == 0) return AMCT_OK;
+    if (!x || !scales || !q) return AMCT_E_BADARG;
     int64_t nb = (M * K + kBlock - 1) / kBlock;
     if (nb > 65536) nb = 65536;
     hipStream_t st = (hipStream_t)stream;

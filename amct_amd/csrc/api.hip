@@ -33,7 +33,7 @@ __global__ __launch_bounds__(kBlock) void copy_k(const uint4* src, uint4* dst, i
 }  // namespace amct
 
 extern "C" int amct_copy_bytes(const void* src, void* dst, int64_t nbytes, amct_stream_t stream) {
-    if (!src || !dst || nbytes < 0) return AMCT_E_BADARG;
+    if (nbytes < 0 || (nbytes != 0 && (!src || !dst))) return AMCT_E_BADARG;
     if (nbytes % 16 != 0 || !amct::aligned16(src) || !amct::aligned16(dst)) return AMCT_E_ALIGN;
     const int64_t nvec = nbytes / 16;
     if (nvec == 0) return AMCT_OK;

@@ -545,8 +545,9 @@ using namespace amct;
 
 extern "C" int amct_minmax(const void* w, float* mn, float* mx, int64_t rows, int64_t cols, int group, int dtype,
                            amct_stream_t stream) {
-    if (!w || !mn || !mx || rows < 0 || cols <= 0 || group < 0) return AMCT_E_BADARG;
-    if (rows == 0) return AMCT_OK;
+    if (rows < 0 || cols <= 0 || group < 0) return AMCT_E_BADARG;
+    if (rows == 0) return AMCT_OK;                                // nothing is read: null pointers are fine
+    if (!w || !mn || !mx) return AMCT_E_BADARG;
     if (rows > 0x7FFFFFFF) return AMCT_E_UNSUPPORTED;
     const int seg_len = group > 0 ? group : (int)cols;
     const int spr = group > 0 ? (int)((cols + group - 1) / group) : 1;
@@ -570,9 +571,10 @@ extern "C" int amct_minmax(const void* w, float* mn, float* mx, int64_t rows, in
 extern "C" int amct_scale_offset(const void* mx, const void* mn, float* scale, int32_t* offset, int32_t* bad_count,
                                  int64_t n, int bits, int symmetric, int scope_rule, int in_dtype,
                                  amct_stream_t stream) {
-    if (!mx || !mn || !scale || n < 0 || (bits != 4 && bits != 8)) return AMCT_E_BADARG;
-    if (!symmetric && !offset) return AMCT_E_BADARG;
+    if (n < 0 || (bits != 4 && bits != 8)) return AMCT_E_BADARG;
     if (n == 0) return AMCT_OK;
+    if (!mx || !mn || !scale) return AMCT_E_BADARG;
+    if (!symmetric && !offset) return AMCT_E_BADARG;
     const unsigned nb = (unsigned)((n + kBlock - 1) / kBlock);
     hipStream_t st = (hipStream_t)stream;
     switch (in_dtype) {
@@ -594,12 +596,14 @@ extern "C" int amct_quant_with_params(const void* w, const float* scale, const i
                                       int codes_kind, const void* col_scale, int col_mode, int64_t rows, int64_t cols,
                                       int group, int qmin, int qmax, int round_via_src_dtype, int stage, int dtype,
                                       amct_stream_t stream) {
-    if (!w || !scale || rows < 0 || cols <= 0 || group < -1 || qmin > qmax) return AMCT_E_BADARG;
+    if (rows < 0 || cols <= 0 || group < -1 || qmin > qmax) return AMCT_E_BADARG;
     if (stage < AMCT_STAGE_FULL || stage > AMCT_STAGE_COL) return AMCT_E_BADARG;
-    if (stage != AMCT_STAGE_FULL && (codes || !dq)) return AMCT_E_BADARG;
     if (codes && codes_kind != AMCT_CODES_I8 && codes_kind != AMCT_CODES_I32) return AMCT_E_BADARG;
-    if (col_mode < 0 || col_mode > 3 || (col_mode != AMCT_COL_NONE && !col_scale)) return AMCT_E_BADARG;
+    if (col_mode < 0 || col_mode > 3) return AMCT_E_BADARG;
     if (rows == 0) return AMCT_OK;
+    if (!w || !scale) return AMCT_E_BADARG;
+    if (stage != AMCT_STAGE_FULL && (codes || !dq)) return AMCT_E_BADARG;
+    if (col_mode != AMCT_COL_NONE && !col_scale) return AMCT_E_BADARG;
     FqArgs a{};
     if (!fill_geometry(a, rows, cols, group)) return AMCT_E_UNSUPPORTED;
     a.w = w; a.dq = dq; a.codes = codes; a.codes_kind = codes ? codes_kind : AMCT_CODES_NONE;
@@ -618,13 +622,15 @@ extern "C" int amct_fakequant_int(const void* w, void* dq, void* codes, int code
                                   int32_t* bad_count, const void* col_scale, int col_mode, int64_t rows, int64_t cols,
                                   int group, int bits, int symmetric, int scope_rule, int qmin, int qmax,
                                   int round_via_src_dtype, int dtype, amct_stream_t stream) {
-    if (!w || !scale || rows < 0 || cols <= 0 || group < 0 || qmin > qmax) return AMCT_E_BADARG;
+    if (rows < 0 || cols <= 0 || group < 0 || qmin > qmax) return AMCT_E_BADARG;
     if (bits != 4 && bits != 8) return AMCT_E_BADARG;
-    if (!symmetric && !offset) return AMCT_E_BADARG;
     if (codes && codes_kind != AMCT_CODES_I8 && codes_kind != AMCT_CODES_I32) return AMCT_E_BADARG;
-    if (col_mode < 0 || col_mode > 3 || (col_mode != AMCT_COL_NONE && !col_scale)) return AMCT_E_BADARG;
+    if (col_mode < 0 || col_mode > 3) return AMCT_E_BADARG;
     if (scope_rule != AMCT_SCOPE_AMCT && scope_rule != AMCT_SCOPE_ABSMAX) return AMCT_E_BADARG;
     if (rows == 0) return AMCT_OK;
+    if (!w || !scale) return AMCT_E_BADARG;
+    if (!symmetric && !offset) return AMCT_E_BADARG;
+    if (col_mode != AMCT_COL_NONE && !col_scale) return AMCT_E_BADARG;
     FqArgs a{};
     if (!fill_geometry(a, rows, cols, group)) return AMCT_E_UNSUPPORTED;
     a.w = w; a.dq = dq; a.codes = codes; a.codes_kind = codes ? codes_kind : AMCT_CODES_NONE;

@@ -903,7 +903,8 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
                                int scale_dtype, const uint8_t* zeros, const float* bias, void* out, int64_t M,
                                int64_t N, int64_t K, int group, int dtype, void* workspace, size_t workspace_bytes,
                                amct_stream_t stream) {
-    if (!x || !wq || !scales || !zeros || !out || M < 0 || N <= 0 || K <= 0 || group <= 0) return AMCT_E_BADARG;
+    if (M < 0 || N <= 0 || K <= 0 || group <= 0) return AMCT_E_BADARG;
+    if (M != 0 && (!x || !wq || !scales || !zeros || !out)) return AMCT_E_BADARG;   // M == 0 reads nothing
     if (scale_dtype != AMCT_F16 && scale_dtype != AMCT_BF16) return AMCT_E_BADARG;
     if (dtype != AMCT_BF16) return AMCT_E_UNSUPPORTED;
     if (K % group != 0 || K % 2 != 0) return AMCT_E_ALIGN;

@@ -614,8 +614,8 @@ using namespace amct;
 extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s_tok, const float* s_ch,
                               const void* bias, int bias_kind, void* out, int32_t* acc_out, int64_t M, int64_t N,
                               int64_t K, int out_dtype, amct_stream_t stream) {
-    if (!xq || !wq || !s_ch || !out || M < 0 || N <= 0 || K <= 0) return AMCT_E_BADARG;
-    if (bias_kind < 0 || bias_kind > 2 || (bias_kind != 0 && !bias)) return AMCT_E_BADARG;
+    if (M < 0 || N <= 0 || K <= 0 || bias_kind < 0 || bias_kind > 2) return AMCT_E_BADARG;
+    if (M != 0 && (!xq || !wq || !s_ch || !out || (bias_kind != 0 && !bias))) return AMCT_E_BADARG;   // M == 0 reads nothing
     if (out_dtype != AMCT_F32 && out_dtype != AMCT_F16 && out_dtype != AMCT_BF16) return AMCT_E_BADARG;
     if (M == 0) return AMCT_OK;
     W8A8Args a{xq, wq, s_tok, s_ch, bias_kind ? bias : nullptr, out, acc_out, M, N, K, bias_kind, out_dtype};

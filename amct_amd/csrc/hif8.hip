@@ -195,7 +195,7 @@ __global__ __launch_bounds__(kBlock) void hif8_decode_k(const uint8_t* x, void* 
 using namespace amct;
 
 extern "C" int amct_hif8_encode(const void* x, uint8_t* y, int64_t n, int dtype, int saturate, amct_stream_t stream) {
-    if (!x || !y || n < 0) return AMCT_E_BADARG;
+    if (n < 0 || (n != 0 && (!x || !y))) return AMCT_E_BADARG;   // n == 0 reads nothing: null pointers are fine
     if (!aligned16(x) || (reinterpret_cast<uintptr_t>(y) & 7u) != 0) return AMCT_E_ALIGN;
     if (n == 0) return AMCT_OK;
     constexpr int U = 4;
@@ -219,7 +219,7 @@ extern "C" int amct_hif8_encode(const void* x, uint8_t* y, int64_t n, int dtype,
 }
 
 extern "C" int amct_hif8_decode(const uint8_t* x, void* y, int64_t n, int dtype, amct_stream_t stream) {
-    if (!x || !y || n < 0) return AMCT_E_BADARG;
+    if (n < 0 || (n != 0 && (!x || !y))) return AMCT_E_BADARG;   // n == 0 reads nothing: null pointers are fine
     if (!aligned16(y) || (reinterpret_cast<uintptr_t>(x) & 7u) != 0) return AMCT_E_ALIGN;
     if (n == 0) return AMCT_OK;
     hipStream_t st = (hipStream_t)stream;

@@ -411,9 +411,10 @@ extern "C" int amct_quant_int4_group_pack(const void* w, uint8_t* packed, void* 
                                           float* scales32, uint8_t* zeros, int32_t* bad_count, const void* col_scale,
                                           int col_mode, int64_t rows, int64_t cols, int group, int symmetric, int dtype,
                                           amct_stream_t stream) {
-    if (!w || !packed || rows < 0 || cols <= 0 || group <= 0) return AMCT_E_BADARG;
+    if (rows < 0 || cols <= 0 || group <= 0) return AMCT_E_BADARG;
     if (scales16 && scale_dtype != AMCT_F16 && scale_dtype != AMCT_BF16) return AMCT_E_BADARG;
-    if (col_mode < 0 || col_mode > 2 || (col_mode != AMCT_COL_NONE && !col_scale)) return AMCT_E_BADARG;
+    if (col_mode < 0 || col_mode > 2) return AMCT_E_BADARG;
+    if (rows != 0 && (!w || !packed || (col_mode != AMCT_COL_NONE && !col_scale))) return AMCT_E_BADARG;   // rows == 0 reads nothing
     if (cols % group != 0 || group % 32 != 0) return AMCT_E_ALIGN;
     if (rows == 0) return AMCT_OK;
     PackArgs a{};
@@ -430,7 +431,7 @@ extern "C" int amct_quant_int4_group_pack(const void* w, uint8_t* packed, void* 
 }
 
 extern "C" int amct_pack_int4_words(const int32_t* codes, int32_t* words, int64_t k, int64_t n, amct_stream_t stream) {
-    if (!codes || !words || k < 0 || n < 0) return AMCT_E_BADARG;
+    if (k < 0 || n < 0 || (k * n != 0 && (!codes || !words))) return AMCT_E_BADARG;
     if (n % 8 != 0 || !aligned16(codes)) return AMCT_E_ALIGN;
     const int64_t nwords = k * (n / 8);
     if (nwords == 0) return AMCT_OK;
@@ -440,7 +441,7 @@ extern "C" int amct_pack_int4_words(const int32_t* codes, int32_t* words, int64_
 }
 
 extern "C" int amct_words_to_nibbles_nk(const int32_t* words, uint8_t* packed, int64_t k, int64_t n, amct_stream_t stream) {
-    if (!words || !packed || k < 0 || n < 0) return AMCT_E_BADARG;
+    if (k < 0 || n < 0 || (k * n != 0 && (!words || !packed))) return AMCT_E_BADARG;
     if (n % 8 != 0 || k % 2 != 0) return AMCT_E_ALIGN;
     const int64_t total = (k / 2) * (n / 8);
     if (total == 0) return AMCT_OK;
@@ -450,7 +451,7 @@ extern "C" int amct_words_to_nibbles_nk(const int32_t* words, uint8_t* packed, i
 }
 
 extern "C" int amct_pack_nibbles_nk(const int8_t* codes, uint8_t* packed, int64_t rows, int64_t cols, amct_stream_t stream) {
-    if (!codes || !packed || rows < 0 || cols < 0) return AMCT_E_BADARG;
+    if (rows < 0 || cols < 0 || (rows * cols != 0 && (!codes || !packed))) return AMCT_E_BADARG;
     if (cols % 2 != 0) return AMCT_E_ALIGN;
     const int64_t nbytes = rows * (cols / 2);
     if (nbytes == 0) return AMCT_OK;
@@ -460,7 +461,7 @@ extern "C" int amct_pack_nibbles_nk(const int8_t* codes, uint8_t* packed, int64_
 }
 
 extern "C" int amct_nibbles_nk_to_codes_kn(const uint8_t* packed, int32_t* codes, int64_t k, int64_t n, amct_stream_t stream) {
-    if (!packed || !codes || k < 0 || n < 0) return AMCT_E_BADARG;
+    if (k < 0 || n < 0 || (k * n != 0 && (!packed || !codes))) return AMCT_E_BADARG;
     if (k % 2 != 0) return AMCT_E_ALIGN;
     if (k * n == 0) return AMCT_OK;
     hipLaunchKernelGGL(nibbles_to_codes_kn_k, dim3((unsigned)((k * n + kBlock - 1) / kBlock)), dim3(kBlock), 0,

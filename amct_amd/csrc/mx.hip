@@ -255,7 +255,7 @@ using namespace amct;
 // instead of the hardware conversion instructions (both give identical codes).
 extern "C" int amct_mx_quant(const void* x, uint8_t* elems, uint8_t* e8m0, int64_t rows, int64_t cols, int fmt,
                              int scale_mode, int dtype, amct_stream_t stream) {
-    if (!x || !elems || !e8m0 || rows < 0 || cols <= 0) return AMCT_E_BADARG;
+    if (rows < 0 || cols <= 0 || (rows != 0 && (!x || !elems || !e8m0))) return AMCT_E_BADARG;   // rows == 0 reads nothing
     if (fmt != kFmtE4M3 && fmt != kFmtE2M1) return AMCT_E_BADARG;
     if ((scale_mode & ~0x101) != 0) return AMCT_E_BADARG;
     if (cols % 32 != 0 || !aligned16(x) || (reinterpret_cast<uintptr_t>(elems) & 7u) != 0) return AMCT_E_ALIGN;
@@ -278,7 +278,7 @@ extern "C" int amct_mx_quant(const void* x, uint8_t* elems, uint8_t* e8m0, int64
 
 extern "C" int amct_mx_dequant(const uint8_t* elems, const uint8_t* e8m0, void* y, int64_t rows, int64_t cols, int fmt,
                                int dtype, amct_stream_t stream) {
-    if (!elems || !e8m0 || !y || rows < 0 || cols <= 0) return AMCT_E_BADARG;
+    if (rows < 0 || cols <= 0 || (rows != 0 && (!elems || !e8m0 || !y))) return AMCT_E_BADARG;
     if (fmt != kFmtE4M3 && fmt != kFmtE2M1) return AMCT_E_BADARG;
     if (cols % 32 != 0 || !aligned16(y) || (reinterpret_cast<uintptr_t>(elems) & 7u) != 0) return AMCT_E_ALIGN;
     if (rows == 0) return AMCT_OK;

@@ -11,6 +11,10 @@
  *     enqueues work on `stream` and returns;
  *   - return value: 0 on success, a negative AMCT_E_* code otherwise
  *     (amct_hip_strerror gives the text); no exception crosses the boundary;
+ *     a call that fails enqueues nothing and leaves its outputs untouched;
+ *   - an empty problem (rows, M or n equal to 0) succeeds without enqueuing
+ *     anything, and its tensor pointers may then be null (an empty torch
+ *     tensor has a null data pointer);
  *   - dtype arguments use AMCT_F32 / AMCT_F16 / AMCT_BF16, numbered like the
  *     reference's DATA_MAP (amct_pytorch/utils/data_utils.py:19-23).
  *
