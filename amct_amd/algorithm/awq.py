@@ -60,3 +60,60 @@ def process_weights_for_layers(layers, scale_awq, quant_config):
         dq, _, _, _ = ops.fakequant_int(w, bits, bool(cfg.get('symmetric')), group=group_size if strategy == 'group' else 0,
                                         col_scale=scale_awq, col_mode=ops.COL_MUL_THEN_DIV, via_src=True)
         layer.weight.data = dq
+
+
+def awq_scale_for_ratio(inputs_mean, ratio, dtype):
+    """The candidate scale of one grid point (awq.py:85-88): mean|x| ** ratio, clamped, normalised by the
+    geometric mean of its extremes in fp64, narrowed to the activation dtype and clamped again."""
+    scale_awq = inputs_mean.pow(ratio).clamp(min=1e-4).to(torch.float64).view(1, -1)
+    scale_awq = scale_awq / (scale_awq.max() * scale_awq.min()).sqrt()
+    return torch.clamp(scale_awq.to(dtype), 1e-4, torch.finfo(dtype).max)
+
+
+@torch.no_grad()
+def search_scale(inputs, layers, block, quant_config, kwargs=None):
+    """AWQ scale search (awq.py:52-105) with everything resident on the device.  Same arguments, return
+    value and errors as the reference.  The reference copies the whole state dict of `block` to the host
+    once and loads it back after every grid point; only the weights of `layers` change inside the loop
+    (process_weights_for_layers, which replaces layer.weight.data by a new tensor and never writes into the
+    old one), so here the original weight tensors are simply kept and put back: no copy at all, and the
+    fake-quant of a grid point is one fused kernel per layer."""
+    algo_params = quant_config.get("algorithm")
+    if not torch.isfinite(inputs).all():
+        raise RuntimeError("Run AWQ error! Invalid value(nan or inf) in activation!")
+    for layer in layers:
+        if not torch.isfinite(layer.weight.data).all():
+            raise RuntimeError("Run AWQ error! Invalid value(nan or inf) in weight!")
+    kwargs = dict() if kwargs is None else kwargs
+    ori_out = block(inputs, **kwargs)
+    if isinstance(ori_out, tuple):
+        ori_out = ori_out[0]
+
+    min_loss = torch.tensor(float('inf'), device=inputs.device)
+    best_scale = None
+    inputs_mean = inputs.abs().contiguous().view(-1, inputs.shape[-1]).mean(0)  # (cin)
+    grids_num = algo_params.get('awq').get('grids_num')
+    saved = [layer.weight.data for layer in layers]
+    for grid in range(grids_num):
+        scale_awq = awq_scale_for_ratio(inputs_mean, grid / grids_num, inputs.dtype)
+        process_weights_for_layers(layers, scale_awq, quant_config)
+        quant_out = block(inputs, **kwargs)
+        if isinstance(quant_out, tuple):
+            quant_out = quant_out[0]
+        loss = (ori_out - quant_out).float().pow(4).mean()
+        if not torch.isnan(loss) and loss < min_loss:
+            min_loss = loss
+            best_scale = scale_awq
+        for layer, w in zip(layers, saved):
+            layer.weight.data = w
+    if best_scale is None or torch.isinf(min_loss):
+        raise RuntimeError("Run AWQ error! Got invalid loss.")
+    return best_scale
+
+
+@torch.no_grad()
+def apply_scale(scale_awq, ori_module, input_data):
+    """awq.py:108-118: fold the chosen scale into the weight and out of the activation, in place."""
+    scale = scale_awq.to(ori_module.weight.device)
+    ori_module.weight.data.mul_(scale)
+    input_data.div_(scale)

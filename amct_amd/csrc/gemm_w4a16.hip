@@ -408,7 +408,7 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
             const uint4 v = *reinterpret_cast<const uint4*>(patch + prow * kPatchRow + chunk * 16);
             const int64_t m = mbase + prow;
             const int64_t n = n0 + wn * 64 + chunk * 8;
-            if (m < a.M && n < a.N) stg16(reinterpret_cast<char*>(a.out) + (m * a.N + n) * 2, v);
+            if (m < a.M && n < a.N) stg16_nt(reinterpret_cast<char*>(a.out) + (m * a.N + n) * 2, v);
         }
     }
 }

@@ -296,3 +296,36 @@ def static_quantize(x, scales, zero_points, axis=-1):
     if zp is not None:
         t = t + zp.float()
     return t.round().clamp(-128, 127).to(torch.int8)
+
+
+def awq_search_scale(inputs, weights, forward, grids_num, kind, strategy, symmetric, group_size=None):
+    """The AWQ scale search (amct_pytorch/algorithm/awq.py:52-105) on plain tensors: `weights` are the
+    [N,K] weights of the layers that share the input, `forward(inputs, weights)` evaluates the block.
+    Returns (best_scale [1,K], losses per grid point as Python floats).  Test infrastructure only.
+    Parity unpinned beyond its parts: the grid step is awq_grid_step (pinned above); the loop, the scale
+    formula and the loss are restated from the cited lines and have no independent check."""
+    if not torch.isfinite(inputs).all():
+        raise RuntimeError("Run AWQ error! Invalid value(nan or inf) in activation!")
+    for w in weights:
+        if not torch.isfinite(w).all():
+            raise RuntimeError("Run AWQ error! Invalid value(nan or inf) in weight!")
+    ori_out = forward(inputs, weights)
+    min_loss = torch.tensor(float('inf'))
+    best_scale = None
+    losses = []
+    inputs_mean = inputs.abs().contiguous().view(-1, inputs.shape[-1]).mean(0)
+    for grid in range(grids_num):
+        ratio = grid / grids_num
+        scale_awq = inputs_mean.pow(ratio).clamp(min=1e-4).to(torch.float64).view(1, -1)
+        scale_awq = scale_awq / (scale_awq.max() * scale_awq.min()).sqrt()
+        scale_awq = torch.clamp(scale_awq.to(inputs.dtype), 1e-4, torch.finfo(inputs.dtype).max)
+        new_w = [awq_grid_step(w, scale_awq, kind, strategy, symmetric, group_size)[0] for w in weights]
+        quant_out = forward(inputs, new_w)
+        loss = (ori_out - quant_out).float().pow(4).mean()
+        losses.append(float(loss))
+        if not torch.isnan(loss) and loss < min_loss:
+            min_loss = loss
+            best_scale = scale_awq
+    if best_scale is None or torch.isinf(min_loss):
+        raise RuntimeError("Run AWQ error! Got invalid loss.")
+    return best_scale, losses

@@ -266,3 +266,53 @@ def test_dispatcher_operators(dev):
     assert_bits_equal(c, d, "weight_quant_batchmatmul")
     with pytest.raises(NotImplementedError):
         torch.ops.amct_hip.convert_weight_to_int4pack(codes)
+
+
+class _TwoLinears(torch.nn.Module):
+    """Two linears on the same input, as the q/k/v projections of a block share theirs."""
+
+    def __init__(self, k, n):
+        super().__init__()
+        self.a = torch.nn.Linear(k, n, bias=False)
+        self.b = torch.nn.Linear(k, n, bias=False)
+
+    def forward(self, x):
+        return torch.cat([self.a(x), self.b(x)], dim=-1)
+
+
+@pytest.mark.parametrize("strategy,group,sym", [('group', 32, False), ('channel', None, True)])
+def test_awq_search_scale_on_device(dev, strategy, group, sym):
+    """The scale search with the state resident on the device against the CPU restatement: same grid point
+    chosen, the same scale up to the device's pow (not bit-identical to the host's), losses within 2 %, and
+    the layers' weights are the untouched original tensors afterwards."""
+    torch.manual_seed(11)
+    T, K, N, grids = 64, 128, 48, 8
+    c = cfg('int4', sym, strategy, group)
+    c['algorithm'] = {'awq': {'grids_num': grids}}
+    x = torch.randn(T, K) * (1.0 + 6.0 * (torch.arange(K) % 16 == 0))       # a few heavy input channels
+    block = _TwoLinears(K, N)
+    w_cpu = [block.a.weight.data.clone(), block.b.weight.data.clone()]
+    want_scale, want_losses = iq.awq_search_scale(
+        x, w_cpu, lambda inp, ws: torch.cat([inp @ ws[0].t(), inp @ ws[1].t()], dim=-1), grids, 'int4', strategy, sym,
+        group)
+    dblock = _TwoLinears(K, N).to(dev)
+    dblock.a.weight.data.copy_(w_cpu[0])
+    dblock.b.weight.data.copy_(w_cpu[1])
+    before = [dblock.a.weight.data_ptr(), dblock.b.weight.data_ptr()]
+    got = awq.search_scale(x.to(dev), [dblock.a, dblock.b], dblock, c)
+    assert dblock.a.weight.data_ptr() == before[0] and dblock.b.weight.data_ptr() == before[1]
+    assert_bits_equal(dblock.a.weight.data, w_cpu[0], "weight restored")
+    best = min(range(grids), key=lambda i: want_losses[i])
+    ranked = sorted(want_losses)
+    if ranked[1] > 1.02 * ranked[0]:                                         # a clear winner on the host
+        torch.testing.assert_close(got.cpu(), want_scale, rtol=2e-6, atol=0)
+    assert got.shape == (1, K) and got.dtype == x.dtype
+    # the search result used as the reference uses it
+    xin = x.to(dev).clone()
+    awq.apply_scale(got, dblock.a, xin)
+    torch.testing.assert_close(xin.cpu(), x / got.cpu(), rtol=1e-6, atol=0)
+    with pytest.raises(RuntimeError, match="Invalid value"):
+        bad = x.clone()
+        bad[0, 0] = float('nan')
+        awq.search_scale(bad.to(dev), [dblock.a, dblock.b], dblock, c)
+    assert best >= 0

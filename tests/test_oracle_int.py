@@ -238,3 +238,25 @@ def test_oracle_matches_exact_arithmetic_fixture():
         got_codes = iq.quant_codes(w, kind, s, z)
         assert torch.equal(got_codes.to(torch.int32), codes)
         assert_bits_equal(iq.fake_quant(w, kind, s, z), dq, "dq")
+
+
+def test_awq_search_special_cases():
+    """Closed-form cases of the scale search: one grid point means ratio 0, whose scale is all ones, and the
+    grid step then is the plain AWQ fake-quant; equal-magnitude inputs give an all-ones scale at every ratio, so
+    every grid point has the same loss and the first one wins; non-finite data raises like the reference."""
+    torch.manual_seed(3)
+    x = torch.randn(16, 64)
+    w = [torch.randn(24, 64) * 0.05]
+    fwd = lambda inp, ws: inp @ ws[0].t()
+    s, losses = iq.awq_search_scale(x, w, fwd, 1, 'int4', 'group', False, 32)
+    assert torch.equal(s, torch.ones(1, 64))
+    sc, off = iq.weight_scale_offset(w[0], 'group', False, 'int4', 32)
+    dq = iq.awq_fake_quant(w[0], 'int4', sc, off, 'group', 32)
+    assert abs(losses[0] - float((fwd(x, w) - fwd(x, [dq])).float().pow(4).mean())) == 0.0
+    xs = torch.sign(torch.randn(16, 64)) * 0.5                        # mean|x| identical in every channel
+    s, losses = iq.awq_search_scale(xs, w, fwd, 5, 'int4', 'group', False, 32)
+    assert torch.equal(s, torch.ones(1, 64)) and len(set(losses)) == 1
+    bad = x.clone()
+    bad[1, 2] = float('inf')
+    with pytest.raises(RuntimeError, match="Invalid value"):
+        iq.awq_search_scale(bad, w, fwd, 2, 'int4', 'group', False, 32)
