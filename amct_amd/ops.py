@@ -65,6 +65,27 @@ def minmax(w, group=0):
     return mn, mx
 
 
+def col_minmax(x, col_max=None, col_min=None, absolute=False):
+    """Per-column (input channel) max and min over all rows of x [rows, cols] -> fp32 [cols] each.
+    With col_max / col_min given (fp32 [cols]) the running update `batch > old ? batch : old` is applied to
+    them in place and they are returned; absolute=True reduces |x| and returns only the maximum."""
+    dev = _dev(x, col_max, col_min)
+    x = _c(x)
+    rows, cols = x.shape
+    accumulate = col_max is not None or col_min is not None
+    if col_max is None:
+        col_max = torch.empty(cols, dtype=torch.float32, device=dev)
+    if col_min is None and not absolute:
+        col_min = torch.empty(cols, dtype=torch.float32, device=dev)
+    lib = _lib.load()
+    nbytes = lib.amct_col_minmax_workspace_bytes(rows, cols)
+    ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(lib.amct_col_minmax(_p(x), _p(col_max), None if absolute else _p(col_min), rows, cols, int(absolute),
+                                       int(accumulate), dtype_code(x.dtype), _p(ws), nbytes, _stream(dev)))
+    return col_max if absolute else (col_max, col_min)
+
+
 def scale_offset(vmax, vmin, bits, symmetric, scope_rule=SCOPE_AMCT, bad=None):
     """Elementwise (max, min) -> (scale fp32, offset int32 | None), same shape as the inputs."""
     dev = _dev(vmax, vmin, bad)

@@ -197,6 +197,25 @@ def build_cases(dev, only):
         cases.append(Case("act_quant_per_token", "hbm", work, "B", launch, ns, "f32",
                           "dynamic per-token INT8 quantize, X[2048,4096] bf16 (config 4)"))
 
+    # ---- column statistics over tokens (SmoothQuant calibration), X[8192,4096] bf16 ----------------------
+    if want("col_minmax"):
+        xc = workloads.c3_activations()
+        Rc, Cc = xc.shape
+        work = Rc * Cc * 2 + 2 * Cc * 4
+        nsc2 = sets_for(work)
+        xcs = dev_copies(xc, nsc2)
+        cmx = torch.empty(Cc, dtype=torch.float32, device=dev)
+        cmn = torch.empty(Cc, dtype=torch.float32, device=dev)
+        wsb = lib.amct_col_minmax_workspace_bytes(Rc, Cc)
+        wsc = torch.empty(wsb, dtype=torch.uint8, device=dev)
+
+        def launch(i, xcs=xcs, cmx=cmx, cmn=cmn, wsc=wsc, wsb=wsb, Rc=Rc, Cc=Cc):
+            rc = lib.amct_col_minmax(xcs[i % len(xcs)].data_ptr(), cmx.data_ptr(), cmn.data_ptr(), Rc, Cc, 0, 0, _lib.BF16,
+                                     wsc.data_ptr(), wsb, st)
+            assert rc == 0, rc
+        cases.append(Case("col_minmax", "hbm", work, "B", launch, nsc2, "f32",
+                          "per-channel max/min over tokens, X[8192,4096] bf16 (two kernels per call)"))
+
     # ---- K6: W8A8 Linear, W[14336,4096] int8 ----------------------------------------------------------
     if want("w8a8_m2048") or want("w8a8_m16"):
         x6, wq6, sw6 = workloads.c4_w8a8()

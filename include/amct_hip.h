@@ -77,6 +77,19 @@ const char* amct_hip_strerror(int code);
  * the yardstick for the bandwidth figures and for scaling hardware traffic counters. */
 int amct_copy_bytes(const void* src, void* dst, int64_t nbytes, amct_stream_t stream);
 
+/* ---- column statistics over tokens (calibration of the smoothing factor) -----------------
+ * Replaces the reductions of amct_pytorch/quantize_op/smooth_quant_module.py: :79-80 batch amax / amin over
+ * all tokens per input channel, :88-91 the running update data_max = batch_max > data_max ? batch_max :
+ * data_max (and the mirror image for the minimum), :121 |W|.amax(dim=0).
+ * x [rows, cols]; col_max, col_min fp32 [cols] (either may be null).  absolute != 0 reduces |x|.
+ * accumulate = 0 overwrites the outputs with this batch's values; accumulate != 0 applies the running update
+ * to the values already there (a NaN batch value leaves them unchanged, as torch.where does).
+ * max / min propagate NaN like torch.amax / amin.  workspace: amct_col_minmax_workspace_bytes(rows, cols)
+ * bytes of device memory, 4-byte aligned, contents irrelevant before and after the call. */
+size_t amct_col_minmax_workspace_bytes(int64_t rows, int64_t cols);
+int amct_col_minmax(const void* x, float* col_max, float* col_min, int64_t rows, int64_t cols, int absolute,
+                    int accumulate, int dtype, void* workspace, size_t workspace_bytes, amct_stream_t stream);
+
 /* ---- A1: min / max per row (group = 0) or per group of `group` columns ----------------
  * Replaces get_weight_min_max_by_granularity (amct_pytorch/quantize_op/utils.py:111-136)
  * and the per-token reductions of amct_pytorch/quantize_op/minmax_module.py:96-105.

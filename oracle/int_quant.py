@@ -329,3 +329,23 @@ def awq_search_scale(inputs, weights, forward, grids_num, kind, strategy, symmet
     if best_scale is None or torch.isinf(min_loss):
         raise RuntimeError("Run AWQ error! Got invalid loss.")
     return best_scale, losses
+
+
+# --------------------------------------------------------------------------
+# SmoothQuant calibration statistics (amct_pytorch/quantize_op/smooth_quant_module.py)
+# --------------------------------------------------------------------------
+def channel_min_max_update(inputs, data_max, data_min):
+    """:79-80, :88-91 -- batch amax / amin per input channel over all tokens, then the running update."""
+    batch_max = inputs.reshape(-1, inputs.shape[-1]).amax(dim=0, keepdim=True)
+    batch_min = inputs.reshape(-1, inputs.shape[-1]).amin(dim=0, keepdim=True)
+    data_max = torch.where(batch_max > data_max, batch_max, data_max)
+    data_min = torch.where(batch_min < data_min, batch_min, data_min)
+    return data_max, data_min
+
+
+def smooth_factor(act_max, weight, smooth_strength):
+    """:113-133 -- act_max^a / (|W|.amax(dim=0))^(1-a), 1 where below eps or not finite."""
+    wts_max = weight.abs().amax(dim=0, keepdim=True)
+    f = (act_max ** smooth_strength) / (wts_max ** (1 - smooth_strength))
+    bad = (f < torch.finfo(act_max.dtype).eps) | ~torch.isfinite(f)
+    return torch.where(bad, torch.tensor(1.0, dtype=f.dtype), f)

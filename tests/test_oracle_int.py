@@ -260,3 +260,22 @@ def test_awq_search_special_cases():
     bad[1, 2] = float('inf')
     with pytest.raises(RuntimeError, match="Invalid value"):
         iq.awq_search_scale(bad, w, fwd, 2, 'int4', 'group', False, 32)
+
+
+def test_channel_stats_known_answers():
+    """Column statistics: hand-checkable values, the running update over two batches, a NaN batch value
+    that the update ignores (NaN > x is false), and the smoothing factor's closed forms (strength 1 gives
+    act_max, strength 0 gives 1 / wts_max, non-positive or non-finite factors become 1)."""
+    x1 = torch.tensor([[1.0, -2.0, 0.5], [3.0, -1.0, float('nan')]])
+    dmax = torch.full((1, 3), float('-inf'))
+    dmin = torch.full((1, 3), float('inf'))
+    dmax, dmin = iq.channel_min_max_update(x1, dmax, dmin)
+    assert dmax.tolist() == [[3.0, -1.0, float('-inf')]] and dmin.tolist() == [[1.0, -2.0, float('inf')]]
+    x2 = torch.tensor([[[2.0, -5.0, 0.25]], [[-4.0, 0.0, 0.75]]])          # rank 3: all leading dims are tokens
+    dmax, dmin = iq.channel_min_max_update(x2, dmax, dmin)
+    assert dmax.tolist() == [[3.0, 0.0, 0.75]] and dmin.tolist() == [[-4.0, -5.0, 0.25]]
+    w = torch.tensor([[0.5, -4.0, 0.0], [-2.0, 1.0, 0.0]])
+    act = torch.tensor([[4.0, 9.0, 1.0]])
+    assert torch.equal(iq.smooth_factor(act, w, 1.0), act)
+    assert torch.equal(iq.smooth_factor(act, w, 0.0)[:, :2], torch.tensor([[0.5, 0.25]]))
+    assert torch.equal(iq.smooth_factor(act, w, 0.5), torch.tensor([[2.0 / 2.0 ** 0.5, 1.5, 1.0]]))   # x / 0 -> inf -> 1
