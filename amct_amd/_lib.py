@@ -26,6 +26,9 @@ SIGNATURES = {
     "amct_hip_strerror": (ctypes.c_char_p, [_I]),
     "amct_copy_bytes": (_I, [_P, _P, _L, _P]),
     "amct_minmax": (_I, [_P, _P, _P, _L, _L, _I, _I, _P]),
+    "amct_fp8_block_dequant": (_I, [_P, _P, _P, _L, _L, _I, _I, _P]),
+    "amct_pack_int4_pairs_n": (_I, [_P, _P, _L, _L, _P]),
+    "amct_scale_f32_to_u64": (_I, [_P, _P, _L, _P]),
     "amct_col_minmax_workspace_bytes": (ctypes.c_size_t, [_L, _L]),
     "amct_col_minmax": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _P, ctypes.c_size_t, _P]),
     "amct_scale_offset": (_I, [_P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _P]),

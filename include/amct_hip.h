@@ -224,6 +224,18 @@ int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t* wq, const 
                     int64_t M, int64_t N, int64_t K, int group, int dtype,
                     void* workspace, size_t workspace_bytes, amct_stream_t stream);
 
+/* ---- interchange formats of the checkpoint converter ---------------------------------------
+ * (amct_pytorch/experimental/quantization/DeepSeekV3.2/deploy.py)
+ * amct_fp8_block_dequant: weight_dequant :48-92.  w E4M3FN codes [rows, cols], scale fp32
+ *   [ceil(rows/block), ceil(cols/block)]; out[r][c] = out_dtype(fp32(w[r][c]) * scale[r/block][c/block]).
+ * amct_pack_int4_pairs_n: pack_4bit :110-127.  x int8 [n, k] holding int4 values, n even;
+ *   y int8 [n/2, k] = (x[2i+1][k] << 4) | (x[2i][k] & 15): two output channels per byte.
+ * amct_scale_f32_to_u64: scale_fp32_to_u64 :95-107.  out[i] = the bits of s[i] in the low 32 bits, 0 above. */
+int amct_fp8_block_dequant(const uint8_t* w, const float* scale, void* out, int64_t rows, int64_t cols,
+                           int block, int out_dtype, amct_stream_t stream);
+int amct_pack_int4_pairs_n(const int8_t* x, int8_t* y, int64_t n, int64_t k, amct_stream_t stream);
+int amct_scale_f32_to_u64(const float* s, uint64_t* out, int64_t n, amct_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

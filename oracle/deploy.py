@@ -259,3 +259,31 @@ def w4a16_forward_f64(x, codes_nk, scale_ng, antioffset_ng, group_size, bias=Non
         x2 = torch.mul(x2, scale_factor.to(x2.dtype))
     wdq = dequant_weight(codes_nk, scale_ng, antioffset_ng, group_size, x.dtype)
     return weight_quant_matmul_f64(x2, wdq, bias).reshape(*shp[:-1], -1)
+
+
+# --------------------------------------------------------------------------
+# interchange formats of the checkpoint converter
+# (amct_pytorch/experimental/quantization/DeepSeekV3.2/deploy.py)
+# --------------------------------------------------------------------------
+def fp8_block_dequant(weight, scale, block_size=128, out_dtype=torch.bfloat16):
+    """weight_dequant :48-92 -- fp32(weight) * scale expanded per block, one rounding to out_dtype.
+    Pinned by tests/test_oracle_int.py::test_interchange_known_answers (exact products of powers of two)."""
+    m, n = weight.shape
+    s = scale.repeat_interleave(block_size, dim=0).repeat_interleave(block_size, dim=1)[:m, :n]
+    return (weight.to(torch.float32) * s).to(out_dtype)
+
+
+def pack_4bit(x):
+    """pack_4bit :110-127 -- pairs of output channels per byte, returned [n/2, k]."""
+    x = x.T.contiguous()
+    shape = x.shape
+    x = x.view(-1, 2)
+    y = torch.bitwise_or(x[:, 0] & 0b00001111, torch.bitwise_left_shift(x[:, 1], 4))
+    return y.view(shape[0], shape[1] // 2).T.contiguous()
+
+
+def scale_fp32_to_u64(weight_scale):
+    """scale_fp32_to_u64 :95-107 -- the fp32 bits in the low half of a 64-bit word (as int64 here)."""
+    import numpy as np
+    bits = weight_scale.float().cpu().numpy().view(np.uint32).astype(np.uint64)
+    return torch.from_numpy(bits.astype(np.int64))

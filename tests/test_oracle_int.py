@@ -279,3 +279,19 @@ def test_channel_stats_known_answers():
     assert torch.equal(iq.smooth_factor(act, w, 1.0), act)
     assert torch.equal(iq.smooth_factor(act, w, 0.0)[:, :2], torch.tensor([[0.5, 0.25]]))
     assert torch.equal(iq.smooth_factor(act, w, 0.5), torch.tensor([[2.0 / 2.0 ** 0.5, 1.5, 1.0]]))   # x / 0 -> inf -> 1
+
+
+def test_interchange_known_answers():
+    """fp8 block dequant, pair packing and scale widening on values whose results are known exactly."""
+    from oracle import deploy as od
+    codes = torch.tensor([[0x38, 0xB8, 0x40, 0x01], [0x7E, 0x00, 0x80, 0x30]], dtype=torch.uint8)   # 1, -1, 2, 2^-9; 448, 0, -0, 0.5
+    w = codes.view(torch.float8_e4m3fn)
+    scale = torch.tensor([[0.5, 4.0]])
+    out = od.fp8_block_dequant(w, scale, block_size=2, out_dtype=torch.float32)
+    assert out.tolist() == [[0.5, -0.5, 8.0, 2.0 ** -7], [224.0, 0.0, -0.0, 2.0]]
+    x = torch.tensor([[5, -7], [-8, 7], [0, 1], [-1, -2]], dtype=torch.int8)
+    y = od.pack_4bit(x)
+    # rows (0,1) -> (x1 << 4) | (x0 & 15): 5,-8 -> 0x85 ; -7,7 -> 0x79 ; rows (2,3): 0,-1 -> 0xF0 ; 1,-2 -> 0xE1
+    assert y.view(torch.uint8).tolist() == [[0x85, 0x79], [0xF0, 0xE1]]
+    s = torch.tensor([[1.0, -2.0]])
+    assert od.scale_fp32_to_u64(s).tolist() == [[0x3F800000, 0xC0000000]]
