@@ -216,6 +216,27 @@ def build_cases(dev, only):
         cases.append(Case("col_minmax", "hbm", work, "B", launch, nsc2, "f32",
                           "per-channel max/min over tokens, X[8192,4096] bf16 (two kernels per call)"))
 
+    # ---- GPTQ inner block: 128 columns of W[14336,4096] fp32, int4 asymmetric per-channel ----------------
+    if want("gptq_block"):
+        Ng, Kg, cnt = 14336, 4096, 128
+        gq = torch.Generator().manual_seed(1013)
+        wg = [(torch.randn(Ng, Kg, generator=gq) * 0.02).to(dev) for _ in range(2)]
+        hq = torch.triu(torch.randn(cnt, cnt, generator=gq) * 0.05 + torch.eye(cnt)).to(dev).contiguous()
+        sg = (torch.rand(Ng, generator=gq) * 0.01 + 0.002).to(dev)
+        zg = torch.randint(-8, 8, (Ng,), generator=gq, dtype=torch.int32).to(dev)
+        eg = torch.empty(Ng, cnt, dtype=torch.float32, device=dev)
+        gi = torch.zeros(cnt, dtype=torch.int32, device=dev)
+        work = Ng * cnt * 4 * 3 + cnt * cnt * 4
+
+        def launch(i, wg=wg, hq=hq, sg=sg, zg=zg, eg=eg, gi=gi, Ng=Ng, Kg=Kg, cnt=cnt):
+            # successive launches walk over the column blocks of two matrices: the data is not cache-resident
+            wsel = wg[(i // 32) % 2]
+            rc = lib.amct_gptq_block(wsel.data_ptr() + (i % 32) * cnt * 4, Kg, eg.data_ptr(), cnt, hq.data_ptr(), cnt,
+                                     sg.data_ptr(), zg.data_ptr(), 1, gi.data_ptr(), Ng, cnt, -8, 7, st)
+            assert rc == 0, rc
+        cases.append(Case("gptq_block", "hbm", work, "B", launch, 2, "f32",
+                          "GPTQ column loop of one 128-column block, W[14336,4096] fp32 (latency/ALU-bound: 128 dependent steps)"))
+
     # ---- K6: W8A8 Linear, W[14336,4096] int8 ----------------------------------------------------------
     if want("w8a8_m2048") or want("w8a8_m16"):
         x6, wq6, sw6 = workloads.c4_w8a8()

@@ -224,6 +224,21 @@ int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t* wq, const 
                     int64_t M, int64_t N, int64_t K, int group, int dtype,
                     void* workspace, size_t workspace_bytes, amct_stream_t stream);
 
+/* ---- GPTQ inner block ------------------------------------------------------------------------
+ * The column loop of amct_pytorch/quantize_op/gptq_module.py:128-151 for one block of count <= 128 columns,
+ * all rows in one launch.  For i = 0 .. count-1, per row n:
+ *   wq = ((clamp(rne(w[n][i] / s + z), qmin, qmax)) - z) * s;  err = (w[n][i] - wq) / hinv[i][i];
+ *   w[n][j] -= err * hinv[i][j] for j = i .. count-1;  err_out[n][i] = err
+ * with s = scale[n * scale_stride + gidx[i]], z = offset[same index] (offset null: symmetric).  scale_stride = 0
+ * shares one row of factors among all rows (per-tensor); gidx[i] is the factor column of block column i
+ * (perm[i1 + i] / group_size for per-group factors, 0 otherwise).  w points at the block's first column inside
+ * the column-sorted fp32 weight (row stride ld_w), hinv at the block's diagonal element (row stride ld_h);
+ * err_out [rows, count] (row stride ld_e) feeds the reference's trailing update
+ * weight[:, i2:] -= err_block @ hinv[i1:i2, i2:], which stays a library GEMM. */
+int amct_gptq_block(float* w, int64_t ld_w, float* err_out, int64_t ld_e, const float* hinv, int64_t ld_h,
+                    const float* scale, const int32_t* offset, int64_t scale_stride, const int32_t* gidx,
+                    int64_t rows, int count, int qmin, int qmax, amct_stream_t stream);
+
 /* ---- interchange formats of the checkpoint converter ---------------------------------------
  * (amct_pytorch/experimental/quantization/DeepSeekV3.2/deploy.py)
  * amct_fp8_block_dequant: weight_dequant :48-92.  w E4M3FN codes [rows, cols], scale fp32

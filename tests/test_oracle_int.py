@@ -295,3 +295,36 @@ def test_interchange_known_answers():
     assert y.view(torch.uint8).tolist() == [[0x85, 0x79], [0xF0, 0xE1]]
     s = torch.tensor([[1.0, -2.0]])
     assert od.scale_fp32_to_u64(s).tolist() == [[0x3F800000, 0xC0000000]]
+
+
+def test_gptq_block_loop_against_scalar_model():
+    """The block loop restated with numpy float32 scalars, one rounding per operation written out, and the
+    invariant that a finished column holds w - err * d."""
+    from oracle import gptq as og
+    rng = np.random.default_rng(4)
+    n, count = 5, 7
+    w0 = (rng.standard_normal((n, count)) * 0.1).astype(np.float32)
+    a = rng.standard_normal((count, count)).astype(np.float32)
+    hinv = np.triu(a * 0.1 + np.eye(count, dtype=np.float32))
+    for sym in (True, False):
+        wt = torch.from_numpy(w0.copy())
+        s, z = iq.weight_scale_offset(wt, 'channel', sym, 'int4')
+        got_w, got_e = og.block_loop(wt.clone(), torch.from_numpy(hinv), 'int4', [s.reshape(-1, 1)] * count,
+                                     None if z is None else [z.reshape(-1, 1)] * count)
+        w = w0.copy()
+        e = np.zeros_like(w)
+        sn = s.numpy().reshape(-1)
+        zn = None if z is None else z.numpy().reshape(-1).astype(np.float32)
+        for i in range(count):
+            for r in range(n):
+                t = np.float32(w[r, i] / sn[r])
+                if zn is not None:
+                    t = np.float32(t + zn[r])
+                q = np.float32(min(max(np.rint(t), -8), 7))
+                wq = np.float32(np.float32(q - (zn[r] if zn is not None else np.float32(0))) * sn[r])
+                err = np.float32(np.float32(w[r, i] - wq) / hinv[i, i])
+                e[r, i] = err
+                for j in range(i, count):
+                    w[r, j] = np.float32(w[r, j] - np.float32(err * hinv[i, j]))
+        assert np.array_equal(got_w.numpy().view(np.uint32), w.view(np.uint32))
+        assert np.array_equal(got_e.numpy().view(np.uint32), e.view(np.uint32))
