@@ -658,7 +658,9 @@ __global__ __launch_bounds__(WAVES * 64) void w4a16_decode(W4A16Args a) {
 // per-lane traffic left; a lane's loads come in pairs that cover both 64-byte halves of a 128-byte
 // line back to back (k-slots h = 0, 1 of a 256-wide iteration), two iterations are in flight.
 // ---------------------------------------------------------------------------
-template <int WAVES, bool SMOOTH, int XJ, int TN>
+// SMOOTH: 0 no smoothing; 1 every vector a thread stages has the same k position (the thread count is a multiple
+// of the vectors per row), so one smoothing vector serves them all; 2 one smoothing vector per staged vector
+template <int WAVES, int SMOOTH, int XJ, int TN>
 __global__ __launch_bounds__(WAVES * 64) void w4a16_decode_lds(W4A16Args a) {
     extern __shared__ __align__(16) uint8_t lds_raw[];
     constexpr int NT = WAVES * 64;
@@ -699,17 +701,17 @@ __global__ __launch_bounds__(WAVES * 64) void w4a16_decode_lds(W4A16Args a) {
         zv[j] = ldg16(a.zeros + (i < zv_total ? i : zv_total - 1) * 16);
     }
     const uint32_t KV = K / 8, n_xv = M * KV;
-    uint4 xv[XJ], cv[XJ];
+    uint4 xv[XJ], cv[SMOOTH == 2 ? XJ : 1];
     uint32_t xdst[XJ];
-    const bool cv_same = NT % KV == 0;                            // a thread's vectors then share their k position
 #pragma unroll
     for (int j = 0; j < XJ; ++j) {
         const uint32_t v = tid + NT * j;
         const uint32_t vc = v < n_xv ? v : n_xv - 1;
         const uint32_t row = vc / KV, kv = vc - row * KV;
         xv[j] = ldg16(a.x + (int64_t)row * K + kv * 8);
-        if constexpr (SMOOTH) {
-            if (j == 0 || !cv_same) cv[j] = ldg16(a.smooth + kv * 8);
+        if constexpr (SMOOTH == 2) cv[j] = ldg16(a.smooth + kv * 8);
+        if constexpr (SMOOTH == 1) {
+            if (j == 0) cv[0] = ldg16(a.smooth + kv * 8);
         }
         xdst[j] = row * xstride + kv * 16;
     }
@@ -747,7 +749,7 @@ __global__ __launch_bounds__(WAVES * 64) void w4a16_decode_lds(W4A16Args a) {
 #pragma unroll
     for (int j = 0; j < XJ; ++j) {
         const uint32_t v = tid + NT * j;
-        if constexpr (SMOOTH) xv[j] = smooth8(xv[j], cv_same ? cv[0] : cv[j]);
+        if constexpr (SMOOTH != 0) xv[j] = smooth8(xv[j], cv[SMOOTH == 2 ? j : 0]);
         if (v < n_xv) *reinterpret_cast<uint4*>(xs + xdst[j]) = xv[j];
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -843,7 +845,7 @@ static size_t decode_lds_bytes(int64_t M, int64_t K, int group, int waves, int t
     return total <= 150 * 1024 ? total : 0;
 }
 
-template <int WAVES, bool SMOOTH, int XJ, int TN>
+template <int WAVES, int SMOOTH, int XJ, int TN>
 static int launch_decode_lds(const W4A16Args& a, size_t lds, hipStream_t st) {
     // only launches above the default 64 KiB of dynamic LDS need the attribute; it is per device and cheap,
     // so it is simply set on every such launch and no state is kept in the library
@@ -858,13 +860,20 @@ static int launch_decode_lds(const W4A16Args& a, size_t lds, hipStream_t st) {
     return hip_status();
 }
 
-template <int WAVES, bool SMOOTH, int TN>
-static int launch_decode_lds_xj(const W4A16Args& a, size_t lds, hipStream_t st) {
+template <int WAVES, int SMOOTH, int TN>
+static int launch_decode_lds_sm(const W4A16Args& a, size_t lds, hipStream_t st) {
     const int64_t per_thread = (a.M * (a.K / 8) + WAVES * 64 - 1) / (WAVES * 64);
     if (per_thread <= 1) return launch_decode_lds<WAVES, SMOOTH, 1, TN>(a, lds, st);
     if (per_thread <= 4) return launch_decode_lds<WAVES, SMOOTH, 4, TN>(a, lds, st);
     if (per_thread <= 16) return launch_decode_lds<WAVES, SMOOTH, 16, TN>(a, lds, st);
     return AMCT_E_UNSUPPORTED;                                    // caller falls through to the register kernel
+}
+
+template <int WAVES, bool SMOOTH, int TN>
+static int launch_decode_lds_xj(const W4A16Args& a, size_t lds, hipStream_t st) {
+    if constexpr (!SMOOTH) return launch_decode_lds_sm<WAVES, 0, TN>(a, lds, st);
+    else if ((WAVES * 64) % (a.K / 8) == 0) return launch_decode_lds_sm<WAVES, 1, TN>(a, lds, st);
+    else return launch_decode_lds_sm<WAVES, 2, TN>(a, lds, st);
 }
 
 template <bool SMOOTH, int TN>
