@@ -3,14 +3,15 @@
 //   wdq = bf16((u[n,k] - zero[n,k/g]) * scale[n,k/g]) (the operator called at :116-117)
 // wq holds u = code + 8 as nibbles, even k in the low nibble.
 //
-//   tile kernel   : 128x128 block tile, BK = 64, bf16 MFMA 32x32x16.  The weight tile is
-//                   dequantised on its way from global memory to LDS: byte-wise nibble split,
-//                   v_cvt_f32_ubyteN, one fma per element ((u - z) * s == fma(u, s, -z*s) exactly),
-//                   v_cvt_pk_bf16_f32.  The smooth multiply is applied to the activation tile on the
-//                   same path.
-//   skinny kernel : M <= 64 (decode): weights streamed once from HBM, dequantised in registers,
-//                   bf16 MFMA 16x16x32, split-K over the 4 waves of a block.
+//   large-tile kernel (M >= 256): 256x256 block tile, 8 waves, activations direct-to-LDS, packed weights
+//                   fetched by asm loads four steps ahead, dequantised one step ahead into LDS.
+//   tile kernel   : 128x128 block tile, BK = 64, bf16 MFMA 32x32x16; the weight tile is dequantised on its
+//                   way from global memory to LDS (64 < M < 256 and shapes the large-tile kernel does not take).
+//   decode kernels (M <= 16 with the activations staged in LDS, M <= 64 straight from L2): the weight is
+//                   streamed once, dequantised in registers, bf16 MFMA 16x16x32, split-K over the waves.
 //   general kernel: any shape, one output per thread.
+// Dequantisation everywhere: byte-wise nibble split, v_cvt_f32_ubyteN, one fma per element
+// ((u - z) * s == fma(u, s, -z*s) exactly), one v_cvt_pk_bf16_f32 per pair.
 #include <type_traits>
 
 #include "amct_common.h"
@@ -409,94 +410,6 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
             const int64_t m = mbase + prow;
             const int64_t n = n0 + wn * 64 + chunk * 8;
             if (m < a.M && n < a.N) stg16_nt(reinterpret_cast<char*>(a.out) + (m * a.N + n) * 2, v);
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------
-// skinny kernel: M <= 16 * MT.  One block = 16 output columns, its 4 waves split K.
-// Per iteration a wave covers 128 k: lane (r = l%16, g = l/16) loads the 32 nibbles
-// k = kb + 32g .. +32 of weight row n0 + r; MFMA s (0..3) consumes nibbles 8s..8s+7 of every lane,
-// and the activation fragment of that MFMA is x[m][kb + 32g + 8s .. +8]: the k order inside an MFMA
-// is permuted identically for both operands, which leaves the dot product unchanged.
-// ---------------------------------------------------------------------------
-template <int MT>
-__global__ __launch_bounds__(kBlock) void w4a16_skinny(W4A16Args a) {
-    __shared__ float red[3][MT][64][4];
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int r16 = lane & 15, g = lane >> 4;
-    const int64_t n0 = (int64_t)blockIdx.x * 16;
-    const int64_t nrow = (n0 + r16 < a.N) ? n0 + r16 : a.N - 1;
-    const int64_t G = a.K / a.group;
-    const uint8_t* wrow = a.wq + nrow * (a.K / 2);
-    const int64_t iters_total = a.K / 128;
-    const int64_t per_wave = (iters_total + 3) / 4;
-    const int64_t it_begin = wave * per_wave;
-    const int64_t it_end = (it_begin + per_wave < iters_total) ? it_begin + per_wave : iters_total;
-
-    const uint16_t* xrow[MT];
-#pragma unroll
-    for (int t = 0; t < MT; ++t) {
-        const int64_t m = t * 16 + r16;
-        xrow[t] = a.x + (m < a.M ? m : a.M - 1) * a.K;
-    }
-    v4f acc[MT];
-#pragma unroll
-    for (int t = 0; t < MT; ++t) acc[t] = v4f{0.f, 0.f, 0.f, 0.f};
-
-    constexpr int UN = 2;
-    for (int64_t it = it_begin; it < it_end; it += UN) {
-        uint4 wv[UN];
-        float sc[UN], nzs[UN];
-#pragma unroll
-        for (int u = 0; u < UN; ++u) {
-            const bool ok = it + u < it_end;
-            const int64_t k = (it + u) * 128 + g * 32;
-            wv[u] = ok ? ldg16(wrow + k / 2) : make_uint4(0, 0, 0, 0);
-            const int64_t gi = nrow * G + (ok ? k / a.group : 0);
-            sc[u] = load_scale(a, gi);
-            nzs[u] = -((float)a.zeros[gi] * sc[u]);
-        }
-#pragma unroll
-        for (int u = 0; u < UN; ++u) {
-            const bool ok = it + u < it_end;
-            const int64_t k = (it + u) * 128 + g * 32;
-            const uint32_t ws[4] = {wv[u].x, wv[u].y, wv[u].z, wv[u].w};
-#pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const uint4 bq = ok ? dequant8(ws[s], sc[u], nzs[u]) : make_uint4(0, 0, 0, 0);
-                const v8bf fb = __builtin_bit_cast(v8bf, bq);
-                uint4 cs = make_uint4(0, 0, 0, 0);
-                if (a.smooth && ok) cs = ldg16(a.smooth + k + s * 8);
-#pragma unroll
-                for (int t = 0; t < MT; ++t) {
-                    uint4 xv = ok ? ldg16(xrow[t] + k + s * 8) : make_uint4(0, 0, 0, 0);
-                    if (a.smooth) xv = smooth8(xv, cs);
-                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, xv), fb, acc[t], 0, 0, 0);
-                }
-            }
-        }
-    }
-    if (wave > 0) {
-#pragma unroll
-        for (int t = 0; t < MT; ++t)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) red[wave - 1][t][lane][r] = acc[t][r];
-    }
-    __syncthreads();
-    if (wave == 0) {
-        const int64_t n = n0 + r16;
-        const float b = (a.bias && n < a.N) ? a.bias[n] : 0.f;
-#pragma unroll
-        for (int t = 0; t < MT; ++t) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                float v = ((acc[t][r] + red[0][t][lane][r]) + red[1][t][lane][r]) + red[2][t][lane][r];
-                if (a.bias) v = v + b;
-                const int64_t m = t * 16 + 4 * g + r;
-                if (n < a.N && m < a.M) a.out[m * a.N + n] = (uint16_t)f32_to_bf16_bits(v);
-            }
         }
     }
 }
@@ -959,14 +872,6 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
         else AMCT_DEC(4)
 #undef AMCT_DEC2
 #undef AMCT_DEC
-        return hip_status();
-    }
-    if (vec_ok && M <= 64 && K % 128 == 0) {
-        const dim3 grid((unsigned)((N + 15) / 16));
-        if (M <= 16) hipLaunchKernelGGL((w4a16_skinny<1>), grid, dim3(kBlock), 0, st, a);
-        else if (M <= 32) hipLaunchKernelGGL((w4a16_skinny<2>), grid, dim3(kBlock), 0, st, a);
-        else if (M <= 48) hipLaunchKernelGGL((w4a16_skinny<3>), grid, dim3(kBlock), 0, st, a);
-        else hipLaunchKernelGGL((w4a16_skinny<4>), grid, dim3(kBlock), 0, st, a);
         return hip_status();
     }
     if (vec_ok && M >= 256 && K % 128 == 0 && N % 8 == 0 && group % 16 == 0 && aligned16(out)) {

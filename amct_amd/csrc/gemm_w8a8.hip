@@ -7,8 +7,10 @@
 //                   direct global->LDS loads, fragment reads software-pipelined against the MFMAs.
 //   tile kernel   : 128x128 block tile, 4 waves of 64x64, BK = 128 bytes, two register stages of
 //                   prefetch (shapes the large-tile kernel does not take).
-//   skinny kernel : M <= 64 (decode): the weight is streamed once straight from HBM into MFMA
-//                   operands (v_mfma_i32_16x16x64_i8), split-K across the 4 waves of a block.
+//   decode kernel : M <= 16: activations staged once per block in LDS, the weight streamed once straight
+//                   from HBM into MFMA operands (v_mfma_i32_16x16x64_i8), split-K across the waves.
+//   skinny kernel : 16 < M <= 64 (and M <= 16 shapes the decode kernel does not take): as above with the
+//                   activations read from L2 per MFMA.
 //   general kernel: any shape, one output per thread.
 #include "amct_common.h"
 
