@@ -9,7 +9,7 @@
 //                   prefetch (shapes the large-tile kernel does not take).
 //   decode kernel : M <= 16: activations staged once per block in LDS, the weight streamed once straight
 //                   from HBM into MFMA operands (v_mfma_i32_16x16x64_i8), split-K across the waves.
-//   skinny kernel : 16 < M <= 64 (and M <= 16 shapes the decode kernel does not take): as above with the
+//   skinny kernel : 16 < M <= 32 (and M <= 16 shapes the decode kernel does not take): as above with the
 //                   activations read from L2 per MFMA.
 //   general kernel: any shape, one output per thread.
 #include "amct_common.h"
@@ -636,12 +636,12 @@ extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s
         if (lds) rc = tn == 1 ? launch_w8a8_decode_w<1>(a, waves, lds, st) : launch_w8a8_decode_w<2>(a, waves, lds, st);
         if (rc != AMCT_E_UNSUPPORTED) return rc;
     }
-    if (vec_ok && M <= 64) {
+    // measured on W[14336,4096]: the skinny kernel re-reads the activations once per 16 output columns and
+    // loses to the 128x128 tile kernel from M = 48 on (33.9 us against 30.5 us; M = 64: 41.7 against 32.9)
+    if (vec_ok && M <= 32) {
         const dim3 grid((unsigned)((N + 15) / 16));
         if (M <= 16) hipLaunchKernelGGL((w8a8_skinny<1>), grid, dim3(kBlock), 0, st, a);
-        else if (M <= 32) hipLaunchKernelGGL((w8a8_skinny<2>), grid, dim3(kBlock), 0, st, a);
-        else if (M <= 48) hipLaunchKernelGGL((w8a8_skinny<3>), grid, dim3(kBlock), 0, st, a);
-        else hipLaunchKernelGGL((w8a8_skinny<4>), grid, dim3(kBlock), 0, st, a);
+        else hipLaunchKernelGGL((w8a8_skinny<2>), grid, dim3(kBlock), 0, st, a);
         return hip_status();
     }
     if (vec_ok && M >= 256 && K % kLK == 0 && K >= kLK && N % 8 == 0 && aligned16(out)) {
