@@ -235,6 +235,7 @@ constexpr float kEps = 1.1920928955078125e-7f;   // fp32(1.192092896e-7), utils.
 struct Factors {
     float s;
     float z;
+    float y;      // RN(1 / s) of the final scale: computed once here, reused for the element divisions
     bool bad;     // scale, 1/scale or offset not finite (utils.py:54-72)
 };
 
@@ -251,13 +252,16 @@ AMCT_DEV Factors make_factors(float vmax, float vmin, int bits, bool symmetric, 
             // quotient of a tensor by a Python number keeps the tensor's dtype
             r.s = round_to<DT>(fmax_nan(amax, amin) / qpos);
             r.z = 0.f;
-            r.bad = !finite_f(r.s) || !finite_f(1.0f / r.s);
+            r.y = 1.0f / r.s;
+            r.bad = !finite_f(r.s) || !finite_f(r.y);
             return r;
         }
         const float scope = (amax < amin) ? qpos + 1.0f : qpos;
         const float bound = (amax > amin) ? amax : amin;
-        r.s = bound / scope;
+        const float s_raw = bound / scope;
+        r.s = (s_raw < kEps) ? 1.0f : s_raw;
         r.z = 0.f;
+        r.y = 1.0f / r.s;
     } else {
         // torch.clamp propagates NaN; (x < 0 ? 0 : x) keeps NaN as well
         vmax = (vmax < 0.f) ? 0.f : vmax;
@@ -266,23 +270,39 @@ AMCT_DEV Factors make_factors(float vmax, float vmin, int bits, bool symmetric, 
         const float half = (float)(1 << (bits - 1));        // ceil(scope / 2)
         const float diff = vmax - vmin;
         const uint32_t ed = (__float_as_uint(diff) >> 23) & 0xFFu;
-        if (ed >= 67u && ed <= 187u) {
-            // diff in [2^-60, 2^61): both quotients by the exact fma sequence (same results as '/')
-            r.s = div_const(diff, scope, bits == 8 ? (1.0f / 255.0f) : (1.0f / 15.0f));
-            const Divisor ds = make_divisor(r.s);
-            r.z = (vmax != vmin) ? (-half - div_fast<true>(vmin, ds)) : -half;
+        const bool exact_fma = ed >= 67u && ed <= 187u;     // diff in [2^-60, 2^61)
+        // both quotients by the exact fma sequence where it is valid (same results as '/')
+        const float s_raw = exact_fma ? div_const(diff, scope, bits == 8 ? (1.0f / 255.0f) : (1.0f / 15.0f)) : diff / scope;
+        const bool tiny = s_raw < kEps;
+        r.s = tiny ? 1.0f : s_raw;
+        r.y = 1.0f / r.s;                                   // the one reciprocal per segment
+        float q;
+        if (exact_fma) {
+            Divisor ds;
+            ds.s = r.s;
+            ds.y = r.y;
+            ds.fast = true;
+            q = div_fast<true>(vmin, ds);                   // a tiny scale overrides the offset below
         } else {
-            r.s = diff / scope;
-            r.z = (vmax != vmin) ? (-half - vmin / r.s) : -half;
+            q = vmin / r.s;
         }
+        r.z = (vmax != vmin) ? (-half - q) : -half;
+        r.z = tiny ? -half : r.z;
     }
-    const bool tiny = r.s < kEps;
-    if (!symmetric) r.z = tiny ? -(float)(1 << (bits - 1)) : r.z;
-    r.s = tiny ? 1.0f : r.s;
-    r.bad = !finite_f(r.s) || !finite_f(1.0f / r.s) || !finite_f(r.z);
+    r.bad = !finite_f(r.s) || !finite_f(r.y) || !finite_f(r.z);
     // round-half-even, then through int32 as the reference does: a rounded -0.0 becomes +0.0
     r.z = (float)(int)__builtin_rintf(r.z);
     return r;
+}
+
+// the element divisor of a segment from its factors (no second reciprocal)
+AMCT_DEV Divisor divisor_of(const Factors& f) {
+    Divisor d;
+    d.s = f.s;
+    d.y = f.y;
+    const uint32_t e = (__float_as_uint(f.s) >> 23) & 0xFFu;
+    d.fast = (e >= 67u) && (e <= 187u) && f.s > 0.f;
+    return d;
 }
 
 // One element of the integer (fake-)quantiser.

@@ -189,7 +189,7 @@ __global__ __launch_bounds__(kBlock) void fq_fused(FqArgs a) {
         float mx_my, mn_my;
         team_minmax_scatter4<T>(mn, mx, lt, mn_my, mx_my);
         const Factors f = make_factors<DT>(mx_my, mn_my, a.bits, a.symmetric != 0, a.scope_rule);
-        const Divisor dmy = make_divisor(f.s);
+        const Divisor dmy = divisor_of(f);
         const uint32_t big = max(__float_as_uint(mx_my) & 0x7FFFFFFFu, __float_as_uint(mn_my) & 0x7FFFFFFFu);
         fast = wave_all(dmy.fast && big < 0x5D800000u);
         if (lt < 4 && seg0 + my < a.nseg) {
@@ -206,7 +206,7 @@ __global__ __launch_bounds__(kBlock) void fq_fused(FqArgs a) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const Factors f = make_factors<DT>(mx[u], mn[u], a.bits, a.symmetric != 0, a.scope_rule);
-            dv[u] = make_divisor(f.s);
+            dv[u] = divisor_of(f);
             z[u] = f.z;
             const uint32_t big = max(__float_as_uint(mx[u]) & 0x7FFFFFFFu, __float_as_uint(mn[u]) & 0x7FFFFFFFu);
             ok = ok && dv[u].fast && big < 0x5D800000u;

@@ -143,14 +143,21 @@ __global__ __launch_bounds__(kBlock) void int4_group_pack4(PackArgs a) {
 #pragma unroll
     for (int v = 0; v < NV; ++v) vl[v] = (lt + T * v < S) ? lt + T * v : S - 1;
 
+    // one 64-bit base per lane (first group of the team, clamped into the tensor), then 32-bit offsets per group:
+    // group u of the team is u groups further, or the last group of the tensor if the team hangs over its end
     uint4 raw[U][NV];
     int64_t segc[U];
+    const int64_t seg_first = seg0 < a.nseg ? seg0 : a.nseg - 1;
+    const int64_t left = a.nseg - 1 - seg_first;                    // groups after the first one
+    const int left32 = left < U ? (int)left : U - 1;
+    const char* base = reinterpret_cast<const char*>(a.w) + seg_first * a.seg_len * BYTES;
+    const uint32_t seg_bytes = (uint32_t)a.seg_len * BYTES;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-        segc[u] = (seg0 + u < a.nseg) ? seg0 + u : a.nseg - 1;
+        const int uc = u < left32 ? u : left32;
+        segc[u] = seg_first + uc;
 #pragma unroll
-        for (int v = 0; v < NV; ++v)
-            raw[u][v] = ldg16_nt(reinterpret_cast<const char*>(a.w) + (segc[u] * a.seg_len + (int64_t)vl[v] * VEC) * BYTES);
+        for (int v = 0; v < NV; ++v) raw[u][v] = ldg16_nt(base + (uint32_t)uc * seg_bytes + (uint32_t)vl[v] * 16u);
     }
     float x[U][NV][VEC];
 #pragma unroll
@@ -189,7 +196,7 @@ __global__ __launch_bounds__(kBlock) void int4_group_pack4(PackArgs a) {
     float mx_my, mn_my;
     team_minmax_scatter4<T>(mn, mx, lt, mn_my, mx_my);
     const Factors f = make_factors<AMCT_F32>(mx_my, mn_my, 4, a.symmetric != 0, AMCT_SCOPE_AMCT);
-    const Divisor dmy = make_divisor(f.s);
+    const Divisor dmy = divisor_of(f);
     const uint32_t big = max(__float_as_uint(mx_my) & 0x7FFFFFFFu, __float_as_uint(mn_my) & 0x7FFFFFFFu);
     const bool fast = wave_all(dmy.fast && big < 0x5D800000u);       // |x| < 2^60, finite
     if (lt < 4 && seg0 + my < a.nseg) {
