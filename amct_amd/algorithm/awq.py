@@ -70,6 +70,18 @@ def awq_scale_for_ratio(inputs_mean, ratio, dtype):
     return torch.clamp(scale_awq.to(dtype), 1e-4, torch.finfo(dtype).max)
 
 
+def _first_output(block, inputs, kwargs):
+    out = block(inputs, **kwargs)
+    return out[0] if isinstance(out, tuple) else out
+
+
+def _require_finite(inputs, layers):
+    if not bool(torch.isfinite(inputs).all()):
+        raise RuntimeError("Run AWQ error! Invalid value(nan or inf) in activation!")
+    if not all(bool(torch.isfinite(layer.weight.data).all()) for layer in layers):
+        raise RuntimeError("Run AWQ error! Invalid value(nan or inf) in weight!")
+
+
 @torch.no_grad()
 def search_scale(inputs, layers, block, quant_config, kwargs=None):
     """AWQ scale search (awq.py:52-105) with everything resident on the device.  Same arguments, return
@@ -78,37 +90,28 @@ def search_scale(inputs, layers, block, quant_config, kwargs=None):
     (process_weights_for_layers, which replaces layer.weight.data by a new tensor and never writes into the
     old one), so here the original weight tensors are simply kept and put back: no copy at all, and the
     fake-quant of a grid point is one fused kernel per layer."""
-    algo_params = quant_config.get("algorithm")
-    if not torch.isfinite(inputs).all():
-        raise RuntimeError("Run AWQ error! Invalid value(nan or inf) in activation!")
-    for layer in layers:
-        if not torch.isfinite(layer.weight.data).all():
-            raise RuntimeError("Run AWQ error! Invalid value(nan or inf) in weight!")
-    kwargs = dict() if kwargs is None else kwargs
-    ori_out = block(inputs, **kwargs)
-    if isinstance(ori_out, tuple):
-        ori_out = ori_out[0]
-
-    min_loss = torch.tensor(float('inf'), device=inputs.device)
-    best_scale = None
-    inputs_mean = inputs.abs().contiguous().view(-1, inputs.shape[-1]).mean(0)  # (cin)
-    grids_num = algo_params.get('awq').get('grids_num')
-    saved = [layer.weight.data for layer in layers]
-    for grid in range(grids_num):
-        scale_awq = awq_scale_for_ratio(inputs_mean, grid / grids_num, inputs.dtype)
-        process_weights_for_layers(layers, scale_awq, quant_config)
-        quant_out = block(inputs, **kwargs)
-        if isinstance(quant_out, tuple):
-            quant_out = quant_out[0]
-        loss = (ori_out - quant_out).float().pow(4).mean()
-        if not torch.isnan(loss) and loss < min_loss:
-            min_loss = loss
-            best_scale = scale_awq
-        for layer, w in zip(layers, saved):
+    _require_finite(inputs, layers)
+    kwargs = kwargs or {}
+    grids_num = quant_config.get("algorithm").get('awq').get('grids_num')
+    target = _first_output(block, inputs, kwargs)
+    channel_mean = inputs.abs().contiguous().view(-1, inputs.shape[-1]).mean(0)     # one value per input channel
+    originals = [layer.weight.data for layer in layers]
+    winner, winner_loss = None, torch.tensor(float('inf'), device=inputs.device)
+    try:
+        for grid in range(grids_num):
+            candidate = awq_scale_for_ratio(channel_mean, grid / grids_num, inputs.dtype)
+            process_weights_for_layers(layers, candidate, quant_config)
+            loss = (target - _first_output(block, inputs, kwargs)).float().pow(4).mean()
+            if not torch.isnan(loss) and loss < winner_loss:
+                winner, winner_loss = candidate, loss
+            for layer, w in zip(layers, originals):
+                layer.weight.data = w
+    finally:
+        for layer, w in zip(layers, originals):                                     # also after an exception
             layer.weight.data = w
-    if best_scale is None or torch.isinf(min_loss):
+    if winner is None or torch.isinf(winner_loss):
         raise RuntimeError("Run AWQ error! Got invalid loss.")
-    return best_scale
+    return winner
 
 
 @torch.no_grad()
