@@ -4,7 +4,8 @@
 // Both operands are K-contiguous, which is the natural operand order of the gfx950 int8 MFMA
 // (v_mfma_i32_32x32x32_i8: lane l supplies 16 consecutive k-bytes of row l%32, k-half l/32).
 //   large tiles   : 256x256 block tile, 8 waves of 128x64, BK = 64 bytes, 4 LDS stages filled by
-//                   direct global->LDS loads, fragment reads software-pipelined against the MFMAs.
+//                   direct global->LDS loads, fragment reads software-pipelined against the MFMAs;
+//                   when the tile count does not fill the CUs evenly, one launch mixes in 256x192 tiles.
 //   tile kernel   : 128x128 block tile, 4 waves of 64x64, BK = 128 bytes, two register stages of
 //                   prefetch (shapes the large-tile kernel does not take).
 //   decode kernel : M <= 16: activations staged once per block in LDS, the weight streamed once straight
@@ -12,6 +13,8 @@
 //   skinny kernel : 16 < M <= 32 (and M <= 16 shapes the decode kernel does not take): as above with the
 //                   activations read from L2 per MFMA.
 //   general kernel: any shape, one output per thread.
+#include <queue>
+#include <vector>
 #include "amct_common.h"
 
 namespace amct {
@@ -192,21 +195,26 @@ AMCT_DEV void dma16(uint32_t lds_addr, const void* gptr) {
 }
 template <int N> AMCT_DEV void wait_dma_lds() { asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"(N) : "memory"); }
 
-// WM x WN waves of 128x64 each: block tile (128*WM) x (64*WN); STAGES LDS stages of BK = 64 bytes
-template <int ODT, int WM, int WN, int STAGES>
-__global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void w8a8_tile_dma(W8A8Args a) {
-    constexpr int kLM = 128 * WM, kLN = 64 * WN, kWaves = WM * WN;
-    constexpr int kLStageBytes = (kLM + kLN) * kLK;
-    constexpr int kPieces = (kLM + kLN) / 16;                      // 1 KiB pieces per stage
-    constexpr int kPPW = kPieces / kWaves;                         // pieces per wave
-    static_assert(kPieces % kWaves == 0, "pieces must divide evenly among the waves");
-    constexpr int kEpiBytes = kWaves * 16384;
-    constexpr int kSmem = STAGES * kLStageBytes > kEpiBytes ? STAGES * kLStageBytes : kEpiBytes;
-    __shared__ __attribute__((aligned(1024))) int8_t smem[kSmem];
+// WM x WN waves of (32*TI) x (32*TJ) each: block tile (32*TI*WM) x (32*TJ*WN); STAGES LDS stages of BK = 64 bytes.
+// The body is a device function so that one launch can mix block shapes (see w8a8_tile_mix).
+template <int WM, int WN, int TI, int TJ, int STAGES>
+struct DmaTile {
+    static constexpr int kLM = 32 * TI * WM, kLN = 32 * TJ * WN, kWaves = WM * WN;
+    static constexpr int kLStageBytes = (kLM + kLN) * kLK;
+    static constexpr int kPieces = (kLM + kLN) / 16;               // 1 KiB pieces per stage
+    static constexpr int kPPW = (kPieces + kWaves - 1) / kWaves;   // pieces per wave (the last wave may repeat one)
+    static constexpr int kEpiBytes = kWaves * 16384;
+    static constexpr int kSmem = STAGES * kLStageBytes > kEpiBytes ? STAGES * kLStageBytes : kEpiBytes;
+};
+
+template <int ODT, int WM, int WN, int TI, int TJ, int STAGES>
+AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, const int64_t n0) {
+    using Sh = DmaTile<WM, WN, TI, TJ, STAGES>;
+    constexpr int kLM = Sh::kLM, kLN = Sh::kLN, kWaves = Sh::kWaves;
+    constexpr int kLStageBytes = Sh::kLStageBytes, kPieces = Sh::kPieces, kPPW = Sh::kPPW;
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
-    const int64_t m0 = (int64_t)blockIdx.y * kLM, n0 = (int64_t)blockIdx.x * kLN;
     const int nsteps = (int)(a.K / kLK);
     const int last = nsteps - 1;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t*)smem;
@@ -218,7 +226,8 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2,
         const int lc = (lane & 3) ^ ((rin >> 2) & 3);               // logical chunk this lane fetches
 #pragma unroll
         for (int j = 0; j < kPPW; ++j) {
-            const int piece = wave * kPPW + j;
+            // a wave beyond the last piece fetches the last piece again: same bytes to the same place
+            const int piece = (kPieces % kWaves == 0 || wave * kPPW + j < kPieces) ? wave * kPPW + j : kPieces - 1;
             if (piece < kLM / 16) {
                 const int64_t r = m0 + piece * 16 + rin;
                 gp[j] = a.xq + (r < a.M ? r : a.M - 1) * a.K + lc * 16;
@@ -229,9 +238,11 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2,
         }
     }
     auto dma_stage = [&](int stage, int step) {
-        const uint32_t base = __builtin_amdgcn_readfirstlane(lds0 + stage * kLStageBytes + wave * kPPW * 1024);
 #pragma unroll
-        for (int j = 0; j < kPPW; ++j) dma16(base + j * 1024, gp[j] + (int64_t)step * kLK);
+        for (int j = 0; j < kPPW; ++j) {
+            const int piece = (kPieces % kWaves == 0 || wave * kPPW + j < kPieces) ? wave * kPPW + j : kPieces - 1;
+            dma16(__builtin_amdgcn_readfirstlane(lds0 + stage * kLStageBytes + piece * 1024), gp[j] + (int64_t)step * kLK);
+        }
     };
 
     // fragment offsets: lane reads row (tile base + lane%32), logical chunk 2*ks + lane/32
@@ -240,40 +251,40 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2,
     for (int ks = 0; ks < 2; ++ks) {
         const int r = lane & 31;
         const int phys = (ks * 2 + (lane >> 5)) ^ ((r >> 2) & 3);
-        offA[ks] = (wm * 128 + r) * kLK + phys * 16;
-        offB[ks] = kLM * kLK + (wn * 64 + r) * kLK + phys * 16;
+        offA[ks] = (wm * 32 * TI + r) * kLK + phys * 16;
+        offB[ks] = kLM * kLK + (wn * 32 * TJ + r) * kLK + phys * 16;
     }
 
-    v16i acc[4][2];
+    v16i acc[TI][TJ];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TI; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TJ; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s) dma_stage(s, s < last ? s : last);
 
-    auto read_frags = [&](int stage, int ks, v4i (&fa)[4], v4i (&fb)[2]) {
+    auto read_frags = [&](int stage, int ks, v4i (&fa)[TI], v4i (&fb)[TJ]) {
         const int8_t* st = smem + stage * kLStageBytes;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) fa[i] = *reinterpret_cast<const v4i*>(st + offA[ks] + i * 32 * kLK);
+        for (int i = 0; i < TI; ++i) fa[i] = *reinterpret_cast<const v4i*>(st + offA[ks] + i * 32 * kLK);
 #pragma unroll
-        for (int j = 0; j < 2; ++j) fb[j] = *reinterpret_cast<const v4i*>(st + offB[ks] + j * 32 * kLK);
+        for (int j = 0; j < TJ; ++j) fb[j] = *reinterpret_cast<const v4i*>(st + offB[ks] + j * 32 * kLK);
     };
-    auto mfma_half = [&](const v4i (&fa)[4], const v4i (&fb)[2]) {
+    auto mfma_half = [&](const v4i (&fa)[TI], const v4i (&fb)[TJ]) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < TI; ++i)
 #pragma unroll
-            for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+            for (int j = 0; j < TJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
     };
 
     // software pipeline over half K-steps: while the 8 MFMAs of one half run, the fragments of the
     // next half are read from LDS.  At the barrier of iteration s every wave holds the last fragments
     // of stage s % STAGES in registers (lgkmcnt(0)), so that stage is free for the loads of step
     // s + STAGES; the loads of the STAGES-2 steps after s+1 stay in flight.
-    v4i fa0[4], fb0[2], fa1[4], fb1[2];
+    v4i fa0[TI], fb0[TJ], fa1[TI], fb1[TJ];
     wait_dma_lds<(STAGES - 2) * kPPW>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
@@ -298,25 +309,26 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2,
     asm volatile("" ::: "memory");
 
     // epilogue: fp32(acc + ibias) * s_ch * s_tok + fbias, narrowed, transposed through a per-wave LDS
-    // patch of 32 rows x 64 columns, stored as 16-byte pieces of full rows
+    // patch of 32 rows x 32*TJ columns, stored as 16-byte pieces of full rows
     constexpr int ES = (ODT == AMCT_F32) ? 4 : 2;                   // bytes per output element
-    constexpr int kPatchRow = 64 * ES + 16;                        // padded patch row
-    constexpr int CPR = 64 * ES / 16;                              // 16-byte chunks per patch row
-    constexpr int RPI = 64 / CPR;                                  // patch rows covered by one wave-wide read
+    constexpr int kPW = 32 * TJ;                                   // patch width in columns
+    constexpr int kPatchRow = kPW * ES + 16;                       // padded patch row
+    constexpr int CPR = kPW * ES / 16;                             // 16-byte chunks per patch row
+    static_assert(32 * kPatchRow <= 16384 && (32 * CPR) % 64 == 0, "patch must fit its 16 KiB and split into wave-wide reads");
     int8_t* patch = smem + wave * 16384;
-    float sc[2], fb2[2];
-    int32_t ib[2];
+    float sc[TJ], fb2[TJ];
+    int32_t ib[TJ];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int64_t n = n0 + wn * 64 + j * 32 + (lane & 31);
+    for (int j = 0; j < TJ; ++j) {
+        const int64_t n = n0 + wn * kPW + j * 32 + (lane & 31);
         const int64_t nc = n < a.N ? n : a.N - 1;
         sc[j] = a.s_ch[nc];
         ib[j] = a.bias_kind == 1 ? reinterpret_cast<const int32_t*>(a.bias)[nc] : 0;
         fb2[j] = a.bias_kind == 2 ? reinterpret_cast<const float*>(a.bias)[nc] : 0.f;
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int64_t mbase = m0 + wm * 128 + i * 32;
+    for (int i = 0; i < TI; ++i) {
+        const int64_t mbase = m0 + wm * 32 * TI + i * 32;
         float tks[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {                              // all 16 row factors in flight together
@@ -329,10 +341,10 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2,
             const int64_t m = mbase + prow;
             const float tk = tks[r];
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
+            for (int j = 0; j < TJ; ++j) {
                 const int32_t v = acc[i][j][r] + ib[j];
                 if (a.acc_out) {
-                    const int64_t n = n0 + wn * 64 + j * 32 + (lane & 31);
+                    const int64_t n = n0 + wn * kPW + j * 32 + (lane & 31);
                     if (m < a.M && n < a.N) a.acc_out[m * a.N + n] = v;
                 }
                 float f = (float)v * sc[j];
@@ -346,14 +358,48 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2,
         }
         // LDS operations of one wave complete in order: the reads below see the writes above
 #pragma unroll
-        for (int it = 0; it < 32 / RPI; ++it) {
-            const int prow = it * RPI + lane / CPR;
-            const int chunk = lane % CPR;
+        for (int it = 0; it < 32 * CPR / 64; ++it) {
+            const int idx = it * 64 + lane;                        // 16-byte chunk of the patch, row-major
+            const int prow = idx / CPR;
+            const int chunk = idx % CPR;
             const uint4 v = *reinterpret_cast<const uint4*>(patch + prow * kPatchRow + chunk * 16);
             const int64_t m = mbase + prow;
-            const int64_t n = n0 + wn * 64 + chunk * (16 / ES);
+            const int64_t n = n0 + wn * kPW + chunk * (16 / ES);
             if (m < a.M && n < a.N) stg16_nt(reinterpret_cast<char*>(a.out) + (m * a.N + n) * ES, v);
         }
+    }
+}
+
+template <int ODT, int WM, int WN, int STAGES>
+__global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void w8a8_tile_dma(W8A8Args a) {
+    using Sh = DmaTile<WM, WN, 4, 2, STAGES>;
+    __shared__ __attribute__((aligned(1024))) int8_t smem[Sh::kSmem];
+    w8a8_dma_body<ODT, WM, WN, 4, 2, STAGES>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
+}
+
+// One launch, two block shapes: the first `big` blocks compute 256x256 tiles of the first `nbig` column tiles,
+// the rest 256x192 tiles of the columns after them.  The host picks the split so that the blocks fill the
+// CUs evenly (a 256x192 tile costs 3/4 of a 256x256 one): with uniform tiles the last round of a launch
+// leaves CUs idle, e.g. 448 tiles on 256 CUs take two rounds for 1.75 rounds of work.
+struct MixPlan {
+    int mtiles;                                                     // row tiles (256 rows each)
+    int nbig;                                                       // 256-column tiles, columns [0, 256*nbig)
+    int big;                                                        // mtiles * nbig
+    int nsmall;                                                     // 192-column tiles after them
+};
+
+template <int ODT>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void w8a8_tile_mix(W8A8Args a, MixPlan p) {
+    using Big = DmaTile<2, 4, 4, 2, 4>;
+    using Small = DmaTile<4, 2, 2, 3, 4>;
+    __shared__ __attribute__((aligned(1024))) int8_t smem[Big::kSmem > Small::kSmem ? Big::kSmem : Small::kSmem];
+    const int b = blockIdx.x;
+    if (b < p.big) {
+        w8a8_dma_body<ODT, 2, 4, 4, 2, 4>(a, smem, (int64_t)(b / p.nbig) * 256, (int64_t)(b % p.nbig) * 256);
+    } else {
+        const int s = b - p.big;
+        w8a8_dma_body<ODT, 4, 2, 2, 3, 4>(a, smem, (int64_t)(s / p.nsmall) * 256,
+                                          (int64_t)p.nbig * 256 + (int64_t)(s % p.nsmall) * 192);
     }
 }
 
@@ -609,6 +655,46 @@ __global__ __launch_bounds__(kBlock) void w8a8_general(W8A8Args a) {
     w8a8_epilogue(a, m, n, acc);
 }
 
+// Finish time, in quarters of a 256x256 tile, of `big` blocks of cost 4 followed by `small` blocks of cost 3
+// handed in that order to `cus` CUs holding one block each (the hardware gives the next block to the first
+// CU that becomes free).
+static int64_t mix_makespan(int64_t big, int64_t small, int cus) {
+    std::priority_queue<int64_t, std::vector<int64_t>, std::greater<int64_t>> busy;
+    int64_t end = 0;
+    for (int64_t t = 0; t < big + small; ++t) {
+        int64_t start = 0;
+        if ((int64_t)busy.size() >= cus) {
+            start = busy.top();
+            busy.pop();
+        }
+        const int64_t done = start + (t < big ? 4 : 3);
+        busy.push(done);
+        if (done > end) end = done;
+    }
+    return end;
+}
+
+// Split of the N columns into 256-wide and 192-wide column tiles that finishes first; nbig = -1 when plain
+// 256x256 tiles are as good (or the launch is so large that its last round does not matter).
+static MixPlan plan_mix(int64_t M, int64_t N, int cus) {
+    MixPlan best{(int)((M + 255) / 256), -1, 0, 0};
+    const int64_t mt = best.mtiles;
+    const int64_t uniform_tiles = mt * ((N + 255) / 256);
+    if (cus <= 0 || uniform_tiles > 16 * (int64_t)cus) return best;
+    int64_t best_t = mix_makespan(uniform_tiles, 0, cus);
+    for (int64_t nb = (N + 255) / 256 - 1; nb >= 0; --nb) {         // nb big column tiles, the rest 192 wide
+        const int64_t ns = (N - 256 * nb + 191) / 192;
+        const int64_t t = mix_makespan(mt * nb, mt * ns, cus);
+        if (t < best_t) {
+            best_t = t;
+            best.nbig = (int)nb;
+            best.big = (int)(mt * nb);
+            best.nsmall = (int)ns;
+        }
+    }
+    return best;
+}
+
 }  // namespace amct
 
 using namespace amct;
@@ -649,6 +735,20 @@ extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s
         // the traffic from L2 into LDS matters more than decoupling the barriers)
         const dim3 grid((unsigned)((N + 255) / 256), (unsigned)((M + 255) / 256));
         if (grid.y > 65535) return AMCT_E_UNSUPPORTED;
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+            (void)hipGetLastError();
+            cus = 0;
+        }
+        const MixPlan plan = plan_mix(M, N, cus);
+        if (plan.nbig >= 0) {
+            const dim3 g1((unsigned)(plan.big + plan.mtiles * plan.nsmall));
+            if (out_dtype == AMCT_BF16) hipLaunchKernelGGL((w8a8_tile_mix<AMCT_BF16>), g1, dim3(512), 0, st, a, plan);
+            else if (out_dtype == AMCT_F16) hipLaunchKernelGGL((w8a8_tile_mix<AMCT_F16>), g1, dim3(512), 0, st, a, plan);
+            else hipLaunchKernelGGL((w8a8_tile_mix<AMCT_F32>), g1, dim3(512), 0, st, a, plan);
+            return hip_status();
+        }
         if (out_dtype == AMCT_BF16) hipLaunchKernelGGL((w8a8_tile_dma<AMCT_BF16, 2, 4, 4>), grid, dim3(512), 0, st, a);
         else if (out_dtype == AMCT_F16) hipLaunchKernelGGL((w8a8_tile_dma<AMCT_F16, 2, 4, 4>), grid, dim3(512), 0, st, a);
         else hipLaunchKernelGGL((w8a8_tile_dma<AMCT_F32, 2, 4, 4>), grid, dim3(512), 0, st, a);

@@ -67,6 +67,19 @@ def test_w8a8_vs_oracle(dev, M, N, K, per_token, bias):
         assert ((out.cpu().double() - f64).abs() <= tol * f64.abs().clamp_min(f64.abs().max() * 1e-3)).all()
 
 
+@pytest.mark.parametrize("M,N,K", [(300, 1000, 320), (256, 448, 128), (512, 832, 256), (2048, 14336, 192), (1100, 9000, 64),
+                                   (2000, 14328, 128)])
+def test_w8a8_large_shapes_mixed_blocks(dev, M, N, K):
+    """Launches with M >= 256 may mix two block shapes (256x256 and 256x192 tiles) so that the blocks fill the
+    CUs evenly; ragged edges in M and N, every output dtype, accumulators bit for bit."""
+    xq, wq, s_ch, s_tok, b = w8a8_case(M, N, K, 131, True, 'float')
+    want_acc = od.int8_matmul_exact(xq, wq.t())
+    for odt in (torch.bfloat16, torch.float32):
+        out, acc = ops.gemm_w8a8(xq.to(dev), wq.to(dev), s_ch.to(dev), s_tok.to(dev), b.to(dev), out_dtype=odt, want_acc=True)
+        assert torch.equal(acc.cpu().to(torch.int64), want_acc), "accumulators"
+        assert_bits_equal(out, od.quant_matmul(xq, wq.t(), s_ch, s_tok, b, odt), "out %s" % odt)
+
+
 def w4a16_case(M, N, K, group, seed, sdt=torch.float16):
     g = torch.Generator().manual_seed(seed)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)
