@@ -193,6 +193,10 @@ constexpr int kLK = 64;
 AMCT_DEV void dma16(uint32_t lds_addr, const void* gptr) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(gptr) : "memory");
 }
+// the same with a wave-uniform 64-bit base in SGPRs and a 32-bit byte offset per lane: no vector ALU work per load
+AMCT_DEV void dma16s(uint32_t lds_addr, const void* sbase, uint32_t voff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
 template <int N> AMCT_DEV void wait_dma_lds() { asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"(N) : "memory"); }
 
 // WM x WN waves of (32*TI) x (32*TJ) each: block tile (32*TI*WM) x (32*TJ*WN); STAGES LDS stages of BK = 64 bytes.
@@ -212,15 +216,20 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
     using Sh = DmaTile<WM, WN, TI, TJ, STAGES>;
     constexpr int kLM = Sh::kLM, kLN = Sh::kLN, kWaves = Sh::kWaves;
     constexpr int kLStageBytes = Sh::kLStageBytes, kPieces = Sh::kPieces, kPPW = Sh::kPPW;
+    static_assert((kLM / 16) % kPPW == 0, "a wave's pieces are all A rows or all B rows");
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
     const int nsteps = (int)(a.K / kLK);
     const int last = nsteps - 1;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t*)smem;
 
-    // this wave's 1 KiB pieces of a stage: pieces 0 .. kLM/16-1 are A rows, the rest B rows
-    const int8_t* gp[kPPW];
+    // this wave's 1 KiB pieces of a stage: pieces 0 .. kLM/16-1 are A rows, the rest B rows.  A wave's pieces
+    // all come from one operand, so a load is addressed as (operand base + 64 * step) in SGPRs plus a constant
+    // 32-bit byte offset per lane and piece (the host admits only operands below 4 GiB to this kernel).
+    const bool wave_is_a = wave * kPPW < kLM / 16;
+    const int8_t* const opbase = wave_is_a ? a.xq : a.wq;
+    uint32_t goff[kPPW];
     {
         const int rin = lane >> 2;                                  // row inside the 16-row piece
         const int lc = (lane & 3) ^ ((rin >> 2) & 3);               // logical chunk this lane fetches
@@ -228,21 +237,32 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
         for (int j = 0; j < kPPW; ++j) {
             // a wave beyond the last piece fetches the last piece again: same bytes to the same place
             const int piece = (kPieces % kWaves == 0 || wave * kPPW + j < kPieces) ? wave * kPPW + j : kPieces - 1;
-            if (piece < kLM / 16) {
-                const int64_t r = m0 + piece * 16 + rin;
-                gp[j] = a.xq + (r < a.M ? r : a.M - 1) * a.K + lc * 16;
+            int64_t r;
+            if (wave_is_a) {
+#ifdef AMCT_ABL_SAMETILE
+                r = piece * 16 + rin;
+#else
+                r = m0 + piece * 16 + rin;
+#endif
+                r = r < a.M ? r : a.M - 1;
             } else {
-                const int64_t r = n0 + (piece - kLM / 16) * 16 + rin;
-                gp[j] = a.wq + (r < a.N ? r : a.N - 1) * a.K + lc * 16;
+#ifdef AMCT_ABL_SAMETILE
+                r = (piece - kLM / 16) * 16 + rin;
+#else
+                r = n0 + (piece - kLM / 16) * 16 + rin;
+#endif
+                r = r < a.N ? r : a.N - 1;
             }
+            goff[j] = (uint32_t)(r * a.K + lc * 16);
         }
     }
+    auto dma_one = [&](int stg, int step, int j) {
+        const int piece = (kPieces % kWaves == 0 || wave * kPPW + j < kPieces) ? wave * kPPW + j : kPieces - 1;
+        dma16s(lds0 + stg * kLStageBytes + piece * 1024, opbase + (int64_t)step * kLK, goff[j]);
+    };
     auto dma_stage = [&](int stage, int step) {
 #pragma unroll
-        for (int j = 0; j < kPPW; ++j) {
-            const int piece = (kPieces % kWaves == 0 || wave * kPPW + j < kPieces) ? wave * kPPW + j : kPieces - 1;
-            dma16(__builtin_amdgcn_readfirstlane(lds0 + stage * kLStageBytes + piece * 1024), gp[j] + (int64_t)step * kLK);
-        }
+        for (int j = 0; j < kPPW; ++j) dma_one(stage, step, j);
     };
 
     // fragment offsets: lane reads row (tile base + lane%32), logical chunk 2*ks + lane/32
@@ -280,42 +300,129 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
             for (int j = 0; j < TJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
     };
 
-    // software pipeline over half K-steps: while the 8 MFMAs of one half run, the fragments of the
-    // next half are read from LDS.  At the barrier of iteration s every wave holds the last fragments
-    // of stage s % STAGES in registers (lgkmcnt(0)), so that stage is free for the loads of step
-    // s + STAGES; the loads of the STAGES-2 steps after s+1 stay in flight.
+    // software pipeline over half K-steps: while the MFMAs of one half run, the fragments of the next half
+    // are read from LDS.  At the barrier of iteration s every wave holds the last fragments of stage
+    // s % STAGES in registers (lgkmcnt(0)), so that stage is free for the loads of step s + STAGES; the loads
+    // of the STAGES-2 steps after s+1 stay in flight.
+    // The issue order is pinned instruction by instruction (a scheduling barrier after each): one memory
+    // instruction in the shadow of each MFMA, the MFMAs of the first half issued BEFORE the wait and the barrier,
+    // the first MFMA of the second half right after it.  Left alone, the optimiser moves the first half's MFMAs
+    // behind the barrier (the matrix pipe then idles while the waves meet) and, with a conditional read at the
+    // end of the loop, waits for the youngest LDS reads before the second half.  The loop is therefore
+    // branch-free: the last iteration reads one stage too far (valid LDS, values unused).
+    constexpr int kNM = TI * TJ, kNR = TI + TJ;
+#ifndef AMCT_DMA_SPREAD
+#define AMCT_DMA_SPREAD 1
+#endif
+#ifndef AMCT_RPM
+#define AMCT_RPM 2
+#endif
+    constexpr int kRPM = AMCT_RPM;                                  // fragment reads issued behind each MFMA
+    static_assert(kNM >= kNR && kNM >= kPPW, "one memory instruction per MFMA");
+    // fragment q in the order the MFMAs need them: A0, B0, B1, .., A1, A2, ..
+    auto read_one = [&](int stg, int ks, int q, v4i (&fa)[TI], v4i (&fb)[TJ]) {
+        const int8_t* st = smem + stg * kLStageBytes;
+        if (q == 0) fa[0] = *reinterpret_cast<const v4i*>(st + offA[ks]);
+        else if (q <= TJ) fb[q - 1] = *reinterpret_cast<const v4i*>(st + offB[ks] + (q - 1) * 32 * kLK);
+        else fa[q - TJ] = *reinterpret_cast<const v4i*>(st + offA[ks] + (q - TJ) * 32 * kLK);
+    };
+    auto mfma_one = [&](int m, const v4i (&fa)[TI], const v4i (&fb)[TJ]) {
+        const int i = m / TJ, j = m % TJ;
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    };
     v4i fa0[TI], fb0[TJ], fa1[TI], fb1[TJ];
     wait_dma_lds<(STAGES - 2) * kPPW>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    dma_stage(STAGES - 1, STAGES - 1 < last ? STAGES - 1 : last);
+#if AMCT_DMA_SPREAD
+    constexpr int kDH = kPPW / 2;                                   // pieces issued in the half after the barrier
+#else
+    constexpr int kDH = kPPW;
+#endif
+    constexpr int kGapA = kDH > 0 ? kNM / kDH : kNM, kGapB = kPPW > kDH ? kNM / (kPPW - kDH) : kNM;
+    int pstage = STAGES - 1, prefill = STAGES - 1 < last ? STAGES - 1 : last;
+#pragma unroll
+    for (int j = 0; j < kDH; ++j) dma_one(pstage, prefill, j);
     read_frags(0, 0, fa0, fb0);
     int stage = 0;
     for (int step = 0; step < nsteps; ++step) {
         const int next = stage + 1 == STAGES ? 0 : stage + 1;
-        read_frags(stage, 1, fa1, fb1);
-        mfma_half(fa0, fb0);
+        const int refill = step + STAGES < last ? step + STAGES : last;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int m = 0; m < kNM; ++m) {
+            mfma_one(m, fa0, fb0);
+            __builtin_amdgcn_sched_barrier(0);
+#ifndef AMCT_ABL_NODMA
+            if (kPPW > kDH && m % kGapB == 0 && m / kGapB < kPPW - kDH) {   // the rest of the previous refill
+                dma_one(pstage, prefill, kDH + m / kGapB);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#endif
+#pragma unroll
+            for (int q = kRPM * m; q < kRPM * (m + 1); ++q) {
+#ifndef AMCT_ABL_NOREAD
+                if (q < kNR) {
+                    read_one(stage, 1, q, fa1, fb1);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#endif
+            }
+        }
+#if defined(AMCT_ABL_NODMA)
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+#elif defined(AMCT_ABL_NOWAIT)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#else
         wait_dma_lds<(STAGES - 2) * kPPW>();
+#endif
+#ifndef AMCT_ABL_NOBAR
         __builtin_amdgcn_s_barrier();
+#endif
         asm volatile("" ::: "memory");
-        dma_stage(stage, step + STAGES < last ? step + STAGES : last);
-        if (step + 1 < nsteps) read_frags(next, 0, fa0, fb0);
-        mfma_half(fa1, fb1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int m = 0; m < kNM; ++m) {
+            mfma_one(m, fa1, fb1);
+            __builtin_amdgcn_sched_barrier(0);
+#ifndef AMCT_ABL_NODMA
+            if (m % kGapA == 0 && m / kGapA < kDH) {
+                dma_one(stage, refill, m / kGapA);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#endif
+#pragma unroll
+            for (int q = kRPM * m; q < kRPM * (m + 1); ++q) {
+#ifndef AMCT_ABL_NOREAD
+                if (q < kNR) {
+                    read_one(next, 0, q, fa0, fb0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#endif
+            }
+        }
+        pstage = stage;
+        prefill = refill;
         stage = next;
     }
     // all loads landed and every wave is done with the stages before LDS is reused
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 
     // epilogue: fp32(acc + ibias) * s_ch * s_tok + fbias, narrowed, transposed through a per-wave LDS
-    // patch of 32 rows x 32*TJ columns, stored as 16-byte pieces of full rows
+    // patch of 32 rows x 32*TJ columns, stored as 16-byte pieces of full rows.  Branch-free per element:
+    // absent factors are replaced by their neutral elements (x * 1.0f and x + (-0.0f) return x bit for bit),
+    // the row factors of the wave come from a small LDS table, every LDS address is base + immediate.
     constexpr int ES = (ODT == AMCT_F32) ? 4 : 2;                   // bytes per output element
     constexpr int kPW = 32 * TJ;                                   // patch width in columns
     constexpr int kPatchRow = kPW * ES + 16;                       // padded patch row
     constexpr int CPR = kPW * ES / 16;                             // 16-byte chunks per patch row
-    static_assert(32 * kPatchRow <= 16384 && (32 * CPR) % 64 == 0, "patch must fit its 16 KiB and split into wave-wide reads");
+    constexpr int kTokOff = 16384 - 512;                           // 32*TI <= 128 row factors behind the patch
+    static_assert(32 * kPatchRow <= kTokOff && (32 * CPR) % 64 == 0 && TI <= 4,
+                  "patch and row factors must fit the wave's 16 KiB; the patch must split into wave-wide reads");
     int8_t* patch = smem + wave * 16384;
+    float* tokl = reinterpret_cast<float*>(patch + kTokOff);
     float sc[TJ], fb2[TJ];
     int32_t ib[TJ];
 #pragma unroll
@@ -324,33 +431,47 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
         const int64_t nc = n < a.N ? n : a.N - 1;
         sc[j] = a.s_ch[nc];
         ib[j] = a.bias_kind == 1 ? reinterpret_cast<const int32_t*>(a.bias)[nc] : 0;
-        fb2[j] = a.bias_kind == 2 ? reinterpret_cast<const float*>(a.bias)[nc] : 0.f;
+        fb2[j] = a.bias_kind == 2 ? reinterpret_cast<const float*>(a.bias)[nc] : -0.0f;
     }
+#pragma unroll
+    for (int t = lane; t < 32 * TI; t += 64) {
+        const int64_t m = m0 + wm * 32 * TI + t;
+        tokl[t] = a.s_tok ? a.s_tok[m < a.M ? m : a.M - 1] : 1.0f;
+    }
+    if (a.acc_out) {                                                // accumulators on request (tests): plain stores
+#pragma unroll
+        for (int i = 0; i < TI; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+#pragma unroll
+                for (int j = 0; j < TJ; ++j) {
+                    const int64_t m = m0 + wm * 32 * TI + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    const int64_t n = n0 + wn * kPW + j * 32 + (lane & 31);
+                    if (m < a.M && n < a.N) a.acc_out[m * a.N + n] = acc[i][j][r] + ib[j];
+                }
+    }
+    const int h4 = 4 * (lane >> 5);
+    int8_t* wbase = patch + h4 * kPatchRow + (lane & 31) * ES;      // this lane's element of patch row h4
+    const int8_t* rbase = patch + (lane / CPR) * kPatchRow + (lane % CPR) * 16;
+    constexpr int RPI = 64 / CPR;                                   // patch rows per wave-wide read when CPR divides 64
 #pragma unroll
     for (int i = 0; i < TI; ++i) {
         const int64_t mbase = m0 + wm * 32 * TI + i * 32;
         float tks[16];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {                              // all 16 row factors in flight together
-            const int64_t m = mbase + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-            tks[r] = a.s_tok ? a.s_tok[m < a.M ? m : a.M - 1] : 1.0f;
+        for (int q = 0; q < 4; ++q) {                               // rows 8q + h4 .. + 3 are registers 4q .. 4q + 3
+            const float4 t4 = *reinterpret_cast<const float4*>(tokl + i * 32 + 8 * q + h4);
+            tks[4 * q] = t4.x; tks[4 * q + 1] = t4.y; tks[4 * q + 2] = t4.z; tks[4 * q + 3] = t4.w;
         }
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int prow = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-            const int64_t m = mbase + prow;
-            const float tk = tks[r];
+            const int prow0 = 8 * (r >> 2) + (r & 3);               // patch row minus h4
 #pragma unroll
             for (int j = 0; j < TJ; ++j) {
-                const int32_t v = acc[i][j][r] + ib[j];
-                if (a.acc_out) {
-                    const int64_t n = n0 + wn * kPW + j * 32 + (lane & 31);
-                    if (m < a.M && n < a.N) a.acc_out[m * a.N + n] = v;
-                }
-                float f = (float)v * sc[j];
-                if (a.s_tok) f = f * tk;
-                if (a.bias_kind == 2) f = f + fb2[j];
-                int8_t* dst = patch + prow * kPatchRow + (j * 32 + (lane & 31)) * ES;
+                float f = (float)(acc[i][j][r] + ib[j]) * sc[j];
+                f = f * tks[r];
+                f = f + fb2[j];
+                int8_t* dst = wbase + prow0 * kPatchRow + j * 32 * ES;
                 if constexpr (ODT == AMCT_F32) *reinterpret_cast<float*>(dst) = f;
                 else if constexpr (ODT == AMCT_BF16) *reinterpret_cast<uint16_t*>(dst) = (uint16_t)f32_to_bf16_bits(f);
                 else *reinterpret_cast<uint16_t*>(dst) = (uint16_t)f32_to_f16_bits(f);
@@ -359,10 +480,18 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
         // LDS operations of one wave complete in order: the reads below see the writes above
 #pragma unroll
         for (int it = 0; it < 32 * CPR / 64; ++it) {
-            const int idx = it * 64 + lane;                        // 16-byte chunk of the patch, row-major
-            const int prow = idx / CPR;
-            const int chunk = idx % CPR;
-            const uint4 v = *reinterpret_cast<const uint4*>(patch + prow * kPatchRow + chunk * 16);
+            int prow, chunk;
+            uint4 v;
+            if constexpr (64 % CPR == 0) {
+                prow = it * RPI + lane / CPR;
+                chunk = lane % CPR;
+                v = *reinterpret_cast<const uint4*>(rbase + it * RPI * kPatchRow);
+            } else {
+                const int idx = it * 64 + lane;                    // 16-byte chunk of the patch, row-major
+                prow = idx / CPR;
+                chunk = idx % CPR;
+                v = *reinterpret_cast<const uint4*>(patch + prow * kPatchRow + chunk * 16);
+            }
             const int64_t m = mbase + prow;
             const int64_t n = n0 + wn * kPW + chunk * (16 / ES);
             if (m < a.M && n < a.N) stg16_nt(reinterpret_cast<char*>(a.out) + (m * a.N + n) * ES, v);
@@ -730,7 +859,8 @@ extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s
         else hipLaunchKernelGGL((w8a8_skinny<2>), grid, dim3(kBlock), 0, st, a);
         return hip_status();
     }
-    if (vec_ok && M >= 256 && K % kLK == 0 && K >= kLK && N % 8 == 0 && aligned16(out)) {
+    if (vec_ok && M >= 256 && K % kLK == 0 && K >= kLK && N % 8 == 0 && aligned16(out) && M * K < (int64_t(1) << 32) &&
+        N * K < (int64_t(1) << 32)) {
         // 256x256 tiles, 8 waves, 4 stages (measured faster than 256x128 with two blocks per CU:
         // the traffic from L2 into LDS matters more than decoupling the barriers)
         const dim3 grid((unsigned)((N + 255) / 256), (unsigned)((M + 255) / 256));
