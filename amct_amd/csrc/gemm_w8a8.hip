@@ -199,80 +199,85 @@ AMCT_DEV void dma16s(uint32_t lds_addr, const void* sbase, uint32_t voff) {
 }
 template <int N> AMCT_DEV void wait_dma_lds() { asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"(N) : "memory"); }
 
-// WM x WN waves of (32*TI) x (32*TJ) each: block tile (32*TI*WM) x (32*TJ*WN); STAGES LDS stages of BK = 64 bytes.
-// The body is a device function so that one launch can mix block shapes (see w8a8_tile_mix).
-template <int WM, int WN, int TI, int TJ, int STAGES>
+// WM x WN waves of (32*TI) x (32*TJ) each: block tile (32*TI*WM) x (32*TJ*WN); STAGES LDS stages of LK bytes
+// of K (64 or 128).  The body is a device function so that one launch can mix block shapes (see w8a8_tile_mix).
+template <int WM, int WN, int TI, int TJ, int STAGES, int LK>
 struct DmaTile {
     static constexpr int kLM = 32 * TI * WM, kLN = 32 * TJ * WN, kWaves = WM * WN;
-    static constexpr int kLStageBytes = (kLM + kLN) * kLK;
-    static constexpr int kPieces = (kLM + kLN) / 16;               // 1 KiB pieces per stage
-    static constexpr int kPPW = (kPieces + kWaves - 1) / kWaves;   // pieces per wave (the last wave may repeat one)
+    static constexpr int kLStageBytes = (kLM + kLN) * LK;
+    static constexpr int kRP = 1024 / LK;                          // rows per 1 KiB piece
+    static constexpr int kNA = kLM / kRP / kWaves;                 // A pieces per wave and stage
+    static constexpr int kNB = (kLN / kRP + kWaves - 1) / kWaves;  // B pieces per wave (the last ones may repeat)
+    static constexpr int kPPW = kNA + kNB;
     static constexpr int kEpiBytes = kWaves * 16384;
     static constexpr int kSmem = STAGES * kLStageBytes > kEpiBytes ? STAGES * kLStageBytes : kEpiBytes;
+    static_assert((kLM / kRP) % kWaves == 0, "the A pieces must divide evenly among the waves");
+    static_assert(kSmem <= 160 * 1024, "LDS");
 };
 
-template <int ODT, int WM, int WN, int TI, int TJ, int STAGES>
+template <int ODT, int WM, int WN, int TI, int TJ, int STAGES, int LK>
 AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, const int64_t n0) {
-    using Sh = DmaTile<WM, WN, TI, TJ, STAGES>;
-    constexpr int kLM = Sh::kLM, kLN = Sh::kLN, kWaves = Sh::kWaves;
-    constexpr int kLStageBytes = Sh::kLStageBytes, kPieces = Sh::kPieces, kPPW = Sh::kPPW;
-    static_assert((kLM / 16) % kPPW == 0, "a wave's pieces are all A rows or all B rows");
+    using Sh = DmaTile<WM, WN, TI, TJ, STAGES, LK>;
+    constexpr int kLM = Sh::kLM, kLN = Sh::kLN, kRP = Sh::kRP, kNA = Sh::kNA, kNB = Sh::kNB, kPPW = Sh::kPPW;
+    constexpr int kLStageBytes = Sh::kLStageBytes;
+    constexpr int kCH = LK / 16;                                    // 16-byte chunks per row
+    constexpr int kKS = LK / 32;                                    // MFMA k-slices per stage
+    static_assert(LK == 64 || LK == 128, "row length");
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
-    const int nsteps = (int)(a.K / kLK);
+    const int nsteps = (int)(a.K / LK);
     const int last = nsteps - 1;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t*)smem;
+    // Rows are LK bytes, unpadded (a direct-to-LDS load writes the 64 lanes' 16-byte pieces to 1024 contiguous
+    // bytes); 16-byte chunk c of row r lives at chunk position c ^ swz(r), which spreads the 16 rows that one
+    // phase of a 16-byte fragment read touches over all banks.
+    auto swz = [](int r) { return LK == 64 ? (r >> 2) & 3 : (r >> 1) & 7; };
 
-    // this wave's 1 KiB pieces of a stage: pieces 0 .. kLM/16-1 are A rows, the rest B rows.  A wave's pieces
-    // all come from one operand, so a load is addressed as (operand base + 64 * step) in SGPRs plus a constant
-    // 32-bit byte offset per lane and piece (the host admits only operands below 4 GiB to this kernel).
-    const bool wave_is_a = wave * kPPW < kLM / 16;
-    const int8_t* const opbase = wave_is_a ? a.xq : a.wq;
+    // this wave's 1 KiB pieces of a stage: kNA pieces of A rows, then kNB pieces of B rows.  A load is addressed
+    // as (operand base + LK * step) in SGPRs plus a constant 32-bit byte offset per lane and piece (the host
+    // admits only operands below 4 GiB to this kernel).
     uint32_t goff[kPPW];
     {
-        const int rin = lane >> 2;                                  // row inside the 16-row piece
-        const int lc = (lane & 3) ^ ((rin >> 2) & 3);               // logical chunk this lane fetches
+        const int rin = lane / kCH;                                 // row inside the piece
+        const int pc = lane % kCH;                                  // physical chunk this lane fills
 #pragma unroll
         for (int j = 0; j < kPPW; ++j) {
-            // a wave beyond the last piece fetches the last piece again: same bytes to the same place
-            const int piece = (kPieces % kWaves == 0 || wave * kPPW + j < kPieces) ? wave * kPPW + j : kPieces - 1;
             int64_t r;
-            if (wave_is_a) {
-#ifdef AMCT_ABL_SAMETILE
-                r = piece * 16 + rin;
-#else
-                r = m0 + piece * 16 + rin;
-#endif
-                r = r < a.M ? r : a.M - 1;
+            int lr;                                                 // row inside the operand's LDS tile
+            if (j < kNA) {
+                lr = (wave * kNA + j) * kRP + rin;
+                r = m0 + lr < a.M ? m0 + lr : a.M - 1;
             } else {
-#ifdef AMCT_ABL_SAMETILE
-                r = (piece - kLM / 16) * 16 + rin;
-#else
-                r = n0 + (piece - kLM / 16) * 16 + rin;
-#endif
-                r = r < a.N ? r : a.N - 1;
+                // a wave beyond the last piece fetches the last piece again: same bytes to the same place
+                const int pb = wave * kNB + (j - kNA) < kLN / kRP ? wave * kNB + (j - kNA) : kLN / kRP - 1;
+                lr = pb * kRP + rin;
+                r = n0 + lr < a.N ? n0 + lr : a.N - 1;
             }
-            goff[j] = (uint32_t)(r * a.K + lc * 16);
+            goff[j] = (uint32_t)(r * a.K + (pc ^ swz(lr)) * 16);
         }
     }
     auto dma_one = [&](int stg, int step, int j) {
-        const int piece = (kPieces % kWaves == 0 || wave * kPPW + j < kPieces) ? wave * kPPW + j : kPieces - 1;
-        dma16s(lds0 + stg * kLStageBytes + piece * 1024, opbase + (int64_t)step * kLK, goff[j]);
+        if (j < kNA) {
+            dma16s(lds0 + stg * kLStageBytes + (wave * kNA + j) * 1024, a.xq + (int64_t)step * LK, goff[j]);
+        } else {
+            const int pb = wave * kNB + (j - kNA) < kLN / kRP ? wave * kNB + (j - kNA) : kLN / kRP - 1;
+            dma16s(lds0 + stg * kLStageBytes + kLM * LK + pb * 1024, a.wq + (int64_t)step * LK, goff[j]);
+        }
     };
     auto dma_stage = [&](int stage, int step) {
 #pragma unroll
         for (int j = 0; j < kPPW; ++j) dma_one(stage, step, j);
     };
 
-    // fragment offsets: lane reads row (tile base + lane%32), logical chunk 2*ks + lane/32
-    int offA[2], offB[2];
+    // fragment offsets of k-slice ks: lane reads row (tile base + lane%32), logical chunk 2*ks + lane/32
+    int offA[kKS], offB[kKS];
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
+    for (int ks = 0; ks < kKS; ++ks) {
         const int r = lane & 31;
-        const int phys = (ks * 2 + (lane >> 5)) ^ ((r >> 2) & 3);
-        offA[ks] = (wm * 32 * TI + r) * kLK + phys * 16;
-        offB[ks] = kLM * kLK + (wn * 32 * TJ + r) * kLK + phys * 16;
+        const int phys = (ks * 2 + (lane >> 5)) ^ swz(r);
+        offA[ks] = (wm * 32 * TI + r) * LK + phys * 16;
+        offB[ks] = kLM * LK + (wn * 32 * TJ + r) * LK + phys * 16;
     }
 
     v16i acc[TI][TJ];
@@ -286,123 +291,74 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s) dma_stage(s, s < last ? s : last);
 
-    auto read_frags = [&](int stage, int ks, v4i (&fa)[TI], v4i (&fb)[TJ]) {
-        const int8_t* st = smem + stage * kLStageBytes;
-#pragma unroll
-        for (int i = 0; i < TI; ++i) fa[i] = *reinterpret_cast<const v4i*>(st + offA[ks] + i * 32 * kLK);
-#pragma unroll
-        for (int j = 0; j < TJ; ++j) fb[j] = *reinterpret_cast<const v4i*>(st + offB[ks] + j * 32 * kLK);
-    };
-    auto mfma_half = [&](const v4i (&fa)[TI], const v4i (&fb)[TJ]) {
-#pragma unroll
-        for (int i = 0; i < TI; ++i)
-#pragma unroll
-            for (int j = 0; j < TJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
-    };
-
-    // software pipeline over half K-steps: while the MFMAs of one half run, the fragments of the next half
-    // are read from LDS.  At the barrier of iteration s every wave holds the last fragments of stage
-    // s % STAGES in registers (lgkmcnt(0)), so that stage is free for the loads of step s + STAGES; the loads
-    // of the STAGES-2 steps after s+1 stay in flight.
-    // The issue order is pinned instruction by instruction (a scheduling barrier after each): one memory
-    // instruction in the shadow of each MFMA, the MFMAs of the first half issued BEFORE the wait and the barrier,
-    // the first MFMA of the second half right after it.  Left alone, the optimiser moves the first half's MFMAs
-    // behind the barrier (the matrix pipe then idles while the waves meet) and, with a conditional read at the
-    // end of the loop, waits for the youngest LDS reads before the second half.  The loop is therefore
-    // branch-free: the last iteration reads one stage too far (valid LDS, values unused).
+    // Software pipeline over k-slices of 32 bytes: while the MFMAs of one slice run, the fragments of the next
+    // slice are read from LDS.  Before the last slice of a stage the waves meet: every wave then holds that
+    // slice's fragments in registers (lgkmcnt(0)), so the stage is free for the loads of step s + STAGES, and
+    // the loads of step s + 1 have landed (those of the STAGES-2 steps after it stay in flight).
+    // The issue order is pinned instruction by instruction (a scheduling barrier after each): memory
+    // instructions in the shadow of the MFMAs, the MFMAs of the slices before the barrier issued BEFORE the
+    // wait, the first MFMA of the last slice right after it.  Left alone, the optimiser moves MFMAs behind the
+    // barrier (the matrix pipe then idles while the waves meet) and, with a conditional read at the end of the
+    // loop, waits for the youngest LDS reads too early.  The loop is therefore branch-free: the last iteration
+    // reads one stage too far (valid LDS, values unused).
     constexpr int kNM = TI * TJ, kNR = TI + TJ;
-#ifndef AMCT_DMA_SPREAD
-#define AMCT_DMA_SPREAD 1
-#endif
-#ifndef AMCT_RPM
-#define AMCT_RPM 2
-#endif
-    constexpr int kRPM = AMCT_RPM;                                  // fragment reads issued behind each MFMA
-    static_assert(kNM >= kNR && kNM >= kPPW, "one memory instruction per MFMA");
+    constexpr int kDPM = (kPPW + kNM - 1) / kNM;                    // loads issued behind each MFMA of the last slice
+    static_assert(kNM >= kNR, "one fragment read per MFMA");
     // fragment q in the order the MFMAs need them: A0, B0, B1, .., A1, A2, ..
     auto read_one = [&](int stg, int ks, int q, v4i (&fa)[TI], v4i (&fb)[TJ]) {
         const int8_t* st = smem + stg * kLStageBytes;
         if (q == 0) fa[0] = *reinterpret_cast<const v4i*>(st + offA[ks]);
-        else if (q <= TJ) fb[q - 1] = *reinterpret_cast<const v4i*>(st + offB[ks] + (q - 1) * 32 * kLK);
-        else fa[q - TJ] = *reinterpret_cast<const v4i*>(st + offA[ks] + (q - TJ) * 32 * kLK);
+        else if (q <= TJ) fb[q - 1] = *reinterpret_cast<const v4i*>(st + offB[ks] + (q - 1) * 32 * LK);
+        else fa[q - TJ] = *reinterpret_cast<const v4i*>(st + offA[ks] + (q - TJ) * 32 * LK);
     };
     auto mfma_one = [&](int m, const v4i (&fa)[TI], const v4i (&fb)[TJ]) {
         const int i = m / TJ, j = m % TJ;
         acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
     };
-    v4i fa0[TI], fb0[TJ], fa1[TI], fb1[TJ];
+    v4i fa[2][TI], fb[2][TJ];
     wait_dma_lds<(STAGES - 2) * kPPW>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-#if AMCT_DMA_SPREAD
-    constexpr int kDH = kPPW / 2;                                   // pieces issued in the half after the barrier
-#else
-    constexpr int kDH = kPPW;
-#endif
-    constexpr int kGapA = kDH > 0 ? kNM / kDH : kNM, kGapB = kPPW > kDH ? kNM / (kPPW - kDH) : kNM;
-    int pstage = STAGES - 1, prefill = STAGES - 1 < last ? STAGES - 1 : last;
+    dma_stage(STAGES - 1, STAGES - 1 < last ? STAGES - 1 : last);
 #pragma unroll
-    for (int j = 0; j < kDH; ++j) dma_one(pstage, prefill, j);
-    read_frags(0, 0, fa0, fb0);
+    for (int q = 0; q < kNR; ++q) read_one(0, 0, q, fa[0], fb[0]);
     int stage = 0;
     for (int step = 0; step < nsteps; ++step) {
         const int next = stage + 1 == STAGES ? 0 : stage + 1;
         const int refill = step + STAGES < last ? step + STAGES : last;
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int m = 0; m < kNM; ++m) {
-            mfma_one(m, fa0, fb0);
-            __builtin_amdgcn_sched_barrier(0);
-#ifndef AMCT_ABL_NODMA
-            if (kPPW > kDH && m % kGapB == 0 && m / kGapB < kPPW - kDH) {   // the rest of the previous refill
-                dma_one(pstage, prefill, kDH + m / kGapB);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-#endif
+        for (int ks = 0; ks < kKS - 1; ++ks) {
 #pragma unroll
-            for (int q = kRPM * m; q < kRPM * (m + 1); ++q) {
-#ifndef AMCT_ABL_NOREAD
-                if (q < kNR) {
-                    read_one(stage, 1, q, fa1, fb1);
+            for (int m = 0; m < kNM; ++m) {
+                mfma_one(m, fa[ks & 1], fb[ks & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+                if (m < kNR) {
+                    read_one(stage, ks + 1, m, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
                     __builtin_amdgcn_sched_barrier(0);
                 }
-#endif
             }
         }
-#if defined(AMCT_ABL_NODMA)
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-#elif defined(AMCT_ABL_NOWAIT)
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#else
         wait_dma_lds<(STAGES - 2) * kPPW>();
-#endif
-#ifndef AMCT_ABL_NOBAR
         __builtin_amdgcn_s_barrier();
-#endif
         asm volatile("" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int m = 0; m < kNM; ++m) {
-            mfma_one(m, fa1, fb1);
+            mfma_one(m, fa[(kKS - 1) & 1], fb[(kKS - 1) & 1]);
             __builtin_amdgcn_sched_barrier(0);
-#ifndef AMCT_ABL_NODMA
-            if (m % kGapA == 0 && m / kGapA < kDH) {
-                dma_one(stage, refill, m / kGapA);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-#endif
 #pragma unroll
-            for (int q = kRPM * m; q < kRPM * (m + 1); ++q) {
-#ifndef AMCT_ABL_NOREAD
-                if (q < kNR) {
-                    read_one(next, 0, q, fa0, fb0);
+            for (int j = kDPM * m; j < kDPM * (m + 1); ++j) {
+                if (j < kPPW) {
+                    dma_one(stage, refill, j);
                     __builtin_amdgcn_sched_barrier(0);
                 }
-#endif
+            }
+            if (m < kNR) {
+                read_one(next, 0, m, fa[0], fb[0]);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
-        pstage = stage;
-        prefill = refill;
         stage = next;
     }
     // all loads landed and every wave is done with the stages before LDS is reused
@@ -499,11 +455,11 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
     }
 }
 
-template <int ODT, int WM, int WN, int STAGES>
+template <int ODT, int WM, int WN, int STAGES, int LK>
 __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void w8a8_tile_dma(W8A8Args a) {
-    using Sh = DmaTile<WM, WN, 4, 2, STAGES>;
+    using Sh = DmaTile<WM, WN, 4, 2, STAGES, LK>;
     __shared__ __attribute__((aligned(1024))) int8_t smem[Sh::kSmem];
-    w8a8_dma_body<ODT, WM, WN, 4, 2, STAGES>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
+    w8a8_dma_body<ODT, WM, WN, 4, 2, STAGES, LK>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
 }
 
 // One launch, two block shapes: the first `big` blocks compute 256x256 tiles of the first `nbig` column tiles,
@@ -517,18 +473,18 @@ struct MixPlan {
     int nsmall;                                                     // 192-column tiles after them
 };
 
-template <int ODT>
+template <int ODT, int STAGES, int LK>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void w8a8_tile_mix(W8A8Args a, MixPlan p) {
-    using Big = DmaTile<2, 4, 4, 2, 4>;
-    using Small = DmaTile<4, 2, 2, 3, 4>;
+    using Big = DmaTile<2, 4, 4, 2, STAGES, LK>;
+    using Small = DmaTile<4, 2, 2, 3, STAGES, LK>;
     __shared__ __attribute__((aligned(1024))) int8_t smem[Big::kSmem > Small::kSmem ? Big::kSmem : Small::kSmem];
     const int b = blockIdx.x;
     if (b < p.big) {
-        w8a8_dma_body<ODT, 2, 4, 4, 2, 4>(a, smem, (int64_t)(b / p.nbig) * 256, (int64_t)(b % p.nbig) * 256);
+        w8a8_dma_body<ODT, 2, 4, 4, 2, STAGES, LK>(a, smem, (int64_t)(b / p.nbig) * 256, (int64_t)(b % p.nbig) * 256);
     } else {
         const int s = b - p.big;
-        w8a8_dma_body<ODT, 4, 2, 2, 3, 4>(a, smem, (int64_t)(s / p.nsmall) * 256,
-                                          (int64_t)p.nbig * 256 + (int64_t)(s % p.nsmall) * 192);
+        w8a8_dma_body<ODT, 4, 2, 2, 3, STAGES, LK>(a, smem, (int64_t)(s / p.nsmall) * 256,
+                                                   (int64_t)p.nbig * 256 + (int64_t)(s % p.nsmall) * 192);
     }
 }
 
@@ -872,16 +828,25 @@ extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s
             cus = 0;
         }
         const MixPlan plan = plan_mix(M, N, cus);
-        if (plan.nbig >= 0) {
-            const dim3 g1((unsigned)(plan.big + plan.mtiles * plan.nsmall));
-            if (out_dtype == AMCT_BF16) hipLaunchKernelGGL((w8a8_tile_mix<AMCT_BF16>), g1, dim3(512), 0, st, a, plan);
-            else if (out_dtype == AMCT_F16) hipLaunchKernelGGL((w8a8_tile_mix<AMCT_F16>), g1, dim3(512), 0, st, a, plan);
-            else hipLaunchKernelGGL((w8a8_tile_mix<AMCT_F32>), g1, dim3(512), 0, st, a, plan);
-            return hip_status();
-        }
-        if (out_dtype == AMCT_BF16) hipLaunchKernelGGL((w8a8_tile_dma<AMCT_BF16, 2, 4, 4>), grid, dim3(512), 0, st, a);
-        else if (out_dtype == AMCT_F16) hipLaunchKernelGGL((w8a8_tile_dma<AMCT_F16, 2, 4, 4>), grid, dim3(512), 0, st, a);
-        else hipLaunchKernelGGL((w8a8_tile_dma<AMCT_F32, 2, 4, 4>), grid, dim3(512), 0, st, a);
+#ifndef AMCT_LK128
+#define AMCT_LK128 1
+#endif
+        const bool wide = AMCT_LK128 && K % 128 == 0;                // 128-byte rows, 2 stages; else 64-byte rows, 4 stages
+#define AMCT_LAUNCH_DMA(ODT)                                                                                        \
+    {                                                                                                               \
+        if (plan.nbig >= 0) {                                                                                       \
+            const dim3 g1((unsigned)(plan.big + plan.mtiles * plan.nsmall));                                        \
+            if (wide) hipLaunchKernelGGL((w8a8_tile_mix<ODT, 2, 128>), g1, dim3(512), 0, st, a, plan);              \
+            else hipLaunchKernelGGL((w8a8_tile_mix<ODT, 4, 64>), g1, dim3(512), 0, st, a, plan);                    \
+        } else {                                                                                                    \
+            if (wide) hipLaunchKernelGGL((w8a8_tile_dma<ODT, 2, 4, 2, 128>), grid, dim3(512), 0, st, a);            \
+            else hipLaunchKernelGGL((w8a8_tile_dma<ODT, 2, 4, 4, 64>), grid, dim3(512), 0, st, a);                  \
+        }                                                                                                           \
+    }
+        if (out_dtype == AMCT_BF16) AMCT_LAUNCH_DMA(AMCT_BF16)
+        else if (out_dtype == AMCT_F16) AMCT_LAUNCH_DMA(AMCT_F16)
+        else AMCT_LAUNCH_DMA(AMCT_F32)
+#undef AMCT_LAUNCH_DMA
         return hip_status();
     }
     if (vec_ok) {
