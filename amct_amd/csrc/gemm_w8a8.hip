@@ -3,9 +3,10 @@
 //
 // Both operands are K-contiguous, which is the natural operand order of the gfx950 int8 MFMA
 // (v_mfma_i32_32x32x32_i8: lane l supplies 16 consecutive k-bytes of row l%32, k-half l/32).
-//   large tiles   : 256x256 block tile, 8 waves of 128x64, BK = 64 bytes, 4 LDS stages filled by
-//                   direct global->LDS loads, fragment reads software-pipelined against the MFMAs;
-//                   when the tile count does not fill the CUs evenly, one launch mixes in 256x192 tiles.
+//   large tiles   : 256x256 block tile, 8 waves of 128x64, LDS stages of 128 bytes of K filled by direct
+//                   global->LDS loads, fragment reads software-pipelined against the MFMAs in a pinned
+//                   issue order; when the tile count does not fill the CUs evenly, one launch mixes in
+//                   256x192 tiles.
 //   tile kernel   : 128x128 block tile, 4 waves of 64x64, BK = 128 bytes, two register stages of
 //                   prefetch (shapes the large-tile kernel does not take).
 //   decode kernel : M <= 16: activations staged once per block in LDS, the weight streamed once straight
@@ -13,8 +14,7 @@
 //   skinny kernel : 16 < M <= 32 (and M <= 16 shapes the decode kernel does not take): as above with the
 //                   activations read from L2 per MFMA.
 //   general kernel: any shape, one output per thread.
-#include <queue>
-#include <vector>
+#include <map>
 #include "amct_common.h"
 
 namespace amct {
@@ -177,23 +177,19 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2, 2))) 
 }
 
 // ---------------------------------------------------------------------------
-// large-tile kernel: 256x256 block tile, 8 waves (2 x 4) of 128x64, BK = 64 bytes, four LDS stages
-// filled by direct global->LDS loads (global_load_lds_dwordx4: no VGPR staging, no ds_write), three
-// K-steps of loads in flight behind the MFMAs, one barrier per K-step, epilogue transposed through LDS
-// so that every lane stores 16 contiguous bytes.
+// large-tile kernel: 256x256 (or 256x192) block tile, 8 waves, LDS stages of 128 (or 64) bytes of K filled by
+// direct global->LDS loads (global_load_lds_dwordx4: no VGPR staging, no ds_write), one barrier per stage,
+// epilogue transposed through LDS so that every lane stores 16 contiguous bytes.
 //
-// A direct-to-LDS load writes the 64 lanes' 16-byte pieces to 1024 contiguous LDS bytes, so the LDS
-// layout is unpadded [row][64 B]; bank conflicts are avoided by a swizzle instead: 16-byte chunk c of
-// row r lives at chunk position c ^ ((r >> 2) & 3) (measured conflict-free with SQ_LDS_BANK_CONFLICT), applied by choosing which global chunk a lane
-// fetches.  The loads and their s_waitcnt are inline asm: the compiler would otherwise wait for ALL
-// outstanding direct-to-LDS loads before every LDS read.
+// A direct-to-LDS load writes the 64 lanes' 16-byte pieces to 1024 contiguous LDS bytes, so the LDS layout is
+// unpadded [row][LK bytes]; bank conflicts are avoided by a swizzle instead (measured conflict-free with
+// SQ_LDS_BANK_CONFLICT), applied by choosing which global chunk a lane fetches.  The loads and their s_waitcnt
+// are inline asm: the compiler would otherwise wait for ALL outstanding direct-to-LDS loads before every LDS read.
 // ---------------------------------------------------------------------------
-constexpr int kLK = 64;
+constexpr int kLK = 64;                                             // smallest K granule of the large-tile kernel
 
-AMCT_DEV void dma16(uint32_t lds_addr, const void* gptr) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(gptr) : "memory");
-}
-// the same with a wave-uniform 64-bit base in SGPRs and a 32-bit byte offset per lane: no vector ALU work per load
+// one direct-to-LDS load: a wave-uniform 64-bit base in SGPRs and a 32-bit byte offset per lane (no vector ALU
+// work per load); lane l's 16 bytes land at lds_addr + 16 * l
 AMCT_DEV void dma16s(uint32_t lds_addr, const void* sbase, uint32_t voff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
 }
@@ -206,12 +202,13 @@ struct DmaTile {
     static constexpr int kLM = 32 * TI * WM, kLN = 32 * TJ * WN, kWaves = WM * WN;
     static constexpr int kLStageBytes = (kLM + kLN) * LK;
     static constexpr int kRP = 1024 / LK;                          // rows per 1 KiB piece
-    static constexpr int kNA = kLM / kRP / kWaves;                 // A pieces per wave and stage
-    static constexpr int kNB = (kLN / kRP + kWaves - 1) / kWaves;  // B pieces per wave (the last ones may repeat)
+    static constexpr int kLW = kWaves / 2;                         // waves that issue the direct-to-LDS loads
+    static constexpr int kNA = kLM / kRP / kLW;                    // A pieces per loading wave and stage
+    static constexpr int kNB = (kLN / kRP + kLW - 1) / kLW;        // B pieces per loading wave (the last ones may repeat)
     static constexpr int kPPW = kNA + kNB;
     static constexpr int kEpiBytes = kWaves * 16384;
     static constexpr int kSmem = STAGES * kLStageBytes > kEpiBytes ? STAGES * kLStageBytes : kEpiBytes;
-    static_assert((kLM / kRP) % kWaves == 0, "the A pieces must divide evenly among the waves");
+    static_assert((kLM / kRP) % kLW == 0, "the A pieces must divide evenly among the loading waves");
     static_assert(kSmem <= 160 * 1024, "LDS");
 };
 
@@ -219,7 +216,7 @@ template <int ODT, int WM, int WN, int TI, int TJ, int STAGES, int LK>
 AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, const int64_t n0) {
     using Sh = DmaTile<WM, WN, TI, TJ, STAGES, LK>;
     constexpr int kLM = Sh::kLM, kLN = Sh::kLN, kRP = Sh::kRP, kNA = Sh::kNA, kNB = Sh::kNB, kPPW = Sh::kPPW;
-    constexpr int kLStageBytes = Sh::kLStageBytes;
+    constexpr int kLStageBytes = Sh::kLStageBytes, kWaves = Sh::kWaves, kLW = Sh::kLW;
     constexpr int kCH = LK / 16;                                    // 16-byte chunks per row
     constexpr int kKS = LK / 32;                                    // MFMA k-slices per stage
     static_assert(LK == 64 || LK == 128, "row length");
@@ -237,6 +234,8 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
     // this wave's 1 KiB pieces of a stage: kNA pieces of A rows, then kNB pieces of B rows.  A load is addressed
     // as (operand base + LK * step) in SGPRs plus a constant 32-bit byte offset per lane and piece (the host
     // admits only operands below 4 GiB to this kernel).
+    const bool loader = wave >= kWaves - kLW;                       // the last kLW waves: one per SIMD when kLW = 4
+    const int lw = loader ? wave - (kWaves - kLW) : 0;
     uint32_t goff[kPPW];
     {
         const int rin = lane / kCH;                                 // row inside the piece
@@ -246,11 +245,11 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
             int64_t r;
             int lr;                                                 // row inside the operand's LDS tile
             if (j < kNA) {
-                lr = (wave * kNA + j) * kRP + rin;
+                lr = (lw * kNA + j) * kRP + rin;
                 r = m0 + lr < a.M ? m0 + lr : a.M - 1;
             } else {
                 // a wave beyond the last piece fetches the last piece again: same bytes to the same place
-                const int pb = wave * kNB + (j - kNA) < kLN / kRP ? wave * kNB + (j - kNA) : kLN / kRP - 1;
+                const int pb = lw * kNB + (j - kNA) < kLN / kRP ? lw * kNB + (j - kNA) : kLN / kRP - 1;
                 lr = pb * kRP + rin;
                 r = n0 + lr < a.N ? n0 + lr : a.N - 1;
             }
@@ -259,15 +258,17 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
     }
     auto dma_one = [&](int stg, int step, int j) {
         if (j < kNA) {
-            dma16s(lds0 + stg * kLStageBytes + (wave * kNA + j) * 1024, a.xq + (int64_t)step * LK, goff[j]);
+            dma16s(lds0 + stg * kLStageBytes + (lw * kNA + j) * 1024, a.xq + (int64_t)step * LK, goff[j]);
         } else {
-            const int pb = wave * kNB + (j - kNA) < kLN / kRP ? wave * kNB + (j - kNA) : kLN / kRP - 1;
+            const int pb = lw * kNB + (j - kNA) < kLN / kRP ? lw * kNB + (j - kNA) : kLN / kRP - 1;
             dma16s(lds0 + stg * kLStageBytes + kLM * LK + pb * 1024, a.wq + (int64_t)step * LK, goff[j]);
         }
     };
     auto dma_stage = [&](int stage, int step) {
+        if (loader) {
 #pragma unroll
-        for (int j = 0; j < kPPW; ++j) dma_one(stage, step, j);
+            for (int j = 0; j < kPPW; ++j) dma_one(stage, step, j);
+        }
     };
 
     // fragment offsets of k-slice ks: lane reads row (tile base + lane%32), logical chunk 2*ks + lane/32
@@ -295,14 +296,17 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
     // slice are read from LDS.  Before the last slice of a stage the waves meet: every wave then holds that
     // slice's fragments in registers (lgkmcnt(0)), so the stage is free for the loads of step s + STAGES, and
     // the loads of step s + 1 have landed (those of the STAGES-2 steps after it stay in flight).
-    // The issue order is pinned instruction by instruction (a scheduling barrier after each): memory
-    // instructions in the shadow of the MFMAs, the MFMAs of the slices before the barrier issued BEFORE the
-    // wait, the first MFMA of the last slice right after it.  Left alone, the optimiser moves MFMAs behind the
+    // The direct-to-LDS loads of a step are issued by half of the waves (the last WM*WN/2, one per SIMD with
+    // the usual round-robin placement) in one burst right after the barrier: a wave stalls at such a load while
+    // the memory pipeline is busy, and the other wave of its SIMD keeps the matrix pipe fed meanwhile (3 %
+    // faster than every wave issuing its share between its MFMAs).
+    // The issue order is pinned instruction by instruction (a scheduling barrier after each): fragment reads
+    // in the shadow of the MFMAs, the MFMAs of the slices before the barrier issued BEFORE the wait, the first
+    // MFMA of the last slice right after the barrier (and the loads).  Left alone, the optimiser moves MFMAs behind the
     // barrier (the matrix pipe then idles while the waves meet) and, with a conditional read at the end of the
     // loop, waits for the youngest LDS reads too early.  The loop is therefore branch-free: the last iteration
     // reads one stage too far (valid LDS, values unused).
     constexpr int kNM = TI * TJ, kNR = TI + TJ;
-    constexpr int kDPM = (kPPW + kNM - 1) / kNM;                    // loads issued behind each MFMA of the last slice
     static_assert(kNM >= kNR, "one fragment read per MFMA");
     // fragment q in the order the MFMAs need them: A0, B0, B1, .., A1, A2, ..
     auto read_one = [&](int stg, int ks, int q, v4i (&fa)[TI], v4i (&fb)[TJ]) {
@@ -343,17 +347,12 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
+        dma_stage(stage, refill);                                   // loading waves only
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int m = 0; m < kNM; ++m) {
             mfma_one(m, fa[(kKS - 1) & 1], fb[(kKS - 1) & 1]);
             __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int j = kDPM * m; j < kDPM * (m + 1); ++j) {
-                if (j < kPPW) {
-                    dma_one(stage, refill, j);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            }
             if (m < kNR) {
                 read_one(next, 0, m, fa[0], fb[0]);
                 __builtin_amdgcn_sched_barrier(0);
@@ -742,26 +741,29 @@ __global__ __launch_bounds__(kBlock) void w8a8_general(W8A8Args a) {
 
 // Finish time, in quarters of a 256x256 tile, of `big` blocks of cost 4 followed by `small` blocks of cost 3
 // handed in that order to `cus` CUs holding one block each (the hardware gives the next block to the first
-// CU that becomes free).
+// CU that becomes free).  CUs that become free at the same time are handled together, so the cost is a few
+// map operations per round of blocks, not per block.
 static int64_t mix_makespan(int64_t big, int64_t small, int cus) {
-    std::priority_queue<int64_t, std::vector<int64_t>, std::greater<int64_t>> busy;
-    int64_t end = 0;
-    for (int64_t t = 0; t < big + small; ++t) {
-        int64_t start = 0;
-        if ((int64_t)busy.size() >= cus) {
-            start = busy.top();
-            busy.pop();
-        }
-        const int64_t done = start + (t < big ? 4 : 3);
-        busy.push(done);
-        if (done > end) end = done;
+    std::map<int64_t, int64_t> free_at;                            // time -> number of CUs free from then on
+    const int64_t q = big / cus, rem = big % cus;
+    free_at[4 * q] = cus - rem;
+    if (rem) free_at[4 * (q + 1)] = rem;
+    int64_t end = big ? (rem ? 4 * (q + 1) : 4 * q) : 0;
+    while (small > 0) {
+        const auto it = free_at.begin();
+        const int64_t t = it->first, n = it->second < small ? it->second : small;
+        if (n == it->second) free_at.erase(it);
+        else it->second -= n;
+        free_at[t + 3] += n;
+        if (t + 3 > end) end = t + 3;
+        small -= n;
     }
     return end;
 }
 
 // Split of the N columns into 256-wide and 192-wide column tiles that finishes first; nbig = -1 when plain
 // 256x256 tiles are as good (or the launch is so large that its last round does not matter).
-static MixPlan plan_mix(int64_t M, int64_t N, int cus) {
+static MixPlan plan_mix_search(int64_t M, int64_t N, int cus) {
     MixPlan best{(int)((M + 255) / 256), -1, 0, 0};
     const int64_t mt = best.mtiles;
     const int64_t uniform_tiles = mt * ((N + 255) / 256);
@@ -779,6 +781,17 @@ static MixPlan plan_mix(int64_t M, int64_t N, int cus) {
     }
     return best;
 }
+
+static MixPlan plan_mix(int64_t M, int64_t N, int cus) {
+    // the last answer is kept per host thread: a layer is called with the same shape again and again
+    struct Last { int64_t M, N; int cus; MixPlan plan; };
+    static thread_local Last last_plan{-1, -1, -1, {}};
+    if (last_plan.M == M && last_plan.N == N && last_plan.cus == cus) return last_plan.plan;
+    const MixPlan fresh = plan_mix_search(M, N, cus);
+    last_plan = Last{M, N, cus, fresh};
+    return fresh;
+}
+
 
 }  // namespace amct
 
@@ -828,10 +841,9 @@ extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s
             cus = 0;
         }
         const MixPlan plan = plan_mix(M, N, cus);
-#ifndef AMCT_LK128
-#define AMCT_LK128 1
-#endif
-        const bool wide = AMCT_LK128 && K % 128 == 0;                // 128-byte rows, 2 stages; else 64-byte rows, 4 stages
+        // 128-byte LDS rows and 2 stages when K allows (whole cache lines per load, one barrier per 128 bytes of K:
+        // 7 % faster), else 64-byte rows and 4 stages
+        const bool wide = K % 128 == 0;
 #define AMCT_LAUNCH_DMA(ODT)                                                                                        \
     {                                                                                                               \
         if (plan.nbig >= 0) {                                                                                       \
