@@ -246,8 +246,9 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
     u4v mreg[4];
     auto issue = [&](int slot, int stage, int step) {              // the loads of K-step `step`
         const int st = step < last ? step : last;
-        const int64_t k = (int64_t)st * kQK;
-        const int64_t gi = (k + bhalf * 16) / a.group;
+        const uint32_t k = (uint32_t)st * kQK;
+        // k / group without a division (k, group < 2^16); group % 32 == 0 keeps both halves of a step in one group
+        const uint32_t gi = __umulhi(k, a.group_magic);
         gload8(wreg[slot], wp + k / 2);
         gload_u16(sreg[slot], sp + gi * sbytes);
         gload_u8(zreg[slot], zp + gi);
@@ -409,6 +410,244 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
             const uint4 v = *reinterpret_cast<const uint4*>(patch + prow * kPatchRow + chunk * 16);
             const int64_t m = mbase + prow;
             const int64_t n = n0 + wn * 64 + chunk * 8;
+            if (m < a.M && n < a.N) stg16_nt(reinterpret_cast<char*>(a.out) + (m * a.N + n) * 2, v);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// wide large-tile kernel (K % 128 == 0, group % 64 == 0, activations already smoothed): 256x256 block tile,
+// 8 waves (2 x 4) of 128x64, two LDS stages of 64 elements of K (128-byte rows: a direct-to-LDS load covers
+// whole cache lines, one barrier per 64 elements).
+//   activations : direct global->LDS loads issued by waves 4..7 (one per SIMD) in one burst right after the
+//                 barrier that frees the stage; a wave stalls at such a load while the memory pipeline is busy
+//                 and the other wave of its SIMD keeps the matrix pipe fed meanwhile;
+//   weights     : 16 bytes (32 nibbles) per thread and step into registers two steps ahead, with the scale and
+//                 zero-point of their group; dequantised in the shadow of the MFMAs of the first two k-slices
+//                 of the step before and written to the other LDS stage in MFMA operand order.
+// The issue order is pinned: sched_group_barrier interleaves MFMA / VALU / LDS inside a k-slice, scheduling
+// barriers separate the slices, and the MFMAs of the slices before the barrier are issued BEFORE the wait
+// (left alone, the optimiser moves them behind the barrier and the matrix pipe idles while the waves meet).
+// All global loads and their s_waitcnt are inline asm with SGPR bases and constant 32-bit lane offsets; the
+// counter retires in order and every iteration issues the same number of operations per wave.
+// LDS layout: unpadded [row][128 B], 16-byte chunk c of row r at c ^ ((r >> 1) & 7).
+// ---------------------------------------------------------------------------
+constexpr int kWK = 64;                                            // elements of K per stage
+constexpr int kWRow = 128;                                         // bytes per LDS row
+constexpr int kWStageBytes = (kQM + kQN) * kWRow;                  // 64 KiB
+constexpr int kWNA = (kQM * kWRow / 1024) / 4;                     // activation pieces per loading wave: 8
+
+AMCT_DEV void dma16s(uint32_t lds_addr, const void* sbase, uint32_t voff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
+AMCT_DEV void gload16s(u4v& dst, const void* sbase, uint32_t voff) {
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(dst) : "v"(voff), "s"(sbase) : "memory");
+}
+AMCT_DEV void gload_u16s(uint32_t& dst, const void* sbase, uint32_t voff) {
+    asm volatile("global_load_ushort %0, %1, %2" : "=v"(dst) : "v"(voff), "s"(sbase) : "memory");
+}
+AMCT_DEV void gload_u8s(uint32_t& dst, const void* sbase, uint32_t voff) {
+    asm volatile("global_load_ubyte %0, %1, %2" : "=v"(dst) : "v"(voff), "s"(sbase) : "memory");
+}
+
+template <bool SF16>
+__global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void w4a16_tile_wide(W4A16Args a) {
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[2 * kWStageBytes];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 2, wn = wave & 3;
+    const int64_t m0 = (int64_t)blockIdx.y * kQM, n0 = (int64_t)blockIdx.x * kQN;
+    const int nsteps = (int)(a.K / kWK);
+    const int last = nsteps - 1;
+    const uint32_t G = (uint32_t)(a.K / a.group);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
+    auto swz = [](int r) { return (r >> 1) & 7; };
+
+    // activation pieces (8 rows x 128 B) of the loading waves
+    const bool loader = wave >= 4;
+    const int lw = loader ? wave - 4 : 0;
+    uint32_t goff[kWNA];
+    {
+        const int rin = lane >> 3, pc = lane & 7;
+#pragma unroll
+        for (int j = 0; j < kWNA; ++j) {
+            const int lr = (lw * kWNA + j) * 8 + rin;
+            const int64_t r = m0 + lr < a.M ? m0 + lr : a.M - 1;
+            goff[j] = (uint32_t)((r * a.K + (pc ^ swz(lr)) * 8) * 2);
+        }
+    }
+    auto dma_a = [&](int stg, int step) {
+        if (loader) {
+            const int st = step < last ? step : last;
+#pragma unroll
+            for (int j = 0; j < kWNA; ++j)
+                dma16s(lds0 + stg * kWStageBytes + (lw * kWNA + j) * 1024, a.x + (int64_t)st * kWK, goff[j]);
+        }
+    };
+    // weight row of this thread: row tid/2, 32 weights (16 bytes) per step, which half from tid%2
+    const int brow = tid >> 1, bhalf = tid & 1;
+    const int64_t wrow = (n0 + brow < a.N) ? n0 + brow : a.N - 1;
+    const uint32_t woff = (uint32_t)(wrow * (a.K / 2) + bhalf * 16);
+    const uint32_t soff = (uint32_t)(wrow * G * 2), zoff = (uint32_t)(wrow * G);
+    int bdst[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) bdst[c] = kQM * kWRow + brow * kWRow + ((4 * bhalf + c) ^ swz(brow)) * 16;
+
+    u4v wreg[2];
+    uint32_t sreg[2], zreg[2];
+    auto issue_b = [&](int slot, int step) {                       // the weight loads of K-step `step`
+        const int st = step < last ? step : last;
+        const uint32_t k = (uint32_t)st * kWK;
+        const uint32_t gi = __umulhi(k, a.group_magic);             // k / group (k, group < 2^16); group % 64 == 0
+        gload16s(wreg[slot], a.wq + k / 2, woff);
+        gload_u16s(sreg[slot], reinterpret_cast<const uint8_t*>(a.scales) + gi * 2, soff);
+        gload_u8s(zreg[slot], a.zeros + gi, zoff);
+    };
+    float sc = 0.f, nzs = 0.f;
+    auto factors = [&](int slot) {
+        sc = SF16 ? f16_bits_to_f32(sreg[slot]) : bf16_bits_to_f32(sreg[slot]);
+        nzs = -((float)zreg[slot] * sc);
+    };
+    auto write_b = [&](int slot, int stg, int c) {                 // dequantise 8 weights into LDS
+        *reinterpret_cast<uint4*>(smem + stg * kWStageBytes + bdst[c]) = dequant8(wreg[slot][c], sc, nzs);
+    };
+    // wait for every outstanding load and LDS operation of this wave; the slot's registers are tied to the
+    // statement so that their uses stay behind it
+#define AMCT_WAIT_ALL(slot) \
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : "+v"(wreg[slot]), "+v"(sreg[slot]), "+v"(zreg[slot]) : : "memory")
+
+    int offA[4], offB[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+        const int r = lane & 31;
+        const int phys = (ks * 2 + (lane >> 5)) ^ swz(r);
+        offA[ks] = (wm * 128 + r) * kWRow + phys * 16;
+        offB[ks] = kQM * kWRow + (wn * 64 + r) * kWRow + phys * 16;
+    }
+    v16f acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    // fragment q in the order the MFMAs need them: A0, B0, B1, A1, A2, A3
+    auto read_one = [&](int stg, int ks, int q, v8bf (&fa)[4], v8bf (&fb)[2]) {
+        const uint8_t* st = smem + stg * kWStageBytes;
+        if (q == 0) fa[0] = *reinterpret_cast<const v8bf*>(st + offA[ks]);
+        else if (q <= 2) fb[q - 1] = *reinterpret_cast<const v8bf*>(st + offB[ks] + (q - 1) * 32 * kWRow);
+        else fa[q - 2] = *reinterpret_cast<const v8bf*>(st + offA[ks] + (q - 2) * 32 * kWRow);
+    };
+    auto mfma_one = [&](int m, const v8bf (&fa)[4], const v8bf (&fb)[2]) {
+        const int i = m >> 1, j = m & 1;
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    };
+
+    // prologue: A(0) and B(0) into stage 0, A(1) on its way to stage 1, B(1) and B(2) on their way to registers
+    v8bf fa[2][4], fb[2][2];
+    dma_a(0, 0);
+    issue_b(0, 0);
+    issue_b(1, 1);
+    AMCT_WAIT_ALL(0);
+    AMCT_WAIT_ALL(1);
+    factors(0);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) write_b(0, 0, c);
+    dma_a(1, 1);
+    issue_b(0, 2);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int q = 0; q < 6; ++q) read_one(0, 0, q, fa[0], fb[0]);
+
+    // iteration s (stage CUR = s % 2, NXT the other; slot NXT holds B(s+1), slot CUR holds B(s+2) in flight):
+    //   k-slices 0, 1 : MFMAs, fragment reads of the next slice, dequantisation of B(s+1) into stage NXT
+    //   k-slice 2     : MFMAs, fragment reads of slice 3
+    //   wait (A(s+1) and B(s+2) have landed: both were issued a whole iteration ago; own LDS operations done),
+    //   barrier: stage CUR is free, stage NXT complete
+    //   loads         : A(s+2) into stage CUR (loading waves), B(s+3) into slot NXT
+    //   k-slice 3     : MFMAs, fragment reads of slice 0 of stage NXT
+#define AMCT_WSLICE_DQ(CUR, NXT, KS)                                                   \
+    {                                                                                  \
+        __builtin_amdgcn_sched_barrier(0);                                             \
+        _Pragma("unroll") for (int m_ = 0; m_ < 8; ++m_) mfma_one(m_, fa[(KS) & 1], fb[(KS) & 1]); \
+        _Pragma("unroll") for (int q_ = 0; q_ < 6; ++q_) read_one(CUR, (KS) + 1, q_, fa[((KS) + 1) & 1], fb[((KS) + 1) & 1]); \
+        write_b(NXT, NXT, 2 * (KS));                                                   \
+        write_b(NXT, NXT, 2 * (KS) + 1);                                               \
+        _Pragma("unroll") for (int g_ = 0; g_ < 8; ++g_) {                             \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* 1 MFMA */            \
+            __builtin_amdgcn_sched_group_barrier(0x002, 7, 0); /* 7 VALU */            \
+            __builtin_amdgcn_sched_group_barrier(0x080, 1, 0); /* 1 DS      */         \
+        }                                                                              \
+        __builtin_amdgcn_sched_barrier(0);                                             \
+    }
+#define AMCT_WSLICE_PIN(STG, KSREAD, KS)                                               \
+    {                                                                                  \
+        _Pragma("unroll") for (int m_ = 0; m_ < 8; ++m_) {                             \
+            mfma_one(m_, fa[(KS) & 1], fb[(KS) & 1]);                                  \
+            __builtin_amdgcn_sched_barrier(0);                                         \
+            if (m_ < 6) {                                                              \
+                read_one(STG, KSREAD, m_, fa[((KS) + 1) & 1], fb[((KS) + 1) & 1]);     \
+                __builtin_amdgcn_sched_barrier(0);                                     \
+            }                                                                          \
+        }                                                                              \
+    }
+#define AMCT_WITER(CUR, NXT, step)                                                     \
+    {                                                                                  \
+        factors(NXT);                                                                  \
+        AMCT_WSLICE_DQ(CUR, NXT, 0)                                                    \
+        AMCT_WSLICE_DQ(CUR, NXT, 1)                                                    \
+        AMCT_WSLICE_PIN(CUR, 3, 2)                                                     \
+        AMCT_WAIT_ALL(CUR);                                                            \
+        __builtin_amdgcn_s_barrier();                                                  \
+        asm volatile("" ::: "memory");                                                 \
+        __builtin_amdgcn_sched_barrier(0);                                             \
+        dma_a(CUR, (step) + 2);                                                        \
+        issue_b(NXT, (step) + 3);                                                      \
+        __builtin_amdgcn_sched_barrier(0);                                             \
+        AMCT_WSLICE_PIN(NXT, 0, 3)                                                     \
+    }
+    for (int step = 0; step < nsteps; step += 2) {
+        AMCT_WITER(0, 1, step)
+        AMCT_WITER(1, 0, step + 1)
+    }
+#undef AMCT_WITER
+#undef AMCT_WSLICE_PIN
+#undef AMCT_WSLICE_DQ
+#undef AMCT_WAIT_ALL
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+
+    // epilogue: + bias (or + (-0.0f), which returns the value bit for bit), narrow to bf16, transpose through a
+    // per-wave LDS patch, 16-byte stores of full rows
+    constexpr int kPatchRow = 64 * 2 + 16;
+    uint8_t* patch = smem + wave * 16384;
+    float bs[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int64_t n = n0 + wn * 64 + j * 32 + (lane & 31);
+        bs[j] = a.bias ? a.bias[n < a.N ? n : a.N - 1] : -0.0f;
+    }
+    uint8_t* wbase = patch + 4 * (lane >> 5) * kPatchRow + (lane & 31) * 2;
+    const uint8_t* rbase = patch + (lane >> 3) * kPatchRow + (lane & 7) * 16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int64_t mbase = m0 + wm * 128 + i * 32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int prow0 = 8 * (r >> 2) + (r & 3);
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                *reinterpret_cast<uint16_t*>(wbase + prow0 * kPatchRow + j * 64) = (uint16_t)f32_to_bf16_bits(acc[i][j][r] + bs[j]);
+        }
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const uint4 v = *reinterpret_cast<const uint4*>(rbase + it * 8 * kPatchRow);
+            const int64_t m = mbase + it * 8 + (lane >> 3);
+            const int64_t n = n0 + wn * 64 + (lane & 7) * 8;
             if (m < a.M && n < a.N) stg16_nt(reinterpret_cast<char*>(a.out) + (m * a.N + n) * 2, v);
         }
     }
@@ -874,7 +1113,7 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
 #undef AMCT_DEC
         return hip_status();
     }
-    if (vec_ok && M >= 256 && K % 128 == 0 && N % 8 == 0 && group % 16 == 0 && aligned16(out)) {
+    if (vec_ok && M >= 256 && K % 128 == 0 && K < 65536 && N % 8 == 0 && aligned16(out)) {
         const dim3 grid((unsigned)((N + kQN - 1) / kQN), (unsigned)((M + kQM - 1) / kQM));
         if (grid.y > 65535) return AMCT_E_UNSUPPORTED;
         if (smooth && workspace && workspace_bytes >= (size_t)(M * K * 2) && aligned16(workspace)) {
@@ -887,7 +1126,12 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
             a.smooth = nullptr;
             smooth = nullptr;
         }
-        if (smooth) hipLaunchKernelGGL((w4a16_tile_dma<true>), grid, dim3(kQThreads), 0, st, a);
+        const int64_t G = K / group;
+        const bool wide = !smooth && group % 64 == 0 && M * K * 2 < (int64_t(1) << 32) && N * (K / 2) < (int64_t(1) << 32) &&
+                          N * G * 2 < (int64_t(1) << 32);
+        if (wide && scale_dtype == AMCT_F16) hipLaunchKernelGGL((w4a16_tile_wide<true>), grid, dim3(kQThreads), 0, st, a);
+        else if (wide) hipLaunchKernelGGL((w4a16_tile_wide<false>), grid, dim3(kQThreads), 0, st, a);
+        else if (smooth) hipLaunchKernelGGL((w4a16_tile_dma<true>), grid, dim3(kQThreads), 0, st, a);
         else hipLaunchKernelGGL((w4a16_tile_dma<false>), grid, dim3(kQThreads), 0, st, a);
         return hip_status();
     }
