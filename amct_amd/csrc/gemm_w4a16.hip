@@ -450,13 +450,16 @@ AMCT_DEV void gload_u8s(uint32_t& dst, const void* sbase, uint32_t voff) {
     asm volatile("global_load_ubyte %0, %1, %2" : "=v"(dst) : "v"(voff), "s"(sbase) : "memory");
 }
 
-template <bool SF16>
-__global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void w4a16_tile_wide(W4A16Args a) {
-    __shared__ __attribute__((aligned(1024))) uint8_t smem[2 * kWStageBytes];
+// WM x WN = 8 waves of (32*TI) x (32*TJ); used as 2 x 4 waves of 128 x 64 for the 256x256 tile.  (4 x 2 waves of
+// 64 x 96 give a 256x192 tile in the same 64 KiB stage, every wave still dequantising its 32 weight rows.)
+template <bool SF16, int WM, int WN, int TI, int TJ>
+AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m0, const int64_t n0) {
+    static_assert(WM * WN == 8 && 32 * TI * WM == kQM && 32 * TJ * WN <= kQN, "tile shape");
+    constexpr int kNM = TI * TJ, kNR = TI + TJ;                    // MFMAs and fragment reads per k-slice
+    static_assert(kNM >= kNR, "one fragment read per MFMA");
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 2, wn = wave & 3;
-    const int64_t m0 = (int64_t)blockIdx.y * kQM, n0 = (int64_t)blockIdx.x * kQN;
+    const int wm = wave / WN, wn = wave % WN;
     const int nsteps = (int)(a.K / kWK);
     const int last = nsteps - 1;
     const uint32_t G = (uint32_t)(a.K / a.group);
@@ -521,31 +524,31 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
     for (int ks = 0; ks < 4; ++ks) {
         const int r = lane & 31;
         const int phys = (ks * 2 + (lane >> 5)) ^ swz(r);
-        offA[ks] = (wm * 128 + r) * kWRow + phys * 16;
-        offB[ks] = kQM * kWRow + (wn * 64 + r) * kWRow + phys * 16;
+        offA[ks] = (wm * 32 * TI + r) * kWRow + phys * 16;
+        offB[ks] = kQM * kWRow + (wn * 32 * TJ + r) * kWRow + phys * 16;
     }
-    v16f acc[4][2];
+    v16f acc[TI][TJ];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TI; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TJ; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    // fragment q in the order the MFMAs need them: A0, B0, B1, A1, A2, A3
-    auto read_one = [&](int stg, int ks, int q, v8bf (&fa)[4], v8bf (&fb)[2]) {
+    // fragment q in the order the MFMAs need them: A0, B0, B1, .., A1, A2, ..
+    auto read_one = [&](int stg, int ks, int q, v8bf (&fa)[TI], v8bf (&fb)[TJ]) {
         const uint8_t* st = smem + stg * kWStageBytes;
         if (q == 0) fa[0] = *reinterpret_cast<const v8bf*>(st + offA[ks]);
-        else if (q <= 2) fb[q - 1] = *reinterpret_cast<const v8bf*>(st + offB[ks] + (q - 1) * 32 * kWRow);
-        else fa[q - 2] = *reinterpret_cast<const v8bf*>(st + offA[ks] + (q - 2) * 32 * kWRow);
+        else if (q <= TJ) fb[q - 1] = *reinterpret_cast<const v8bf*>(st + offB[ks] + (q - 1) * 32 * kWRow);
+        else fa[q - TJ] = *reinterpret_cast<const v8bf*>(st + offA[ks] + (q - TJ) * 32 * kWRow);
     };
-    auto mfma_one = [&](int m, const v8bf (&fa)[4], const v8bf (&fb)[2]) {
-        const int i = m >> 1, j = m & 1;
+    auto mfma_one = [&](int m, const v8bf (&fa)[TI], const v8bf (&fb)[TJ]) {
+        const int i = m / TJ, j = m % TJ;
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
     };
 
     // prologue: A(0) and B(0) into stage 0, A(1) on its way to stage 1, B(1) and B(2) on their way to registers
-    v8bf fa[2][4], fb[2][2];
+    v8bf fa[2][TI], fb[2][TJ];
     dma_a(0, 0);
     issue_b(0, 0);
     issue_b(1, 1);
@@ -560,7 +563,7 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 #pragma unroll
-    for (int q = 0; q < 6; ++q) read_one(0, 0, q, fa[0], fb[0]);
+    for (int q = 0; q < kNR; ++q) read_one(0, 0, q, fa[0], fb[0]);
 
     // iteration s (stage CUR = s % 2, NXT the other; slot NXT holds B(s+1), slot CUR holds B(s+2) in flight):
     //   k-slices 0, 1 : MFMAs, fragment reads of the next slice, dequantisation of B(s+1) into stage NXT
@@ -572,23 +575,23 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
 #define AMCT_WSLICE_DQ(CUR, NXT, KS)                                                   \
     {                                                                                  \
         __builtin_amdgcn_sched_barrier(0);                                             \
-        _Pragma("unroll") for (int m_ = 0; m_ < 8; ++m_) mfma_one(m_, fa[(KS) & 1], fb[(KS) & 1]); \
-        _Pragma("unroll") for (int q_ = 0; q_ < 6; ++q_) read_one(CUR, (KS) + 1, q_, fa[((KS) + 1) & 1], fb[((KS) + 1) & 1]); \
+        _Pragma("unroll") for (int m_ = 0; m_ < kNM; ++m_) mfma_one(m_, fa[(KS) & 1], fb[(KS) & 1]); \
+        _Pragma("unroll") for (int q_ = 0; q_ < kNR; ++q_) read_one(CUR, (KS) + 1, q_, fa[((KS) + 1) & 1], fb[((KS) + 1) & 1]); \
         write_b(NXT, NXT, 2 * (KS));                                                   \
         write_b(NXT, NXT, 2 * (KS) + 1);                                               \
-        _Pragma("unroll") for (int g_ = 0; g_ < 8; ++g_) {                             \
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* 1 MFMA */            \
-            __builtin_amdgcn_sched_group_barrier(0x002, 7, 0); /* 7 VALU */            \
-            __builtin_amdgcn_sched_group_barrier(0x080, 1, 0); /* 1 DS      */         \
+        _Pragma("unroll") for (int g_ = 0; g_ < kNM; ++g_) {                           \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                      /* 1 MFMA */ \
+            __builtin_amdgcn_sched_group_barrier(0x002, (56 + kNM - 1) / kNM, 0);   /* VALU   */ \
+            __builtin_amdgcn_sched_group_barrier(0x080, kNM >= kNR + 2 ? 1 : 2, 0); /* DS     */ \
         }                                                                              \
         __builtin_amdgcn_sched_barrier(0);                                             \
     }
 #define AMCT_WSLICE_PIN(STG, KSREAD, KS)                                               \
     {                                                                                  \
-        _Pragma("unroll") for (int m_ = 0; m_ < 8; ++m_) {                             \
+        _Pragma("unroll") for (int m_ = 0; m_ < kNM; ++m_) {                           \
             mfma_one(m_, fa[(KS) & 1], fb[(KS) & 1]);                                  \
             __builtin_amdgcn_sched_barrier(0);                                         \
-            if (m_ < 6) {                                                              \
+            if (m_ < kNR) {                                                              \
                 read_one(STG, KSREAD, m_, fa[((KS) + 1) & 1], fb[((KS) + 1) & 1]);     \
                 __builtin_amdgcn_sched_barrier(0);                                     \
             }                                                                          \
@@ -622,35 +625,45 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
     asm volatile("" ::: "memory");
 
     // epilogue: + bias (or + (-0.0f), which returns the value bit for bit), narrow to bf16, transpose through a
-    // per-wave LDS patch, 16-byte stores of full rows
-    constexpr int kPatchRow = 64 * 2 + 16;
+    // per-wave LDS patch of 32 rows x 32*TJ columns, 16-byte stores of full rows
+    constexpr int kPW = 32 * TJ;                                   // patch width in columns
+    constexpr int kPatchRow = kPW * 2 + 16;
+    constexpr int CPR = kPW * 2 / 16;                              // 16-byte chunks per patch row
+    static_assert(32 * kPatchRow <= 16384 && (32 * CPR) % 64 == 0, "patch");
     uint8_t* patch = smem + wave * 16384;
-    float bs[2];
+    float bs[TJ];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int64_t n = n0 + wn * 64 + j * 32 + (lane & 31);
+    for (int j = 0; j < TJ; ++j) {
+        const int64_t n = n0 + wn * kPW + j * 32 + (lane & 31);
         bs[j] = a.bias ? a.bias[n < a.N ? n : a.N - 1] : -0.0f;
     }
     uint8_t* wbase = patch + 4 * (lane >> 5) * kPatchRow + (lane & 31) * 2;
-    const uint8_t* rbase = patch + (lane >> 3) * kPatchRow + (lane & 7) * 16;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int64_t mbase = m0 + wm * 128 + i * 32;
+    for (int i = 0; i < TI; ++i) {
+        const int64_t mbase = m0 + wm * 32 * TI + i * 32;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int prow0 = 8 * (r >> 2) + (r & 3);
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < TJ; ++j)
                 *reinterpret_cast<uint16_t*>(wbase + prow0 * kPatchRow + j * 64) = (uint16_t)f32_to_bf16_bits(acc[i][j][r] + bs[j]);
         }
 #pragma unroll
-        for (int it = 0; it < 4; ++it) {
-            const uint4 v = *reinterpret_cast<const uint4*>(rbase + it * 8 * kPatchRow);
-            const int64_t m = mbase + it * 8 + (lane >> 3);
-            const int64_t n = n0 + wn * 64 + (lane & 7) * 8;
+        for (int it = 0; it < 32 * CPR / 64; ++it) {
+            const int idx = it * 64 + lane;                        // 16-byte chunk of the patch, row-major
+            const int prow = idx / CPR, chunk = idx % CPR;
+            const uint4 v = *reinterpret_cast<const uint4*>(patch + prow * kPatchRow + chunk * 16);
+            const int64_t m = mbase + prow;
+            const int64_t n = n0 + wn * kPW + chunk * 8;
             if (m < a.M && n < a.N) stg16_nt(reinterpret_cast<char*>(a.out) + (m * a.N + n) * 2, v);
         }
     }
+}
+
+template <bool SF16>
+__global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void w4a16_tile_wide(W4A16Args a) {
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[2 * kWStageBytes];
+    w4a16_wide_body<SF16, 2, 4, 4, 2>(a, smem, (int64_t)blockIdx.y * kQM, (int64_t)blockIdx.x * kQN);
 }
 
 // x' = bf16(x * smooth[k]) over the whole activation matrix (K % 8 == 0): used when the caller lends a
@@ -1129,6 +1142,8 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
         const int64_t G = K / group;
         const bool wide = !smooth && group % 64 == 0 && M * K * 2 < (int64_t(1) << 32) && N * (K / 2) < (int64_t(1) << 32) &&
                           N * G * 2 < (int64_t(1) << 32);
+        // (mixing in 256x192 blocks as the W8A8 launch does was measured neutral here: the narrow tile dequantises
+        // as many weights as the full one)
         if (wide && scale_dtype == AMCT_F16) hipLaunchKernelGGL((w4a16_tile_wide<true>), grid, dim3(kQThreads), 0, st, a);
         else if (wide) hipLaunchKernelGGL((w4a16_tile_wide<false>), grid, dim3(kQThreads), 0, st, a);
         else if (smooth) hipLaunchKernelGGL((w4a16_tile_dma<true>), grid, dim3(kQThreads), 0, st, a);

@@ -14,8 +14,8 @@
 //   skinny kernel : 16 < M <= 32 (and M <= 16 shapes the decode kernel does not take): as above with the
 //                   activations read from L2 per MFMA.
 //   general kernel: any shape, one output per thread.
-#include <map>
 #include "amct_common.h"
+#include "gemm_plan.h"
 
 namespace amct {
 
@@ -461,17 +461,6 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2,
     w8a8_dma_body<ODT, WM, WN, 4, 2, STAGES, LK>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
 }
 
-// One launch, two block shapes: the first `big` blocks compute 256x256 tiles of the first `nbig` column tiles,
-// the rest 256x192 tiles of the columns after them.  The host picks the split so that the blocks fill the
-// CUs evenly (a 256x192 tile costs 3/4 of a 256x256 one): with uniform tiles the last round of a launch
-// leaves CUs idle, e.g. 448 tiles on 256 CUs take two rounds for 1.75 rounds of work.
-struct MixPlan {
-    int mtiles;                                                     // row tiles (256 rows each)
-    int nbig;                                                       // 256-column tiles, columns [0, 256*nbig)
-    int big;                                                        // mtiles * nbig
-    int nsmall;                                                     // 192-column tiles after them
-};
-
 template <int ODT, int STAGES, int LK>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void w8a8_tile_mix(W8A8Args a, MixPlan p) {
     using Big = DmaTile<2, 4, 4, 2, STAGES, LK>;
@@ -739,60 +728,6 @@ __global__ __launch_bounds__(kBlock) void w8a8_general(W8A8Args a) {
     w8a8_epilogue(a, m, n, acc);
 }
 
-// Finish time, in quarters of a 256x256 tile, of `big` blocks of cost 4 followed by `small` blocks of cost 3
-// handed in that order to `cus` CUs holding one block each (the hardware gives the next block to the first
-// CU that becomes free).  CUs that become free at the same time are handled together, so the cost is a few
-// map operations per round of blocks, not per block.
-static int64_t mix_makespan(int64_t big, int64_t small, int cus) {
-    std::map<int64_t, int64_t> free_at;                            // time -> number of CUs free from then on
-    const int64_t q = big / cus, rem = big % cus;
-    free_at[4 * q] = cus - rem;
-    if (rem) free_at[4 * (q + 1)] = rem;
-    int64_t end = big ? (rem ? 4 * (q + 1) : 4 * q) : 0;
-    while (small > 0) {
-        const auto it = free_at.begin();
-        const int64_t t = it->first, n = it->second < small ? it->second : small;
-        if (n == it->second) free_at.erase(it);
-        else it->second -= n;
-        free_at[t + 3] += n;
-        if (t + 3 > end) end = t + 3;
-        small -= n;
-    }
-    return end;
-}
-
-// Split of the N columns into 256-wide and 192-wide column tiles that finishes first; nbig = -1 when plain
-// 256x256 tiles are as good (or the launch is so large that its last round does not matter).
-static MixPlan plan_mix_search(int64_t M, int64_t N, int cus) {
-    MixPlan best{(int)((M + 255) / 256), -1, 0, 0};
-    const int64_t mt = best.mtiles;
-    const int64_t uniform_tiles = mt * ((N + 255) / 256);
-    if (cus <= 0 || uniform_tiles > 16 * (int64_t)cus) return best;
-    int64_t best_t = mix_makespan(uniform_tiles, 0, cus);
-    for (int64_t nb = (N + 255) / 256 - 1; nb >= 0; --nb) {         // nb big column tiles, the rest 192 wide
-        const int64_t ns = (N - 256 * nb + 191) / 192;
-        const int64_t t = mix_makespan(mt * nb, mt * ns, cus);
-        if (t < best_t) {
-            best_t = t;
-            best.nbig = (int)nb;
-            best.big = (int)(mt * nb);
-            best.nsmall = (int)ns;
-        }
-    }
-    return best;
-}
-
-static MixPlan plan_mix(int64_t M, int64_t N, int cus) {
-    // the last answer is kept per host thread: a layer is called with the same shape again and again
-    struct Last { int64_t M, N; int cus; MixPlan plan; };
-    static thread_local Last last_plan{-1, -1, -1, {}};
-    if (last_plan.M == M && last_plan.N == N && last_plan.cus == cus) return last_plan.plan;
-    const MixPlan fresh = plan_mix_search(M, N, cus);
-    last_plan = Last{M, N, cus, fresh};
-    return fresh;
-}
-
-
 }  // namespace amct
 
 using namespace amct;
@@ -834,12 +769,7 @@ extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s
         // the traffic from L2 into LDS matters more than decoupling the barriers)
         const dim3 grid((unsigned)((N + 255) / 256), (unsigned)((M + 255) / 256));
         if (grid.y > 65535) return AMCT_E_UNSUPPORTED;
-        int dev = 0, cus = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
-            (void)hipGetLastError();
-            cus = 0;
-        }
+        const int cus = current_cu_count();
         const MixPlan plan = plan_mix(M, N, cus);
         // 128-byte LDS rows and 2 stages when K allows (whole cache lines per load, one barrier per 128 bytes of K:
         // 7 % faster), else 64-byte rows and 4 stages

@@ -97,6 +97,19 @@ def w4a16_oracle(x, codes, scales, zeros, group, smooth, bias):
     return od.w4a16_forward_f64(x, signed, scales, anti, group, bias, None if smooth is None else smooth.reshape(1, -1))
 
 
+@pytest.mark.parametrize("M,N,K,group", [(300, 1000, 256, 64), (256, 448, 128, 128), (2048, 14336, 256, 128), (2000, 14328, 128, 64)])
+def test_w4a16_large_shapes_ragged(dev, M, N, K, group):
+    """The wide large-tile kernel (M >= 256, group % 64 == 0) on ragged edges in M and N, both scale dtypes."""
+    for sdt in (torch.float16, torch.bfloat16):
+        x, codes, scales, zeros, smooth, bias = w4a16_case(M, N, K, group, 137, sdt)
+        packed = workloads.pack_nibbles(codes)
+        out = ops.gemm_w4a16(x.to(dev), packed.to(dev), scales.to(dev), zeros.to(dev), group, None, bias.to(dev))
+        want = w4a16_oracle(x, codes, scales, zeros, group, None, bias)
+        err = (out.cpu().double() - want).abs()
+        tol = 1e-3 * want.abs().amax(dim=1, keepdim=True) + want.abs() * 2.0 ** -8
+        assert (err <= tol).all(), (err.max().item(), tol.min().item())
+
+
 @pytest.mark.parametrize("M,N,K,group", [(1, 64, 256, 128), (16, 128, 512, 128), (7, 33, 128, 32), (64, 64, 256, 64),
                                          (130, 200, 384, 128), (256, 256, 1024, 128), (2048, 128, 4096, 128),
                                          (16, 136, 4096, 128), (3, 72, 1024, 256), (20, 64, 768, 128),
