@@ -25,6 +25,7 @@ SIGNATURES = {
     "amct_hip_version": (_I, []),
     "amct_hip_strerror": (ctypes.c_char_p, [_I]),
     "amct_copy_bytes": (_I, [_P, _P, _L, _P]),
+    "amct_mfma_yardstick": (_I, [_I, _I, _I, _P, _P, _P]),
     "amct_minmax": (_I, [_P, _P, _P, _L, _L, _I, _I, _P]),
     "amct_gptq_block": (_I, [_P, _L, _P, _L, _P, _L, _P, _P, _L, _P, _L, _I, _I, _I, _P]),
     "amct_fp8_block_dequant": (_I, [_P, _P, _P, _L, _L, _I, _I, _P]),

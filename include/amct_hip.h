@@ -77,6 +77,13 @@ const char* amct_hip_strerror(int code);
  * the yardstick for the bandwidth figures and for scaling hardware traffic counters. */
 int amct_copy_bytes(const void* src, void* dst, int64_t nbytes, amct_stream_t stream);
 
+/* Register-only MFMA loop on every CU (8 waves per CU, no memory traffic), int8 32x32x32 or bf16 32x32x16, with
+ * constant or pseudo-random operand values.  No counterpart in the reference: it is the yardstick for the GEMM
+ * figures, the rate the matrix pipe sustains under the power limit for that kind of data.  sink: >= 2 KiB of
+ * device memory (never written in practice); *ops receives the number of operations (2 per multiply-add) the
+ * launch performs. */
+int amct_mfma_yardstick(int bf16, int random_operands, int iters, void* sink, int64_t* ops, amct_stream_t stream);
+
 /* ---- column statistics over tokens (calibration of the smoothing factor) -----------------
  * Replaces the reductions of amct_pytorch/quantize_op/smooth_quant_module.py: :79-80 batch amax / amin over
  * all tokens per input channel, :88-91 the running update data_max = batch_max > data_max ? batch_max :
