@@ -34,9 +34,9 @@ MEASURED_TRAFFIC_BYTES = {
     "fakequant_int8": 134442394,
     "mxfp8_quant": 101803014,
     "hif8_encode": 100722479,
-    "w8a8_m2048": 252233414,
+    "w8a8_m2048": 254904953,
     "w8a8_m16": 59904148,
-    "w4a16_m2048": 271015110,
+    "w4a16_m2048": 269965424,
     "w4a16_m1": 36949937,
 }
 
