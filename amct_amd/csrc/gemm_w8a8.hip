@@ -11,8 +11,10 @@
 //                   prefetch (shapes the large-tile kernel does not take).
 //   decode kernel : M <= 16: activations staged once per block in LDS, the weight streamed once straight
 //                   from HBM into MFMA operands (v_mfma_i32_16x16x64_i8), split-K across the waves.
-//   skinny kernel : 16 < M <= 32 (and M <= 16 shapes the decode kernel does not take): as above with the
-//                   activations read from L2 per MFMA.
+//   medium tiles  : 16 < M up to a few hundred rows: the large-tile body with 128x128 (4 waves) or 128x256 blocks and
+//                   three LDS stages, chosen so that all blocks of the launch run at once.
+//   skinny kernel : 16 < M <= 32 when K is not a multiple of 128 (and M <= 16 shapes the decode kernel does not
+//                   take): as above with the activations read from L2 per MFMA.
 //   general kernel: any shape, one output per thread.
 #include "amct_common.h"
 #include "gemm_plan.h"
@@ -476,6 +478,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
+// any block shape the body supports, uniform over the launch (blockIdx.x: column tile, blockIdx.y: row tile)
+template <int ODT, int WM, int WN, int TI, int TJ, int STAGES, int LK>
+__global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void w8a8_tile_shape(W8A8Args a) {
+    using Sh = DmaTile<WM, WN, TI, TJ, STAGES, LK>;
+    __shared__ __attribute__((aligned(1024))) int8_t smem[Sh::kSmem];
+    w8a8_dma_body<ODT, WM, WN, TI, TJ, STAGES, LK>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
+}
+
 // ---------------------------------------------------------------------------
 // skinny kernel: M <= 16 * MT.  One block = 16 output columns; its 4 waves split K.
 // Lane l of a wave streams row n0 + l%16 of the weight, 16 bytes per MFMA, k-slot l/16.
@@ -754,6 +764,30 @@ extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s
         int rc = AMCT_E_UNSUPPORTED;
         if (lds) rc = tn == 1 ? launch_w8a8_decode_w<1>(a, waves, lds, st) : launch_w8a8_decode_w<2>(a, waves, lds, st);
         if (rc != AMCT_E_UNSUPPORTED) return rc;
+    }
+    // Medium M: as long as all tiles of a launch run at once (one or two blocks per CU), small tiles on many CUs beat
+    // large tiles on few.  128x128 tiles of 4 waves (measured on W[14336,4096]: 22 us for M = 24 .. 256 against
+    // 26 .. 42 us for the skinny / first-generation / 256x256 kernels), then 128x256 tiles of 8 waves (M = 384, 512:
+    // 32 us against 43 us); three LDS stages, because a short step exposes the load latency that two stages cover
+    // for a 256x256 tile.
+    if (vec_ok && M > 16 && K % 128 == 0 && N % 8 == 0 && aligned16(out) && M * K < (int64_t(1) << 32) && N * K < (int64_t(1) << 32)) {
+        const int64_t cus = current_cu_count();
+        const int64_t mt = (M + 127) / 128, nt128 = (N + 127) / 128, nt256 = (N + 255) / 256;
+        int shape = 0;
+        if (cus > 0 && mt * nt128 <= cus) shape = 1;
+        else if (cus > 0 && (mt * nt256 <= cus || M < 256)) shape = 2;
+        if (shape && mt <= 65535) {
+#define AMCT_LAUNCH_MID(ODT)                                                                                          \
+    {                                                                                                                 \
+        if (shape == 1) hipLaunchKernelGGL((w8a8_tile_shape<ODT, 2, 2, 2, 2, 3, 128>), dim3((unsigned)nt128, (unsigned)mt), dim3(256), 0, st, a); \
+        else hipLaunchKernelGGL((w8a8_tile_shape<ODT, 2, 4, 2, 2, 3, 128>), dim3((unsigned)nt256, (unsigned)mt), dim3(512), 0, st, a);            \
+    }
+            if (out_dtype == AMCT_BF16) AMCT_LAUNCH_MID(AMCT_BF16)
+            else if (out_dtype == AMCT_F16) AMCT_LAUNCH_MID(AMCT_F16)
+            else AMCT_LAUNCH_MID(AMCT_F32)
+#undef AMCT_LAUNCH_MID
+            return hip_status();
+        }
     }
     // measured on W[14336,4096]: the skinny kernel re-reads the activations once per 16 output columns and
     // loses to the 128x128 tile kernel from M = 48 on (33.9 us against 30.5 us; M = 64: 41.7 against 32.9)

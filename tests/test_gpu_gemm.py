@@ -68,10 +68,11 @@ def test_w8a8_vs_oracle(dev, M, N, K, per_token, bias):
 
 
 @pytest.mark.parametrize("M,N,K", [(300, 1000, 320), (256, 448, 128), (512, 832, 256), (2048, 14336, 192), (1100, 9000, 64),
-                                   (2000, 14328, 128)])
+                                   (2000, 14328, 128), (100, 1000, 256), (200, 520, 384), (384, 14336, 128), (17, 72, 128),
+                                   (640, 14336, 128), (33, 40000, 128)])
 def test_w8a8_large_shapes_mixed_blocks(dev, M, N, K):
-    """Launches with M >= 256 may mix two block shapes (256x256 and 256x192 tiles) so that the blocks fill the
-    CUs evenly; ragged edges in M and N, every output dtype, accumulators bit for bit."""
+    """Block shapes of the tile kernels: 128x128 and 128x256 blocks for medium M, 256x256 for large M, where a launch
+    may mix in 256x192 blocks so that the blocks fill the CUs evenly; ragged edges in M and N, accumulators bit for bit."""
     xq, wq, s_ch, s_tok, b = w8a8_case(M, N, K, 131, True, 'float')
     want_acc = od.int8_matmul_exact(xq, wq.t())
     for odt in (torch.bfloat16, torch.float32):
