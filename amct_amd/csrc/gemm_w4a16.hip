@@ -15,6 +15,7 @@
 #include <type_traits>
 
 #include "amct_common.h"
+#include "gemm_plan.h"
 
 namespace amct {
 
@@ -416,15 +417,18 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
 }
 
 // ---------------------------------------------------------------------------
-// wide large-tile kernel (K % 128 == 0, group % 64 == 0, activations already smoothed): 256x256 block tile,
-// 8 waves (2 x 4) of 128x64, two LDS stages of 64 elements of K (128-byte rows: a direct-to-LDS load covers
-// whole cache lines, one barrier per 64 elements).
-//   activations : direct global->LDS loads issued by waves 4..7 (one per SIMD) in one burst right after the
-//                 barrier that frees the stage; a wave stalls at such a load while the memory pipeline is busy
-//                 and the other wave of its SIMD keeps the matrix pipe fed meanwhile;
-//   weights     : 16 bytes (32 nibbles) per thread and step into registers two steps ahead, with the scale and
+// wide tile kernels (K % 128 == 0, group % 64 == 0, activations already smoothed): block tile (32*TI*WM) x
+// (32*TJ*WN), WM x WN waves, STAGES LDS stages of 64 elements of K (128-byte rows: a direct-to-LDS load covers
+// whole cache lines, one barrier per 64 elements).  256x256 with 8 waves of 128x64 and two stages for large M;
+// 128x128 (4 waves of 64x64) and 128x256 (8 waves of 64x64) with three stages for medium M, where a short step
+// would expose the load latency that two stages cover for the large tile.
+//   activations : direct global->LDS loads issued by the upper half of the waves (one per SIMD) in one burst
+//                 right after the barrier that frees the stage; a wave stalls at such a load while the memory
+//                 pipeline is busy and the other wave of its SIMD keeps the matrix pipe fed meanwhile;
+//   weights     : 16 bytes (32 nibbles) per thread and step into registers two steps ahead (two register slots,
+//                 the loop is unrolled by two; the LDS stage index is a run-time value), with the scale and
 //                 zero-point of their group; dequantised in the shadow of the MFMAs of the first two k-slices
-//                 of the step before and written to the other LDS stage in MFMA operand order.
+//                 of the step before and written to the next LDS stage in MFMA operand order.
 // The issue order is pinned: sched_group_barrier interleaves MFMA / VALU / LDS inside a k-slice, scheduling
 // barriers separate the slices, and the MFMAs of the slices before the barrier are issued BEFORE the wait
 // (left alone, the optimiser moves them behind the barrier and the matrix pipe idles while the waves meet).
@@ -434,8 +438,6 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
 // ---------------------------------------------------------------------------
 constexpr int kWK = 64;                                            // elements of K per stage
 constexpr int kWRow = 128;                                         // bytes per LDS row
-constexpr int kWStageBytes = (kQM + kQN) * kWRow;                  // 64 KiB
-constexpr int kWNA = (kQM * kWRow / 1024) / 4;                     // activation pieces per loading wave: 8
 
 AMCT_DEV void dma16s(uint32_t lds_addr, const void* sbase, uint32_t voff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
@@ -449,14 +451,27 @@ AMCT_DEV void gload_u16s(uint32_t& dst, const void* sbase, uint32_t voff) {
 AMCT_DEV void gload_u8s(uint32_t& dst, const void* sbase, uint32_t voff) {
     asm volatile("global_load_ubyte %0, %1, %2" : "=v"(dst) : "v"(voff), "s"(sbase) : "memory");
 }
+template <int N> AMCT_DEV void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory"); }
 
-// WM x WN = 8 waves of (32*TI) x (32*TJ); used as 2 x 4 waves of 128 x 64 for the 256x256 tile.  (4 x 2 waves of
-// 64 x 96 give a 256x192 tile in the same 64 KiB stage, every wave still dequantising its 32 weight rows.)
-template <bool SF16, int WM, int WN, int TI, int TJ>
+template <int WM, int WN, int TI, int TJ, int STAGES>
+struct WideTile {
+    static constexpr int kLM = 32 * TI * WM, kLN = 32 * TJ * WN, kWaves = WM * WN, kThreads = kWaves * 64;
+    static constexpr int kStageBytes = (kLM + kLN) * kWRow;
+    static constexpr int kLW = kWaves / 2;                         // waves that issue the direct-to-LDS loads
+    static constexpr int kNA = (kLM * kWRow / 1024) / kLW;         // activation pieces (8 rows x 128 B) per loading wave
+    static constexpr int kEpi = kWaves * 16384;
+    static constexpr int kSmem = STAGES * kStageBytes > kEpi ? STAGES * kStageBytes : kEpi;
+    static_assert(kThreads == 2 * kLN, "every thread dequantises half a weight row of the tile per step");
+    static_assert((kLM * kWRow / 1024) % kLW == 0 && kSmem <= 160 * 1024, "tile shape");
+    static_assert(kNA < 64, "vmcnt range");
+};
+
+template <bool SF16, int WM, int WN, int TI, int TJ, int STAGES>
 AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m0, const int64_t n0) {
-    static_assert(WM * WN == 8 && 32 * TI * WM == kQM && 32 * TJ * WN <= kQN, "tile shape");
+    using Sh = WideTile<WM, WN, TI, TJ, STAGES>;
+    constexpr int kLM = Sh::kLM, kStageBytes = Sh::kStageBytes, kWaves = Sh::kWaves, kLW = Sh::kLW, kNA = Sh::kNA;
     constexpr int kNM = TI * TJ, kNR = TI + TJ;                    // MFMAs and fragment reads per k-slice
-    static_assert(kNM >= kNR, "one fragment read per MFMA");
+    static_assert(kNM >= kNR && (STAGES == 2 || STAGES == 3), "one fragment read per MFMA; 2 or 3 stages");
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
@@ -467,14 +482,14 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
     auto swz = [](int r) { return (r >> 1) & 7; };
 
     // activation pieces (8 rows x 128 B) of the loading waves
-    const bool loader = wave >= 4;
-    const int lw = loader ? wave - 4 : 0;
-    uint32_t goff[kWNA];
+    const bool loader = wave >= kWaves - kLW;
+    const int lw = loader ? wave - (kWaves - kLW) : 0;
+    uint32_t goff[kNA];
     {
         const int rin = lane >> 3, pc = lane & 7;
 #pragma unroll
-        for (int j = 0; j < kWNA; ++j) {
-            const int lr = (lw * kWNA + j) * 8 + rin;
+        for (int j = 0; j < kNA; ++j) {
+            const int lr = (lw * kNA + j) * 8 + rin;
             const int64_t r = m0 + lr < a.M ? m0 + lr : a.M - 1;
             goff[j] = (uint32_t)((r * a.K + (pc ^ swz(lr)) * 8) * 2);
         }
@@ -483,18 +498,18 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
         if (loader) {
             const int st = step < last ? step : last;
 #pragma unroll
-            for (int j = 0; j < kWNA; ++j)
-                dma16s(lds0 + stg * kWStageBytes + (lw * kWNA + j) * 1024, a.x + (int64_t)st * kWK, goff[j]);
+            for (int j = 0; j < kNA; ++j)
+                dma16s(lds0 + stg * kStageBytes + (lw * kNA + j) * 1024, a.x + (int64_t)st * kWK, goff[j]);
         }
     };
-    // weight row of this thread: row tid/2, 32 weights (16 bytes) per step, which half from tid%2
+    // weight row of this thread: row tid/2 of the tile, 32 weights (16 bytes) per step, which half from tid%2
     const int brow = tid >> 1, bhalf = tid & 1;
     const int64_t wrow = (n0 + brow < a.N) ? n0 + brow : a.N - 1;
     const uint32_t woff = (uint32_t)(wrow * (a.K / 2) + bhalf * 16);
     const uint32_t soff = (uint32_t)(wrow * G * 2), zoff = (uint32_t)(wrow * G);
     int bdst[4];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) bdst[c] = kQM * kWRow + brow * kWRow + ((4 * bhalf + c) ^ swz(brow)) * 16;
+    for (int c = 0; c < 4; ++c) bdst[c] = kLM * kWRow + brow * kWRow + ((4 * bhalf + c) ^ swz(brow)) * 16;
 
     u4v wreg[2];
     uint32_t sreg[2], zreg[2];
@@ -512,12 +527,23 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
         nzs = -((float)zreg[slot] * sc);
     };
     auto write_b = [&](int slot, int stg, int c) {                 // dequantise 8 weights into LDS
-        *reinterpret_cast<uint4*>(smem + stg * kWStageBytes + bdst[c]) = dequant8(wreg[slot][c], sc, nzs);
+        *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[c]) = dequant8(wreg[slot][c], sc, nzs);
     };
-    // wait for every outstanding load and LDS operation of this wave; the slot's registers are tied to the
-    // statement so that their uses stay behind it
-#define AMCT_WAIT_ALL(slot) \
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : "+v"(wreg[slot]), "+v"(sreg[slot]), "+v"(zreg[slot]) : : "memory")
+    // Wait until the weight loads of the previous iteration and the activation loads issued STAGES-1 iterations ago
+    // have landed and this wave's LDS operations are done.  An iteration issues its 3 weight loads first and then, in
+    // a loading wave, kNA direct-to-LDS loads; with three stages the latter may stay in flight, hence the
+    // wave-uniform choice of the count.  The slot's registers are tied to a statement behind the wait so that
+    // their uses (and any copies the register allocator makes) stay behind it.
+    auto wait_older = [&]() {
+        if constexpr (STAGES == 2) {
+            wait_vm<0>();
+        } else {
+            if (loader) wait_vm<kNA>();
+            else wait_vm<0>();
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+#define AMCT_TIE_SLOT(slot) asm volatile("" : "+v"(wreg[slot]), "+v"(sreg[slot]), "+v"(zreg[slot]) : : "memory")
 
     int offA[4], offB[4];
 #pragma unroll
@@ -525,7 +551,7 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
         const int r = lane & 31;
         const int phys = (ks * 2 + (lane >> 5)) ^ swz(r);
         offA[ks] = (wm * 32 * TI + r) * kWRow + phys * 16;
-        offB[ks] = kQM * kWRow + (wn * 32 * TJ + r) * kWRow + phys * 16;
+        offB[ks] = kLM * kWRow + (wn * 32 * TJ + r) * kWRow + phys * 16;
     }
     v16f acc[TI][TJ];
 #pragma unroll
@@ -537,7 +563,7 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
 
     // fragment q in the order the MFMAs need them: A0, B0, B1, .., A1, A2, ..
     auto read_one = [&](int stg, int ks, int q, v8bf (&fa)[TI], v8bf (&fb)[TJ]) {
-        const uint8_t* st = smem + stg * kWStageBytes;
+        const uint8_t* st = smem + stg * kStageBytes;
         if (q == 0) fa[0] = *reinterpret_cast<const v8bf*>(st + offA[ks]);
         else if (q <= TJ) fb[q - 1] = *reinterpret_cast<const v8bf*>(st + offB[ks] + (q - 1) * 32 * kWRow);
         else fa[q - TJ] = *reinterpret_cast<const v8bf*>(st + offA[ks] + (q - TJ) * 32 * kWRow);
@@ -547,38 +573,41 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
     };
 
-    // prologue: A(0) and B(0) into stage 0, A(1) on its way to stage 1, B(1) and B(2) on their way to registers
+    // prologue: B(0), B(1) and A(0 .. STAGES-2); once B(0) is dequantised into stage 0 its slot takes B(2), and
+    // A(STAGES-1) follows (weights first, as in the loop)
     v8bf fa[2][TI], fb[2][TJ];
-    dma_a(0, 0);
     issue_b(0, 0);
     issue_b(1, 1);
-    AMCT_WAIT_ALL(0);
-    AMCT_WAIT_ALL(1);
+#pragma unroll
+    for (int j = 0; j < STAGES - 1; ++j) dma_a(j, j);
+    wait_vm<0>();
+    AMCT_TIE_SLOT(0);
+    AMCT_TIE_SLOT(1);
     factors(0);
 #pragma unroll
     for (int c = 0; c < 4; ++c) write_b(0, 0, c);
-    dma_a(1, 1);
     issue_b(0, 2);
+    dma_a(STAGES - 1, STAGES - 1);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 #pragma unroll
     for (int q = 0; q < kNR; ++q) read_one(0, 0, q, fa[0], fb[0]);
 
-    // iteration s (stage CUR = s % 2, NXT the other; slot NXT holds B(s+1), slot CUR holds B(s+2) in flight):
-    //   k-slices 0, 1 : MFMAs, fragment reads of the next slice, dequantisation of B(s+1) into stage NXT
+    // iteration s (LDS stage cur, the next one nxt; register slot SL holds B(s+1), landed; the other slot B(s+2)):
+    //   k-slices 0, 1 : MFMAs, fragment reads of the next slice, dequantisation of B(s+1) into stage nxt
     //   k-slice 2     : MFMAs, fragment reads of slice 3
-    //   wait (A(s+1) and B(s+2) have landed: both were issued a whole iteration ago; own LDS operations done),
-    //   barrier: stage CUR is free, stage NXT complete
-    //   loads         : A(s+2) into stage CUR (loading waves), B(s+3) into slot NXT
-    //   k-slice 3     : MFMAs, fragment reads of slice 0 of stage NXT
-#define AMCT_WSLICE_DQ(CUR, NXT, KS)                                                   \
+    //   wait (A(s+1) and B(s+2) have landed; own LDS operations done), barrier: stage cur is free, nxt complete
+    //   loads         : B(s+3) into slot SL, A(s+STAGES) into stage cur (loading waves)
+    //   k-slice 3     : MFMAs, fragment reads of slice 0 of stage nxt
+    int cur = 0, nxt = 1;
+#define AMCT_WSLICE_DQ(CUR, NXT, SL, KS)                                                 \
     {                                                                                  \
         __builtin_amdgcn_sched_barrier(0);                                             \
         _Pragma("unroll") for (int m_ = 0; m_ < kNM; ++m_) mfma_one(m_, fa[(KS) & 1], fb[(KS) & 1]); \
         _Pragma("unroll") for (int q_ = 0; q_ < kNR; ++q_) read_one(CUR, (KS) + 1, q_, fa[((KS) + 1) & 1], fb[((KS) + 1) & 1]); \
-        write_b(NXT, NXT, 2 * (KS));                                                   \
-        write_b(NXT, NXT, 2 * (KS) + 1);                                               \
+        write_b(SL, NXT, 2 * (KS));                                                    \
+        write_b(SL, NXT, 2 * (KS) + 1);                                                \
         _Pragma("unroll") for (int g_ = 0; g_ < kNM; ++g_) {                           \
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                      /* 1 MFMA */ \
             __builtin_amdgcn_sched_group_barrier(0x002, (56 + kNM - 1) / kNM, 0);   /* VALU   */ \
@@ -591,35 +620,38 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
         _Pragma("unroll") for (int m_ = 0; m_ < kNM; ++m_) {                           \
             mfma_one(m_, fa[(KS) & 1], fb[(KS) & 1]);                                  \
             __builtin_amdgcn_sched_barrier(0);                                         \
-            if (m_ < kNR) {                                                              \
+            if (m_ < kNR) {                                                            \
                 read_one(STG, KSREAD, m_, fa[((KS) + 1) & 1], fb[((KS) + 1) & 1]);     \
                 __builtin_amdgcn_sched_barrier(0);                                     \
             }                                                                          \
         }                                                                              \
     }
-#define AMCT_WITER(CUR, NXT, step)                                                     \
+#define AMCT_WITER(SL, step)                                                           \
     {                                                                                  \
-        factors(NXT);                                                                  \
-        AMCT_WSLICE_DQ(CUR, NXT, 0)                                                    \
-        AMCT_WSLICE_DQ(CUR, NXT, 1)                                                    \
-        AMCT_WSLICE_PIN(CUR, 3, 2)                                                     \
-        AMCT_WAIT_ALL(CUR);                                                            \
+        AMCT_TIE_SLOT(SL);                                                             \
+        factors(SL);                                                                   \
+        AMCT_WSLICE_DQ(cur, nxt, SL, 0)                                                \
+        AMCT_WSLICE_DQ(cur, nxt, SL, 1)                                                \
+        AMCT_WSLICE_PIN(cur, 3, 2)                                                     \
+        wait_older();                                                                  \
         __builtin_amdgcn_s_barrier();                                                  \
         asm volatile("" ::: "memory");                                                 \
         __builtin_amdgcn_sched_barrier(0);                                             \
-        dma_a(CUR, (step) + 2);                                                        \
-        issue_b(NXT, (step) + 3);                                                      \
+        issue_b(SL, (step) + 3);                                                       \
+        dma_a(cur, (step) + STAGES);                                                   \
         __builtin_amdgcn_sched_barrier(0);                                             \
-        AMCT_WSLICE_PIN(NXT, 0, 3)                                                     \
+        AMCT_WSLICE_PIN(nxt, 0, 3)                                                     \
+        cur = nxt;                                                                     \
+        nxt = nxt + 1 == STAGES ? 0 : nxt + 1;                                         \
     }
-    for (int step = 0; step < nsteps; step += 2) {
-        AMCT_WITER(0, 1, step)
-        AMCT_WITER(1, 0, step + 1)
+    for (int step = 0; step < nsteps; step += 2) {                  // K % 128 == 0: an even number of steps
+        AMCT_WITER(1, step)
+        AMCT_WITER(0, step + 1)
     }
 #undef AMCT_WITER
 #undef AMCT_WSLICE_PIN
 #undef AMCT_WSLICE_DQ
-#undef AMCT_WAIT_ALL
+#undef AMCT_TIE_SLOT
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
@@ -660,10 +692,12 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
     }
 }
 
-template <bool SF16>
-__global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void w4a16_tile_wide(W4A16Args a) {
-    __shared__ __attribute__((aligned(1024))) uint8_t smem[2 * kWStageBytes];
-    w4a16_wide_body<SF16, 2, 4, 4, 2>(a, smem, (int64_t)blockIdx.y * kQM, (int64_t)blockIdx.x * kQN);
+// blockIdx.x: column tile, blockIdx.y: row tile
+template <bool SF16, int WM, int WN, int TI, int TJ, int STAGES>
+__global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM * WN / 4, WM * WN / 4))) void w4a16_tile_wide(W4A16Args a) {
+    using Sh = WideTile<WM, WN, TI, TJ, STAGES>;
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[Sh::kSmem];
+    w4a16_wide_body<SF16, WM, WN, TI, TJ, STAGES>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
 }
 
 // x' = bf16(x * smooth[k]) over the whole activation matrix (K % 8 == 0): used when the caller lends a
@@ -1126,9 +1160,14 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
 #undef AMCT_DEC
         return hip_status();
     }
-    if (vec_ok && M >= 256 && K % 128 == 0 && K < 65536 && N % 8 == 0 && aligned16(out)) {
+    // 16 < M <= 64 stays with the weight-streaming decode kernel above (25 .. 40 us on W[14336,4096] against 51 us for
+    // the smallest tile shape here)
+    if (vec_ok && M > 64 && K % 128 == 0 && K < 65536 && N % 8 == 0 && aligned16(out)) {
         const dim3 grid((unsigned)((N + kQN - 1) / kQN), (unsigned)((M + kQM - 1) / kQM));
         if (grid.y > 65535) return AMCT_E_UNSUPPORTED;
+        const int64_t G = K / group;
+        const bool fits = group % 64 == 0 && M * K * 2 < (int64_t(1) << 32) && N * (K / 2) < (int64_t(1) << 32) &&
+                          N * G * 2 < (int64_t(1) << 32);
         if (smooth && workspace && workspace_bytes >= (size_t)(M * K * 2) && aligned16(workspace)) {
             // smoothing once into the lent workspace, then the kernel without the in-tile multiply
             const int64_t nvec = M * K / 8;
@@ -1139,16 +1178,34 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
             a.smooth = nullptr;
             smooth = nullptr;
         }
-        const int64_t G = K / group;
-        const bool wide = !smooth && group % 64 == 0 && M * K * 2 < (int64_t(1) << 32) && N * (K / 2) < (int64_t(1) << 32) &&
-                          N * G * 2 < (int64_t(1) << 32);
-        // (mixing in 256x192 blocks as the W8A8 launch does was measured neutral here: the narrow tile dequantises
-        // as many weights as the full one)
-        if (wide && scale_dtype == AMCT_F16) hipLaunchKernelGGL((w4a16_tile_wide<true>), grid, dim3(kQThreads), 0, st, a);
-        else if (wide) hipLaunchKernelGGL((w4a16_tile_wide<false>), grid, dim3(kQThreads), 0, st, a);
-        else if (smooth) hipLaunchKernelGGL((w4a16_tile_dma<true>), grid, dim3(kQThreads), 0, st, a);
-        else hipLaunchKernelGGL((w4a16_tile_dma<false>), grid, dim3(kQThreads), 0, st, a);
-        return hip_status();
+        const bool wide = !smooth && fits;
+        if (wide) {
+            // Block shape: as long as all tiles of a launch run at once, small tiles on many CUs beat large tiles on
+            // few (the weight stream is the bulk of the traffic for medium M): 128x128 blocks of 4 waves, then 128x256
+            // blocks of 8 waves, each with three LDS stages; 256x256 with two stages otherwise.  (Mixing in 256x192
+            // blocks as the W8A8 launch does was measured neutral here: the narrow tile dequantises as many weights.)
+            const int64_t cus = current_cu_count();
+            const int64_t mt = (M + 127) / 128, nt128 = (N + 127) / 128, nt256 = (N + 255) / 256;
+            int shape = 0;
+            if (cus > 0 && mt * nt128 <= cus) shape = 1;
+            else if (cus > 0 && (mt * nt256 <= cus || M < 256)) shape = 2;
+            if (mt > 65535) return AMCT_E_UNSUPPORTED;
+#define AMCT_LAUNCH_WIDE(SF)                                                                                           \
+    {                                                                                                                  \
+        if (shape == 1) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 2, 2, 3>), dim3((unsigned)nt128, (unsigned)mt), dim3(256), 0, st, a);      \
+        else if (shape == 2) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 4, 2, 2, 3>), dim3((unsigned)nt256, (unsigned)mt), dim3(512), 0, st, a); \
+        else hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 4, 4, 2, 2>), grid, dim3(kQThreads), 0, st, a);                \
+    }
+            if (scale_dtype == AMCT_F16) AMCT_LAUNCH_WIDE(true)
+            else AMCT_LAUNCH_WIDE(false)
+#undef AMCT_LAUNCH_WIDE
+            return hip_status();
+        }
+        if (M >= 256) {
+            if (smooth) hipLaunchKernelGGL((w4a16_tile_dma<true>), grid, dim3(kQThreads), 0, st, a);
+            else hipLaunchKernelGGL((w4a16_tile_dma<false>), grid, dim3(kQThreads), 0, st, a);
+            return hip_status();
+        }
     }
     if (vec_ok && K % kTK == 0) {
         const dim3 grid((unsigned)((N + kTN - 1) / kTN), (unsigned)((M + kTM - 1) / kTM));
