@@ -700,6 +700,237 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM
     w4a16_wide_body<SF16, WM, WN, TI, TJ, STAGES>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
 }
 
+// ---------------------------------------------------------------------------
+// medium-M kernel with specialised waves: 128x128 block tile, 8 waves.  Waves 0..3 (2 x 2 of 64x64) only read
+// fragments and issue MFMAs; waves 4..7 only move data: the direct-to-LDS loads of the activation tile, the
+// packed weights into registers, their dequantisation and the LDS writes.  With the usual round-robin placement
+// every SIMD holds one wave of each kind, so the dequantisation (92 vector instructions per thread and step)
+// runs under the other wave's MFMAs instead of between a wave's own: a block of 4 waves that does both, alone on
+// its CU (three 32 KiB stages), has nobody to overlap with.  Same LDS layout, stage protocol and load pipeline
+// as w4a16_wide_body; both kinds of wave pass the same number of barriers (one per step, one before the loop,
+// one behind it).
+// ---------------------------------------------------------------------------
+template <bool SF16, int STAGES>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void w4a16_tile_spec(W4A16Args a) {
+    constexpr int kLM = 128, kLN = 128, TI = 2, TJ = 2, WN = 2;
+    constexpr int kStageBytes = (kLM + kLN) * kWRow;                // 32 KiB
+    constexpr int kNA = (kLM * kWRow / 1024) / 4;                   // activation pieces per moving wave: 4
+    constexpr int kNM = TI * TJ, kNR = TI + TJ;
+    static_assert(STAGES == 2 || STAGES == 3, "stages");
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[STAGES * kStageBytes > 65536 ? STAGES * kStageBytes : 65536];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t m0 = (int64_t)blockIdx.y * kLM, n0 = (int64_t)blockIdx.x * kLN;
+    const int nsteps = (int)(a.K / kWK);
+    const int last = nsteps - 1;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
+    auto swz = [](int r) { return (r >> 1) & 7; };
+
+    if (wave >= 4) {
+        // ---------------- data movement ----------------
+        const int pw = wave - 4, ptid = tid - 256;
+        const uint32_t G = (uint32_t)(a.K / a.group);
+        uint32_t goff[kNA];
+        {
+            const int rin = lane >> 3, pc = lane & 7;
+#pragma unroll
+            for (int j = 0; j < kNA; ++j) {
+                const int lr = (pw * kNA + j) * 8 + rin;
+                const int64_t r = m0 + lr < a.M ? m0 + lr : a.M - 1;
+                goff[j] = (uint32_t)((r * a.K + (pc ^ swz(lr)) * 8) * 2);
+            }
+        }
+        auto dma_a = [&](int stg, int step) {
+            const int st = step < last ? step : last;
+#pragma unroll
+            for (int j = 0; j < kNA; ++j)
+                dma16s(lds0 + stg * kStageBytes + (pw * kNA + j) * 1024, a.x + (int64_t)st * kWK, goff[j]);
+        };
+        const int brow = ptid >> 1, bhalf = ptid & 1;
+        const int64_t wrow = (n0 + brow < a.N) ? n0 + brow : a.N - 1;
+        const uint32_t woff = (uint32_t)(wrow * (a.K / 2) + bhalf * 16);
+        const uint32_t soff = (uint32_t)(wrow * G * 2), zoff = (uint32_t)(wrow * G);
+        int bdst[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) bdst[c] = kLM * kWRow + brow * kWRow + ((4 * bhalf + c) ^ swz(brow)) * 16;
+        // The weights stream from HBM and a step of this small tile is shorter than that latency, so the packed
+        // weights of a step are fetched kD steps ahead into kD register slots (the loop is unrolled by kD).
+        constexpr int kD = 4;
+        u4v wreg[kD];
+        uint32_t sreg[kD], zreg[kD];
+        auto issue_b = [&](int slot, int step) {
+            const int st = step < last ? step : last;
+            const uint32_t k = (uint32_t)st * kWK;
+            const uint32_t gi = __umulhi(k, a.group_magic);         // k / group (k, group < 2^16); group % 64 == 0
+            gload16s(wreg[slot], a.wq + k / 2, woff);
+            gload_u16s(sreg[slot], reinterpret_cast<const uint8_t*>(a.scales) + gi * 2, soff);
+            gload_u8s(zreg[slot], a.zeros + gi, zoff);
+        };
+        auto dequant_into = [&](int slot, int stg) {
+            const float sc = SF16 ? f16_bits_to_f32(sreg[slot]) : bf16_bits_to_f32(sreg[slot]);
+            const float nzs = -((float)zreg[slot] * sc);
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[c]) = dequant8(wreg[slot][c], sc, nzs);
+        };
+#define AMCT_TIE_SLOT(slot) asm volatile("" : "+v"(wreg[slot]), "+v"(sreg[slot]), "+v"(zreg[slot]) : : "memory")
+        // prologue: B(0 .. kD-1) into their slots and A(0 .. STAGES-2); everything lands; B(0) is dequantised into
+        // stage 0 and its slot takes B(kD); A(STAGES-1) follows (weights first, as in the loop)
+#pragma unroll
+        for (int j = 0; j < kD; ++j) issue_b(j, j);
+#pragma unroll
+        for (int j = 0; j < STAGES - 1; ++j) dma_a(j, j);
+        wait_vm<0>();
+#pragma unroll
+        for (int j = 0; j < kD; ++j) AMCT_TIE_SLOT(j);
+        dequant_into(0, 0);
+        issue_b(0, kD);
+        dma_a(STAGES - 1, STAGES - 1);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        // iteration s: wait for B(s+1) (slot SL; issued kD iterations ago: the kNA activation loads of that
+        // iteration and the 3 + kNA operations of each iteration since may stay in flight); B(s+1) -> stage nxt;
+        // wait for A(s+1) (issued STAGES-1 iterations ago); barrier; B(s+1+kD) into slot SL, A(s+STAGES) into stage cur
+        int cur = 0, nxt = 1;
+#define AMCT_MOVE_ITER(SL, step)                                                       \
+    {                                                                                  \
+        wait_vm<kNA + (kD - 1) * (3 + kNA)>();                                         \
+        AMCT_TIE_SLOT(SL);                                                             \
+        dequant_into(SL, nxt);                                                         \
+        wait_vm<(STAGES - 2) * (3 + kNA)>();                                           \
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                             \
+        __builtin_amdgcn_s_barrier();                                                  \
+        asm volatile("" ::: "memory");                                                 \
+        issue_b(SL, (step) + 1 + kD);                                                  \
+        dma_a(cur, (step) + STAGES);                                                   \
+        cur = nxt;                                                                     \
+        nxt = nxt + 1 == STAGES ? 0 : nxt + 1;                                         \
+    }
+        for (int step = 0; step < nsteps; step += kD) {             // K % 256 == 0: a multiple of kD steps
+            AMCT_MOVE_ITER(1, step)
+            AMCT_MOVE_ITER(2, step + 1)
+            AMCT_MOVE_ITER(3, step + 2)
+            AMCT_MOVE_ITER(0, step + 3)
+        }
+#undef AMCT_MOVE_ITER
+#undef AMCT_TIE_SLOT
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        return;
+    }
+
+    // ---------------- matrix work ----------------
+    const int wm = wave / WN, wn = wave % WN;
+    int offA[4], offB[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+        const int r = lane & 31;
+        const int phys = (ks * 2 + (lane >> 5)) ^ swz(r);
+        offA[ks] = (wm * 32 * TI + r) * kWRow + phys * 16;
+        offB[ks] = kLM * kWRow + (wn * 32 * TJ + r) * kWRow + phys * 16;
+    }
+    v16f acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    auto read_one = [&](int stg, int ks, int q, v8bf (&fa)[TI], v8bf (&fb)[TJ]) {
+        const uint8_t* st = smem + stg * kStageBytes;
+        if (q == 0) fa[0] = *reinterpret_cast<const v8bf*>(st + offA[ks]);
+        else if (q <= TJ) fb[q - 1] = *reinterpret_cast<const v8bf*>(st + offB[ks] + (q - 1) * 32 * kWRow);
+        else fa[q - TJ] = *reinterpret_cast<const v8bf*>(st + offA[ks] + (q - TJ) * 32 * kWRow);
+    };
+    auto mfma_one = [&](int m, const v8bf (&fa)[TI], const v8bf (&fb)[TJ]) {
+        const int i = m / TJ, j = m % TJ;
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    };
+    // One fragment buffer per k-slice: a 64x64 wave tile has only 4 MFMAs per slice, fewer cycles than an LDS read
+    // takes, so the reads of slices 1..3 of a step are all issued behind the MFMAs of slice 0 (the stage is complete
+    // when the step starts) and their latency is paid once per step instead of once per slice.
+    v8bf fa[4][TI], fb[4][TJ];
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int q = 0; q < kNR; ++q) read_one(0, 0, q, fa[0], fb[0]);
+    {
+        int cur = 0, nxt = 1;
+        constexpr int kRPM = (3 * kNR + kNM - 1) / kNM;             // reads behind each MFMA of slice 0
+        for (int step = 0; step < nsteps; ++step) {
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int m = 0; m < kNM; ++m) {
+                mfma_one(m, fa[0], fb[0]);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int q = kRPM * m; q < kRPM * (m + 1); ++q) {
+                    if (q < 3 * kNR) {
+                        read_one(cur, 1 + q / kNR, q % kNR, fa[1 + q / kNR], fb[1 + q / kNR]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            }
+#pragma unroll
+            for (int ks = 1; ks < 3; ++ks) {
+#pragma unroll
+                for (int m = 0; m < kNM; ++m) {
+                    mfma_one(m, fa[ks], fb[ks]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int m = 0; m < kNM; ++m) {
+                mfma_one(m, fa[3], fb[3]);
+                __builtin_amdgcn_sched_barrier(0);
+                read_one(nxt, 0, m, fa[0], fb[0]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            cur = nxt;
+            nxt = nxt + 1 == STAGES ? 0 : nxt + 1;
+        }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+
+    // epilogue (matrix waves only): + bias (or + (-0.0f)), narrow to bf16, transpose through a per-wave LDS patch
+    constexpr int kPW = 32 * TJ, kPatchRow = kPW * 2 + 16, CPR = kPW * 2 / 16;
+    uint8_t* patch = smem + wave * 16384;
+    float bs[TJ];
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) {
+        const int64_t n = n0 + wn * kPW + j * 32 + (lane & 31);
+        bs[j] = a.bias ? a.bias[n < a.N ? n : a.N - 1] : -0.0f;
+    }
+    uint8_t* wbase = patch + 4 * (lane >> 5) * kPatchRow + (lane & 31) * 2;
+#pragma unroll
+    for (int i = 0; i < TI; ++i) {
+        const int64_t mbase = m0 + wm * 32 * TI + i * 32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int prow0 = 8 * (r >> 2) + (r & 3);
+#pragma unroll
+            for (int j = 0; j < TJ; ++j)
+                *reinterpret_cast<uint16_t*>(wbase + prow0 * kPatchRow + j * 64) = (uint16_t)f32_to_bf16_bits(acc[i][j][r] + bs[j]);
+        }
+#pragma unroll
+        for (int it = 0; it < 32 * CPR / 64; ++it) {
+            const int idx = it * 64 + lane;
+            const int prow = idx / CPR, chunk = idx % CPR;
+            const uint4 v = *reinterpret_cast<const uint4*>(patch + prow * kPatchRow + chunk * 16);
+            const int64_t m = mbase + prow;
+            const int64_t n = n0 + wn * kPW + chunk * 8;
+            if (m < a.M && n < a.N) stg16_nt(reinterpret_cast<char*>(a.out) + (m * a.N + n) * 2, v);
+        }
+    }
+}
+
 // x' = bf16(x * smooth[k]) over the whole activation matrix (K % 8 == 0): used when the caller lends a
 // workspace, so that the multiply is done once instead of once per column tile
 __global__ __launch_bounds__(kBlock) void smooth_rows(const uint16_t* x, const uint16_t* smooth, uint16_t* y, int64_t nvec, int kvec) {
@@ -1181,8 +1412,10 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
         const bool wide = !smooth && fits;
         if (wide) {
             // Block shape: as long as all tiles of a launch run at once, small tiles on many CUs beat large tiles on
-            // few (the weight stream is the bulk of the traffic for medium M): 128x128 blocks of 4 waves, then 128x256
-            // blocks of 8 waves, each with three LDS stages; 256x256 with two stages otherwise.  (Mixing in 256x192
+            // few (the weight stream is the bulk of the traffic for medium M): 128x128 blocks (with specialised waves
+            // when K % 256 == 0: 43 us against 51 us on W[14336,4096], M = 65 .. 256; the first-generation kernel took
+            // 97 us), then 128x256 blocks of 8 waves (M = 384, 512: 72 .. 75 us against 96 us), each with three LDS
+            // stages; 256x256 with two stages otherwise.  (Mixing in 256x192
             // blocks as the W8A8 launch does was measured neutral here: the narrow tile dequantises as many weights.)
             const int64_t cus = current_cu_count();
             const int64_t mt = (M + 127) / 128, nt128 = (N + 127) / 128, nt256 = (N + 255) / 256;
@@ -1192,7 +1425,8 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
             if (mt > 65535) return AMCT_E_UNSUPPORTED;
 #define AMCT_LAUNCH_WIDE(SF)                                                                                           \
     {                                                                                                                  \
-        if (shape == 1) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 2, 2, 3>), dim3((unsigned)nt128, (unsigned)mt), dim3(256), 0, st, a);      \
+        if (shape == 1 && K % 256 == 0) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3>), dim3((unsigned)nt128, (unsigned)mt), dim3(512), 0, st, a); \
+        else if (shape == 1) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 2, 2, 3>), dim3((unsigned)nt128, (unsigned)mt), dim3(256), 0, st, a); \
         else if (shape == 2) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 4, 2, 2, 3>), dim3((unsigned)nt256, (unsigned)mt), dim3(512), 0, st, a); \
         else hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 4, 4, 2, 2>), grid, dim3(kQThreads), 0, st, a);                \
     }
