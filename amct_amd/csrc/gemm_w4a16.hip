@@ -438,6 +438,7 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
 // ---------------------------------------------------------------------------
 constexpr int kWK = 64;                                            // elements of K per stage
 constexpr int kWRow = 128;                                         // bytes per LDS row
+constexpr int kSpecMaxG = 32;                                      // groups per weight row the specialised kernel's factor table holds
 
 AMCT_DEV void dma16s(uint32_t lds_addr, const void* sbase, uint32_t voff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
@@ -717,7 +718,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     constexpr int kNA = (kLM * kWRow / 1024) / 4;                   // activation pieces per moving wave: 4
     constexpr int kNM = TI * TJ, kNR = TI + TJ;
     static_assert(STAGES == 2 || STAGES == 3, "stages");
-    __shared__ __attribute__((aligned(1024))) uint8_t smem[STAGES * kStageBytes > 65536 ? STAGES * kStageBytes : 65536];
+    constexpr int kStages = STAGES * kStageBytes > 65536 ? STAGES * kStageBytes : 65536;
+    // behind the stages: scale (low 16 bits) and zero-point of every (weight row of the tile, group), one row of
+    // kSpecMaxG + 1 words per weight row (odd stride: the 32 rows a wave reads hit different banks)
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[kStages + kLN * (kSpecMaxG + 1) * 4];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int64_t m0 = (int64_t)blockIdx.y * kLM, n0 = (int64_t)blockIdx.x * kLN;
@@ -725,6 +729,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int last = nsteps - 1;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
     auto swz = [](int r) { return (r >> 1) & 7; };
+    uint32_t* const tab = reinterpret_cast<uint32_t*>(smem + kStages);
+    {
+        // Per-step loads of a 2-byte scale and a 1-byte zero-point per thread touch 48 cache lines per wave
+        // instruction; all of the tile's factors are fetched once instead, by all 512 threads.
+        const uint32_t G = (uint32_t)(a.K / a.group);
+        for (uint32_t e = tid; e < (uint32_t)kLN * G; e += 512) {
+            const uint32_t row = e / G, g = e - row * G;
+            const int64_t wr = (n0 + row < a.N) ? n0 + row : a.N - 1;
+            const uint32_t sbits = reinterpret_cast<const uint16_t*>(a.scales)[wr * G + g];
+            tab[row * (kSpecMaxG + 1) + g] = sbits | ((uint32_t)a.zeros[wr * G + g] << 16);
+        }
+        __syncthreads();
+    }
 
     if (wave >= 4) {
         // ---------------- data movement ----------------
@@ -749,7 +766,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int brow = ptid >> 1, bhalf = ptid & 1;
         const int64_t wrow = (n0 + brow < a.N) ? n0 + brow : a.N - 1;
         const uint32_t woff = (uint32_t)(wrow * (a.K / 2) + bhalf * 16);
-        const uint32_t soff = (uint32_t)(wrow * G * 2), zoff = (uint32_t)(wrow * G);
+        const uint32_t* const trow = tab + brow * (kSpecMaxG + 1);
         int bdst[4];
 #pragma unroll
         for (int c = 0; c < 4; ++c) bdst[c] = kLM * kWRow + brow * kWRow + ((4 * bhalf + c) ^ swz(brow)) * 16;
@@ -757,23 +774,21 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         // weights of a step are fetched kD steps ahead into kD register slots (the loop is unrolled by kD).
         constexpr int kD = 4;
         u4v wreg[kD];
-        uint32_t sreg[kD], zreg[kD];
         auto issue_b = [&](int slot, int step) {
             const int st = step < last ? step : last;
-            const uint32_t k = (uint32_t)st * kWK;
-            const uint32_t gi = __umulhi(k, a.group_magic);         // k / group (k, group < 2^16); group % 64 == 0
-            gload16s(wreg[slot], a.wq + k / 2, woff);
-            gload_u16s(sreg[slot], reinterpret_cast<const uint8_t*>(a.scales) + gi * 2, soff);
-            gload_u8s(zreg[slot], a.zeros + gi, zoff);
+            gload16s(wreg[slot], a.wq + (uint32_t)st * (kWK / 2), woff);
         };
-        auto dequant_into = [&](int slot, int stg) {
-            const float sc = SF16 ? f16_bits_to_f32(sreg[slot]) : bf16_bits_to_f32(sreg[slot]);
-            const float nzs = -((float)zreg[slot] * sc);
+        auto dequant_into = [&](int slot, int step, int stg) {      // the weights of K-step `step` (in `slot`) -> stage stg
+            const int st = step < last ? step : last;
+            const uint32_t gi = __umulhi((uint32_t)st * kWK, a.group_magic);   // k / group (k, group < 2^16); group % 64 == 0
+            const uint32_t e = trow[gi];
+            const float sc = SF16 ? f16_bits_to_f32(e & 0xFFFFu) : bf16_bits_to_f32(e & 0xFFFFu);
+            const float nzs = -((float)(e >> 16) * sc);
 #pragma unroll
             for (int c = 0; c < 4; ++c)
                 *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[c]) = dequant8(wreg[slot][c], sc, nzs);
         };
-#define AMCT_TIE_SLOT(slot) asm volatile("" : "+v"(wreg[slot]), "+v"(sreg[slot]), "+v"(zreg[slot]) : : "memory")
+#define AMCT_TIE_SLOT(slot) asm volatile("" : "+v"(wreg[slot]) : : "memory")
         // prologue: B(0 .. kD-1) into their slots and A(0 .. STAGES-2); everything lands; B(0) is dequantised into
         // stage 0 and its slot takes B(kD); A(STAGES-1) follows (weights first, as in the loop)
 #pragma unroll
@@ -783,22 +798,22 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         wait_vm<0>();
 #pragma unroll
         for (int j = 0; j < kD; ++j) AMCT_TIE_SLOT(j);
-        dequant_into(0, 0);
+        dequant_into(0, 0, 0);
         issue_b(0, kD);
         dma_a(STAGES - 1, STAGES - 1);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         // iteration s: wait for B(s+1) (slot SL; issued kD iterations ago: the kNA activation loads of that
-        // iteration and the 3 + kNA operations of each iteration since may stay in flight); B(s+1) -> stage nxt;
+        // iteration and the 1 + kNA operations of each iteration since may stay in flight); B(s+1) -> stage nxt;
         // wait for A(s+1) (issued STAGES-1 iterations ago); barrier; B(s+1+kD) into slot SL, A(s+STAGES) into stage cur
         int cur = 0, nxt = 1;
 #define AMCT_MOVE_ITER(SL, step)                                                       \
     {                                                                                  \
-        wait_vm<kNA + (kD - 1) * (3 + kNA)>();                                         \
+        wait_vm<kNA + (kD - 1) * (1 + kNA)>();                                         \
         AMCT_TIE_SLOT(SL);                                                             \
-        dequant_into(SL, nxt);                                                         \
-        wait_vm<(STAGES - 2) * (3 + kNA)>();                                           \
+        dequant_into(SL, (step) + 1, nxt);                                             \
+        wait_vm<(STAGES - 2) * (1 + kNA)>();                                           \
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                             \
         __builtin_amdgcn_s_barrier();                                                  \
         asm volatile("" ::: "memory");                                                 \
@@ -1425,7 +1440,7 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
             if (mt > 65535) return AMCT_E_UNSUPPORTED;
 #define AMCT_LAUNCH_WIDE(SF)                                                                                           \
     {                                                                                                                  \
-        if (shape == 1 && K % 256 == 0) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3>), dim3((unsigned)nt128, (unsigned)mt), dim3(512), 0, st, a); \
+        if (shape == 1 && K % 256 == 0 && G <= kSpecMaxG) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3>), dim3((unsigned)nt128, (unsigned)mt), dim3(512), 0, st, a); \
         else if (shape == 1) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 2, 2, 3>), dim3((unsigned)nt128, (unsigned)mt), dim3(256), 0, st, a); \
         else if (shape == 2) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 4, 2, 2, 3>), dim3((unsigned)nt256, (unsigned)mt), dim3(512), 0, st, a); \
         else hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 4, 4, 2, 2>), grid, dim3(kQThreads), 0, st, a);                \
