@@ -438,6 +438,7 @@ __global__ __launch_bounds__(kQThreads) __attribute__((amdgpu_waves_per_eu(2, 2)
 // ---------------------------------------------------------------------------
 constexpr int kWK = 64;                                            // elements of K per stage
 constexpr int kWRow = 128;                                         // bytes per LDS row
+constexpr int kSpecThreads = 768;                                  // 4 matrix waves + 8 data-movement waves
 constexpr int kSpecMaxG = 32;                                      // groups per weight row the specialised kernel's factor table holds
 
 AMCT_DEV void dma16s(uint32_t lds_addr, const void* sbase, uint32_t voff) {
@@ -702,20 +703,22 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM
 }
 
 // ---------------------------------------------------------------------------
-// medium-M kernel with specialised waves: 128x128 block tile, 8 waves.  Waves 0..3 (2 x 2 of 64x64) only read
-// fragments and issue MFMAs; waves 4..7 only move data: the direct-to-LDS loads of the activation tile, the
-// packed weights into registers, their dequantisation and the LDS writes.  With the usual round-robin placement
-// every SIMD holds one wave of each kind, so the dequantisation (92 vector instructions per thread and step)
-// runs under the other wave's MFMAs instead of between a wave's own: a block of 4 waves that does both, alone on
-// its CU (three 32 KiB stages), has nobody to overlap with.  Same LDS layout, stage protocol and load pipeline
-// as w4a16_wide_body; both kinds of wave pass the same number of barriers (one per step, one before the loop,
-// one behind it).
+// medium-M kernel with specialised waves: 128x128 block tile, 12 waves.  Waves 0..3 (2 x 2 of 64x64, one per
+// SIMD) only read fragments and issue MFMAs; waves 4..11 (two per SIMD) only move data: the direct-to-LDS loads of
+// the activation tile, the packed weights into registers (8 bytes per thread and step, four steps ahead), their
+// dequantisation and the LDS writes.  The dequantisation then runs under the other waves' MFMAs instead of
+// between a wave's own: a block of 4 waves that does both, alone on its CU (three 32 KiB stages), has nobody to
+// overlap with.  Same LDS layout and stage protocol as w4a16_wide_body; every wave passes the same number of
+// barriers (one per step, two before the loop, one behind it).  Measured on W[14336,4096], M = 128: 38 us (8
+// data-movement waves), 43 us (4), 51 us (4 waves doing everything); of the 38 us, 22 us are the matrix waves and
+// the barriers alone, the LDS writes of the dequantised weights add 8 us, the loads 7 us, the arithmetic 4 us.
 // ---------------------------------------------------------------------------
 template <bool SF16, int STAGES>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void w4a16_tile_spec(W4A16Args a) {
+__global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) void w4a16_tile_spec(W4A16Args a) {
     constexpr int kLM = 128, kLN = 128, TI = 2, TJ = 2, WN = 2;
     constexpr int kStageBytes = (kLM + kLN) * kWRow;                // 32 KiB
-    constexpr int kNA = (kLM * kWRow / 1024) / 4;                   // activation pieces per moving wave: 4
+    constexpr int kMW = kSpecThreads / 64 - 4;                      // data-movement waves: 8
+    constexpr int kNA = (kLM * kWRow / 1024) / kMW;                 // activation pieces per moving wave: 2
     constexpr int kNM = TI * TJ, kNR = TI + TJ;
     static_assert(STAGES == 2 || STAGES == 3, "stages");
     constexpr int kStages = STAGES * kStageBytes > 65536 ? STAGES * kStageBytes : 65536;
@@ -734,7 +737,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         // Per-step loads of a 2-byte scale and a 1-byte zero-point per thread touch 48 cache lines per wave
         // instruction; all of the tile's factors are fetched once instead, by all 512 threads.
         const uint32_t G = (uint32_t)(a.K / a.group);
-        for (uint32_t e = tid; e < (uint32_t)kLN * G; e += 512) {
+        for (uint32_t e = tid; e < (uint32_t)kLN * G; e += kSpecThreads) {
             const uint32_t row = e / G, g = e - row * G;
             const int64_t wr = (n0 + row < a.N) ? n0 + row : a.N - 1;
             const uint32_t sbits = reinterpret_cast<const uint16_t*>(a.scales)[wr * G + g];
@@ -763,20 +766,21 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             for (int j = 0; j < kNA; ++j)
                 dma16s(lds0 + stg * kStageBytes + (pw * kNA + j) * 1024, a.x + (int64_t)st * kWK, goff[j]);
         };
-        const int brow = ptid >> 1, bhalf = ptid & 1;
+        // weight row ptid/4 of the tile, 16 weights (8 bytes) per step, which quarter from ptid%4
+        const int brow = ptid >> 2, bq = ptid & 3;
         const int64_t wrow = (n0 + brow < a.N) ? n0 + brow : a.N - 1;
-        const uint32_t woff = (uint32_t)(wrow * (a.K / 2) + bhalf * 16);
+        const uint32_t woff = (uint32_t)(wrow * (a.K / 2) + bq * 8);
         const uint32_t* const trow = tab + brow * (kSpecMaxG + 1);
-        int bdst[4];
+        int bdst[2];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) bdst[c] = kLM * kWRow + brow * kWRow + ((4 * bhalf + c) ^ swz(brow)) * 16;
+        for (int c = 0; c < 2; ++c) bdst[c] = kLM * kWRow + brow * kWRow + ((2 * bq + c) ^ swz(brow)) * 16;
         // The weights stream from HBM and a step of this small tile is shorter than that latency, so the packed
         // weights of a step are fetched kD steps ahead into kD register slots (the loop is unrolled by kD).
         constexpr int kD = 4;
-        u4v wreg[kD];
+        uint64_t wreg[kD];
         auto issue_b = [&](int slot, int step) {
             const int st = step < last ? step : last;
-            gload16s(wreg[slot], a.wq + (uint32_t)st * (kWK / 2), woff);
+            asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(wreg[slot]) : "v"(woff), "s"(a.wq + (uint32_t)st * (kWK / 2)) : "memory");
         };
         auto dequant_into = [&](int slot, int step, int stg) {      // the weights of K-step `step` (in `slot`) -> stage stg
             const int st = step < last ? step : last;
@@ -784,9 +788,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             const uint32_t e = trow[gi];
             const float sc = SF16 ? f16_bits_to_f32(e & 0xFFFFu) : bf16_bits_to_f32(e & 0xFFFFu);
             const float nzs = -((float)(e >> 16) * sc);
-#pragma unroll
-            for (int c = 0; c < 4; ++c)
-                *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[c]) = dequant8(wreg[slot][c], sc, nzs);
+            *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[0]) = dequant8((uint32_t)wreg[slot], sc, nzs);
+            *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[1]) = dequant8((uint32_t)(wreg[slot] >> 32), sc, nzs);
         };
 #define AMCT_TIE_SLOT(slot) asm volatile("" : "+v"(wreg[slot]) : : "memory")
         // prologue: B(0 .. kD-1) into their slots and A(0 .. STAGES-2); everything lands; B(0) is dequantised into
@@ -1428,7 +1431,7 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
         if (wide) {
             // Block shape: as long as all tiles of a launch run at once, small tiles on many CUs beat large tiles on
             // few (the weight stream is the bulk of the traffic for medium M): 128x128 blocks (with specialised waves
-            // when K % 256 == 0: 43 us against 51 us on W[14336,4096], M = 65 .. 256; the first-generation kernel took
+            // when K % 256 == 0: 38 us against 51 us on W[14336,4096], M = 65 .. 256; the first-generation kernel took
             // 97 us), then 128x256 blocks of 8 waves (M = 384, 512: 72 .. 75 us against 96 us), each with three LDS
             // stages; 256x256 with two stages otherwise.  (Mixing in 256x192
             // blocks as the W8A8 launch does was measured neutral here: the narrow tile dequantises as many weights.)
@@ -1440,7 +1443,7 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
             if (mt > 65535) return AMCT_E_UNSUPPORTED;
 #define AMCT_LAUNCH_WIDE(SF)                                                                                           \
     {                                                                                                                  \
-        if (shape == 1 && K % 256 == 0 && G <= kSpecMaxG) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3>), dim3((unsigned)nt128, (unsigned)mt), dim3(512), 0, st, a); \
+        if (shape == 1 && K % 256 == 0 && G <= kSpecMaxG) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3>), dim3((unsigned)nt128, (unsigned)mt), dim3(kSpecThreads), 0, st, a); \
         else if (shape == 1) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 2, 2, 3>), dim3((unsigned)nt128, (unsigned)mt), dim3(256), 0, st, a); \
         else if (shape == 2) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 4, 2, 2, 3>), dim3((unsigned)nt256, (unsigned)mt), dim3(512), 0, st, a); \
         else hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 4, 4, 2, 2>), grid, dim3(kQThreads), 0, st, a);                \
