@@ -81,3 +81,60 @@ def int_weight_quant(tensor, bits=8, weight_clip_factor=None):
         bias = int4_assistance_bias(codes, scale)
         return pack_4bit(codes), scale_fp32_to_u64(scale), bias
     return codes, scale.to(torch.float32), None
+
+
+# ---- compressed-tensors description of a converted checkpoint ------------------------------------------
+# Host-side mirror of experimental/quantization/DeepSeekV3.2/deploy.py:171-238: the `quantization_config` block
+# that the converter writes into config.json, so that a checkpoint quantised here is described exactly as one the
+# reference converted.  Pure dictionaries; the field names are those of the compressed-tensors format.
+
+_PER_LAYER_UNQUANTISED = ("self_attn.indexer.wk", "self_attn.indexer.weights_proj", "self_attn.kv_b_proj",
+                          "self_attn.kv_a_proj_with_mqa", "self_attn.q_a_proj")
+
+
+def generate_ignore_item(num_layers, num_hidden_layers, first_k_dense_replace):
+    """Names of the modules that stay unquantised (deploy.py:171-188): five attention projections of every layer,
+    the MoE router of the sparse layers, the two extra heads of the multi-token-prediction layers, `lm_head`."""
+    names = []
+    for layer in range(num_layers):
+        prefix = "model.layers.%d." % layer
+        names.extend(prefix + leaf for leaf in _PER_LAYER_UNQUANTISED)
+        if layer >= first_k_dense_replace:
+            names.append(prefix + "mlp.gate")
+        if layer >= num_hidden_layers:
+            names.extend((prefix + "eh_proj", prefix + "shared_head.head"))
+    names.append("lm_head")
+    return names
+
+
+def generate_w4a8_quant(num_layers, first_k_dense_replace):
+    """The expert blocks of the sparse layers, which take the W4A8 scheme (deploy.py:191-196)."""
+    return ["model.layers.%d.mlp.experts" % layer for layer in range(first_k_dense_replace, num_layers)]
+
+
+def _tensor_scheme(num_bits, dynamic, observer, strategy):
+    return {"actorder": None, "block_structure": None, "dynamic": dynamic, "group_size": None, "num_bits": num_bits,
+            "observer": observer, "observer_kwargs": {}, "strategy": strategy, "symmetric": True, "type": "int"}
+
+
+def generate_quant_group(a_num_bits=8, w_num_bits=8, targets=None, activation_use_clip=False):
+    """One config group (deploy.py:199-211): dynamic per-token symmetric activations, static per-channel symmetric
+    weights."""
+    return {"input_activations": _tensor_scheme(a_num_bits, True, "memoryless", "token"),
+            "activation_use_clip": activation_use_clip,
+            "output_activations": None,
+            "targets": targets,
+            "weights": _tensor_scheme(w_num_bits, False, "minmax", "channel")}
+
+
+def generate_quant_config(c8, ignores, w4a8=False, clip=False):
+    """The whole `quantization_config` (deploy.py:214-238): group_0 = W8A8 on every Linear; with `w4a8` group_1 = W4A8
+    on the grouped expert GEMM; with `c8` an fp8 group-128 KV-cache scheme (its two flags are the strings the
+    reference writes, not booleans)."""
+    groups = {"group_0": generate_quant_group(8, 8, ["Linear"])}
+    if w4a8:
+        groups["group_1"] = generate_quant_group(8, 4, ["MoEGMM"], activation_use_clip=clip)
+    kv = {"num_bits": 8, "type": "float", "strategy": "group", "group_size": 128, "dynamic": "true",
+          "symmetric": "true"} if c8 else None
+    return {"config_groups": groups, "format": "int-quantized", "global_compression_ratio": 1, "ignore": ignores,
+            "kv_cache_scheme": kv, "quant_method": "compressed-tensors", "quantization_status": "compressed"}

@@ -55,3 +55,18 @@ def test_check_scale_offset_messages():
         qutils.check_scale_offset(torch.tensor([0.0]), None)
     with pytest.raises(RuntimeError, match="Param offset has invalid value inf or nan!"):
         qutils.check_scale_offset(torch.tensor([1.0]), torch.tensor([float('inf')]))
+
+
+def test_compressed_tensors_config_matches_the_fixture():
+    """The quantization_config block of a converted checkpoint (experimental/.../deploy.py:171-238) against
+    expected dictionaries written out by hand in tests/golden/quant_config_kat.json."""
+    import json
+    import os
+    from amct_amd import interchange as ic
+    kat = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "quant_config_kat.json")))
+    assert ic.generate_ignore_item(3, 2, 1) == kat["ignore_3_2_1"]
+    assert ic.generate_w4a8_quant(3, 1) == kat["w4a8_3_1"]
+    assert ic.generate_quant_config(True, ["lm_head"], w4a8=True, clip=True) == kat["config_c8_w4a8_clip"]
+    plain = ic.generate_quant_config(False, [])
+    assert plain["kv_cache_scheme"] is None and list(plain["config_groups"]) == ["group_0"]
+    assert json.loads(json.dumps(plain)) == plain          # serialisable as written
