@@ -108,3 +108,21 @@ def test_single_element_and_single_group(dev):
     got = ops.hif8_encode(x.to(dev)).cpu()
     want = oh.encode_bruteforce(x.float().numpy())
     assert torch.equal(got, torch.as_tensor(want).to(torch.uint8).reshape(-1))
+
+
+def test_mfma_yardstick_counts_its_operations(dev):
+    """The measurement aid of bench.py: one block of 8 waves per CU, 8 MFMAs per wave and iteration; the operation count
+    it reports follows from that, a zero-iteration call enqueues nothing, a null sink is refused."""
+    import ctypes
+    lib = _lib.load()
+    sink = torch.zeros(1024, dtype=torch.int32, device=dev)
+    ops_out = ctypes.c_int64(-1)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    for bf, per_mfma in ((0, 65536), (1, 32768)):
+        for rnd in (0, 1):
+            assert lib.amct_mfma_yardstick(bf, rnd, 3, sink.data_ptr(), ctypes.addressof(ops_out), _st(dev)) == 0
+            assert ops_out.value == cus * 8 * 8 * 3 * per_mfma
+    assert lib.amct_mfma_yardstick(0, 1, 0, sink.data_ptr(), ctypes.addressof(ops_out), _st(dev)) == 0 and ops_out.value == 0
+    assert lib.amct_mfma_yardstick(0, 1, 3, None, ctypes.addressof(ops_out), _st(dev)) == E_BADARG
+    torch.cuda.synchronize(dev)
+    assert int(sink.abs().sum()) == 0                      # the sink is never written in practice
