@@ -79,6 +79,13 @@ def test_w8a8_large_shapes_mixed_blocks(dev, M, N, K):
         out, acc = ops.gemm_w8a8(xq.to(dev), wq.to(dev), s_ch.to(dev), s_tok.to(dev), b.to(dev), out_dtype=odt, want_acc=True)
         assert torch.equal(acc.cpu().to(torch.int64), want_acc), "accumulators"
         assert_bits_equal(out, od.quant_matmul(xq, wq.t(), s_ch, s_tok, b, odt), "out %s" % odt)
+    # the other epilogue variants on the same operands: no per-token factor with an int32 bias (fp16 out), no bias at all
+    _, _, _, _, ib = w8a8_case(M, N, K, 133, False, 'int')
+    out, acc = ops.gemm_w8a8(xq.to(dev), wq.to(dev), s_ch.to(dev), None, ib.to(dev), out_dtype=torch.float16, want_acc=True)
+    assert torch.equal(acc.cpu().to(torch.int64), want_acc + ib.to(torch.int64)), "accumulators with int bias"
+    assert_bits_equal(out, od.quant_matmul(xq, wq.t(), s_ch, None, ib, torch.float16), "out fp16, int bias")
+    out = ops.gemm_w8a8(xq.to(dev), wq.to(dev), s_ch.to(dev), s_tok.to(dev), None)
+    assert_bits_equal(out, od.quant_matmul(xq, wq.t(), s_ch, s_tok, None, torch.bfloat16), "out bf16, no bias")
 
 
 def w4a16_case(M, N, K, group, seed, sdt=torch.float16):
