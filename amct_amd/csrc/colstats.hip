@@ -16,6 +16,7 @@ constexpr int kCsVecs = 32;            // column vectors per block
 constexpr int kCsLanes = 8;            // row lanes per block
 constexpr int kCsRows = 256;           // rows per chunk (before the chunk count is capped)
 constexpr int kCsMaxChunks = 64;
+constexpr int kCsUnroll = 16;          // rows in flight per lane (measured: 16.8 us against 17.5 us with 4)
 
 struct ColArgs {
     const void* x;
@@ -42,18 +43,18 @@ __global__ __launch_bounds__(kCsVecs * kCsLanes) void col_partial_k(ColArgs a) {
 
     float mx[VEC], mn[VEC];
     bool first = true;
-    // rows r0 + rl, + 8, + 16, ... of the chunk, four per iteration; the first iteration always runs (a row
+    // rows r0 + rl, + 8, + 16, ... of the chunk, kCsUnroll per iteration; the first iteration always runs (a row
     // lane beyond a short chunk re-reads the chunk's last row, which changes nothing)
     int64_t r = r0 + rl;
     do {
-        uint4 raw[4];
+        uint4 raw[kCsUnroll];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < kCsUnroll; ++u) {
             const int64_t rr = r + u * kCsLanes;
             raw[u] = ldg16_nt(base + (rr < r1 ? rr : r1 - 1) * row_bytes);   // duplicates do not change a max / min
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < kCsUnroll; ++u) {
             float x[VEC];
             unpack16<DT>(raw[u], x);
 #pragma unroll
@@ -64,7 +65,7 @@ __global__ __launch_bounds__(kCsVecs * kCsLanes) void col_partial_k(ColArgs a) {
             }
             first = false;
         }
-        r += 4 * kCsLanes;
+        r += kCsUnroll * kCsLanes;
     } while (r < r1);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
