@@ -480,7 +480,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 // any block shape the body supports, uniform over the launch (blockIdx.x: column tile, blockIdx.y: row tile)
 template <int ODT, int WM, int WN, int TI, int TJ, int STAGES, int LK>
-__global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void w8a8_tile_shape(W8A8Args a) {
+__global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM * WN / 4, WM * WN / 4))) void w8a8_tile_shape(W8A8Args a) {
     using Sh = DmaTile<WM, WN, TI, TJ, STAGES, LK>;
     __shared__ __attribute__((aligned(1024))) int8_t smem[Sh::kSmem];
     w8a8_dma_body<ODT, WM, WN, TI, TJ, STAGES, LK>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
