@@ -89,23 +89,6 @@ def build_cases(dev, only):
             assert rc == 0, rc
         cases.append(Case("copy", "hbm", 2 * nbytes, "B", launch, nsc, "u8", "plain copy of 128 MiB (yardstick)"))
 
-    # ---- matrix-pipe yardsticks: register-only MFMA loop with pseudo-random operands (about 100 us per launch) ---
-    import ctypes
-    for yname, bf, bound, ydesc in (("mfma_i8_yardstick", 0, "mfma_i8", "int8"), ("mfma_bf16_yardstick", 1, "mfma_bf16", "bf16")):
-        if want(yname):
-            sink = torch.zeros(1024, dtype=torch.int32, device=dev)
-            iters = 1500 if bf else 2500
-            ops_out = ctypes.c_int64(0)
-            rc = lib.amct_mfma_yardstick(bf, 1, iters, sink.data_ptr(), ctypes.addressof(ops_out), st)   # also sets ops_out
-            assert rc == 0, rc
-
-            def launch(i, bf=bf, iters=iters, sink=sink, ops_out=ops_out):
-                rc = lib.amct_mfma_yardstick(bf, 1, iters, sink.data_ptr(), ctypes.addressof(ops_out), st)
-                assert rc == 0, rc
-            cases.append(Case(yname, bound, ops_out.value, "OP", launch, 1, ydesc,
-                              "register-only %s MFMA loop on every CU, pseudo-random operands (yardstick: what the "
-                              "matrix pipe sustains under the power limit on such data)" % ydesc))
-
     # ---- K2 (headline): int4 asym g128 quant + pack, W[14336,4096] bf16 -------------------------
     if want("int4_group_pack"):
         w = workloads.c2_weight()
@@ -253,6 +236,24 @@ def build_cases(dev, only):
             assert rc == 0, rc
         cases.append(Case("gptq_block", "hbm", work, "B", launch, 2, "f32",
                           "GPTQ column loop of one 128-column block, W[14336,4096] fp32 (latency/ALU-bound: 128 dependent steps)"))
+
+    # ---- matrix-pipe yardsticks: register-only MFMA loop with pseudo-random operands, measured right before the
+    # GEMMs they are the yardstick for (and behind the bandwidth-bound kernels, which they would only heat up)
+    import ctypes
+    for yname, bf, bound, ydesc in (("mfma_i8_yardstick", 0, "mfma_i8", "int8"), ("mfma_bf16_yardstick", 1, "mfma_bf16", "bf16")):
+        if want(yname):
+            sink = torch.zeros(1024, dtype=torch.int32, device=dev)
+            iters = 1500 if bf else 2500
+            ops_out = ctypes.c_int64(0)
+            rc = lib.amct_mfma_yardstick(bf, 1, iters, sink.data_ptr(), ctypes.addressof(ops_out), st)   # also sets ops_out
+            assert rc == 0, rc
+
+            def launch(i, bf=bf, iters=iters, sink=sink, ops_out=ops_out):
+                rc = lib.amct_mfma_yardstick(bf, 1, iters, sink.data_ptr(), ctypes.addressof(ops_out), st)
+                assert rc == 0, rc
+            cases.append(Case(yname, bound, ops_out.value, "OP", launch, 1, ydesc,
+                              "register-only %s MFMA loop on every CU, pseudo-random operands (yardstick: what the "
+                              "matrix pipe sustains under the power limit on such data)" % ydesc))
 
     # ---- K6: W8A8 Linear, W[14336,4096] int8 ----------------------------------------------------------
     if want("w8a8_m2048") or want("w8a8_m16"):
