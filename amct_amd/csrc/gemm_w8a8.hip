@@ -309,7 +309,7 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
     // loop, waits for the youngest LDS reads too early.  The loop is therefore branch-free: the last iteration
     // reads one stage too far (valid LDS, values unused).
     constexpr int kNM = TI * TJ, kNR = TI + TJ;
-    static_assert(kNM >= kNR, "one fragment read per MFMA");
+    constexpr int kRPM = (kNR + kNM - 1) / kNM;                     // fragment reads behind each MFMA
     // fragment q in the order the MFMAs need them: A0, B0, B1, .., A1, A2, ..
     auto read_one = [&](int stg, int ks, int q, v4i (&fa)[TI], v4i (&fb)[TJ]) {
         const int8_t* st = smem + stg * kLStageBytes;
@@ -339,9 +339,12 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
             for (int m = 0; m < kNM; ++m) {
                 mfma_one(m, fa[ks & 1], fb[ks & 1]);
                 __builtin_amdgcn_sched_barrier(0);
-                if (m < kNR) {
-                    read_one(stage, ks + 1, m, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
-                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int q = kRPM * m; q < kRPM * (m + 1); ++q) {
+                    if (q < kNR) {
+                        read_one(stage, ks + 1, q, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
             }
         }
@@ -355,9 +358,12 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
         for (int m = 0; m < kNM; ++m) {
             mfma_one(m, fa[(kKS - 1) & 1], fb[(kKS - 1) & 1]);
             __builtin_amdgcn_sched_barrier(0);
-            if (m < kNR) {
-                read_one(next, 0, m, fa[0], fb[0]);
-                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int q = kRPM * m; q < kRPM * (m + 1); ++q) {
+                if (q < kNR) {
+                    read_one(next, 0, q, fa[0], fb[0]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
         }
         stage = next;
@@ -752,7 +758,11 @@ extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s
     W8A8Args a{xq, wq, s_tok, s_ch, bias_kind ? bias : nullptr, out, acc_out, M, N, K, bias_kind, out_dtype};
     hipStream_t st = (hipStream_t)stream;
     const bool vec_ok = (K % 16 == 0) && aligned16(xq) && aligned16(wq);
-    if (vec_ok && M <= 16 && K % 256 == 0) {
+    // the tile kernels (direct-to-LDS loads, MFMA 32x32x32): K a multiple of 128, 16-byte pieces of whole output rows,
+    // operands below 4 GiB (32-bit lane offsets)
+    const bool tile_ok = vec_ok && K % 128 == 0 && N % 8 == 0 && aligned16(out) && M * K < (int64_t(1) << 32) &&
+                         N * K < (int64_t(1) << 32);
+    if (vec_ok && M <= 16 && K % 256 == 0 && (M <= 2 || !tile_ok)) {
         const int iters = (int)(K / 256);
         // measured: blocks of 2 or 4 waves, several per CU, stream best (one block's start-up and reduction
         // overlap with another's loads); wider blocks only pay when the activations are large
@@ -765,21 +775,28 @@ extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s
         if (lds) rc = tn == 1 ? launch_w8a8_decode_w<1>(a, waves, lds, st) : launch_w8a8_decode_w<2>(a, waves, lds, st);
         if (rc != AMCT_E_UNSUPPORTED) return rc;
     }
-    // Medium M: as long as all tiles of a launch run at once (one or two blocks per CU), small tiles on many CUs beat
-    // large tiles on few.  128x128 tiles of 4 waves (measured on W[14336,4096]: 22 us for M = 24 .. 256 against
-    // 26 .. 42 us for the skinny / first-generation / 256x256 kernels), then 128x256 tiles of 8 waves (M = 384, 512:
-    // 32 us against 43 us); three LDS stages, because a short step exposes the load latency that two stages cover
-    // for a 256x256 tile.
-    if (vec_ok && M > 16 && K % 128 == 0 && N % 8 == 0 && aligned16(out) && M * K < (int64_t(1) << 32) && N * K < (int64_t(1) << 32)) {
+    // Small and medium M: as long as all tiles of a launch run at once, small tiles on many CUs beat large tiles on
+    // few, and a short step exposes the load latency that two LDS stages cover for a 256x256 tile.  The smallest block
+    // shape whose blocks fit the CUs in one round is taken (measured on W[14336,4096], us per call):
+    //   64x64,   4 waves of 32x32, 4 stages : M = 3 .. 64   15.2 .. 16.1  (weight-streaming decode kernel: 16.4 .. 19.5 at
+    //                                                        M = 3 .. 16; it stays for M <= 2: 14.4 against 15.1)
+    //   128x64,  4 waves of 64x32, 4 stages : M = 65 .. 128 17.5 .. 19.3
+    //   128x128, 4 waves of 64x64, 3 stages : M <= 256      25     (first-generation 128x128 kernel: 39 .. 42)
+    //   128x256, 8 waves of 64x64, 3 stages : M <= 512      32     (256x256 tiles: 43)
+    if (tile_ok) {
         const int64_t cus = current_cu_count();
-        const int64_t mt = (M + 127) / 128, nt128 = (N + 127) / 128, nt256 = (N + 255) / 256;
+        const int64_t mt = (M + 127) / 128, nt64 = (N + 63) / 64, nt128 = (N + 127) / 128, nt256 = (N + 255) / 256;
         int shape = 0;
-        if (cus > 0 && mt * nt128 <= cus) shape = 1;
-        else if (cus > 0 && (mt * nt256 <= cus || M < 256)) shape = 2;
+        if (cus > 0 && M <= 64 && nt64 <= cus) shape = 1;
+        else if (cus > 0 && mt * nt64 <= cus) shape = 2;
+        else if (cus > 0 && mt * nt128 <= cus) shape = 3;
+        else if (cus > 0 && (mt * nt256 <= cus || M < 256)) shape = 4;
         if (shape && mt <= 65535) {
 #define AMCT_LAUNCH_MID(ODT)                                                                                          \
     {                                                                                                                 \
-        if (shape == 1) hipLaunchKernelGGL((w8a8_tile_shape<ODT, 2, 2, 2, 2, 3, 128>), dim3((unsigned)nt128, (unsigned)mt), dim3(256), 0, st, a); \
+        if (shape == 1) hipLaunchKernelGGL((w8a8_tile_shape<ODT, 2, 2, 1, 1, 4, 128>), dim3((unsigned)nt64, 1), dim3(256), 0, st, a);             \
+        else if (shape == 2) hipLaunchKernelGGL((w8a8_tile_shape<ODT, 2, 2, 2, 1, 4, 128>), dim3((unsigned)nt64, (unsigned)mt), dim3(256), 0, st, a);  \
+        else if (shape == 3) hipLaunchKernelGGL((w8a8_tile_shape<ODT, 2, 2, 2, 2, 3, 128>), dim3((unsigned)nt128, (unsigned)mt), dim3(256), 0, st, a); \
         else hipLaunchKernelGGL((w8a8_tile_shape<ODT, 2, 4, 2, 2, 3, 128>), dim3((unsigned)nt256, (unsigned)mt), dim3(512), 0, st, a);            \
     }
             if (out_dtype == AMCT_BF16) AMCT_LAUNCH_MID(AMCT_BF16)

@@ -69,9 +69,10 @@ def test_w8a8_vs_oracle(dev, M, N, K, per_token, bias):
 
 @pytest.mark.parametrize("M,N,K", [(300, 1000, 320), (256, 448, 128), (512, 832, 256), (2048, 14336, 192), (1100, 9000, 64),
                                    (2000, 14328, 128), (100, 1000, 256), (200, 520, 384), (384, 14336, 128), (17, 72, 128),
-                                   (640, 14336, 128), (33, 40000, 128)])
+                                   (640, 14336, 128), (33, 40000, 128), (5, 64, 128), (3, 14336, 384), (64, 200, 384),
+                                   (33, 14336, 256), (100, 14336, 128), (128, 8200, 256), (16, 40000, 128), (1, 16392, 128)])
 def test_w8a8_large_shapes_mixed_blocks(dev, M, N, K):
-    """Block shapes of the tile kernels: 128x128 and 128x256 blocks for medium M, 256x256 for large M, where a launch
+    """Block shapes of the tile kernels: 64x64 and 128x64 blocks for small M, 128x128 and 128x256 for medium M, 256x256 for large M, where a launch
     may mix in 256x192 blocks so that the blocks fill the CUs evenly; ragged edges in M and N, accumulators bit for bit."""
     xq, wq, s_ch, s_tok, b = w8a8_case(M, N, K, 131, True, 'float')
     want_acc = od.int8_matmul_exact(xq, wq.t())
