@@ -447,6 +447,9 @@ AMCT_DEV void dma16s(uint32_t lds_addr, const void* sbase, uint32_t voff) {
 AMCT_DEV void gload16s(u4v& dst, const void* sbase, uint32_t voff) {
     asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(dst) : "v"(voff), "s"(sbase) : "memory");
 }
+AMCT_DEV void gload16s(u2v& dst, const void* sbase, uint32_t voff) {   // 8 bytes: the quarter-row share of a step
+    asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(dst) : "v"(voff), "s"(sbase) : "memory");
+}
 AMCT_DEV void gload_u16s(uint32_t& dst, const void* sbase, uint32_t voff) {
     asm volatile("global_load_ushort %0, %1, %2" : "=v"(dst) : "v"(voff), "s"(sbase) : "memory");
 }
@@ -463,7 +466,9 @@ struct WideTile {
     static constexpr int kNA = (kLM * kWRow / 1024) / kLW;         // activation pieces (8 rows x 128 B) per loading wave
     static constexpr int kEpi = kWaves * 16384;
     static constexpr int kSmem = STAGES * kStageBytes > kEpi ? STAGES * kStageBytes : kEpi;
-    static_assert(kThreads == 2 * kLN, "every thread dequantises half a weight row of the tile per step");
+    static constexpr int kQ = kThreads / kLN;                     // threads per weight row of the tile
+    static constexpr int kBC = 8 / kQ;                             // 8-weight chunks a thread dequantises per step
+    static_assert(kThreads == 2 * kLN || kThreads == 4 * kLN, "every thread dequantises a half or a quarter of a weight row of the tile per step");
     static_assert((kLM * kWRow / 1024) % kLW == 0 && kSmem <= 160 * 1024, "tile shape");
     static_assert(kNA < 64, "vmcnt range");
 };
@@ -473,7 +478,8 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
     using Sh = WideTile<WM, WN, TI, TJ, STAGES>;
     constexpr int kLM = Sh::kLM, kStageBytes = Sh::kStageBytes, kWaves = Sh::kWaves, kLW = Sh::kLW, kNA = Sh::kNA;
     constexpr int kNM = TI * TJ, kNR = TI + TJ;                    // MFMAs and fragment reads per k-slice
-    static_assert(kNM >= kNR && (STAGES == 2 || STAGES == 3), "one fragment read per MFMA; 2 or 3 stages");
+    constexpr int kRPM = (kNR + kNM - 1) / kNM;                    // fragment reads issued behind each MFMA
+    static_assert(STAGES == 2 || STAGES == 3, "2 or 3 stages");
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
@@ -504,16 +510,17 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
                 dma16s(lds0 + stg * kStageBytes + (lw * kNA + j) * 1024, a.x + (int64_t)st * kWK, goff[j]);
         }
     };
-    // weight row of this thread: row tid/2 of the tile, 32 weights (16 bytes) per step, which half from tid%2
-    const int brow = tid >> 1, bhalf = tid & 1;
+    // weight row of this thread: row tid/kQ of the tile, 8*kBC weights (4*kBC bytes) per step, which part from tid%kQ
+    constexpr int kQ = Sh::kQ, kBC = Sh::kBC;
+    const int brow = tid / kQ, bpart = tid % kQ;
     const int64_t wrow = (n0 + brow < a.N) ? n0 + brow : a.N - 1;
-    const uint32_t woff = (uint32_t)(wrow * (a.K / 2) + bhalf * 16);
+    const uint32_t woff = (uint32_t)(wrow * (a.K / 2) + bpart * (4 * kBC));
     const uint32_t soff = (uint32_t)(wrow * G * 2), zoff = (uint32_t)(wrow * G);
-    int bdst[4];
+    int bdst[kBC];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) bdst[c] = kLM * kWRow + brow * kWRow + ((4 * bhalf + c) ^ swz(brow)) * 16;
+    for (int c = 0; c < kBC; ++c) bdst[c] = kLM * kWRow + brow * kWRow + ((kBC * bpart + c) ^ swz(brow)) * 16;
 
-    u4v wreg[2];
+    typename std::conditional<kBC == 4, u4v, u2v>::type wreg[2];
     uint32_t sreg[2], zreg[2];
     auto issue_b = [&](int slot, int step) {                       // the weight loads of K-step `step`
         const int st = step < last ? step : last;
@@ -587,7 +594,7 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
     AMCT_TIE_SLOT(1);
     factors(0);
 #pragma unroll
-    for (int c = 0; c < 4; ++c) write_b(0, 0, c);
+    for (int c = 0; c < kBC; ++c) write_b(0, 0, c);
     issue_b(0, 2);
     dma_a(STAGES - 1, STAGES - 1);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -608,12 +615,11 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
         __builtin_amdgcn_sched_barrier(0);                                             \
         _Pragma("unroll") for (int m_ = 0; m_ < kNM; ++m_) mfma_one(m_, fa[(KS) & 1], fb[(KS) & 1]); \
         _Pragma("unroll") for (int q_ = 0; q_ < kNR; ++q_) read_one(CUR, (KS) + 1, q_, fa[((KS) + 1) & 1], fb[((KS) + 1) & 1]); \
-        write_b(SL, NXT, 2 * (KS));                                                    \
-        write_b(SL, NXT, 2 * (KS) + 1);                                                \
+        _Pragma("unroll") for (int c_ = 0; c_ < kBC / 2; ++c_) write_b(SL, NXT, (kBC / 2) * (KS) + c_); \
         _Pragma("unroll") for (int g_ = 0; g_ < kNM; ++g_) {                           \
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                      /* 1 MFMA */ \
-            __builtin_amdgcn_sched_group_barrier(0x002, (56 + kNM - 1) / kNM, 0);   /* VALU   */ \
-            __builtin_amdgcn_sched_group_barrier(0x080, kNM >= kNR + 2 ? 1 : 2, 0); /* DS     */ \
+            __builtin_amdgcn_sched_group_barrier(0x002, (14 * kBC + kNM - 1) / kNM, 0); /* VALU */ \
+            __builtin_amdgcn_sched_group_barrier(0x080, (kNR + kBC / 2 + kNM - 1) / kNM, 0); /* DS */ \
         }                                                                              \
         __builtin_amdgcn_sched_barrier(0);                                             \
     }
@@ -622,8 +628,8 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
         _Pragma("unroll") for (int m_ = 0; m_ < kNM; ++m_) {                           \
             mfma_one(m_, fa[(KS) & 1], fb[(KS) & 1]);                                  \
             __builtin_amdgcn_sched_barrier(0);                                         \
-            if (m_ < kNR) {                                                            \
-                read_one(STG, KSREAD, m_, fa[((KS) + 1) & 1], fb[((KS) + 1) & 1]);     \
+            _Pragma("unroll") for (int q_ = m_ * kRPM; q_ < (m_ + 1) * kRPM && q_ < kNR; ++q_) { \
+                read_one(STG, KSREAD, q_, fa[((KS) + 1) & 1], fb[((KS) + 1) & 1]);     \
                 __builtin_amdgcn_sched_barrier(0);                                     \
             }                                                                          \
         }                                                                              \
@@ -1388,7 +1394,15 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
         }
         if (rc != AMCT_E_UNSUPPORTED) return rc;
     }
-    if (vec_ok && M <= 64 && K % 128 == 0 && K < 65536 && group % 32 == 0) {
+    // The weight-streaming kernel below serves M <= 24 (25 us on W[14336,4096] at M = 17, 29 us at M = 32, 40 us at
+    // M = 64; 64x64 tiles take 26 us for any M <= 64), and larger M up to 64 where the tile kernels do not apply; when
+    // the activations are to be smoothed the tile path pays a pre-pass, so the switch comes later.
+    const bool tiles_apply = vec_ok && K % 128 == 0 && K < 65536 && N % 8 == 0 && aligned16(out) && group % 64 == 0 &&
+                             M * K * 2 < (int64_t(1) << 32) && N * (K / 2) < (int64_t(1) << 32) &&
+                             N * (K / group) * 2 < (int64_t(1) << 32) &&
+                             (!smooth || (workspace && workspace_bytes >= (size_t)(M * K * 2) && aligned16(workspace)));
+    const int64_t small_tiles_from = smooth ? 41 : 25;
+    if (vec_ok && M <= 64 && K % 128 == 0 && K < 65536 && group % 32 == 0 && !(tiles_apply && M >= small_tiles_from)) {
         const dim3 grid((unsigned)((N + kDN - 1) / kDN));
         const int iters = (int)(K / 128);
 #define AMCT_DEC2(MT, SM)                                                                                    \
@@ -1409,9 +1423,7 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
 #undef AMCT_DEC
         return hip_status();
     }
-    // 16 < M <= 64 stays with the weight-streaming decode kernel above (25 .. 40 us on W[14336,4096] against 51 us for
-    // the smallest tile shape here)
-    if (vec_ok && M > 64 && K % 128 == 0 && K < 65536 && N % 8 == 0 && aligned16(out)) {
+    if (vec_ok && (M > 64 || (tiles_apply && M >= small_tiles_from)) && K % 128 == 0 && K < 65536 && N % 8 == 0 && aligned16(out)) {
         const dim3 grid((unsigned)((N + kQN - 1) / kQN), (unsigned)((M + kQM - 1) / kQM));
         if (grid.y > 65535) return AMCT_E_UNSUPPORTED;
         const int64_t G = K / group;
@@ -1431,19 +1443,24 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
         if (wide) {
             // Block shape: as long as all tiles of a launch run at once, small tiles on many CUs beat large tiles on
             // few (the weight stream is the bulk of the traffic for medium M): 128x128 blocks (with specialised waves
-            // when K % 256 == 0: 38 us against 51 us on W[14336,4096], M = 65 .. 256; the first-generation kernel took
-            // 97 us), then 128x256 blocks of 8 waves (M = 384, 512: 72 .. 75 us against 96 us), each with three LDS
+            // when K % 256 == 0: 38 us against 51 us on W[14336,4096], M = 129 .. 256; the first-generation kernel took
+            // 97 us; 64-column blocks of 4 waves, a quarter of a weight row per thread and step, while they still fit the
+            // CUs in one round: 64x64 for M <= 64, 26 us, and 128x64 for M <= 128, 34 us), then 128x256 blocks of 8 waves (M = 384, 512: 72 .. 75 us against 96 us), each with three LDS
             // stages; 256x256 with two stages otherwise.  (Mixing in 256x192
             // blocks as the W8A8 launch does was measured neutral here: the narrow tile dequantises as many weights.)
             const int64_t cus = current_cu_count();
-            const int64_t mt = (M + 127) / 128, nt128 = (N + 127) / 128, nt256 = (N + 255) / 256;
+            const int64_t mt = (M + 127) / 128, nt64 = (N + 63) / 64, nt128 = (N + 127) / 128, nt256 = (N + 255) / 256;
             int shape = 0;
-            if (cus > 0 && mt * nt128 <= cus) shape = 1;
+            if (cus > 0 && M <= 64 && nt64 <= cus) shape = 3;
+            else if (cus > 0 && mt * nt64 <= cus) shape = 4;
+            else if (cus > 0 && mt * nt128 <= cus) shape = 1;
             else if (cus > 0 && (mt * nt256 <= cus || M < 256)) shape = 2;
             if (mt > 65535) return AMCT_E_UNSUPPORTED;
 #define AMCT_LAUNCH_WIDE(SF)                                                                                           \
     {                                                                                                                  \
-        if (shape == 1 && K % 256 == 0 && G <= kSpecMaxG) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3>), dim3((unsigned)nt128, (unsigned)mt), dim3(kSpecThreads), 0, st, a); \
+        if (shape == 3) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 1, 1, 3>), dim3((unsigned)nt64, 1), dim3(256), 0, st, a);          \
+        else if (shape == 4) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 2, 1, 3>), dim3((unsigned)nt64, (unsigned)mt), dim3(256), 0, st, a); \
+        else if (shape == 1 && K % 256 == 0 && G <= kSpecMaxG) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3>), dim3((unsigned)nt128, (unsigned)mt), dim3(kSpecThreads), 0, st, a); \
         else if (shape == 1) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 2, 2, 3>), dim3((unsigned)nt128, (unsigned)mt), dim3(256), 0, st, a); \
         else if (shape == 2) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 4, 2, 2, 3>), dim3((unsigned)nt256, (unsigned)mt), dim3(512), 0, st, a); \
         else hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 4, 4, 2, 2>), grid, dim3(kQThreads), 0, st, a);                \

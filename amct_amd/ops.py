@@ -395,8 +395,9 @@ def gemm_w4a16(x, wq_packed, scales, zeros, group, smooth=None, bias=None):
     if bias is not None:
         bias = _c(bias.to(torch.float32))
     out = torch.empty(M, N, dtype=x.dtype, device=dev)
-    # with smoothing and a large M the caller-owned workspace lets the multiply run once up front
-    ws = torch.empty(M, K, dtype=x.dtype, device=dev) if (smooth is not None and M >= 256) else None
+    # with smoothing the caller-owned workspace lets the multiply run once up front (the tile kernels need that;
+    # below 41 rows the library takes its weight-streaming kernels, which smooth in place)
+    ws = torch.empty(M, K, dtype=x.dtype, device=dev) if (smooth is not None and M > 40) else None
     with torch.cuda.device(dev):
         _lib.check(_lib.load().amct_gemm_w4a16(_p(x), _p(smooth), _p(wq_packed), _p(scales), dtype_code(scales.dtype),
                                                _p(zeros), _p(bias), _p(out), M, N, K, group, dtype_code(x.dtype),

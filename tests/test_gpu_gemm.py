@@ -109,10 +109,11 @@ def w4a16_oracle(x, codes, scales, zeros, group, smooth, bias):
 @pytest.mark.parametrize("M,N,K,group", [(300, 1000, 256, 64), (256, 448, 128, 128), (2048, 14336, 256, 128), (2000, 14328, 128, 64),
                                          (65, 72, 128, 64), (100, 1000, 384, 128), (200, 520, 640, 64), (384, 14336, 128, 128),
                                          (130, 40000, 128, 64), (640, 14336, 256, 128), (100, 1000, 512, 128), (256, 136, 1024, 64),
-                                         (65, 14336, 256, 256)])
+                                         (65, 14336, 256, 256), (25, 200, 128, 64), (40, 14336, 256, 128), (48, 40000, 128, 64),
+                                         (100, 14336, 128, 128), (128, 8200, 256, 64), (64, 14336, 128, 128)])
 def test_w4a16_large_shapes_ragged(dev, M, N, K, group):
-    """The wide tile kernels (M > 64, group % 64 == 0) in their block shapes (128x128 with and without specialised waves, 128x256, 256x256;
-    two or three LDS stages) on ragged edges in M and N, both scale dtypes."""
+    """The wide tile kernels (M > 24, group % 64 == 0) in their block shapes (64x64, 128x64, 128x128 with and without specialised
+    waves, 128x256, 256x256; two or three LDS stages) on ragged edges in M and N, both scale dtypes."""
     for sdt in (torch.float16, torch.bfloat16):
         x, codes, scales, zeros, smooth, bias = w4a16_case(M, N, K, group, 137, sdt)
         packed = workloads.pack_nibbles(codes)
@@ -121,6 +122,12 @@ def test_w4a16_large_shapes_ragged(dev, M, N, K, group):
         err = (out.cpu().double() - want).abs()
         tol = 1e-3 * want.abs().amax(dim=1, keepdim=True) + want.abs() * 2.0 ** -8
         assert (err <= tol).all(), (err.max().item(), tol.min().item())
+    # with smoothing: the pre-pass into the workspace, then the same kernels
+    out = ops.gemm_w4a16(x.to(dev), packed.to(dev), scales.to(dev), zeros.to(dev), group, smooth.to(dev), None)
+    want = w4a16_oracle(x, codes, scales, zeros, group, smooth, None)
+    err = (out.cpu().double() - want).abs()
+    tol = 1e-3 * want.abs().amax(dim=1, keepdim=True) + want.abs() * 2.0 ** -8
+    assert (err <= tol).all(), (err.max().item(), tol.min().item())
 
 
 @pytest.mark.parametrize("M,N,K,group", [(1, 64, 256, 128), (16, 128, 512, 128), (7, 33, 128, 32), (64, 64, 256, 64),
