@@ -743,12 +743,21 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
         // Per-step loads of a 2-byte scale and a 1-byte zero-point per thread touch 48 cache lines per wave
         // instruction; all of the tile's factors are fetched once instead, by all 512 threads.
         const uint32_t G = (uint32_t)(a.K / a.group);
-        for (uint32_t e = tid; e < (uint32_t)kLN * G; e += kSpecThreads) {
-            const uint32_t row = e / G, g = e - row * G;
-            const int64_t wr = (n0 + row < a.N) ? n0 + row : a.N - 1;
-            const uint32_t sbits = reinterpret_cast<const uint16_t*>(a.scales)[wr * G + g];
-            tab[row * (kSpecMaxG + 1) + g] = sbits | ((uint32_t)a.zeros[wr * G + g] << 16);
+        // kTPR threads share a row; all loads are issued before the first use (unconditional, clamped): a loop that
+        // loads and stores entry by entry pays one memory latency per trip before the kernel's first MFMA
+        constexpr int kTPR = kSpecThreads / kLN, kIt = (kSpecMaxG + kTPR - 1) / kTPR;
+        const uint32_t row = tid / kTPR, g0 = tid % kTPR;
+        const int64_t wr = (n0 + row < a.N) ? n0 + row : a.N - 1;
+        uint32_t sb[kIt], zb[kIt];
+#pragma unroll
+        for (int j = 0; j < kIt; ++j) {
+            const uint32_t g = g0 + j * kTPR < G ? g0 + j * kTPR : G - 1;
+            sb[j] = reinterpret_cast<const uint16_t*>(a.scales)[wr * G + g];
+            zb[j] = a.zeros[wr * G + g];
         }
+#pragma unroll
+        for (int j = 0; j < kIt; ++j)
+            if (g0 + j * kTPR < G) tab[row * (kSpecMaxG + 1) + g0 + j * kTPR] = sb[j] | (zb[j] << 16);
         __syncthreads();
     }
 
