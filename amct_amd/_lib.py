@@ -33,6 +33,8 @@ SIGNATURES = {
     "amct_scale_f32_to_u64": (_I, [_P, _P, _L, _P]),
     "amct_col_minmax_workspace_bytes": (ctypes.c_size_t, [_L, _L]),
     "amct_col_minmax": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _P, ctypes.c_size_t, _P]),
+    "amct_awq_loss_workspace_bytes": (ctypes.c_size_t, []),
+    "amct_awq_loss": (_I, [_P, _P, _L, _I, _P, _P, ctypes.c_size_t, _P]),
     "amct_scale_offset": (_I, [_P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _P]),
     "amct_quant_with_params": (_I, [_P, _P, _P, _P, _P, _I, _P, _I, _L, _L, _I, _I, _I, _I, _I, _I, _P]),
     "amct_fakequant_int": (_I, [_P, _P, _P, _I, _P, _P, _P, _P, _I, _L, _L, _I, _I, _I, _I, _I, _I, _I, _I, _P]),

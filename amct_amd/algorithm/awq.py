@@ -88,8 +88,8 @@ def search_scale(inputs, layers, block, quant_config, kwargs=None):
     value and errors as the reference.  The reference copies the whole state dict of `block` to the host
     once and loads it back after every grid point; only the weights of `layers` change inside the loop
     (process_weights_for_layers, which replaces layer.weight.data by a new tensor and never writes into the
-    old one), so here the original weight tensors are simply kept and put back: no copy at all, and the
-    fake-quant of a grid point is one fused kernel per layer."""
+    old one), so here the original weight tensors are simply kept and put back: no copy at all, the
+    fake-quant of a grid point is one fused kernel per layer and its loss one pass over the two outputs."""
     _require_finite(inputs, layers)
     kwargs = kwargs or {}
     grids_num = quant_config.get("algorithm").get('awq').get('grids_num')
@@ -101,7 +101,7 @@ def search_scale(inputs, layers, block, quant_config, kwargs=None):
         for grid in range(grids_num):
             candidate = awq_scale_for_ratio(channel_mean, grid / grids_num, inputs.dtype)
             process_weights_for_layers(layers, candidate, quant_config)
-            loss = (target - _first_output(block, inputs, kwargs)).float().pow(4).mean()
+            loss = ops.awq_loss(target, _first_output(block, inputs, kwargs))
             if not torch.isnan(loss) and loss < winner_loss:
                 winner, winner_loss = candidate, loss
             for layer, w in zip(layers, originals):

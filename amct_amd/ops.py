@@ -86,6 +86,22 @@ def col_minmax(x, col_max=None, col_min=None, absolute=False):
     return col_max if absolute else (col_max, col_min)
 
 
+def awq_loss(y, yhat):
+    """mean((y - yhat)^4) as a 0-d fp32 tensor on the device, the difference rounded to the tensors' dtype
+    (algorithm/awq.py:96); one pass over both tensors."""
+    dev = _dev(y, yhat)
+    if y.dtype != yhat.dtype or y.shape != yhat.shape:
+        raise RuntimeError("awq_loss: the two outputs must share dtype and shape")
+    y, yhat = _c(y), _c(yhat)
+    lib = _lib.load()
+    nbytes = lib.amct_awq_loss_workspace_bytes()
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    loss = torch.empty((), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(lib.amct_awq_loss(_p(y), _p(yhat), y.numel(), dtype_code(y.dtype), _p(loss), _p(ws), nbytes, _stream(dev)))
+    return loss
+
+
 def scale_offset(vmax, vmin, bits, symmetric, scope_rule=SCOPE_AMCT, bad=None):
     """Elementwise (max, min) -> (scale fp32, offset int32 | None), same shape as the inputs."""
     dev = _dev(vmax, vmin, bad)

@@ -97,6 +97,18 @@ size_t amct_col_minmax_workspace_bytes(int64_t rows, int64_t cols);
 int amct_col_minmax(const void* x, float* col_max, float* col_min, int64_t rows, int64_t cols, int absolute,
                     int accumulate, int dtype, void* workspace, size_t workspace_bytes, amct_stream_t stream);
 
+/* ---- loss of one AWQ grid point ---------------------------------------------------------------------
+ * Replaces the expression of amct_pytorch/algorithm/awq.py:96, `(ori_out - quant_out).float().pow(4).mean()`:
+ * loss[0] (fp32, device) = mean over the n elements of (dtype(y - yhat))^4, the difference rounded to the
+ * tensors' dtype as the reference's subtraction does, the fourth power and the sum in fp32.  One pass over
+ * both tensors; the summation order is fixed by n (same result on every call and device) but is not torch's,
+ * so the value agrees with the reference's to the rounding of an fp32 sum.  n = 0 gives NaN, as torch does.
+ * y, yhat 16-byte aligned; workspace: amct_awq_loss_workspace_bytes() bytes of device memory, 4-byte aligned,
+ * contents irrelevant before and after the call. */
+size_t amct_awq_loss_workspace_bytes(void);
+int amct_awq_loss(const void* y, const void* yhat, int64_t n, int dtype, float* loss, void* workspace,
+                  size_t workspace_bytes, amct_stream_t stream);
+
 /* ---- A1: min / max per row (group = 0) or per group of `group` columns ----------------
  * Replaces get_weight_min_max_by_granularity (amct_pytorch/quantize_op/utils.py:111-136)
  * and the per-token reductions of amct_pytorch/quantize_op/minmax_module.py:96-105.

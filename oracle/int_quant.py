@@ -298,6 +298,16 @@ def static_quantize(x, scales, zero_points, axis=-1):
     return t.round().clamp(-128, 127).to(torch.int8)
 
 
+def awq_loss(ori_out, quant_out):
+    """The loss of one AWQ grid point (amct_pytorch/algorithm/awq.py:96): the difference in the tensors' own
+    dtype (one rounding), its fourth power and the mean in fp64 (the reference's fp32 mean is one rounding of
+    this sum order-for-order; comparisons against it carry that tolerance).  Pinned by closed forms in the
+    tests: a constant difference d gives d^4, a single non-zero difference d gives d^4 / n, the sign of the
+    difference does not matter, and a difference that the dtype cannot represent is rounded first."""
+    d = (ori_out - quant_out).double()
+    return float((d * d * d * d).mean()) if d.numel() else float('nan')
+
+
 def awq_search_scale(inputs, weights, forward, grids_num, kind, strategy, symmetric, group_size=None):
     """The AWQ scale search (amct_pytorch/algorithm/awq.py:52-105) on plain tensors: `weights` are the
     [N,K] weights of the layers that share the input, `forward(inputs, weights)` evaluates the block.

@@ -5,7 +5,7 @@ import types
 import pytest
 import torch
 
-from amct_amd import torch_hip
+from amct_amd import ops, torch_hip
 from amct_amd.algorithm import awq
 from amct_amd.deploy_op import HipQuantizationLinear, HipWeightQuantizedLinear
 from amct_amd.quantize_op import utils as qutils
@@ -316,3 +316,26 @@ def test_awq_search_scale_on_device(dev, strategy, group, sym):
         bad[0, 0] = float('nan')
         awq.search_scale(bad.to(dev), [dblock.a, dblock.b], dblock, c)
     assert best >= 0
+
+
+@pytest.mark.parametrize("dt", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n", [1, 7, 8, 1000, 4099, 262144, 8 * 1024 * 1024 + 5])
+def test_awq_loss_kernel(dev, dt, n):
+    """mean((y - yhat)^4) in one pass against the fp64 restatement: 2e-6 relative (fp32 sum in a fixed order that
+    is not torch's), identical bits on a second call, NaN for an empty tensor and for a NaN element."""
+    g = torch.Generator().manual_seed(n % 1000 + 3)
+    y = (3.0 * torch.randn(n, generator=g)).to(dt)
+    yh = (y.float() + 0.2 * torch.randn(n, generator=g)).to(dt)
+    got = ops.awq_loss(y.to(dev), yh.to(dev))
+    want = iq.awq_loss(y, yh)
+    assert got.dtype == torch.float32 and got.dim() == 0
+    assert abs(float(got) - want) <= 2e-6 * want, (float(got), want)
+    again = ops.awq_loss(y.to(dev), yh.to(dev))
+    assert torch.equal(got.cpu().view(torch.int32), again.cpu().view(torch.int32))
+    if n == 1000:
+        bad = y.clone()
+        bad[n // 2] = float('nan')
+        assert torch.isnan(ops.awq_loss(bad.to(dev), yh.to(dev)))
+        assert torch.isnan(ops.awq_loss(y[:0].to(dev), yh[:0].to(dev)))
+        with pytest.raises(RuntimeError):
+            ops.awq_loss(y.to(dev), yh[:-1].to(dev))

@@ -328,3 +328,26 @@ def test_gptq_block_loop_against_scalar_model():
                     w[r, j] = np.float32(w[r, j] - np.float32(err * hinv[i, j]))
         assert np.array_equal(got_w.numpy().view(np.uint32), w.view(np.uint32))
         assert np.array_equal(got_e.numpy().view(np.uint32), e.view(np.uint32))
+
+
+def test_awq_loss_closed_forms():
+    """oracle.int_quant.awq_loss against what the expression fixes: constant difference, one non-zero
+    difference, sign symmetry, the rounding of the difference to the dtype, and torch's own evaluation of the
+    reference's expression (awq.py:96)."""
+    n = 1000
+    a = torch.full((n,), 3.0)
+    assert iq.awq_loss(a, a - 0.5) == 0.5 ** 4
+    assert iq.awq_loss(a - 0.5, a) == 0.5 ** 4
+    b = a.clone()
+    b[17] += 2.0
+    assert iq.awq_loss(a, b) == 16.0 / n
+    # bf16: 512 - 1 = 511 is not a bf16 value (8 significant bits): the difference is rounded to 512 first
+    y, yh = torch.tensor([512.0], dtype=torch.bfloat16), torch.tensor([1.0], dtype=torch.bfloat16)
+    assert iq.awq_loss(y, yh) == 512.0 ** 4
+    g = torch.Generator().manual_seed(5)
+    for dt in (torch.float32, torch.float16, torch.bfloat16):
+        y = torch.randn(64, 96, generator=g).to(dt)
+        yh = (y.float() + 0.1 * torch.randn(64, 96, generator=g)).to(dt)
+        ref = float((y - yh).float().pow(4).mean())
+        assert abs(iq.awq_loss(y, yh) - ref) <= 1e-5 * ref
+    assert iq.awq_loss(torch.zeros(0), torch.zeros(0)) != iq.awq_loss(torch.zeros(0), torch.zeros(0))   # NaN
