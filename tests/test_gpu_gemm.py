@@ -161,3 +161,27 @@ def test_w4a16_reduces_to_plain_matmul(dev):
     out = ops.gemm_w4a16(x.to(dev), workloads.pack_nibbles(codes).to(dev), scales.to(dev), zeros.to(dev), 128)
     want = torch.matmul(x.float(), (codes.float() - 8).t())          # small integers: exact in fp32
     assert_bits_equal(out, want.to(torch.bfloat16), "plain matmul")
+
+
+BOUNDARY_M = [1, 2, 3, 15, 16, 17, 24, 25, 32, 33, 40, 41, 63, 64, 65, 127, 128, 129, 255, 256, 257, 300, 513]
+
+
+@pytest.mark.parametrize("N,K", [(136, 256), (4104, 128)])
+def test_gemm_dispatch_boundaries_in_m(dev, N, K):
+    """Every row count at which the libraries switch kernels (decode, 64x64, 128x64, 128x128, 128x256, 256x256 tiles;
+    with smoothing the W4A16 switch points move), on one weight: W8A8 bit for bit, W4A16 within its tolerance."""
+    xq, wq, s_ch, s_tok, b = w8a8_case(max(BOUNDARY_M), N, K, 211, True, 'float')
+    x, codes, scales, zeros, smooth, bias = w4a16_case(max(BOUNDARY_M), N, K, 64, 212)
+    packed = workloads.pack_nibbles(codes).to(dev)
+    want8 = od.quant_matmul(xq, wq.t(), s_ch, s_tok, b, torch.bfloat16)
+    want4 = [w4a16_oracle(x, codes, scales, zeros, 64, sm, bias) for sm in (None, smooth)]
+    dwq, dsc, db = wq.to(dev), s_ch.to(dev), b.to(dev)
+    dscales, dzeros, dbias, dsmooth = scales.to(dev), zeros.to(dev), bias.to(dev), smooth.to(dev)
+    for M in BOUNDARY_M:
+        out = ops.gemm_w8a8(xq[:M].contiguous().to(dev), dwq, dsc, s_tok[:M].contiguous().to(dev), db)
+        assert_bits_equal(out, want8[:M], "w8a8 M=%d" % M)
+        for sm, want in ((None, want4[0]), (dsmooth, want4[1])):
+            out = ops.gemm_w4a16(x[:M].contiguous().to(dev), packed, dscales, dzeros, 64, sm, dbias)
+            err = (out.cpu().double() - want[:M]).abs()
+            tol = 1e-3 * want[:M].abs().amax(dim=1, keepdim=True) + want[:M].abs() * 2.0 ** -8
+            assert (err <= tol).all(), (M, sm is not None, err.max().item())
