@@ -235,7 +235,7 @@ def build_cases(dev, only):
                                      sg.data_ptr(), zg.data_ptr(), 1, gi.data_ptr(), Ng, cnt, -8, 7, st)
             assert rc == 0, rc
         cases.append(Case("gptq_block", "hbm", work, "B", launch, 2, "f32",
-                          "GPTQ column loop of one 128-column block, W[14336,4096] fp32 (latency/ALU-bound: 128 dependent steps)"))
+                          "GPTQ column loop of one 128-column block, W[14336,4096] fp32 (latency/ALU-bound: 128 dependent steps; bytes = block in, block and errors out)"))
 
     # ---- matrix-pipe yardsticks: register-only MFMA loop with pseudo-random operands, measured right before the
     # GEMMs they are the yardstick for (and behind the bandwidth-bound kernels, which they would only heat up)

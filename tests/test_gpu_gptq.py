@@ -53,6 +53,25 @@ def test_gptq_block_bit_exact(dev, kind, sym, n, count, strategy):
     assert_bits_equal(dw.cpu(), want_w, "weight block (columns outside the block untouched)")
 
 
+@pytest.mark.parametrize("n,count", [(70, 128), (33, 40)])
+def test_gptq_block_full_matrix_hinv(dev, n, count):
+    """A step only touches the columns at and behind its own (gptq_module.py:141): with an inverse-Hessian block
+    that is NOT triangular the entries in front of the diagonal must be ignored, in both kernels (full 128-column
+    blocks and shorter ones)."""
+    g = torch.Generator().manual_seed(count)
+    w = (torch.randn(n, count, generator=g) * 0.05).float()
+    hinv = _hinv(count, 3) + 0.01 * torch.randn(count, count, generator=g)       # dense, diagonal still dominant
+    s, z = iq.weight_scale_offset(w, 'channel', False, 'int4')
+    gidx = torch.zeros(count, dtype=torch.int32)
+    want_w = w.clone()
+    _, want_e = og.block_loop(want_w, hinv, 'int4', [s.reshape(-1, 1)] * count, [z.reshape(-1, 1)] * count)
+    dw = w.clone().to(dev)
+    got_e = gptq.gptq_block(dw, 0, count, hinv.to(dev), s.reshape(-1).contiguous().to(dev),
+                            z.reshape(-1).to(torch.int32).contiguous().to(dev), gidx.to(dev), -8, 7)
+    assert_bits_equal(got_e.cpu(), want_e, "err block")
+    assert_bits_equal(dw.cpu(), want_w, "weight block")
+
+
 @pytest.mark.parametrize("strategy,group,sym", [('channel', None, True), ('group', 32, False)])
 def test_gptq_whole_routine(dev, strategy, group, sym):
     """End to end.  The two sides factorise and multiply with different libraries, so a weight that sits next
