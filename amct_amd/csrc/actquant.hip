@@ -141,8 +141,7 @@ __global__ __launch_bounds__(kBlock) void act_quant_token_general(const void* x,
     }
 }
 
-// static quantise, scalar indexing (shapes are small / irregular; the hot serving path is the
-// dynamic kernel above)
+// static quantise, scalar indexing: the fallback for shapes and pointers the vector kernel below does not take
 template <int DT>
 __global__ __launch_bounds__(kBlock) void quantize_static(const void* x, const void* smooth, const void* scales,
                                                           const void* zps, int8_t* q, int64_t M, int64_t K,
@@ -157,6 +156,52 @@ __global__ __launch_bounds__(kBlock) void quantize_static(const void* x, const v
         if (zps) t = t + load_scalar<DT>(zps, si);
         t = __builtin_amdgcn_fmed3f(__builtin_rintf(t), -128.f, 127.f);
         q[e] = (int8_t)(int)t;
+    }
+}
+
+// static quantise, 16 bytes of x per thread and iteration (K a multiple of the vector length, aligned pointers):
+// same arithmetic per element as the scalar kernel above
+template <int DT>
+__global__ __launch_bounds__(kBlock) void quantize_static_vec(const void* x, const void* smooth, const void* scales,
+                                                              const void* zps, int8_t* q, int64_t nvec, uint32_t S,
+                                                              int64_t n_scales, int per_token) {
+    constexpr int VEC = Tr<DT>::VEC;
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    const bool small = nvec <= 0xFFFFFFFFll;
+    for (int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += stride) {
+        const int64_t m = small ? (int64_t)((uint32_t)v / S) : v / S;      // row of this vector
+        const uint32_t kv = (uint32_t)(v - m * S);                          // vector inside the row
+        float xv[VEC], sc[VEC], zp[VEC];
+        unpack16<DT>(ldg16_nt(reinterpret_cast<const char*>(x) + v * 16), xv);
+        if (smooth) {
+            float c[VEC];
+            unpack16<DT>(ldg16(reinterpret_cast<const char*>(smooth) + (int64_t)kv * 16), c);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) xv[j] = round_to<DT>(xv[j] * c[j]);
+        }
+        if (per_token || n_scales == 1) {
+            const int64_t si = per_token ? m : 0;
+            const float s1 = load_scalar<DT>(scales, si), z1 = zps ? load_scalar<DT>(zps, si) : 0.f;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) { sc[j] = s1; zp[j] = z1; }
+        } else {
+            unpack16<DT>(ldg16(reinterpret_cast<const char*>(scales) + (int64_t)kv * 16), sc);
+            if (zps) unpack16<DT>(ldg16(reinterpret_cast<const char*>(zps) + (int64_t)kv * 16), zp);
+        }
+        uint32_t out[VEC / 4];
+#pragma unroll
+        for (int wd = 0; wd < VEC / 4; ++wd) {
+            out[wd] = 0;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                float t = xv[4 * wd + b] * sc[4 * wd + b];
+                if (zps) t = t + zp[4 * wd + b];
+                t = __builtin_amdgcn_fmed3f(__builtin_rintf(t), -128.f, 127.f);
+                out[wd] |= ((uint32_t)(int)t & 0xFFu) << (8 * b);
+            }
+        }
+        if constexpr (VEC == 8) stg8_nt(q + v * 8, out[0], out[1]);
+        else *reinterpret_cast<uint32_t*>(q + v * 4) = out[0];
     }
 }
 
@@ -201,9 +246,28 @@ extern "C" int amct_quantize(const void* x, const void* smooth, const void* scal
     if (per_token ? (n_scales != M) : (n_scales != 1 && n_scales != K)) return AMCT_E_BADARG;
     if (M == 0) return AMCT_OK;
     if (!x || !scales || !q) return AMCT_E_BADARG;
+    hipStream_t st = (hipStream_t)stream;
+    {
+        const int vec = dtype == AMCT_F32 ? 4 : 8;
+        const bool table = !per_token && n_scales != 1;            // one scale per column: read as vectors too
+        if (K % vec == 0 && K / vec <= 0x7FFFFFFF && aligned16(x) && (!smooth || aligned16(smooth)) &&
+            (!table || (aligned16(scales) && (!zero_points || aligned16(zero_points)))) &&
+            (reinterpret_cast<uintptr_t>(q) & 7u) == 0) {
+            const int64_t nvec = M * (K / vec);
+            int64_t nbv = (nvec + kBlock - 1) / kBlock;
+            if (nbv > 16384) nbv = 16384;
+            const dim3 gridv((unsigned)nbv), blockv(kBlock);
+            const uint32_t S = (uint32_t)(K / vec);
+            switch (dtype) {
+                case AMCT_F32: hipLaunchKernelGGL((quantize_static_vec<AMCT_F32>), gridv, blockv, 0, st, x, smooth, scales, zero_points, q, nvec, S, n_scales, per_token); return hip_status();
+                case AMCT_F16: hipLaunchKernelGGL((quantize_static_vec<AMCT_F16>), gridv, blockv, 0, st, x, smooth, scales, zero_points, q, nvec, S, n_scales, per_token); return hip_status();
+                case AMCT_BF16: hipLaunchKernelGGL((quantize_static_vec<AMCT_BF16>), gridv, blockv, 0, st, x, smooth, scales, zero_points, q, nvec, S, n_scales, per_token); return hip_status();
+                default: return AMCT_E_BADARG;
+            }
+        }
+    }
     int64_t nb = (M * K + kBlock - 1) / kBlock;
     if (nb > 65536) nb = 65536;
-    hipStream_t st = (hipStream_t)stream;
     const dim3 grid((unsigned)nb), block(kBlock);
     switch (dtype) {
         case AMCT_F32: hipLaunchKernelGGL((quantize_static<AMCT_F32>), grid, block, 0, st, x, smooth, scales, zero_points, q, M, K, n_scales, per_token); break;

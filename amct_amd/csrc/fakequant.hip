@@ -384,6 +384,43 @@ __global__ __launch_bounds__(kBlock) void fq_general(FqArgs a) {
 }
 
 // ---------------------------------------------------------------------------
+// min/max only (A1), groups of T vectors (cols % group == 0, so the tensor is one flat array of groups): a team of T
+// lanes owns 4 consecutive groups, 4 x 16 bytes per lane in flight, extrema by lane exchange.  (The general kernel
+// below walks the groups of a row one after another with 16 of its 256 threads busy for a group of 128 bf16 values:
+// 189 us for W[14336,4096], against 18 us for the per-row case.)
+// ---------------------------------------------------------------------------
+template <int DT, int T>
+__global__ __launch_bounds__(kBlock) void minmax_groups(const void* w, float* mn_out, float* mx_out, int64_t nseg) {
+    constexpr int VEC = Tr<DT>::VEC;
+    constexpr int U = 4;
+    const int tid = threadIdx.x;
+    const int lt = tid % T;
+    const int64_t seg0 = ((int64_t)blockIdx.x * (kBlock / T) + tid / T) * U;
+    uint4 raw[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int64_t sg = seg0 + u < nseg ? seg0 + u : nseg - 1;   // clamped: loads are unconditional
+        raw[u] = ldg16_nt(reinterpret_cast<const char*>(w) + (sg * T + lt) * 16);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        float x[VEC];
+        unpack16<DT>(raw[u], x);
+        float mx = x[0], mn = x[0];
+#pragma unroll
+        for (int j = 1; j < VEC; ++j) {
+            mx = fmax_nan(mx, x[j]);
+            mn = fmin_nan(mn, x[j]);
+        }
+        team_minmax<T>(mn, mx);
+        if (lt == 0 && seg0 + u < nseg) {
+            mn_out[seg0 + u] = mn;
+            mx_out[seg0 + u] = mx;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // min/max only (A1) -- general block-per-row kernel with vector fast path
 // ---------------------------------------------------------------------------
 template <int DT>
@@ -552,9 +589,27 @@ extern "C" int amct_minmax(const void* w, float* mn, float* mx, int64_t rows, in
     const int seg_len = group > 0 ? group : (int)cols;
     const int spr = group > 0 ? (int)((cols + group - 1) / group) : 1;
     hipStream_t st = (hipStream_t)stream;
+#define AMCT_MMG(DT, T)                                                                                          \
+    case T:                                                                                                      \
+        hipLaunchKernelGGL((minmax_groups<DT, T>), dim3(nbg), dim3(kBlock), 0, st, w, mn, mx, nseg);              \
+        return hip_status();
 #define AMCT_MM(DT)                                                                                              \
     {                                                                                                            \
         const int vec_ok = aligned16(w) && cols % Tr<DT>::VEC == 0 && seg_len % Tr<DT>::VEC == 0;               \
+        if (vec_ok && group > 0 && cols % group == 0) {                                                          \
+            const int64_t nseg = rows * spr;                                                                     \
+            const int t = seg_len / Tr<DT>::VEC;                                                                 \
+            const int64_t per_block = (int64_t)(kBlock / (t > 0 && t <= 64 ? t : 64)) * 4;                        \
+            const int64_t nb64 = (nseg + per_block - 1) / per_block;                                             \
+            if (nb64 <= 0x7FFFFFFF) {                                                                            \
+                const unsigned nbg = (unsigned)nb64;                                                             \
+                switch (t) {                                                                                     \
+                    AMCT_MMG(DT, 1) AMCT_MMG(DT, 2) AMCT_MMG(DT, 4) AMCT_MMG(DT, 8) AMCT_MMG(DT, 16) AMCT_MMG(DT, 32)  \
+                    AMCT_MMG(DT, 64)                                                                             \
+                    default: break;                                                                              \
+                }                                                                                                \
+            }                                                                                                    \
+        }                                                                                                        \
         hipLaunchKernelGGL((minmax_rows<DT>), dim3((unsigned)rows), dim3(kBlock), 0, st, w, mn, mx, cols, seg_len, \
                            spr, vec_ok);                                                                         \
     }
@@ -565,6 +620,7 @@ extern "C" int amct_minmax(const void* w, float* mn, float* mx, int64_t rows, in
         default: return AMCT_E_BADARG;
     }
 #undef AMCT_MM
+#undef AMCT_MMG
     return hip_status();
 }
 

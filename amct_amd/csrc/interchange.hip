@@ -7,6 +7,8 @@
 
 namespace amct {
 
+typedef float v2f __attribute__((ext_vector_type(2)));
+
 // E4M3FN code -> fp32 (0x7F / 0xFF are NaN, no infinities)
 AMCT_DEV float e4m3fn_to_f32(uint32_t c) {
     const uint32_t a = c & 0x7Fu;
@@ -21,10 +23,7 @@ AMCT_DEV float e4m3fn_to_f32(uint32_t c) {
 template <int ODT>
 __global__ __launch_bounds__(kBlock) void fp8_block_dequant_k(const uint8_t* w, const float* scale, void* out, int64_t rows,
                                                               int64_t cols, int block, int64_t scale_cols, int64_t nvec) {
-    __shared__ float tbl[256];
     const int tid = threadIdx.x;
-    tbl[tid] = e4m3fn_to_f32((uint32_t)tid);
-    __syncthreads();
     const int64_t vec_per_row = cols / 16;
     constexpr int U = 2;
     const int64_t chunk = (int64_t)kBlock * U;
@@ -44,9 +43,16 @@ __global__ __launch_bounds__(kBlock) void fp8_block_dequant_k(const uint8_t* w, 
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const uint32_t ws[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+            // two codes per instruction through the hardware conversion (v_cvt_pk_f32_fp8, exact; a 256-entry table in
+            // LDS made the kernel LDS-bound: 92 us for W[7168,4096] to fp32)
             float v[16];
 #pragma unroll
-            for (int j = 0; j < 16; ++j) v[j] = tbl[(ws[j / 4] >> (8 * (j % 4))) & 0xFFu] * sc[u];
+            for (int j = 0; j < 8; ++j) {
+                const v2f p = (j & 1) ? __builtin_amdgcn_cvt_pk_f32_fp8((int)ws[j / 2], true)
+                                      : __builtin_amdgcn_cvt_pk_f32_fp8((int)ws[j / 2], false);
+                v[2 * j] = p.x * sc[u];
+                v[2 * j + 1] = p.y * sc[u];
+            }
             if (gv[u] < nvec) {
                 constexpr int VEC = Tr<ODT>::VEC;               // elements per 16-byte store
                 char* o = reinterpret_cast<char*>(out) + gv[u] * 16 * Tr<ODT>::BYTES;

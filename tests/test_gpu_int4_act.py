@@ -103,11 +103,14 @@ def test_dynamic_per_token(dev, dtype, shape):
     assert_bits_equal(q, oq.reshape(shape), "codes absmax")
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_static_quantize(dev, dtype):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(2, 24, 96), (1, 300, 4096), (3, 5, 100), (1, 7, 37)])
+def test_static_quantize(dev, dtype, shape):
+    """Vector kernel (K a multiple of 8, or of 4 for fp32) and scalar fallback, per tensor / per channel / per token,
+    with and without zero-points."""
     g = torch.Generator().manual_seed(73)
-    x = (torch.randn(2, 24, 96, generator=g) * 3).to(dtype)
-    for per_token, n in ((False, 1), (False, 96), (True, 24)):
+    x = (torch.randn(*shape, generator=g) * 3).to(dtype)
+    for per_token, n in ((False, 1), (False, shape[-1]), (True, shape[-2])):
         sc = (5 + 20 * torch.rand(n, generator=g)).to(dtype)
         zp = torch.randint(-20, 20, (n,), generator=g).to(dtype)
         for z in (zp, None):

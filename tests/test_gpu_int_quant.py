@@ -26,7 +26,8 @@ def rand_w(rows, cols, dtype, seed, std=0.02):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape,group", [((16, 96), 0), ((16, 96), 32), ((7, 80), 32), ((5, 37), 0),
                                          ((64, 4096), 0), ((64, 4096), 128), ((3, 8200), 0), ((2, 20000), 0),
-                                         ((9, 1024), 512), ((33, 2048), 0)])
+                                         ((9, 1024), 512), ((33, 2048), 0), ((3, 104), 8), ((5, 272), 16), ((7, 448), 64),
+                                         ((3, 768), 256), ((1, 8), 8), ((37, 4096), 128), ((5, 24), 4)])
 def test_minmax(dev, dtype, shape, group):
     w = rand_w(*shape, dtype, 11)
     mn, mx = ops.minmax(w.to(dev), group)
@@ -40,6 +41,22 @@ def test_minmax(dev, dtype, shape, group):
     # the reduction order (also inside torch) and has no effect on the factors derived from it
     assert torch.equal(mn.cpu(), omn.float()), "min"
     assert torch.equal(mx.cpu(), omx.float()), "max"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_minmax_groups_nan_and_inf(dev, dtype):
+    """A NaN makes both extrema of its group NaN and leaves the neighbours alone (torch.amax / amin); infinities are
+    ordinary values."""
+    w = rand_w(6, 512, dtype, 5)
+    w[1, 130] = float('nan')
+    w[2, 3] = float('inf')
+    w[4, 511] = float('-inf')
+    mn, mx = ops.minmax(w.to(dev), 128)
+    omn, omx = iq.weight_min_max(w, 'group', 128)
+    omn, omx = omn.squeeze(-1).float(), omx.squeeze(-1).float()
+    assert torch.isnan(mn[1, 1]) and torch.isnan(mx[1, 1]) and int(torch.isnan(mn).sum()) == 1
+    assert torch.equal(torch.nan_to_num(mn.cpu(), nan=7.0), torch.nan_to_num(omn, nan=7.0))
+    assert torch.equal(torch.nan_to_num(mx.cpu(), nan=7.0), torch.nan_to_num(omx, nan=7.0))
 
 
 @pytest.mark.parametrize("bits", [8, 4])
