@@ -166,42 +166,54 @@ __global__ __launch_bounds__(kBlock) void quantize_static_vec(const void* x, con
                                                               const void* zps, int8_t* q, int64_t nvec, uint32_t S,
                                                               int64_t n_scales, int per_token) {
     constexpr int VEC = Tr<DT>::VEC;
+    constexpr int U = 4;                                           // vectors in flight per thread
     const int64_t stride = (int64_t)gridDim.x * kBlock;
     const bool small = nvec <= 0xFFFFFFFFll;
-    for (int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += stride) {
-        const int64_t m = small ? (int64_t)((uint32_t)v / S) : v / S;      // row of this vector
-        const uint32_t kv = (uint32_t)(v - m * S);                          // vector inside the row
-        float xv[VEC], sc[VEC], zp[VEC];
-        unpack16<DT>(ldg16_nt(reinterpret_cast<const char*>(x) + v * 16), xv);
-        if (smooth) {
-            float c[VEC];
-            unpack16<DT>(ldg16(reinterpret_cast<const char*>(smooth) + (int64_t)kv * 16), c);
+    for (int64_t v0 = (int64_t)blockIdx.x * kBlock + threadIdx.x; v0 < nvec; v0 += stride * U) {
+        uint4 raw[U];
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) xv[j] = round_to<DT>(xv[j] * c[j]);
+        for (int u = 0; u < U; ++u) {
+            const int64_t v = v0 + u * stride;
+            raw[u] = ldg16_nt(reinterpret_cast<const char*>(x) + (v < nvec ? v : nvec - 1) * 16);   // clamped, unconditional
         }
-        if (per_token || n_scales == 1) {
-            const int64_t si = per_token ? m : 0;
-            const float s1 = load_scalar<DT>(scales, si), z1 = zps ? load_scalar<DT>(zps, si) : 0.f;
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) { sc[j] = s1; zp[j] = z1; }
-        } else {
-            unpack16<DT>(ldg16(reinterpret_cast<const char*>(scales) + (int64_t)kv * 16), sc);
-            if (zps) unpack16<DT>(ldg16(reinterpret_cast<const char*>(zps) + (int64_t)kv * 16), zp);
-        }
-        uint32_t out[VEC / 4];
+        for (int u = 0; u < U; ++u) {
+            const int64_t v = v0 + u * stride;
+            if (v >= nvec) break;
+            const int64_t m = small ? (int64_t)((uint32_t)v / S) : v / S;      // row of this vector
+            const uint32_t kv = (uint32_t)(v - m * S);                          // vector inside the row
+            float xv[VEC], sc[VEC], zp[VEC];
+            unpack16<DT>(raw[u], xv);
+            if (smooth) {
+                float c[VEC];
+                unpack16<DT>(ldg16(reinterpret_cast<const char*>(smooth) + (int64_t)kv * 16), c);
 #pragma unroll
-        for (int wd = 0; wd < VEC / 4; ++wd) {
-            out[wd] = 0;
-#pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                float t = xv[4 * wd + b] * sc[4 * wd + b];
-                if (zps) t = t + zp[4 * wd + b];
-                t = __builtin_amdgcn_fmed3f(__builtin_rintf(t), -128.f, 127.f);
-                out[wd] |= ((uint32_t)(int)t & 0xFFu) << (8 * b);
+                for (int j = 0; j < VEC; ++j) xv[j] = round_to<DT>(xv[j] * c[j]);
             }
+            if (per_token || n_scales == 1) {
+                const int64_t si = per_token ? m : 0;
+                const float s1 = load_scalar<DT>(scales, si), z1 = zps ? load_scalar<DT>(zps, si) : 0.f;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) { sc[j] = s1; zp[j] = z1; }
+            } else {
+                unpack16<DT>(ldg16(reinterpret_cast<const char*>(scales) + (int64_t)kv * 16), sc);
+                if (zps) unpack16<DT>(ldg16(reinterpret_cast<const char*>(zps) + (int64_t)kv * 16), zp);
+            }
+            uint32_t out[VEC / 4];
+#pragma unroll
+            for (int wd = 0; wd < VEC / 4; ++wd) {
+                out[wd] = 0;
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    float t = xv[4 * wd + b] * sc[4 * wd + b];
+                    if (zps) t = t + zp[4 * wd + b];
+                    t = __builtin_amdgcn_fmed3f(__builtin_rintf(t), -128.f, 127.f);
+                    out[wd] |= ((uint32_t)(int)t & 0xFFu) << (8 * b);
+                }
+            }
+            if constexpr (VEC == 8) stg8_nt(q + v * 8, out[0], out[1]);
+            else *reinterpret_cast<uint32_t*>(q + v * 4) = out[0];
         }
-        if constexpr (VEC == 8) stg8_nt(q + v * 8, out[0], out[1]);
-        else *reinterpret_cast<uint32_t*>(q + v * 4) = out[0];
     }
 }
 
@@ -254,7 +266,7 @@ extern "C" int amct_quantize(const void* x, const void* smooth, const void* scal
             (!table || (aligned16(scales) && (!zero_points || aligned16(zero_points)))) &&
             (reinterpret_cast<uintptr_t>(q) & 7u) == 0) {
             const int64_t nvec = M * (K / vec);
-            int64_t nbv = (nvec + kBlock - 1) / kBlock;
+            int64_t nbv = (nvec + kBlock * 4 - 1) / (kBlock * 4);
             if (nbv > 16384) nbv = 16384;
             const dim3 gridv((unsigned)nbv), blockv(kBlock);
             const uint32_t S = (uint32_t)(K / vec);

@@ -410,6 +410,78 @@ __global__ __launch_bounds__(kBlock) void nibbles_to_codes_kn_k(const uint8_t* p
     codes[idx] = u - 8;
 }
 
+// ---- the same three conversions for aligned shapes: 16-byte accesses, transposes through an LDS tile ----
+// (the kernels above touch one word or byte per thread with strided partners: 147 us, 41 us and 224 us for
+// W[14336,4096])
+
+// 128 k-rows x 16 words (128 columns) per block: coalesced word loads, then thread (column c, half h) gathers the
+// nibbles of its column over 64 k-rows into 32 consecutive output bytes.  k % 128 == 0, n8 % 16 == 0.
+__global__ __launch_bounds__(kBlock) void words_to_nibbles_tile_k(const int32_t* words, uint8_t* packed, int64_t k, int64_t n8) {
+    __shared__ uint32_t tile[128][17];
+    const int tid = threadIdx.x;
+    const int64_t i0 = (int64_t)blockIdx.x * 16, k0 = (int64_t)blockIdx.y * 128;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int kr = tid / 16 + 16 * j, i = tid % 16;
+        tile[kr][i] = (uint32_t)words[(k0 + kr) * n8 + i0 + i] ^ 0x88888888u;     // +8 mod 16 on every nibble
+    }
+    __syncthreads();
+    const int c = tid >> 1, h = tid & 1;
+    const int i = c >> 3, sh = 4 * (c & 7);
+    uint32_t out[8];
+#pragma unroll
+    for (int wd = 0; wd < 8; ++wd) {
+        uint32_t v = 0;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int kr = 64 * h + 8 * wd + 2 * b;
+            const uint32_t lo = (tile[kr][i] >> sh) & 0xFu, hi = (tile[kr + 1][i] >> sh) & 0xFu;
+            v |= (lo | (hi << 4)) << (8 * b);
+        }
+        out[wd] = v;
+    }
+    uint8_t* dst = packed + (i0 * 8 + c) * (k / 2) + k0 / 2 + 32 * h;
+    stg16_nt(dst, make_uint4(out[0], out[1], out[2], out[3]));
+    stg16_nt(dst + 16, make_uint4(out[4], out[5], out[6], out[7]));
+}
+
+// 16 codes (16 bytes) -> 8 bytes per thread: (c + 8) mod 16 = (c & 15) ^ 8, pairs merged by shifts
+__global__ __launch_bounds__(kBlock) void pack_nibbles_vec_k(const int8_t* codes, uint8_t* packed, int64_t nvec) {
+    const int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (v >= nvec) return;
+    const uint4 in = ldg16_nt(codes + v * 16);
+    const uint32_t ws[4] = {in.x, in.y, in.z, in.w};
+    uint32_t half[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t t = (ws[j] & 0x0F0F0F0Fu) ^ 0x08080808u;   // bytes t0 t1 t2 t3, each below 16
+        const uint32_t u = t | (t >> 4);                           // byte 0 = t0 | t1 << 4, byte 2 = t2 | t3 << 4
+        half[j] = (u & 0xFFu) | ((u >> 8) & 0xFF00u);
+    }
+    stg8_nt(packed + v * 8, half[0] | (half[1] << 16), half[2] | (half[3] << 16));
+}
+
+// 64 rows x 32 bytes (64 values of k) per block: 16-byte loads, then every k-row of the tile is written as 64
+// consecutive int32 codes.  k % 64 == 0, n % 64 == 0.
+__global__ __launch_bounds__(kBlock) void nibbles_to_codes_tile_k(const uint8_t* packed, int32_t* codes, int64_t k, int64_t n) {
+    __shared__ __attribute__((aligned(16))) uint8_t tile[64][48];  // 32 bytes used; rows 12 words apart
+    const int tid = threadIdx.x;
+    const int64_t n0 = (int64_t)blockIdx.x * 64, k0 = (int64_t)blockIdx.y * 64;
+    if (tid < 128) {
+        const int r = tid >> 1, h = tid & 1;
+        *reinterpret_cast<uint4*>(&tile[r][16 * h]) = ldg16_nt(packed + (n0 + r) * (k / 2) + k0 / 2 + 16 * h);
+    }
+    __syncthreads();
+    const int c = tid & 63, kq = tid >> 6;
+#pragma unroll
+    for (int kk = 0; kk < 16; ++kk) {
+        const int kr = 16 * kq + kk;
+        const uint32_t b = tile[c][kr >> 1];
+        const int32_t u = (kr & 1) ? (int32_t)(b >> 4) : (int32_t)(b & 0xFu);
+        __builtin_nontemporal_store(u - 8, codes + (k0 + kr) * n + n0 + c);
+    }
+}
+
 }  // namespace amct
 
 using namespace amct;
@@ -452,6 +524,11 @@ extern "C" int amct_words_to_nibbles_nk(const int32_t* words, uint8_t* packed, i
     if (n % 8 != 0 || k % 2 != 0) return AMCT_E_ALIGN;
     const int64_t total = (k / 2) * (n / 8);
     if (total == 0) return AMCT_OK;
+    if (k % 128 == 0 && (n / 8) % 16 == 0 && aligned16(packed) && k / 128 <= 65535) {
+        hipLaunchKernelGGL(words_to_nibbles_tile_k, dim3((unsigned)(n / 128), (unsigned)(k / 128)), dim3(kBlock), 0,
+                           (hipStream_t)stream, words, packed, k, n / 8);
+        return hip_status();
+    }
     hipLaunchKernelGGL(words_to_nibbles_k, dim3((unsigned)((total + kBlock - 1) / kBlock)), dim3(kBlock), 0,
                        (hipStream_t)stream, words, packed, k, n / 8);
     return hip_status();
@@ -462,6 +539,12 @@ extern "C" int amct_pack_nibbles_nk(const int8_t* codes, uint8_t* packed, int64_
     if (cols % 2 != 0) return AMCT_E_ALIGN;
     const int64_t nbytes = rows * (cols / 2);
     if (nbytes == 0) return AMCT_OK;
+    if (nbytes % 8 == 0 && aligned16(codes) && (reinterpret_cast<uintptr_t>(packed) & 7u) == 0) {
+        const int64_t nvec = nbytes / 8;
+        hipLaunchKernelGGL(pack_nibbles_vec_k, dim3((unsigned)((nvec + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                           (hipStream_t)stream, codes, packed, nvec);
+        return hip_status();
+    }
     hipLaunchKernelGGL(pack_nibbles_k, dim3((unsigned)((nbytes + kBlock - 1) / kBlock)), dim3(kBlock), 0,
                        (hipStream_t)stream, codes, packed, nbytes);
     return hip_status();
@@ -471,6 +554,11 @@ extern "C" int amct_nibbles_nk_to_codes_kn(const uint8_t* packed, int32_t* codes
     if (k < 0 || n < 0 || (k * n != 0 && (!packed || !codes))) return AMCT_E_BADARG;
     if (k % 2 != 0) return AMCT_E_ALIGN;
     if (k * n == 0) return AMCT_OK;
+    if (k % 64 == 0 && n % 64 == 0 && aligned16(packed) && k / 64 <= 65535) {
+        hipLaunchKernelGGL(nibbles_to_codes_tile_k, dim3((unsigned)(n / 64), (unsigned)(k / 64)), dim3(kBlock), 0,
+                           (hipStream_t)stream, packed, codes, k, n);
+        return hip_status();
+    }
     hipLaunchKernelGGL(nibbles_to_codes_kn_k, dim3((unsigned)((k * n + kBlock - 1) / kBlock)), dim3(kBlock), 0,
                        (hipStream_t)stream, packed, codes, k, n);
     return hip_status();

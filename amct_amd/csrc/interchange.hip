@@ -19,46 +19,44 @@ AMCT_DEV float e4m3fn_to_f32(uint32_t c) {
     return (c & 0x80u) ? -f : f;
 }
 
-// out = dtype(fp32(w) * scale[row / B][col / B]); one lane = 16 consecutive codes of a row
+// out = dtype(fp32(w) * scale[row / B][col / B]).  One lane = the codes of one 16-byte output vector (4 for fp32, 8 for
+// the 16-bit types), so that every store instruction of a wave writes 1 KiB of consecutive bytes; 8 rows in flight per
+// lane.  (With 16 codes and up to four strided 16-byte stores per lane the kernel wrote partial lines: 93 us for
+// W[7168,4096] to fp32.)  Codes are decoded two per instruction by the hardware conversion (v_cvt_pk_f32_fp8, exact).
 template <int ODT>
 __global__ __launch_bounds__(kBlock) void fp8_block_dequant_k(const uint8_t* w, const float* scale, void* out, int64_t rows,
-                                                              int64_t cols, int block, int64_t scale_cols, int64_t nvec) {
-    const int tid = threadIdx.x;
-    const int64_t vec_per_row = cols / 16;
-    constexpr int U = 2;
-    const int64_t chunk = (int64_t)kBlock * U;
-    const int64_t nchunks = (nvec + chunk - 1) / chunk;
-    for (int64_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
-        uint4 raw[U];
+                                                              int64_t cols, int block, int64_t scale_cols) {
+    constexpr int VEC = Tr<ODT>::VEC;
+    constexpr int U = 8;
+    const int64_t vpr = cols / VEC;
+    const int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x;   // vector inside the row
+    const int64_t vc = v < vpr ? v : vpr - 1;                       // clamped: loads are unconditional
+    const int64_t sc_col = (vc * VEC) / block;
+    for (int64_t r0 = (int64_t)blockIdx.y * U; r0 < rows; r0 += (int64_t)gridDim.y * U) {
+        uint32_t raw[U][VEC / 4];
         float sc[U];
-        int64_t gv[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            gv[u] = c * chunk + u * kBlock + tid;
-            const int64_t g = gv[u] < nvec ? gv[u] : nvec - 1;  // clamped: loads are unconditional
-            const int64_t row = g / vec_per_row, col = (g - row * vec_per_row) * 16;
-            raw[u] = ldg16_nt(w + g * 16);
-            sc[u] = scale[(row / block) * scale_cols + col / block];
+            const int64_t r = r0 + u < rows ? r0 + u : rows - 1;
+            const uint32_t* src = reinterpret_cast<const uint32_t*>(w + r * cols + vc * VEC);
+#pragma unroll
+            for (int d = 0; d < VEC / 4; ++d) raw[u][d] = __builtin_nontemporal_load(src + d);
+            sc[u] = scale[(r / block) * scale_cols + sc_col];
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const uint32_t ws[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
-            // two codes per instruction through the hardware conversion (v_cvt_pk_f32_fp8, exact; a 256-entry table in
-            // LDS made the kernel LDS-bound: 92 us for W[7168,4096] to fp32)
-            float v[16];
+            float x[VEC];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const v2f p = (j & 1) ? __builtin_amdgcn_cvt_pk_f32_fp8((int)ws[j / 2], true)
-                                      : __builtin_amdgcn_cvt_pk_f32_fp8((int)ws[j / 2], false);
-                v[2 * j] = p.x * sc[u];
-                v[2 * j + 1] = p.y * sc[u];
+            for (int d = 0; d < VEC / 4; ++d) {
+                const v2f lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)raw[u][d], false);
+                const v2f hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)raw[u][d], true);
+                x[4 * d] = lo.x * sc[u];
+                x[4 * d + 1] = lo.y * sc[u];
+                x[4 * d + 2] = hi.x * sc[u];
+                x[4 * d + 3] = hi.y * sc[u];
             }
-            if (gv[u] < nvec) {
-                constexpr int VEC = Tr<ODT>::VEC;               // elements per 16-byte store
-                char* o = reinterpret_cast<char*>(out) + gv[u] * 16 * Tr<ODT>::BYTES;
-#pragma unroll
-                for (int p = 0; p < 16 / VEC; ++p) stg16_nt(o + p * 16, pack16<ODT>(v + p * VEC));
-            }
+            if (v < vpr && r0 + u < rows)
+                stg16_nt(reinterpret_cast<char*>(out) + ((r0 + u) * cols + v * VEC) * Tr<ODT>::BYTES, pack16<ODT>(x));
         }
     }
 }
@@ -114,15 +112,17 @@ extern "C" int amct_fp8_block_dequant(const uint8_t* w, const float* scale, void
     if (!w || !scale || !out) return AMCT_E_BADARG;
     hipStream_t st = (hipStream_t)stream;
     const int64_t scale_cols = (cols + block - 1) / block;
-    const bool vec_ok = cols % 16 == 0 && block % 16 == 0 && aligned16(w) && aligned16(out);
+    const bool vec_ok = cols % 8 == 0 && block % 8 == 0 && aligned16(w) && aligned16(out);
 #define AMCT_FD(DT)                                                                                               \
     {                                                                                                             \
         if (vec_ok) {                                                                                             \
-            const int64_t nvec = rows * cols / 16;                                                                \
-            int64_t nb = (nvec + kBlock * 2 - 1) / (kBlock * 2);                                                  \
-            if (nb > 8192) nb = 8192;                                                                             \
-            hipLaunchKernelGGL((fp8_block_dequant_k<DT>), dim3((unsigned)nb), dim3(kBlock), 0, st, w, scale, out, rows, \
-                               cols, block, scale_cols, nvec);                                                    \
+            const int64_t vpr = cols / Tr<DT>::VEC;                                                               \
+            const int64_t nbx = (vpr + kBlock - 1) / kBlock;                                                      \
+            int64_t nby = (rows + 7) / 8;                                                                         \
+            if (nby > 65535) nby = 65535;                                                                         \
+            if (nbx > 0x7FFFFFFF) return AMCT_E_UNSUPPORTED;                                                      \
+            hipLaunchKernelGGL((fp8_block_dequant_k<DT>), dim3((unsigned)nbx, (unsigned)nby), dim3(kBlock), 0, st, w, scale, \
+                               out, rows, cols, block, scale_cols);                                               \
         } else {                                                                                                  \
             const int64_t nb = (rows * cols + kBlock - 1) / kBlock;                                               \
             if (nb > 0x7FFFFFFF) return AMCT_E_UNSUPPORTED;                                                       \

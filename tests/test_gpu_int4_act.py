@@ -67,14 +67,20 @@ def test_config2_full_size_properties(dev):
     assert (err <= s32.cpu()[rows].unsqueeze(-1) * 0.5001).all()
 
 
-def test_int4_word_layouts(dev):
+@pytest.mark.parametrize("k,n", [(64, 48), (256, 384), (128, 128), (384, 1160), (192, 136), (2, 8)])
+def test_int4_word_layouts(dev, k, n):
+    """The layout converters on shapes that take the tiled / vector kernels (k % 128 == 0 and n % 128 == 0; k, n % 64
+    == 0) and on shapes that take the element-wise ones; every conversion against the oracle and the round trip."""
     g = torch.Generator().manual_seed(67)
-    codes = torch.randint(-8, 8, (64, 48), generator=g, dtype=torch.int32)          # [k, n]
+    codes = torch.randint(-8, 8, (k, n), generator=g, dtype=torch.int32)            # [k, n]
     words = ops.pack_int4_words(codes.to(dev))
     assert_bits_equal(words, od.pack_int4_words(codes), "words")
     assert torch.equal(od.unpack_int4_words(words.cpu()), codes)
-    nib = ops.words_to_nibbles_nk(words, 64, 48)
-    assert_bits_equal(nib, od.pack_nibbles_k(codes.t().contiguous()), "nibbles [n,k/2]")
+    nib = ops.words_to_nibbles_nk(words, k, n)
+    want_nib = od.pack_nibbles_k(codes.t().contiguous())
+    assert_bits_equal(nib, want_nib, "nibbles [n,k/2]")
+    assert_bits_equal(ops.pack_nibbles_nk(codes.t().contiguous().to(torch.int8).to(dev)), want_nib, "nibbles from int8 codes")
+    assert_bits_equal(ops.unpack_nibbles_to_i32_kn(nib), codes, "codes [k,n] back from the nibbles")
     # nibble order agrees with the usual uint4 packing convention: low nibble = even index
     u = torch.tensor([[1, 2, 3, 4]], dtype=torch.int32) - 8
     assert od.pack_nibbles_k(u).tolist() == [[0x21, 0x43]]
