@@ -1454,7 +1454,8 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
             // few (the weight stream is the bulk of the traffic for medium M): 128x128 blocks (with specialised waves
             // when K % 256 == 0: 38 us against 51 us on W[14336,4096], M = 129 .. 256; the first-generation kernel took
             // 97 us; 64-column blocks of 4 waves, a quarter of a weight row per thread and step, while they still fit the
-            // CUs in one round: 64x64 for M <= 64, 26 us, and 128x64 for M <= 128, 34 us), then 128x256 blocks of 8 waves (M = 384, 512: 72 .. 75 us against 96 us), each with three LDS
+            // CUs in one round: 64x64 for M <= 64, 26 us, and 128x64 for M <= 128, 34 us), then blocks of 8 waves: 256x128 for 256 < M <= 512 (65 us; half the
+            // dequantisation of 128x256 blocks, which take 72 .. 75 us; the first-generation kernel took 96 us), 128x256 where those do not fit the CUs, each with three LDS
             // stages; 256x256 with two stages otherwise.  (Mixing in 256x192
             // blocks as the W8A8 launch does was measured neutral here: the narrow tile dequantises as many weights.)
             const int64_t cus = current_cu_count();
@@ -1471,6 +1472,7 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
         else if (shape == 4) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 2, 1, 3>), dim3((unsigned)nt64, (unsigned)mt), dim3(256), 0, st, a); \
         else if (shape == 1 && K % 256 == 0 && G <= kSpecMaxG) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3>), dim3((unsigned)nt128, (unsigned)mt), dim3(kSpecThreads), 0, st, a); \
         else if (shape == 1) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 2, 2, 3>), dim3((unsigned)nt128, (unsigned)mt), dim3(256), 0, st, a); \
+        else if (shape == 2 && M > 256 && (M + 255) / 256 * nt128 <= cus) hipLaunchKernelGGL((w4a16_tile_wide<SF, 4, 2, 2, 2, 3>), dim3((unsigned)nt128, (unsigned)((M + 255) / 256)), dim3(512), 0, st, a); \
         else if (shape == 2) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 4, 2, 2, 3>), dim3((unsigned)nt256, (unsigned)mt), dim3(512), 0, st, a); \
         else hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 4, 4, 2, 2>), grid, dim3(kQThreads), 0, st, a);                \
     }
