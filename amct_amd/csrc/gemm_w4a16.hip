@@ -719,12 +719,15 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM
 // data-movement waves), 43 us (4), 51 us (4 waves doing everything); of the 38 us, 22 us are the matrix waves and
 // the barriers alone, the LDS writes of the dequantised weights add 8 us, the loads 7 us, the arithmetic 4 us.
 // ---------------------------------------------------------------------------
-template <bool SF16, int STAGES>
-__global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) void w4a16_tile_spec(W4A16Args a) {
-    constexpr int kLM = 128, kLN = 128, TI = 2, TJ = 2, WN = 2;
-    constexpr int kStageBytes = (kLM + kLN) * kWRow;                // 32 KiB
-    constexpr int kMW = kSpecThreads / 64 - 4;                      // data-movement waves: 8
-    constexpr int kNA = (kLM * kWRow / 1024) / kMW;                 // activation pieces per moving wave: 2
+// Tile (64*TI) x (64*TJ): 2 x 2 matrix waves of (32*TI) x (32*TJ) and 4*TJ data-movement waves (four threads per
+// weight row of the tile); 128x128 as described above, 64x64 and 128x64 for small M with 4 + 4 waves.
+template <bool SF16, int STAGES, int TI = 2, int TJ = 2, int kD = 4>
+__global__ __launch_bounds__((4 + 4 * TJ) * 64) __attribute__((amdgpu_waves_per_eu(1 + TJ, 1 + TJ))) void w4a16_tile_spec(W4A16Args a) {
+    constexpr int kLM = 64 * TI, kLN = 64 * TJ, WN = 2;
+    constexpr int kThreads = (4 + 4 * TJ) * 64;
+    constexpr int kStageBytes = (kLM + kLN) * kWRow;                // 32 KiB for 128x128
+    constexpr int kMW = 4 * TJ;                                     // data-movement waves
+    constexpr int kNA = (kLM * kWRow / 1024) / kMW;                 // activation pieces per moving wave
     constexpr int kNM = TI * TJ, kNR = TI + TJ;
     static_assert(STAGES == 2 || STAGES == 3, "stages");
     constexpr int kStages = STAGES * kStageBytes > 65536 ? STAGES * kStageBytes : 65536;
@@ -745,7 +748,7 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
         const uint32_t G = (uint32_t)(a.K / a.group);
         // kTPR threads share a row; all loads are issued before the first use (unconditional, clamped): a loop that
         // loads and stores entry by entry pays one memory latency per trip before the kernel's first MFMA
-        constexpr int kTPR = kSpecThreads / kLN, kIt = (kSpecMaxG + kTPR - 1) / kTPR;
+        constexpr int kTPR = kThreads / kLN, kIt = (kSpecMaxG + kTPR - 1) / kTPR;
         const uint32_t row = tid / kTPR, g0 = tid % kTPR;
         const int64_t wr = (n0 + row < a.N) ? n0 + row : a.N - 1;
         uint32_t sb[kIt], zb[kIt];
@@ -791,7 +794,6 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
         for (int c = 0; c < 2; ++c) bdst[c] = kLM * kWRow + brow * kWRow + ((2 * bq + c) ^ swz(brow)) * 16;
         // The weights stream from HBM and a step of this small tile is shorter than that latency, so the packed
         // weights of a step are fetched kD steps ahead into kD register slots (the loop is unrolled by kD).
-        constexpr int kD = 4;
         uint64_t wreg[kD];
         auto issue_b = [&](int slot, int step) {
             const int st = step < last ? step : last;
@@ -840,11 +842,9 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
         cur = nxt;                                                                     \
         nxt = nxt + 1 == STAGES ? 0 : nxt + 1;                                         \
     }
-        for (int step = 0; step < nsteps; step += kD) {             // K % 256 == 0: a multiple of kD steps
-            AMCT_MOVE_ITER(1, step)
-            AMCT_MOVE_ITER(2, step + 1)
-            AMCT_MOVE_ITER(3, step + 2)
-            AMCT_MOVE_ITER(0, step + 3)
+        for (int step = 0; step < nsteps; step += kD) {             // K % (64 * kD) == 0: a multiple of kD steps
+#pragma unroll
+            for (int u = 0; u < kD; ++u) AMCT_MOVE_ITER((u + 1) % kD, step + u)
         }
 #undef AMCT_MOVE_ITER
 #undef AMCT_TIE_SLOT
@@ -891,6 +891,7 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
     {
         int cur = 0, nxt = 1;
         constexpr int kRPM = (3 * kNR + kNM - 1) / kNM;             // reads behind each MFMA of slice 0
+        constexpr int kRP0 = (kNR + kNM - 1) / kNM;                 // reads of the next step's slice 0 behind each MFMA of slice 3
         for (int step = 0; step < nsteps; ++step) {
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -921,8 +922,11 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
             for (int m = 0; m < kNM; ++m) {
                 mfma_one(m, fa[3], fb[3]);
                 __builtin_amdgcn_sched_barrier(0);
-                read_one(nxt, 0, m, fa[0], fb[0]);
-                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int q = kRP0 * m; q < kRP0 * (m + 1) && q < kNR; ++q) {
+                    read_one(nxt, 0, q, fa[0], fb[0]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
             cur = nxt;
             nxt = nxt + 1 == STAGES ? 0 : nxt + 1;
@@ -1403,14 +1407,16 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
         }
         if (rc != AMCT_E_UNSUPPORTED) return rc;
     }
-    // The weight-streaming kernel below serves M <= 24 (25 us on W[14336,4096] at M = 17, 29 us at M = 32, 40 us at
-    // M = 64; 64x64 tiles take 26 us for any M <= 64), and larger M up to 64 where the tile kernels do not apply; when
-    // the activations are to be smoothed the tile path pays a pre-pass, so the switch comes later.
+    // The weight-streaming kernel below serves 16 < M <= 24 (25 us on W[14336,4096] at M = 17, 29 us at M = 32, 40 us
+    // at M = 64; 64x64 tiles take 26 us for any M <= 64, 22 us with specialised waves, which then start at M = 17), and
+    // larger M up to 64 where the tile kernels do not apply; when the activations are to be smoothed the tile path pays
+    // a pre-pass, so the switch of the plain tiles comes later.
     const bool tiles_apply = vec_ok && K % 128 == 0 && K < 65536 && N % 8 == 0 && aligned16(out) && group % 64 == 0 &&
                              M * K * 2 < (int64_t(1) << 32) && N * (K / 2) < (int64_t(1) << 32) &&
                              N * (K / group) * 2 < (int64_t(1) << 32) &&
                              (!smooth || (workspace && workspace_bytes >= (size_t)(M * K * 2) && aligned16(workspace)));
-    const int64_t small_tiles_from = smooth ? 41 : 25;
+    const bool spec_small = K % 256 == 0 && K / group <= kSpecMaxG;   // the 22 us kernel serves this shape
+    const int64_t small_tiles_from = spec_small ? 17 : smooth ? 41 : 25;
     if (vec_ok && M <= 64 && K % 128 == 0 && K < 65536 && group % 32 == 0 && !(tiles_apply && M >= small_tiles_from)) {
         const dim3 grid((unsigned)((N + kDN - 1) / kDN));
         const int iters = (int)(K / 128);
@@ -1454,7 +1460,8 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
             // few (the weight stream is the bulk of the traffic for medium M): 128x128 blocks (with specialised waves
             // when K % 256 == 0: 38 us against 51 us on W[14336,4096], M = 129 .. 256; the first-generation kernel took
             // 97 us; 64-column blocks of 4 waves, a quarter of a weight row per thread and step, while they still fit the
-            // CUs in one round: 64x64 for M <= 64, 26 us, and 128x64 for M <= 128, 34 us), then blocks of 8 waves: 256x128 for 256 < M <= 512 (65 us; half the
+            // CUs in one round: 64x64 for M <= 64, 26 us, and 128x64 for M <= 128, 34 us; with 4 matrix and 4 data-movement
+            // waves when K % 256 == 0: 22 us and 27 us; fetching the weights 8 steps ahead instead of 4 changed nothing), then blocks of 8 waves: 256x128 for 256 < M <= 512 (65 us; half the
             // dequantisation of 128x256 blocks, which take 72 .. 75 us; the first-generation kernel took 96 us), 128x256 where those do not fit the CUs, each with three LDS
             // stages; 256x256 with two stages otherwise.  (Mixing in 256x192
             // blocks as the W8A8 launch does was measured neutral here: the narrow tile dequantises as many weights.)
@@ -1468,7 +1475,9 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
             if (mt > 65535) return AMCT_E_UNSUPPORTED;
 #define AMCT_LAUNCH_WIDE(SF)                                                                                           \
     {                                                                                                                  \
-        if (shape == 3) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 1, 1, 3>), dim3((unsigned)nt64, 1), dim3(256), 0, st, a);          \
+        if (shape == 3 && K % 256 == 0 && G <= kSpecMaxG) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3, 1, 1>), dim3((unsigned)nt64, 1), dim3(512), 0, st, a); \
+        else if (shape == 4 && K % 256 == 0 && G <= kSpecMaxG) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3, 2, 1>), dim3((unsigned)nt64, (unsigned)mt), dim3(512), 0, st, a); \
+        else if (shape == 3) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 1, 1, 3>), dim3((unsigned)nt64, 1), dim3(256), 0, st, a);          \
         else if (shape == 4) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 2, 1, 3>), dim3((unsigned)nt64, (unsigned)mt), dim3(256), 0, st, a); \
         else if (shape == 1 && K % 256 == 0 && G <= kSpecMaxG) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3>), dim3((unsigned)nt128, (unsigned)mt), dim3(kSpecThreads), 0, st, a); \
         else if (shape == 1) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 2, 2, 3>), dim3((unsigned)nt128, (unsigned)mt), dim3(256), 0, st, a); \

@@ -412,8 +412,8 @@ def gemm_w4a16(x, wq_packed, scales, zeros, group, smooth=None, bias=None):
         bias = _c(bias.to(torch.float32))
     out = torch.empty(M, N, dtype=x.dtype, device=dev)
     # with smoothing the caller-owned workspace lets the multiply run once up front (the tile kernels need that;
-    # below 41 rows the library takes its weight-streaming kernels, which smooth in place)
-    ws = torch.empty(M, K, dtype=x.dtype, device=dev) if (smooth is not None and M > 40) else None
+    # up to 16 rows the library takes its weight-streaming kernels, which smooth in place)
+    ws = torch.empty(M, K, dtype=x.dtype, device=dev) if (smooth is not None and M > 16) else None
     with torch.cuda.device(dev):
         _lib.check(_lib.load().amct_gemm_w4a16(_p(x), _p(smooth), _p(wq_packed), _p(scales), dtype_code(scales.dtype),
                                                _p(zeros), _p(bias), _p(out), M, N, K, group, dtype_code(x.dtype),

@@ -237,7 +237,7 @@ int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s_tok, const
  * amct_quant_int4_group_pack; scales [N, K/group] of scale_dtype; zeros uint8 [N, K/group];
  * bias fp32 [N] or null.  out [M, N] bf16 = x' @ bf16((u - zero) * scale)^T + bias, fp32 accumulate.
  * workspace (may be null): M*K*2 bytes the caller lends; with it the smoothing multiply is done once
- * up front instead of inside every column tile (same results; the fast tile kernels for M > 40 need it
+ * up front instead of inside every column tile (same results; the fast tile kernels for M > 16 need it
  * when smooth is given, without it such calls take slower kernels that smooth in place). */
 int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t* wq, const void* scales,
                     int scale_dtype, const uint8_t* zeros, const float* bias, void* out,
