@@ -719,14 +719,16 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM
 // data-movement waves), 43 us (4), 51 us (4 waves doing everything); of the 38 us, 22 us are the matrix waves and
 // the barriers alone, the LDS writes of the dequantised weights add 8 us, the loads 7 us, the arithmetic 4 us.
 // ---------------------------------------------------------------------------
-// Tile (64*TI) x (64*TJ): 2 x 2 matrix waves of (32*TI) x (32*TJ) and 4*TJ data-movement waves (four threads per
-// weight row of the tile); 128x128 as described above, 64x64 and 128x64 for small M with 4 + 4 waves.
+// Tile (64*TI) x (64*TJ): 2 x 2 matrix waves of (32*TI) x (32*TJ) and 8 data-movement waves (512 / (64*TJ) threads per
+// weight row of the tile); 128x128 as described above, 64x64 and 128x64 for small M (8 weights per thread and step).
 template <bool SF16, int STAGES, int TI = 2, int TJ = 2, int kD = 4>
-__global__ __launch_bounds__((4 + 4 * TJ) * 64) __attribute__((amdgpu_waves_per_eu(1 + TJ, 1 + TJ))) void w4a16_tile_spec(W4A16Args a) {
+__global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) void w4a16_tile_spec(W4A16Args a) {
     constexpr int kLM = 64 * TI, kLN = 64 * TJ, WN = 2;
-    constexpr int kThreads = (4 + 4 * TJ) * 64;
+    constexpr int kThreads = kSpecThreads;
     constexpr int kStageBytes = (kLM + kLN) * kWRow;                // 32 KiB for 128x128
-    constexpr int kMW = 4 * TJ;                                     // data-movement waves
+    constexpr int kMW = kSpecThreads / 64 - 4;                      // data-movement waves: 8
+    constexpr int kPPR = kMW * 64 / kLN;                            // threads per weight row: 4 or 8
+    constexpr int kBC = 8 / kPPR;                                   // 8-weight chunks per thread and step: 2 or 1
     constexpr int kNA = (kLM * kWRow / 1024) / kMW;                 // activation pieces per moving wave
     constexpr int kNM = TI * TJ, kNR = TI + TJ;
     static_assert(STAGES == 2 || STAGES == 3, "stages");
@@ -784,29 +786,39 @@ __global__ __launch_bounds__((4 + 4 * TJ) * 64) __attribute__((amdgpu_waves_per_
             for (int j = 0; j < kNA; ++j)
                 dma16s(lds0 + stg * kStageBytes + (pw * kNA + j) * 1024, a.x + (int64_t)st * kWK, goff[j]);
         };
-        // weight row ptid/4 of the tile, 16 weights (8 bytes) per step, which quarter from ptid%4
-        const int brow = ptid >> 2, bq = ptid & 3;
+        // weight row ptid/kPPR of the tile, 8*kBC weights (4*kBC bytes) per step, which part from ptid%kPPR
+        const int brow = ptid / kPPR, bq = ptid % kPPR;
         const int64_t wrow = (n0 + brow < a.N) ? n0 + brow : a.N - 1;
-        const uint32_t woff = (uint32_t)(wrow * (a.K / 2) + bq * 8);
+        const uint32_t woff = (uint32_t)(wrow * (a.K / 2) + bq * (4 * kBC));
         const uint32_t* const trow = tab + brow * (kSpecMaxG + 1);
-        int bdst[2];
+        int bdst[kBC];
 #pragma unroll
-        for (int c = 0; c < 2; ++c) bdst[c] = kLM * kWRow + brow * kWRow + ((2 * bq + c) ^ swz(brow)) * 16;
+        for (int c = 0; c < kBC; ++c) bdst[c] = kLM * kWRow + brow * kWRow + ((kBC * bq + c) ^ swz(brow)) * 16;
         // The weights stream from HBM and a step of this small tile is shorter than that latency, so the packed
         // weights of a step are fetched kD steps ahead into kD register slots (the loop is unrolled by kD).
-        uint64_t wreg[kD];
+        typename std::conditional<kBC == 2, uint64_t, uint32_t>::type wreg[kD];
         auto issue_b = [&](int slot, int step) {
             const int st = step < last ? step : last;
-            asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(wreg[slot]) : "v"(woff), "s"(a.wq + (uint32_t)st * (kWK / 2)) : "memory");
+            if constexpr (kBC == 2)
+                asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(wreg[slot]) : "v"(woff), "s"(a.wq + (uint32_t)st * (kWK / 2)) : "memory");
+            else
+                asm volatile("global_load_dword %0, %1, %2" : "=v"(wreg[slot]) : "v"(woff), "s"(a.wq + (uint32_t)st * (kWK / 2)) : "memory");
         };
-        auto dequant_into = [&](int slot, int step, int stg) {      // the weights of K-step `step` (in `slot`) -> stage stg
+        // the factors of a step are read from the table one iteration before they are used (enext): the LDS latency
+        // would otherwise head the chain table read -> arithmetic -> LDS write -> barrier that bounds a step
+        auto factor_word = [&](int step) {
             const int st = step < last ? step : last;
-            const uint32_t gi = __umulhi((uint32_t)st * kWK, a.group_magic);   // k / group (k, group < 2^16); group % 64 == 0
-            const uint32_t e = trow[gi];
+            return trow[__umulhi((uint32_t)st * kWK, a.group_magic)];          // k / group (k, group < 2^16); group % 64 == 0
+        };
+        uint32_t enext = factor_word(0);
+        auto dequant_into = [&](int slot, int step, int stg) {      // the weights of K-step `step` (in `slot`) -> stage stg
+            const uint32_t e = enext;
             const float sc = SF16 ? f16_bits_to_f32(e & 0xFFFFu) : bf16_bits_to_f32(e & 0xFFFFu);
             const float nzs = -((float)(e >> 16) * sc);
             *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[0]) = dequant8((uint32_t)wreg[slot], sc, nzs);
-            *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[1]) = dequant8((uint32_t)(wreg[slot] >> 32), sc, nzs);
+            if constexpr (kBC == 2)
+                *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[1]) = dequant8((uint32_t)((uint64_t)wreg[slot] >> 32), sc, nzs);
+            enext = factor_word(step + 1);
         };
 #define AMCT_TIE_SLOT(slot) asm volatile("" : "+v"(wreg[slot]) : : "memory")
         // prologue: B(0 .. kD-1) into their slots and A(0 .. STAGES-2); everything lands; B(0) is dequantised into
@@ -1460,8 +1472,9 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
             // few (the weight stream is the bulk of the traffic for medium M): 128x128 blocks (with specialised waves
             // when K % 256 == 0: 38 us against 51 us on W[14336,4096], M = 129 .. 256; the first-generation kernel took
             // 97 us; 64-column blocks of 4 waves, a quarter of a weight row per thread and step, while they still fit the
-            // CUs in one round: 64x64 for M <= 64, 26 us, and 128x64 for M <= 128, 34 us; with 4 matrix and 4 data-movement
-            // waves when K % 256 == 0: 22 us and 27 us; fetching the weights 8 steps ahead instead of 4 changed nothing), then blocks of 8 waves: 256x128 for 256 < M <= 512 (65 us; half the
+            // CUs in one round: 64x64 for M <= 64, 26 us, and 128x64 for M <= 128, 34 us; with 4 matrix and 8 data-movement
+            // waves when K % 256 == 0: 20 us and 24 us; fetching the weights 8 steps ahead instead of 4 changed nothing, and two
+            // row tiles of 128x64 blocks lose to one 128x128 block for 128 < M <= 256: 46 us against 39 us), then blocks of 8 waves: 256x128 for 256 < M <= 512 (65 us; half the
             // dequantisation of 128x256 blocks, which take 72 .. 75 us; the first-generation kernel took 96 us), 128x256 where those do not fit the CUs, each with three LDS
             // stages; 256x256 with two stages otherwise.  (Mixing in 256x192
             // blocks as the W8A8 launch does was measured neutral here: the narrow tile dequantises as many weights.)
@@ -1475,8 +1488,8 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
             if (mt > 65535) return AMCT_E_UNSUPPORTED;
 #define AMCT_LAUNCH_WIDE(SF)                                                                                           \
     {                                                                                                                  \
-        if (shape == 3 && K % 256 == 0 && G <= kSpecMaxG) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3, 1, 1>), dim3((unsigned)nt64, 1), dim3(512), 0, st, a); \
-        else if (shape == 4 && K % 256 == 0 && G <= kSpecMaxG) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3, 2, 1>), dim3((unsigned)nt64, (unsigned)mt), dim3(512), 0, st, a); \
+        if (shape == 3 && K % 256 == 0 && G <= kSpecMaxG) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3, 1, 1>), dim3((unsigned)nt64, 1), dim3(kSpecThreads), 0, st, a); \
+        else if (shape == 4 && K % 256 == 0 && G <= kSpecMaxG) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3, 2, 1>), dim3((unsigned)nt64, (unsigned)mt), dim3(kSpecThreads), 0, st, a); \
         else if (shape == 3) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 1, 1, 3>), dim3((unsigned)nt64, 1), dim3(256), 0, st, a);          \
         else if (shape == 4) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 2, 1, 3>), dim3((unsigned)nt64, (unsigned)mt), dim3(256), 0, st, a); \
         else if (shape == 1 && K % 256 == 0 && G <= kSpecMaxG) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3>), dim3((unsigned)nt128, (unsigned)mt), dim3(kSpecThreads), 0, st, a); \
