@@ -813,16 +813,17 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
         uint32_t enext = factor_word(0);
         auto dequant_into = [&](int slot, int step, int stg) {      // the weights of K-step `step` (in `slot`) -> stage stg
             const uint32_t e = enext;
+            enext = factor_word(step + 1);                          // issued before this step's LDS writes (see the loop)
+            __builtin_amdgcn_sched_barrier(0);                      // keeps the read in front of the writes
             const float sc = SF16 ? f16_bits_to_f32(e & 0xFFFFu) : bf16_bits_to_f32(e & 0xFFFFu);
             const float nzs = -((float)(e >> 16) * sc);
             *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[0]) = dequant8((uint32_t)wreg[slot], sc, nzs);
             if constexpr (kBC == 2)
                 *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[1]) = dequant8((uint32_t)((uint64_t)wreg[slot] >> 32), sc, nzs);
-            enext = factor_word(step + 1);
         };
 #define AMCT_TIE_SLOT(slot) asm volatile("" : "+v"(wreg[slot]) : : "memory")
-        // prologue: B(0 .. kD-1) into their slots and A(0 .. STAGES-2); everything lands; B(0) is dequantised into
-        // stage 0 and its slot takes B(kD); A(STAGES-1) follows (weights first, as in the loop)
+        // prologue: B(0 .. kD-1) into their slots and A(0 .. STAGES-2); everything lands; B(0), B(1) are dequantised into
+        // stages 0, 1 and their slots take B(kD), B(kD+1); A(STAGES-1) follows (weights first, as in the loop)
 #pragma unroll
         for (int j = 0; j < kD; ++j) issue_b(j, j);
 #pragma unroll
@@ -831,32 +832,40 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
 #pragma unroll
         for (int j = 0; j < kD; ++j) AMCT_TIE_SLOT(j);
         dequant_into(0, 0, 0);
+        dequant_into(1, 1, 1);
         issue_b(0, kD);
+        issue_b(1, kD + 1);
         dma_a(STAGES - 1, STAGES - 1);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        // iteration s: wait for B(s+1) (slot SL; issued kD iterations ago: the kNA activation loads of that
-        // iteration and the 1 + kNA operations of each iteration since may stay in flight); B(s+1) -> stage nxt;
-        // wait for A(s+1) (issued STAGES-1 iterations ago); barrier; B(s+1+kD) into slot SL, A(s+STAGES) into stage cur
-        int cur = 0, nxt = 1;
+        // The dequantisation runs TWO steps ahead of the matrix waves, which need stage s+1 behind the barrier of
+        // iteration s: that barrier then waits for the LDS writes of the iteration before (lgkmcnt leaves this
+        // iteration's kBC writes in flight), so their latency is not part of the step's chain.
+        // iteration s: wait for B(s+2) (slot SL; issued kD iterations ago: the kNA activation loads of that iteration
+        // and the 1 + kNA operations of each iteration since may stay in flight; in iteration 2 the loads behind B(4)
+        // are those of the prologue's tail, one activation group fewer); B(s+2) -> stage (s+2) % STAGES, free since the
+        // barrier before; wait for A(s+1) (issued STAGES-1 iterations ago); barrier; B(s+2+kD) into slot SL,
+        // A(s+STAGES) into stage cur
+        int cur = 0, s2 = 2 % STAGES;
 #define AMCT_MOVE_ITER(SL, step)                                                       \
     {                                                                                  \
-        wait_vm<kNA + (kD - 1) * (1 + kNA)>();                                         \
+        if ((step) == kD - 2) wait_vm<(kD - 1) * (1 + kNA)>();                         \
+        else wait_vm<kNA + (kD - 1) * (1 + kNA)>();                                    \
         AMCT_TIE_SLOT(SL);                                                             \
-        dequant_into(SL, (step) + 1, nxt);                                             \
+        dequant_into(SL, (step) + 2, s2);                                              \
         wait_vm<(STAGES - 2) * (1 + kNA)>();                                           \
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                             \
+        asm volatile("s_waitcnt lgkmcnt(%0)" : : "n"(kBC) : "memory");                 \
         __builtin_amdgcn_s_barrier();                                                  \
         asm volatile("" ::: "memory");                                                 \
-        issue_b(SL, (step) + 1 + kD);                                                  \
+        issue_b(SL, (step) + 2 + kD);                                                  \
         dma_a(cur, (step) + STAGES);                                                   \
-        cur = nxt;                                                                     \
-        nxt = nxt + 1 == STAGES ? 0 : nxt + 1;                                         \
+        cur = cur + 1 == STAGES ? 0 : cur + 1;                                         \
+        s2 = s2 + 1 == STAGES ? 0 : s2 + 1;                                            \
     }
         for (int step = 0; step < nsteps; step += kD) {             // K % (64 * kD) == 0: a multiple of kD steps
 #pragma unroll
-            for (int u = 0; u < kD; ++u) AMCT_MOVE_ITER((u + 1) % kD, step + u)
+            for (int u = 0; u < kD; ++u) AMCT_MOVE_ITER((u + 2) % kD, step + u)
         }
 #undef AMCT_MOVE_ITER
 #undef AMCT_TIE_SLOT
