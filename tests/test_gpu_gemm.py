@@ -186,3 +186,29 @@ def test_gemm_dispatch_boundaries_in_m(dev, N, K):
             err = (out.cpu().double() - want[:M]).abs()
             tol = 1e-3 * want[:M].abs().amax(dim=1, keepdim=True) + want[:M].abs() * 2.0 ** -8
             assert (err <= tol).all(), (M, sm is not None, err.max().item())
+
+
+FULL_ROWS = [0, 1, 63, 64, 127, 128, 255, 256, 257, 511, 512, 1023, 1024, 1500, 2046, 2047]
+
+
+@pytest.mark.parametrize("M", [2048, 16, 1])
+def test_gemms_at_the_benchmark_size(dev, M):
+    """N = 14336, K = 4096 (the size the metric is quoted on) for M = 2048 and the decode sizes: sampled rows of the W8A8
+    output bit for bit and of the W4A16 output within its tolerance, every column."""
+    N, K, grp = 14336, 4096, 128
+    rows = [r for r in FULL_ROWS if r < M]
+    xq, wq, s_ch, s_tok, b = w8a8_case(M, N, K, 311, True, 'float')
+    out, acc = ops.gemm_w8a8(xq.to(dev), wq.to(dev), s_ch.to(dev), s_tok.to(dev), b.to(dev), want_acc=True)
+    want_acc = od.int8_matmul_exact(xq[rows], wq.t())
+    assert torch.equal(acc.cpu()[rows].to(torch.int64), want_acc), "accumulators"
+    assert_bits_equal(out.cpu()[rows], od.quant_matmul(xq[rows], wq.t(), s_ch, s_tok[rows], b, torch.bfloat16), "w8a8 out")
+    del out, acc
+    x, codes, scales, zeros, smooth, bias = w4a16_case(M, N, K, grp, 312)
+    packed = workloads.pack_nibbles(codes).to(dev)
+    for sm in (None, smooth):
+        out = ops.gemm_w4a16(x.to(dev), packed, scales.to(dev), zeros.to(dev), grp, None if sm is None else sm.to(dev),
+                             bias.to(dev)).cpu()[rows]
+        want = w4a16_oracle(x[rows], codes, scales, zeros, grp, sm, bias)
+        err = (out.double() - want).abs()
+        tol = 1e-3 * want.abs().amax(dim=1, keepdim=True) + want.abs() * 2.0 ** -8
+        assert (err <= tol).all(), (M, sm is not None, err.max().item())
