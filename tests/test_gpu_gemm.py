@@ -212,3 +212,32 @@ def test_gemms_at_the_benchmark_size(dev, M):
         err = (out.double() - want).abs()
         tol = 1e-3 * want.abs().amax(dim=1, keepdim=True) + want.abs() * 2.0 ** -8
         assert (err <= tol).all(), (M, sm is not None, err.max().item())
+
+
+@pytest.mark.parametrize("seed", [1, 2])
+def test_gemm_random_shapes(dev, seed):
+    """Seeded random (M, N, K, group, scale dtype, smoothing) over the values at which the libraries switch kernels and
+    over ragged ones: W8A8 bit for bit, W4A16 within its tolerance.  Every case is an ordinary supported call."""
+    import random
+    rng = random.Random(seed)
+    done = 0
+    while done < 40:
+        M = rng.choice([1, 2, 3, 9, 16, 17, 24, 25, 31, 40, 41, 64, 65, 100, 128, 129, 200, 256, 257, 300, 511, 512, 513, 700])
+        N = rng.choice([8, 16, 40, 64, 72, 128, 136, 200, 256, 520, 1000, 2056, 4104, 16392, 16400])
+        K = rng.choice([64, 128, 192, 256, 320, 384, 512, 768, 1024, 2048, 4096, 8192, 8448])
+        if M * N * K > 1.2e10:
+            continue
+        done += 1
+        xq, wq, s_ch, s_tok, b = w8a8_case(M, N, K, 1000 * seed + done, True, 'float')
+        out = ops.gemm_w8a8(xq.to(dev), wq.to(dev), s_ch.to(dev), s_tok.to(dev), b.to(dev))
+        assert_bits_equal(out, od.quant_matmul(xq, wq.t(), s_ch, s_tok, b, torch.bfloat16), "w8a8 %d %d %d" % (M, N, K))
+        group = rng.choice([g for g in (32, 64, 128, 256) if K % g == 0])
+        sdt = rng.choice([torch.float16, torch.bfloat16])
+        x, codes, scales, zeros, smooth, bias = w4a16_case(M, N, K, group, 1000 * seed + done, sdt)
+        sm = smooth if rng.random() < 0.4 else None
+        o4 = ops.gemm_w4a16(x.to(dev), workloads.pack_nibbles(codes).to(dev), scales.to(dev), zeros.to(dev), group,
+                            None if sm is None else sm.to(dev), bias.to(dev)).cpu()
+        want = w4a16_oracle(x, codes, scales, zeros, group, sm, bias)
+        err = (o4.double() - want).abs()
+        tol = 1e-3 * want.abs().amax(dim=1, keepdim=True) + want.abs() * 2.0 ** -8
+        assert (err <= tol).all(), (M, N, K, group, sdt, sm is not None, err.max().item())
