@@ -186,13 +186,15 @@ def test_awq_path_differs_only_by_the_cast():
     wf = w.float()
     s, z = iq.weight_scale_offset(wf, 'channel', True, 'int8')
     assert torch.equal(iq.awq_fake_quant(wf, 'int8', s, z, 'channel'), iq.fake_quant(wf, 'int8', s, z))
-    # a bf16 value that the cast moves across a rounding boundary: t = 2.498 -> bf16(2.5) -> 2
-    # while the fp32 path rounds 2.498 -> 2 as well; 3.498 -> bf16 3.5 -> 4 vs fp32 -> 3
-    wv = torch.tensor([[3.498, 100.0]], dtype=torch.float32)
-    s1 = torch.tensor([[1.0]])
-    assert iq.fake_quant(wv, 'int8', s1)[0, 0].item() == 3.0
-    assert iq.awq_fake_quant(wv.to(torch.bfloat16), 'int8', s1, None, 'channel')[0, 0].item() == 4.0 or \
-        wv.to(torch.bfloat16)[0, 0].item() != 3.498
+    # a value that the cast moves across a rounding boundary: bf16 w = 3.5, fp32 s = 1.0003 -> w/s = 3.49895,
+    # which rounds to 3 in fp32 but is 3.5 once narrowed to bf16 and then rounds (half to even) to 4
+    wv = torch.tensor([[3.5, 100.0]], dtype=torch.bfloat16)
+    s1 = torch.tensor([[1.0003]])
+    assert torch.round(wv.float() / s1)[0, 0].item() == 3.0
+    assert iq.quant_codes(wv, 'int8', s1)[0, 0].item() == 3
+    assert iq.fake_quant(wv, 'int8', s1)[0, 0].item() == torch.tensor(3 * 1.0003).to(torch.bfloat16).item()
+    assert iq.awq_fake_quant(wv, 'int8', s1, None, 'channel')[0, 0].item() == \
+        torch.tensor(4 * 1.0003).to(torch.bfloat16).item()
 
 
 def test_dynamic_token_quant():
@@ -238,6 +240,55 @@ def test_oracle_matches_exact_arithmetic_fixture():
         got_codes = iq.quant_codes(w, kind, s, z)
         assert torch.equal(got_codes.to(torch.int32), codes)
         assert_bits_equal(iq.fake_quant(w, kind, s, z), dq, "dq")
+
+
+def test_oracle_matches_exact_arithmetic_fixture_16bit_group_awq():
+    """tests/golden/int_quant_kat16.json: the same exact-fraction model for bf16 / fp16 / fp32 sources, factors per
+    group (ragged last group zero-padded) and the cast-before-round variant of the AWQ search."""
+    from util import load_int_quant_kat16
+    cases = load_int_quant_kat16()
+    assert len(cases) >= 130
+    differs = 0
+    for c in cases:
+        kind = 'int%d' % c["bits"]
+        w, g, sym = c["w"], c["group"], c["symmetric"]
+        strat = 'group' if g else 'channel'
+        s, z = iq.weight_scale_offset(w, strat, sym, kind, g or None)
+        assert_bits_equal(s.reshape(-1), c["scale"], "scale")
+        if sym:
+            assert z is None
+        else:
+            assert torch.equal(z.reshape(-1), c["offset"])
+        codes = iq.quant_codes(w, kind, s, z, g or None).reshape(1, -1)[:, :w.shape[1]]
+        assert torch.equal(codes.to(torch.int32), c["codes"])
+        assert_bits_equal(iq.fake_quant(w, kind, s, z, g or None), c["dq"], "dq")
+        assert_bits_equal(iq.awq_fake_quant(w, kind, s, z, strat, g or None), c["awq_dq"], "awq dq")
+        differs += int(not torch.equal(c["dq"], c["awq_dq"]))
+    assert differs >= 20                                  # the file does separate the two paths
+
+
+def test_dynamic_token_quant_absmax_known_answers():
+    """The experimental tree's per-token form (node.py:39-43,181-204): s = absmax / 127 with s = 1 for a dead row,
+    q = clamp(rne(x / s), -128, 127).  Rows whose absmax is 127 * 2^k have a power-of-two scale, so every quotient
+    and tie is exact in fp32."""
+    x = torch.tensor([[127.0, -63.5, 62.5, 0.5, -0.5, 1.5, -127.0, 0.0],
+                      [-254.0, 3.0, 1.0, -1.0, 5.0, 7.0, 253.0, 2.0],
+                      [0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0],
+                      [-31.75, 0.125, 0.375, 0.625, -0.125, -0.375, 31.5, 0.25]], dtype=torch.float32)
+    q, s = iq.dynamic_token_quant_absmax(x)
+    assert s.tolist() == [1.0, 2.0, 1.0, 0.25]
+    assert q.dtype == torch.int8
+    assert q.tolist() == [[127, -64, 62, 0, 0, 2, -127, 0],
+                          [-127, 2, 0, 0, 2, 4, 126, 1],
+                          [0, 0, 0, 0, 0, 0, 0, 0],
+                          [-127, 0, 2, 2, 0, -2, 126, 1]]
+    # the positive extremum never produces -128, the negative one never exceeds -127 (absmax rule, no 128 scope)
+    xb = torch.tensor([[-1.0, 0.999]], dtype=torch.bfloat16)
+    qb, sb = iq.dynamic_token_quant_absmax(xb)
+    assert sb.dtype == torch.bfloat16 and qb[0, 0].item() == -127 and qb[0, 1].item() == 127
+    # the AMCT rule on the same row uses scope 128 where the negative extremum dominates
+    qa, sa = iq.dynamic_token_quant(x[1:2])
+    assert sa.item() == 254.0 / 128 and qa[0, 0].item() == -128
 
 
 def test_awq_search_special_cases():
