@@ -15,6 +15,7 @@ STAGE_FULL, STAGE_SCALE, STAGE_DEQUANT, STAGE_COL = 0, 1, 2, 3
 CODES_NONE, CODES_I8, CODES_I32 = 0, 1, 2
 MX_E4M3, MX_E2M1 = 0, 1
 MX_FLOOR, MX_RCEIL = 0, 1
+COL_MINMAX_NOALLOC_MAX_COLS = 8192
 
 _P = ctypes.c_void_p
 _I = ctypes.c_int
@@ -33,6 +34,7 @@ SIGNATURES = {
     "amct_scale_f32_to_u64": (_I, [_P, _P, _L, _P]),
     "amct_col_minmax_workspace_bytes": (ctypes.c_size_t, [_L, _L]),
     "amct_col_minmax": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _P, ctypes.c_size_t, _P]),
+    "amct_col_minmax_noalloc": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _P]),
     "amct_awq_loss_workspace_bytes": (ctypes.c_size_t, []),
     "amct_awq_loss": (_I, [_P, _P, _L, _I, _P, _P, ctypes.c_size_t, _P]),
     "amct_scale_offset": (_I, [_P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _P]),

@@ -10,6 +10,7 @@ extern "C" const char* amct_hip_strerror(int code) {
         case AMCT_E_UNSUPPORTED: return "shape or combination not supported by the kernels";
         case AMCT_E_ALIGN: return "alignment or divisibility requirement violated";
         case AMCT_E_HIP: return "HIP runtime reported a launch error";
+        case AMCT_E_TOO_LARGE: return "problem exceeds the fixed scratch buffer of the allocation-free entry point";
         default: return "unknown error code";
     }
 }

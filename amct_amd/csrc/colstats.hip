@@ -8,6 +8,8 @@
 //   pass 2: one lane per column folds the chunks (coalesced across columns) and applies the update rule.
 // max / min propagate NaN like torch.amax / amin; the running update `batch > old ? batch : old` then
 // ignores a NaN batch value, exactly as torch.where does in the reference.
+#include <atomic>
+
 #include "amct_common.h"
 
 namespace amct {
@@ -156,18 +158,12 @@ extern "C" size_t amct_col_minmax_workspace_bytes(int64_t rows, int64_t cols) {
     return (size_t)chunks * 2 * (size_t)cols * sizeof(float);
 }
 
-extern "C" int amct_col_minmax(const void* x, float* col_max, float* col_min, int64_t rows, int64_t cols, int absolute,
-                               int accumulate, int dtype, void* workspace, size_t workspace_bytes, amct_stream_t stream) {
-    if (rows < 0 || cols <= 0) return AMCT_E_BADARG;
-    if (dtype != AMCT_F32 && dtype != AMCT_F16 && dtype != AMCT_BF16) return AMCT_E_BADARG;
-    if (rows == 0) return AMCT_OK;                                  // no batch: the running values stay
-    if (!x || (!col_max && !col_min) || !workspace) return AMCT_E_BADARG;
-    if (workspace_bytes < amct_col_minmax_workspace_bytes(rows, cols)) return AMCT_E_BADARG;
-    if ((reinterpret_cast<uintptr_t>(workspace) & 3u) != 0) return AMCT_E_ALIGN;
+// shared by both entry points: `ws` holds chunks * 2 * cols floats and is fully overwritten by pass 1 before pass 2 reads it
+static int col_minmax_launch(const void* x, float* col_max, float* col_min, int64_t rows, int64_t cols, int absolute,
+                             int accumulate, int dtype, float* ws, hipStream_t st) {
     ColArgs a{};
-    a.x = x; a.ws = reinterpret_cast<float*>(workspace); a.rows = rows; a.cols = cols;
+    a.x = x; a.ws = ws; a.rows = rows; a.cols = cols;
     chunking(rows, a.rows_per_chunk, a.chunks);
-    hipStream_t st = (hipStream_t)stream;
 #define AMCT_CS(DT)                                                                                              \
     {                                                                                                            \
         constexpr int VEC = Tr<DT>::VEC;                                                                         \
@@ -190,4 +186,58 @@ extern "C" int amct_col_minmax(const void* x, float* col_max, float* col_min, in
     hipLaunchKernelGGL(col_final_k, dim3((unsigned)((cols + kBlock - 1) / kBlock)), dim3(kBlock), 0, st, a.ws, col_max,
                        col_min, cols, a.chunks, accumulate);
     return hip_status();
+}
+
+extern "C" int amct_col_minmax(const void* x, float* col_max, float* col_min, int64_t rows, int64_t cols, int absolute,
+                               int accumulate, int dtype, void* workspace, size_t workspace_bytes, amct_stream_t stream) {
+    if (rows < 0 || cols <= 0) return AMCT_E_BADARG;
+    if (dtype != AMCT_F32 && dtype != AMCT_F16 && dtype != AMCT_BF16) return AMCT_E_BADARG;
+    if (rows == 0) return AMCT_OK;                                  // no batch: the running values stay
+    if (!x || (!col_max && !col_min) || !workspace) return AMCT_E_BADARG;
+    if (workspace_bytes < amct_col_minmax_workspace_bytes(rows, cols)) return AMCT_E_BADARG;
+    if ((reinterpret_cast<uintptr_t>(workspace) & 3u) != 0) return AMCT_E_ALIGN;
+    return col_minmax_launch(x, col_max, col_min, rows, cols, absolute, accumulate, dtype,
+                             reinterpret_cast<float*>(workspace), (hipStream_t)stream);
+}
+
+// ---- the same reduction for callers that cannot allocate -----------------------------------------------------
+// The per-chunk partials live in a fixed array in device memory that is part of the library's code object: every
+// GPU the library runs on holds its own copy (4 MiB) until the process ends.  The array's name is only a host-side
+// handle; its device address is asked for once per device and kept.
+static __device__ __align__(256) float scratch[(size_t)kCsMaxChunks * 2 * AMCT_COL_MINMAX_NOALLOC_MAX_COLS];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<float*> scratch_ptr[kMaxDevices];
+
+// device address of `scratch` on the current device (null on failure); first call per device asks the runtime
+static float* scratch_on_current_device() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    float* p = scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        void* q = nullptr;
+        if (hipGetSymbolAddress(&q, HIP_SYMBOL(scratch)) != hipSuccess || !q) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        p = reinterpret_cast<float*>(q);
+        scratch_ptr[dev].store(p, std::memory_order_release);       // racing first calls store the same address
+    }
+    return p;
+}
+
+extern "C" int amct_col_minmax_noalloc(const void* x, float* col_max, float* col_min, int64_t rows, int64_t cols,
+                                       int absolute, int accumulate, int dtype, amct_stream_t stream) {
+    if (rows < 0 || cols <= 0) return AMCT_E_BADARG;
+    if (dtype != AMCT_F32 && dtype != AMCT_F16 && dtype != AMCT_BF16) return AMCT_E_BADARG;
+    if (cols > AMCT_COL_MINMAX_NOALLOC_MAX_COLS) return AMCT_E_TOO_LARGE;
+    if (rows == 0) return AMCT_OK;
+    if (!x || (!col_max && !col_min)) return AMCT_E_BADARG;
+    float* ws = scratch_on_current_device();
+    if (!ws) return AMCT_E_HIP;
+    // pass 1 writes every partial that pass 2 reads, so nothing of an earlier call has to be cleared
+    return col_minmax_launch(x, col_max, col_min, rows, cols, absolute, accumulate, dtype, ws, (hipStream_t)stream);
 }

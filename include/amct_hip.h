@@ -8,7 +8,8 @@
  *     kernels, anything else a slower general kernel (same results);
  *   - the library never allocates, frees or synchronises: the caller owns all
  *     buffers (including workspaces) and supplies the stream; every call only
- *     enqueues work on `stream` and returns;
+ *     enqueues work on `stream` and returns (amct_col_minmax_noalloc keeps its
+ *     workspace in a fixed device array of the library instead);
  *   - return value: 0 on success, a negative AMCT_E_* code otherwise
  *     (amct_hip_strerror gives the text); no exception crosses the boundary;
  *     a call that fails enqueues nothing and leaves its outputs untouched;
@@ -39,7 +40,8 @@ enum {
     AMCT_E_BADARG = -1,                 /* null pointer, negative size, unknown enum */
     AMCT_E_UNSUPPORTED = -2,            /* shape / combination the kernels do not cover */
     AMCT_E_ALIGN = -3,                  /* alignment or divisibility requirement violated */
-    AMCT_E_HIP = -4                     /* the HIP runtime reported a launch error */
+    AMCT_E_HIP = -4,                    /* the HIP runtime reported a launch error */
+    AMCT_E_TOO_LARGE = -5               /* the problem exceeds the fixed scratch buffer of an allocation-free entry point */
 };
 
 /* symmetric scope rule */
@@ -96,6 +98,18 @@ int amct_mfma_yardstick(int bf16, int random_operands, int iters, void* sink, in
 size_t amct_col_minmax_workspace_bytes(int64_t rows, int64_t cols);
 int amct_col_minmax(const void* x, float* col_max, float* col_min, int64_t rows, int64_t cols, int absolute,
                     int accumulate, int dtype, void* workspace, size_t workspace_bytes, amct_stream_t stream);
+
+/* amct_col_minmax without a workspace argument.  No counterpart in the reference: it is for callers that cannot
+ * allocate device memory around the call (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  Same arguments, kernels and results as amct_col_minmax; the per-chunk partials go to a fixed array
+ * inside the library's device image instead (64 chunks x 2 x AMCT_COL_MINMAX_NOALLOC_MAX_COLS floats = 4 MiB, held
+ * by every GPU the library runs on until the process ends).  cols > AMCT_COL_MINMAX_NOALLOC_MAX_COLS returns
+ * AMCT_E_TOO_LARGE and enqueues nothing.  The call allocates and frees nothing.  All calls on one GPU share that
+ * array: calls that overlap on one GPU (different streams or threads) race; calls on one stream do not.  Nothing
+ * has to be cleared between calls (the first pass overwrites every partial the second pass reads). */
+#define AMCT_COL_MINMAX_NOALLOC_MAX_COLS 8192
+int amct_col_minmax_noalloc(const void* x, float* col_max, float* col_min, int64_t rows, int64_t cols, int absolute,
+                            int accumulate, int dtype, amct_stream_t stream);
 
 /* ---- loss of one AWQ grid point ---------------------------------------------------------------------
  * Replaces the expression of amct_pytorch/algorithm/awq.py:96, `(ori_out - quant_out).float().pow(4).mean()`:
