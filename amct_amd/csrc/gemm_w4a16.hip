@@ -1432,6 +1432,10 @@ __global__ __launch_bounds__(kBlock) void w4a16_general(W4A16Args a) {
     a.out[m * a.N + n] = (uint16_t)f32_to_bf16_bits(acc);
 }
 
+int wq16_int4_f16(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
+                  const uint8_t* zeros, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group,
+                  hipStream_t st);                                 // gemm_wq16.hip
+
 }  // namespace amct
 
 using namespace amct;
@@ -1443,9 +1447,12 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
     if (M < 0 || N <= 0 || K <= 0 || group <= 0) return AMCT_E_BADARG;
     if (M != 0 && (!x || !wq || !scales || !zeros || !out)) return AMCT_E_BADARG;   // M == 0 reads nothing
     if (scale_dtype != AMCT_F16 && scale_dtype != AMCT_BF16) return AMCT_E_BADARG;
-    if (dtype != AMCT_BF16) return AMCT_E_UNSUPPORTED;
+    if (dtype != AMCT_BF16 && dtype != AMCT_F16) return AMCT_E_UNSUPPORTED;
     if (K % group != 0 || K % 2 != 0) return AMCT_E_ALIGN;
     if (M == 0) return AMCT_OK;
+    // fp16 activations: the kernels shared with the int8-weight path (gemm_wq16.hip), which smooth in the tile
+    if (dtype == AMCT_F16)
+        return wq16_int4_f16(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, (hipStream_t)stream);
     W4A16Args a{(const uint16_t*)x, (const uint16_t*)smooth, wq, scales, zeros, bias, (uint16_t*)out, M, N, K, group, scale_dtype,
                 (uint32_t)(0x100000000ull / (uint64_t)group) + 1u};
     hipStream_t st = (hipStream_t)stream;

@@ -45,7 +45,10 @@ class HipQuantizationLinear(torch.nn.Module):
         codes = self.quant_wts(weight, scale_w, wts_type, smooth)          # [N,K] int8, K contiguous
         self.register_buffer('quantized_weight', torch.transpose(codes, 1, 0))
         if quant_module.offset_d is not None:
-            # -round(offset_d[1,K] @ Wq[K,N]) with the integer contraction done exactly by the GEMM kernel
+            # -(offset_d[1,K] @ Wq[K,N]) with the integer contraction done exactly by the int8 GEMM kernel.  The
+            # reference forms the same sum with an fp32 matmul and rounds it (npu_quantization_linear.py:56-59): that
+            # is exact while K * |offset_d| * 127 < 2^24 and otherwise carries the rounding of its library's summation
+            # order; the exact integer is what that expression approximates, and is what is registered here.
             zrow = quant_module.offset_d.to(device).reshape(1, 1).to(torch.int8).repeat(1, weight.shape[-1])
             one = torch.ones(weight.shape[0], dtype=torch.float32, device=device)
             _, acc = ops.gemm_w8a8(zrow, codes, one, want_acc=True, out_dtype=torch.float32)
@@ -84,6 +87,9 @@ class HipQuantizationLinear(torch.nn.Module):
         s_tok = self.pertoken_scale
         m = xq.numel() // xq.shape[-1]
         if s_tok is not None and s_tok.numel() != m:
+            if s_tok.numel() != x.shape[-2]:
+                raise RuntimeError("per-token scales were calibrated for {} tokens, the input has {}".format(
+                    s_tok.numel(), x.shape[-2]))
             s_tok = s_tok.repeat(m // s_tok.numel())
         out = ops.gemm_w8a8(xq.reshape(-1, x.shape[-1]), self.quantized_weight.t(), self.deq_scale, s_tok,
                             self.bias, self.output_dtype)
@@ -97,8 +103,10 @@ class HipQuantizationLinear(torch.nn.Module):
 
     def _init_bias(self, module, scale_d, scale_w):
         """npu_quantization_linear.py:105-130."""
-        self._dyn_scale_w = scale_w
-        self._dyn_bias = module.bias.data.float() if module.bias is not None else None
+        # operands of the dynamic_act path: buffers (so that .to(device) moves them) that stay out of state_dict
+        self.register_buffer('_dyn_scale_w', scale_w, persistent=False)
+        self.register_buffer('_dyn_bias', module.bias.data.float() if module.bias is not None else None,
+                             persistent=False)
         if module.bias is not None:
             bias = module.bias
             if self.act_granularity == 'PER_TENSOR':

@@ -39,6 +39,20 @@ def _p(t):
     return None if t is None else t.data_ptr()
 
 
+def _need(cond, msg, *args):
+    """Host-side operand check: the kernels only see pointers, so every size they rely on is verified here,
+    before anything is launched."""
+    if not cond:
+        raise RuntimeError(msg.format(*args))
+
+
+def _segments(rows, cols, group):
+    """Number of (scale, offset) entries for a [rows, cols] tensor: per group, per row (0) or per tensor (-1)."""
+    if group > 0:
+        return rows * ((cols + group - 1) // group)
+    return rows if group == 0 else 1
+
+
 def _stream(dev):
     return torch.cuda.current_stream(dev).cuda_stream
 
@@ -69,14 +83,22 @@ def col_minmax(x, col_max=None, col_min=None, absolute=False):
     """Per-column (input channel) max and min over all rows of x [rows, cols] -> fp32 [cols] each.
     With col_max / col_min given (fp32 [cols]) the running update `batch > old ? batch : old` is applied to
     them in place and they are returned; absolute=True reduces |x| and returns only the maximum."""
+    _need(x.dim() == 2, "col_minmax expects a 2-D tensor, got {} dims", x.dim())
+    rows, cols = x.shape
+    for name, t in (("col_max", col_max), ("col_min", col_min)):
+        _need(t is None or (t.dtype == torch.float32 and t.numel() == cols and t.is_contiguous()),
+              "col_minmax: {} must be a contiguous fp32 tensor of {} elements", name, cols)
     dev = _dev(x, col_max, col_min)
     x = _c(x)
-    rows, cols = x.shape
     accumulate = col_max is not None or col_min is not None
+    # a running tensor the caller did not pass starts at the neutral element of its update, so that the
+    # accumulating kernel never folds uninitialised memory into the result
     if col_max is None:
-        col_max = torch.empty(cols, dtype=torch.float32, device=dev)
+        col_max = torch.full((cols,), float('-inf'), dtype=torch.float32, device=dev) if accumulate else \
+            torch.empty(cols, dtype=torch.float32, device=dev)
     if col_min is None and not absolute:
-        col_min = torch.empty(cols, dtype=torch.float32, device=dev)
+        col_min = torch.full((cols,), float('inf'), dtype=torch.float32, device=dev) if accumulate else \
+            torch.empty(cols, dtype=torch.float32, device=dev)
     lib = _lib.load()
     nbytes = lib.amct_col_minmax_workspace_bytes(rows, cols)
     ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=dev)
@@ -122,9 +144,17 @@ def scale_offset(vmax, vmin, bits, symmetric, scope_rule=SCOPE_AMCT, bad=None):
 def quant_with_params(w, scale, offset, group, qmin, qmax, want_dq=True, codes_kind=CODES_NONE, col_scale=None,
                       col_mode=COL_NONE, via_src=False, stage=STAGE_FULL):
     """group: >0 per group, 0 per row, -1 per tensor.  Returns (dq | None, codes | None)."""
+    _need(w.dim() == 2, "quantise expects a 2-D tensor, got {} dims", w.dim())
+    rows, cols = w.shape
+    nseg = _segments(rows, cols, group)
+    _need(scale.numel() == nseg, "scale has {} entries, the tensor [{}, {}] with group {} needs {}", scale.numel(), rows,
+          cols, group, nseg)
+    _need(offset is None or offset.numel() == nseg, "offset has {} entries, {} expected",
+          0 if offset is None else offset.numel(), nseg)
+    _need(col_scale is None or col_scale.numel() == cols, "column scale has {} entries, {} columns",
+          0 if col_scale is None else col_scale.numel(), cols)
     dev = _dev(w, scale, offset, col_scale)
     w = _c(w)
-    rows, cols = w.shape
     scale = _c(scale.to(torch.float32))
     if offset is not None:
         offset = _c(offset.to(torch.int32))
@@ -159,10 +189,14 @@ def fakequant_int(w, bits, symmetric, group=0, want_dq=True, codes_kind=CODES_NO
                   qmin=None, qmax=None, col_scale=None, col_mode=COL_NONE, via_src=False, bad=None):
     """One pass over w: min/max -> factors -> quantise.  Returns (dq, codes, scale, offset);
     scale/offset are flat [rows] (group=0) or [rows, cols/group]."""
+    _need(w.dim() == 2, "quantise expects a 2-D tensor, got {} dims", w.dim())
+    rows, cols = w.shape
+    _need(group >= 0, "the fused kernel takes per-row (0) or per-group (> 0) factors, got group {}", group)
+    _need(col_scale is None or col_scale.numel() == cols, "column scale has {} entries, {} columns",
+          0 if col_scale is None else col_scale.numel(), cols)
     dev = _dev(w, col_scale, bad)
     w = _c(w)
-    rows, cols = w.shape
-    nseg = rows if group == 0 else rows * ((cols + group - 1) // group)
+    nseg = _segments(rows, cols, group)
     if qmin is None:
         qmin = -(1 << (bits - 1))
     if qmax is None:
@@ -193,11 +227,14 @@ def fakequant_int(w, bits, symmetric, group=0, want_dq=True, codes_kind=CODES_NO
 def quant_int4_group_pack(w, group, symmetric=False, scale_dtype=torch.float16, want_scales32=False, col_scale=None,
                           col_mode=COL_NONE, bad=None):
     """w [N,K] -> (packed uint8 [N,K/2], scales16 [N,K/g], zeros uint8 [N,K/g], scales32 | None)."""
+    _need(w.dim() == 2, "quantise expects a 2-D tensor, got {} dims", w.dim())
+    rows, cols = w.shape
+    if group <= 0 or cols % group or group % 32:
+        raise ValueError("int4 group pack needs cols % group == 0 and group % 32 == 0")
+    _need(col_scale is None or col_scale.numel() == cols, "column scale has {} entries, {} columns",
+          0 if col_scale is None else col_scale.numel(), cols)
     dev = _dev(w, col_scale, bad)
     w = _c(w)
-    rows, cols = w.shape
-    if cols % group or group % 32:
-        raise ValueError("int4 group pack needs cols % group == 0 and group % 32 == 0")
     g = cols // group
     packed = torch.empty(rows, cols // 2, dtype=torch.uint8, device=dev)
     s16 = torch.empty(rows, g, dtype=scale_dtype, device=dev)
@@ -338,10 +375,14 @@ def mx_quant(x, fmt, scale_mode=MX_FLOOR):
 
 
 def mx_dequant(el, e8, fmt, dtype=torch.bfloat16):
+    cols = e8.shape[-1] * 32
+    rows = e8.numel() // max(e8.shape[-1], 1)
+    want = tuple(e8.shape[:-1]) + (cols if fmt == MX_E4M3 else cols // 2,)
+    _need(el.dtype == torch.uint8 and e8.dtype == torch.uint8, "MX elements and shared exponents are uint8 tensors")
+    _need(tuple(el.shape) == want, "MX elements have shape {}, the shared exponents {} imply {}", tuple(el.shape),
+          tuple(e8.shape), want)
     dev = _dev(el, e8)
     el, e8 = _c(el), _c(e8)
-    cols = e8.shape[-1] * 32
-    rows = e8.numel() // e8.shape[-1]
     y = torch.empty(*e8.shape[:-1], cols, dtype=dtype, device=dev)
     with torch.cuda.device(dev):
         _lib.check(_lib.load().amct_mx_dequant(_p(el), _p(e8), _p(y), rows, cols, fmt, dtype_code(dtype), _stream(dev)))
@@ -371,12 +412,19 @@ def hif8_decode(c, dtype=torch.bfloat16):
 # ---------------------------------------------------------------------------
 def gemm_w8a8(xq, wq_nk, s_ch, s_tok=None, bias=None, out_dtype=torch.bfloat16, want_acc=False):
     """xq int8 [M,K], wq_nk int8 [N,K] (K contiguous) -> out [M,N] (and int32 accumulators)."""
-    dev = _dev(xq, wq_nk, s_ch, s_tok, bias)
-    xq, wq_nk = _c(xq), _c(wq_nk)
+    _need(xq.dim() == 2 and wq_nk.dim() == 2, "int8 GEMM expects 2-D operands")
+    _need(xq.dtype == torch.int8 and wq_nk.dtype == torch.int8, "int8 GEMM expects int8 operands")
     M, K = xq.shape
     N = wq_nk.shape[0]
     if wq_nk.shape[1] != K:
         raise RuntimeError("int8 GEMM: K mismatch ({} vs {})".format(K, wq_nk.shape[1]))
+    _need(s_ch.numel() in (1, N), "int8 GEMM: {} channel scales for {} output channels", s_ch.numel(), N)
+    _need(s_tok is None or s_tok.numel() == M, "int8 GEMM: {} token scales for {} rows",
+          0 if s_tok is None else s_tok.numel(), M)
+    _need(bias is None or bias.numel() == N, "int8 GEMM: bias has {} entries, {} output channels",
+          0 if bias is None else bias.numel(), N)
+    dev = _dev(xq, wq_nk, s_ch, s_tok, bias)
+    xq, wq_nk = _c(xq), _c(wq_nk)
     s_ch = _c(s_ch.reshape(-1).to(torch.float32))
     if s_ch.numel() == 1:
         s_ch = s_ch.expand(N).contiguous()
@@ -398,24 +446,66 @@ def gemm_w8a8(xq, wq_nk, s_ch, s_tok=None, bias=None, out_dtype=torch.bfloat16, 
     return (out, acc) if want_acc else out
 
 
+def _check_weight_only(x, N, K, scales, zeros, group, smooth, bias, zeros_dtype, what):
+    _need(x.dim() == 2 and x.shape[1] == K, "{}: activations must be [M, {}], got {}", what, K, tuple(x.shape))
+    _need(x.dtype in (torch.bfloat16, torch.float16), "Not support tensor dtype {}, support dtypes {}.", x.dtype,
+          [torch.bfloat16, torch.float16])
+    _need(group > 0 and K % group == 0, "{}: K = {} is not a multiple of the group size {}", what, K, group)
+    want = (N, K // group)
+    _need(scales.dtype in (torch.float16, torch.bfloat16), "{}: scales must be fp16 or bf16, got {}", what, scales.dtype)
+    _need(tuple(scales.shape) == want, "{}: scales have shape {}, expected {}", what, tuple(scales.shape), want)
+    _need(zeros is None or (zeros.dtype == zeros_dtype and tuple(zeros.shape) == want),
+          "{}: zero-points have shape {} / dtype {}, expected {} / {}", what,
+          None if zeros is None else tuple(zeros.shape), None if zeros is None else zeros.dtype, want, zeros_dtype)
+    _need(smooth is None or smooth.numel() == K, "{}: smooth factor has {} entries, K = {}", what,
+          0 if smooth is None else smooth.numel(), K)
+    _need(bias is None or bias.numel() == N, "{}: bias has {} entries, {} output channels", what,
+          0 if bias is None else bias.numel(), N)
+
+
 def gemm_w4a16(x, wq_packed, scales, zeros, group, smooth=None, bias=None):
-    """x [M,K] bf16; wq_packed uint8 [N,K/2]; scales [N,K/g] f16|bf16; zeros uint8 [N,K/g]."""
+    """x [M,K] bf16|f16; wq_packed uint8 [N,K/2]; scales [N,K/g] f16|bf16; zeros uint8 [N,K/g]."""
+    _need(wq_packed.dim() == 2 and wq_packed.dtype == torch.uint8, "int4 GEMM: the weight must be uint8 [N, K/2]")
+    N, K = wq_packed.shape[0], wq_packed.shape[1] * 2
+    if x.dim() == 2 and x.shape[1] != K:
+        raise RuntimeError("int4 GEMM: K mismatch ({} vs {})".format(x.shape[1], K))
+    _need(zeros is not None, "int4 GEMM: zero-points are required (8 everywhere for symmetric codes)")
+    _check_weight_only(x, N, K, scales, zeros, group, smooth, bias, torch.uint8, "int4 GEMM")
     dev = _dev(x, wq_packed, scales, zeros, smooth, bias)
     x, wq_packed, scales, zeros = _c(x), _c(wq_packed), _c(scales), _c(zeros)
-    M, K = x.shape
-    N = wq_packed.shape[0]
-    if wq_packed.shape[1] * 2 != K:
-        raise RuntimeError("int4 GEMM: K mismatch ({} vs {})".format(K, wq_packed.shape[1] * 2))
+    M = x.shape[0]
     if smooth is not None:
         smooth = _c(smooth.reshape(-1).to(x.dtype))
     if bias is not None:
-        bias = _c(bias.to(torch.float32))
+        bias = _c(bias.reshape(-1).to(torch.float32))
     out = torch.empty(M, N, dtype=x.dtype, device=dev)
-    # with smoothing the caller-owned workspace lets the multiply run once up front (the tile kernels need that;
-    # up to 16 rows the library takes its weight-streaming kernels, which smooth in place)
-    ws = torch.empty(M, K, dtype=x.dtype, device=dev) if (smooth is not None and M > 16) else None
+    # with smoothing the caller-owned workspace lets the multiply run once up front (the bf16 tile kernels need
+    # that; up to 16 rows the library takes its weight-streaming kernels, which smooth in place)
+    ws = torch.empty(M, K, dtype=x.dtype, device=dev) if (smooth is not None and M > 16 and x.dtype == torch.bfloat16) \
+        else None
     with torch.cuda.device(dev):
         _lib.check(_lib.load().amct_gemm_w4a16(_p(x), _p(smooth), _p(wq_packed), _p(scales), dtype_code(scales.dtype),
                                                _p(zeros), _p(bias), _p(out), M, N, K, group, dtype_code(x.dtype),
                                                _p(ws), 0 if ws is None else ws.numel() * 2, _stream(dev)))
+    return out
+
+
+def gemm_w8a16(x, wq_nk, scales, offsets, group, smooth=None, bias=None):
+    """x [M,K] bf16|f16; wq_nk int8 [N,K] (K contiguous); scales [N,K/g] f16|bf16; offsets int8 [N,K/g] | None."""
+    _need(wq_nk.dim() == 2 and wq_nk.dtype == torch.int8, "int8 weight-only GEMM: the weight must be int8 [N, K]")
+    N, K = wq_nk.shape
+    _check_weight_only(x, N, K, scales, offsets, group, smooth, bias, torch.int8, "int8 weight-only GEMM")
+    dev = _dev(x, wq_nk, scales, offsets, smooth, bias)
+    x, wq_nk, scales = _c(x), _c(wq_nk), _c(scales)
+    offsets = None if offsets is None else _c(offsets)
+    M = x.shape[0]
+    if smooth is not None:
+        smooth = _c(smooth.reshape(-1).to(x.dtype))
+    if bias is not None:
+        bias = _c(bias.reshape(-1).to(torch.float32))
+    out = torch.empty(M, N, dtype=x.dtype, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().amct_gemm_w8a16(_p(x), _p(smooth), _p(wq_nk), _p(scales), dtype_code(scales.dtype),
+                                               _p(offsets), _p(bias), _p(out), M, N, K, group, dtype_code(x.dtype),
+                                               _stream(dev)))
     return out

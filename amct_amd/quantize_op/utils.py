@@ -26,11 +26,15 @@ def get_int_quant_scope(data_type, symmetric, abs_max_is_negative=False):
     return abs_max_is_negative + pow(2, quant_bits - 1) - 1
 
 
-def calculate_scale_offset(data_max, data_min, symmetric, data_type):
+def calculate_scale_offset(data_max, data_min, symmetric, data_type, check=True):
     """(scale fp32, offset int32 | None), shaped like data_max (utils.py:75-108).  Raises the
-    reference's RuntimeError when a factor is not finite."""
+    reference's RuntimeError when a factor is not finite.  That check reads a flag back from the device, which
+    synchronises the stream: check=False skips it for callers inside a loop (the factors are computed the same
+    way, a non-finite one is simply not reported) -- validate once afterwards with check_scale_offset."""
     bits = int(data_type.replace('int', ''))
     dev = data_max.device
+    if not check:
+        return ops.scale_offset(data_max, data_min, bits, bool(symmetric))
     bad = torch.zeros(2, dtype=torch.int32, device=dev)
     scale, offset = ops.scale_offset(data_max, data_min, bits, bool(symmetric), bad=bad[:1])
     if int(bad[0].item()):

@@ -60,8 +60,11 @@ def npu_quant_matmul(x1, x2, scale, offset=None, bias=None, pertoken_scale=None,
     x2d = x1.reshape(-1, x1.shape[-1])
     s_tok = pertoken_scale
     if s_tok is not None and s_tok.numel() != x2d.shape[0]:
-        reps = x2d.shape[0] // s_tok.numel()
-        s_tok = s_tok.reshape(-1).repeat(reps)
+        # one scale per token of the last-but-one dim, shared by every leading batch index
+        if s_tok.numel() == 0 or s_tok.numel() != x1.shape[-2]:
+            raise RuntimeError("npu_quant_matmul: {} token scales for inputs of shape {}".format(
+                s_tok.numel(), tuple(x1.shape)))
+        s_tok = s_tok.reshape(-1).repeat(x2d.shape[0] // s_tok.numel())
     out = ops.gemm_w8a8(x2d, _weight_nk(x2), scale, s_tok, bias, output_dtype)
     return out.reshape(*lead, -1)
 
@@ -71,43 +74,96 @@ def npu_convert_weight_to_int4pack(weight, inner_k_tiles=0):
     return ops.pack_int4_words(weight)
 
 
+class _LayoutCache:
+    """Converted operands of npu_weight_quant_batchmatmul, keyed on the identity and version of the tensors the
+    caller passed.  A deploy module calls the operator with the same registered buffers on every forward; their
+    kernel layout ([N, K] weights, [N, K/g] factors) is computed on the first call only.  Entries hold weak
+    references to their sources, so a buffer that is freed, replaced or written in place is converted again."""
+
+    def __init__(self, capacity=256):
+        self.capacity = capacity
+        self.entries = {}
+
+    @staticmethod
+    def _key(tensors, extra):
+        return tuple((t.data_ptr(), t._version, tuple(t.shape), t.dtype) if t is not None else None
+                     for t in tensors) + (extra,)
+
+    def get(self, tensors, extra, make):
+        import weakref
+        key = self._key(tensors, extra)
+        hit = self.entries.get(key)
+        if hit is not None and all((r is None and t is None) or (r is not None and r() is t)
+                                   for r, t in zip(hit[0], tensors)):
+            return hit[1]
+        value = make()
+        if len(self.entries) >= self.capacity:
+            self.entries.pop(next(iter(self.entries)))
+        self.entries[key] = ([None if t is None else weakref.ref(t) for t in tensors], value)
+        return value
+
+    def clear(self):
+        self.entries.clear()
+
+
+_layout_cache = _LayoutCache()
+
+
 def npu_weight_quant_batchmatmul(x, weight, antiquant_scale, antiquant_offset=None, quant_scale=None,
                                  quant_offset=None, bias=None, antiquant_group_size=0, inner_precise=0):
-    """x [M, K] @ ((weight + antiquant_offset) * antiquant_scale) + bias with weight int4 packed
-    [K, N/8] int32, factors [K/g, N] (or [1|N-broadcast, N] when antiquant_group_size == 0)."""
+    """x [..., K] @ ((weight + antiquant_offset) * antiquant_scale) + bias.  weight: int8 [K, N], or int4 packed
+    [K, N/8] int32; factors [K/g, N] (or broadcastable to [1, N] when antiquant_group_size == 0), in x's dtype.
+    The kernels stream [N, K] weights and [N, K/g] factors: the conversion of the operands a caller passes is done
+    once per (tensor, version) and cached."""
     if quant_scale is not None or quant_offset is not None:
         raise RuntimeError("npu_weight_quant_batchmatmul: output quantisation is not supported")
-    if weight.dtype != torch.int32:
-        raise RuntimeError("npu_weight_quant_batchmatmul: only packed int4 weights (int32 words) are supported")
+    if weight.dtype not in (torch.int32, torch.int8) or weight.dim() != 2:
+        raise RuntimeError("npu_weight_quant_batchmatmul: the weight must be int8 [K, N] or packed int4 (int32 [K, N/8])")
     K = x.shape[-1]
     if weight.shape[0] != K:
-        raise RuntimeError("npu_weight_quant_batchmatmul: weight must be [K, N/8]")
-    N = weight.shape[1] * 8
+        raise RuntimeError("npu_weight_quant_batchmatmul: weight must be [K, N] / [K, N/8]")
+    int4 = weight.dtype == torch.int32
+    N = weight.shape[1] * (8 if int4 else 1)
     group = antiquant_group_size if antiquant_group_size else K
-    packed = ops.words_to_nibbles_nk(weight, K, N)
-    scales, zeros = factors_to_native(antiquant_scale, antiquant_offset, N, K // group)
+    if K % group:
+        raise RuntimeError("npu_weight_quant_batchmatmul: K is not a multiple of antiquant_group_size")
+
+    def convert():
+        if int4:
+            wq = ops.words_to_nibbles_nk(weight, K, N)
+        else:
+            wq = weight.t().contiguous()
+        return (wq,) + factors_to_native(antiquant_scale, antiquant_offset, N, K // group, int4)
+
+    wq, scales, zeros = _layout_cache.get((weight, antiquant_scale, antiquant_offset), (group, x.dtype), convert)
     lead = x.shape[:-1]
-    out = ops.gemm_w4a16(x.reshape(-1, K), packed, scales, zeros, group, None, bias)
+    x2 = x.reshape(-1, K)
+    out = ops.gemm_w4a16(x2, wq, scales, zeros, group, None, bias) if int4 else \
+        ops.gemm_w8a16(x2, wq, scales, zeros, group, None, bias)
     return out.reshape(*lead, N)
 
 
-def factors_to_native(antiquant_scale, antiquant_offset, N, G):
-    """Reference factor layout ([G, N], offset stored negated in the float dtype) -> kernel layout
-    (scales [N, G] f16|bf16, zeros uint8 [N, G] = 8 - antiquant_offset)."""
+def factors_to_native(antiquant_scale, antiquant_offset, N, G, int4=True):
+    """Reference factor layout ([G, N], offset stored negated in the float dtype) -> kernel layout: scales [N, G]
+    f16|bf16; int4: zeros uint8 [N, G] = 8 - antiquant_offset; int8: offsets int8 [N, G] = -antiquant_offset
+    (None when there is no antiquant_offset)."""
     sc = antiquant_scale.reshape(-1, N) if antiquant_scale.dim() > 1 else antiquant_scale.reshape(1, -1)
     if sc.shape[0] not in (1, G):
         raise RuntimeError("antiquant_scale has {} groups, expected {}".format(sc.shape[0], G))
     sc = sc.expand(G, N).t().contiguous()
     if sc.dtype not in (torch.float16, torch.bfloat16):
         sc = sc.to(torch.bfloat16)
+    lo, hi, base = (0, 15, 8) if int4 else (-128, 127, 0)
     if antiquant_offset is None:
-        zeros = torch.full((N, G), 8, dtype=torch.uint8, device=sc.device)
+        zeros = torch.full((N, G), 8, dtype=torch.uint8, device=sc.device) if int4 else None
     else:
         off = antiquant_offset.reshape(-1, N) if antiquant_offset.dim() > 1 else antiquant_offset.reshape(1, -1)
-        z = 8 - off.expand(G, N).t().to(torch.int32)
-        if int(z.min()) < 0 or int(z.max()) > 15:
-            raise RuntimeError("antiquant_offset outside the int4 range")
-        zeros = z.to(torch.uint8).contiguous()
+        if off.shape[0] not in (1, G):
+            raise RuntimeError("antiquant_offset has {} groups, expected {}".format(off.shape[0], G))
+        z = base - off.expand(G, N).t().to(torch.int32)
+        if int(z.min()) < lo or int(z.max()) > hi:
+            raise RuntimeError("antiquant_offset outside the {} range".format("int4" if int4 else "int8"))
+        zeros = z.to(torch.uint8 if int4 else torch.int8).contiguous()
     return sc, zeros
 
 

@@ -247,16 +247,29 @@ int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s_tok, const
 /* ---- K7: W4A16 Linear -------------------------------------------------------------------------------------
  * Replaces torch_npu.npu_weight_quant_batchmatmul as called at
  * amct_pytorch/deploy_op/weight_npu_quant_module.py:116-117 (with the x * scale_factor of :113-114
- * fused in).  x [M, K] bf16; smooth [K] bf16 or null; wq uint8 [N, K/2] as written by
+ * fused in).  x [M, K] of dtype (AMCT_BF16 or AMCT_F16, the source dtypes of
+ * amct_pytorch/utils/vars.py:43-47); smooth [K] of dtype or null; wq uint8 [N, K/2] as written by
  * amct_quant_int4_group_pack; scales [N, K/group] of scale_dtype; zeros uint8 [N, K/group];
- * bias fp32 [N] or null.  out [M, N] bf16 = x' @ bf16((u - zero) * scale)^T + bias, fp32 accumulate.
+ * bias fp32 [N] or null.  out [M, N] of dtype = x' @ dtype((u - zero) * scale)^T + bias, fp32 accumulate.
  * workspace (may be null): M*K*2 bytes the caller lends; with it the smoothing multiply is done once
- * up front instead of inside every column tile (same results; the fast tile kernels for M > 16 need it
+ * up front instead of inside every column tile (same results; the fast bf16 tile kernels for M > 16 need it
  * when smooth is given, without it such calls take slower kernels that smooth in place). */
 int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t* wq, const void* scales,
                     int scale_dtype, const uint8_t* zeros, const float* bias, void* out,
                     int64_t M, int64_t N, int64_t K, int group, int dtype,
                     void* workspace, size_t workspace_bytes, amct_stream_t stream);
+
+/* ---- W8A16 Linear (int8 weight-only) ---------------------------------------------------------------------
+ * The same operator with the int8 weight the reference's module registers when wts_type is int8
+ * (amct_pytorch/deploy_op/weight_npu_quant_module.py:51-53: quant_weight yields int8 codes, only int4 is packed).
+ * x [M, K] of dtype (AMCT_BF16 or AMCT_F16); smooth [K] of dtype or null; wq int8 [N, K] signed codes, K contiguous
+ * (the transpose of the [K, N] buffer of :53); scales [N, K/group] of scale_dtype (group = K: one per output
+ * channel, the reference's antiquant_group_size = 0); offsets int8 [N, K/group] = the quantiser's offset_w, null
+ * when symmetric (the module registers its negation as antiquant_offset, :62-64); bias fp32 [N] or null.
+ * out [M, N] of dtype = x' @ dtype((q - offset) * scale)^T + bias, fp32 accumulate. */
+int amct_gemm_w8a16(const void* x, const void* smooth, const int8_t* wq, const void* scales, int scale_dtype,
+                    const int8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K,
+                    int group, int dtype, amct_stream_t stream);
 
 /* ---- GPTQ inner block ------------------------------------------------------------------------
  * The column loop of amct_pytorch/quantize_op/gptq_module.py:128-151 for one block of count <= 128 columns,

@@ -70,3 +70,51 @@ def test_compressed_tensors_config_matches_the_fixture():
     plain = ic.generate_quant_config(False, [])
     assert plain["kv_cache_scheme"] is None and list(plain["config_groups"]) == ["group_0"]
     assert json.loads(json.dumps(plain)) == plain          # serialisable as written
+
+
+def test_operand_sizes_are_checked_before_any_launch():
+    """The kernels only see pointers: every factor / bias / scale length they rely on is verified on the host and
+    raises before a device is touched (so CPU tensors are enough to show it)."""
+    import pytest
+    import torch
+    from amct_amd import ops, torch_hip
+    w = torch.zeros(8, 64)
+    with pytest.raises(RuntimeError, match="scale has 7 entries"):
+        ops.quant_with_params(w, torch.ones(7), None, 0, -128, 127)
+    with pytest.raises(RuntimeError, match="scale has 8 entries"):
+        ops.quant_with_params(w, torch.ones(8), None, 32, -8, 7)
+    with pytest.raises(RuntimeError, match="offset has 3 entries"):
+        ops.quant_with_params(w, torch.ones(16), torch.zeros(3, dtype=torch.int32), 32, -8, 7)
+    with pytest.raises(RuntimeError, match="column scale has 63 entries"):
+        ops.quant_with_params(w, torch.ones(8), None, 0, -128, 127, col_scale=torch.ones(63), col_mode=ops.COL_MUL)
+    with pytest.raises(RuntimeError, match="column scale has 65 entries"):
+        ops.fakequant_int(w, 8, True, col_scale=torch.ones(65), col_mode=ops.COL_MUL)
+    with pytest.raises(RuntimeError, match="column scale"):
+        ops.quant_int4_group_pack(w, 32, col_scale=torch.ones(1), col_mode=ops.COL_MUL)
+    xq = torch.zeros(6, 64, dtype=torch.int8)
+    wq = torch.zeros(16, 64, dtype=torch.int8)
+    with pytest.raises(RuntimeError, match="15 channel scales"):
+        ops.gemm_w8a8(xq, wq, torch.ones(15))
+    with pytest.raises(RuntimeError, match="4 token scales for 6 rows"):
+        ops.gemm_w8a8(xq, wq, torch.ones(16), s_tok=torch.ones(4))
+    with pytest.raises(RuntimeError, match="bias has 17 entries"):
+        ops.gemm_w8a8(xq, wq, torch.ones(16), bias=torch.zeros(17))
+    # the operator level repeats a per-token scale over leading batch dims only when it divides evenly
+    with pytest.raises(RuntimeError, match="token scales"):
+        torch_hip.npu_quant_matmul(xq, wq.t(), torch.ones(16), pertoken_scale=torch.ones(4))
+    x = torch.zeros(4, 64, dtype=torch.bfloat16)
+    wp = torch.zeros(16, 32, dtype=torch.uint8)
+    with pytest.raises(RuntimeError, match="scales have shape"):
+        ops.gemm_w4a16(x, wp, torch.ones(16, 1, dtype=torch.float16), torch.zeros(16, 2, dtype=torch.uint8), 32)
+    with pytest.raises(RuntimeError, match="zero-points have shape"):
+        ops.gemm_w4a16(x, wp, torch.ones(16, 2, dtype=torch.float16), torch.zeros(16, 1, dtype=torch.uint8), 32)
+    with pytest.raises(RuntimeError, match="smooth factor has 10 entries"):
+        ops.gemm_w4a16(x, wp, torch.ones(16, 2, dtype=torch.float16), torch.zeros(16, 2, dtype=torch.uint8), 32,
+                       smooth=torch.ones(10, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="bias has 3 entries"):
+        ops.gemm_w4a16(x, wp, torch.ones(16, 2, dtype=torch.float16), torch.zeros(16, 2, dtype=torch.uint8), 32,
+                       bias=torch.zeros(3))
+    with pytest.raises(RuntimeError, match="MX elements have shape"):
+        ops.mx_dequant(torch.zeros(4, 60, dtype=torch.uint8), torch.zeros(4, 2, dtype=torch.uint8), ops.MX_E4M3)
+    with pytest.raises(RuntimeError, match="col_max must be"):
+        ops.col_minmax(torch.zeros(4, 64), col_max=torch.zeros(63))

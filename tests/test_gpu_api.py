@@ -167,6 +167,29 @@ def test_w8a8_module(dev, mode, with_bias):
     assert {'act_scale', 'act_offset', 'quantized_weight', 'deq_scale'} <= keys
 
 
+def test_w8a8_offset_bias_at_k4096_is_the_exact_integer(dev):
+    """With an activation offset the module folds -(offset_d @ Wq) into an int32 bias.  The reference evaluates that
+    sum with an fp32 matmul (npu_quantization_linear.py:56-59), which stops being exact once
+    K * |offset| * 127 > 2^24; the module registers the exact integer.  At K = 4096 the two differ by at most the
+    rounding of an fp32 sum of that magnitude, and the module's value equals the int64 sum."""
+    torch.manual_seed(21)
+    N, K = 64, 4096
+    w = (torch.randn(N, K) * 0.05).to(torch.bfloat16)
+    scale_w, _ = iq.weight_scale_offset(w, 'channel', True, 'int8')
+    scale_d = torch.tensor([0.037])
+    offset_d = torch.tensor([-77], dtype=torch.int32)
+    buf = od.w8a8_buffers(w, None, scale_w, scale_d, offset_d, None)
+    qm = quant_module(w.to(dev), None, scale_w=scale_w.to(dev), scale_d=scale_d.to(dev), offset_d=offset_d.to(dev))
+    mod = HipQuantizationLinear(qm)
+    exact = 77 * buf['quantized_weight'].to(torch.int64).sum(dim=0)       # -(offset * sum_k Wq[k, n])
+    assert mod.bias.dtype == torch.int32 and torch.equal(mod.bias.cpu().to(torch.int64), exact)
+    # the reference's fp32 evaluation: within one rounding per partial sum of the exact value
+    ref_bias = buf['bias'].to(torch.int64)
+    bound = exact.abs().max().item() * 2.0 ** -23 * 8 + 1
+    assert (ref_bias - exact).abs().max().item() <= bound
+    assert 'quantized_weight' in mod.state_dict() and '_dyn_scale_w' not in mod.state_dict()
+
+
 def test_w8a8_module_dynamic(dev):
     torch.manual_seed(4)
     N, K, M = 64, 256, 40
@@ -220,6 +243,72 @@ def test_w4a16_module(dev, group, sym, with_awq):
     out2 = torch_hip.npu_weight_quant_batchmatmul(xs.reshape(-1, K), words, sw, antiquant_offset=ow if not sym else None,
                                                   bias=mod.bias, antiquant_group_size=group or 0)
     assert_bits_equal(out2.reshape(3, M, N), got.cpu(), "operator vs module")
+
+
+@pytest.mark.parametrize("kind", ['int8', 'int4'])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("strategy,group,sym,with_awq", [('group', 32, False, False), ('channel', None, True, False),
+                                                         ('tensor', None, False, False), ('group', 64, True, True),
+                                                         ('channel', None, False, True)])
+@pytest.mark.parametrize("M", [9, 70])
+def test_weight_only_module_matrix(dev, kind, dtype, strategy, group, sym, with_awq, M):
+    """The weight-only half of the reference's deploy matrix (tests/amct_pytorch/test_minmax.py:56-381 followed by
+    convert): int8 and int4 weights, bf16 and fp16 models, every granularity; buffers against the restatement of
+    amct_pytorch/deploy_op/weight_npu_quant_module.py:29-100, the forward against the fp64 anchor."""
+    torch.manual_seed(15)
+    N, K = 72, 256
+    w = (torch.randn(N, K) * 0.05).to(dtype)
+    b = torch.randn(N).to(dtype)
+    x = torch.randn(2, M, K).to(dtype)
+    awq_scale = (0.5 + torch.rand(1, K)).to(dtype) if with_awq else None
+    wa = iq.awq_weight(w, awq_scale) if with_awq else w
+    scale_w, offset_w = iq.weight_scale_offset(wa, strategy, sym, kind, group)
+    buf = od.w4a16_buffers(w, b, scale_w, offset_w, kind, group, awq_scale)
+    qm = quant_module(w.to(dev), torch.nn.Parameter(b.to(dev), requires_grad=False), wts_type=kind,
+                      scale_w=scale_w.to(dev), offset_w=None if offset_w is None else offset_w.to(dev),
+                      scale=None if awq_scale is None else awq_scale.to(dev), group_size=group)
+    mod = HipWeightQuantizedLinear(qm)
+    qw, sw, ow = mod.reference_layout()
+    assert_bits_equal(qw, buf['quantized_weight'], "quantized_weight in the reference's layout")
+    assert qw.dtype == (torch.int8 if kind == 'int8' else torch.int32)
+    assert_bits_equal(sw, buf['scale_w'], "scale_w [K/g,N]")
+    if buf['offset_w'] is None:
+        assert ow is None
+    else:
+        assert_bits_equal(ow, buf['offset_w'], "offset_w [K/g,N]")
+    assert mod.group_size == buf['group_size']
+    got = mod(x.to(dev))
+    assert got.shape == (2, M, N) and got.dtype == dtype
+    g = group or K
+    want = od.w4a16_forward_f64(x, buf['codes_nk'].reshape(N, K), buf['scale_w'].t(),
+                                None if buf['offset_w'] is None else buf['offset_w'].t().float(), g,
+                                buf['bias'], awq_scale)
+    err = (got.cpu().double() - want).abs()
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    tol = 1e-3 * want.abs().amax(dim=-1, keepdim=True) + want.abs() * ulp
+    assert (err <= tol).all(), float((err / tol).max())
+    # operator-level drop-in with the reference's operand layouts: same bits as the module
+    xs = x.to(dev) if awq_scale is None else torch.mul(x.to(dev), awq_scale.to(dev))
+    for _ in range(2):                                               # the second call takes the cached layouts
+        out2 = torch_hip.npu_weight_quant_batchmatmul(xs.reshape(-1, K), qw, sw, antiquant_offset=ow, bias=mod.bias,
+                                                      antiquant_group_size=group or 0)
+        assert_bits_equal(out2.reshape(2, M, N), got.cpu(), "operator vs module")
+    keys = set(mod.state_dict().keys())
+    assert {'quantized_weight', 'scale_w', 'bias'} <= keys and ('offset_w' in keys) == (not sym or kind == 'int4')
+
+
+def test_weight_only_layout_cache_follows_in_place_updates(dev):
+    """The operator-level path caches the converted weight per (tensor, version): an in-place write to the buffer
+    must be seen by the next call."""
+    torch.manual_seed(16)
+    M, K, N = 8, 128, 32
+    x = torch.randn(M, K).to(torch.bfloat16).to(dev)
+    wq = torch.randint(-128, 128, (K, N), dtype=torch.int8).to(dev)
+    sw = (torch.rand(1, N) * 0.01 + 0.001).to(torch.bfloat16).to(dev)
+    a = torch_hip.npu_weight_quant_batchmatmul(x, wq, sw)
+    wq.zero_()
+    b = torch_hip.npu_weight_quant_batchmatmul(x, wq, sw)
+    assert float(a.float().abs().max()) > 0 and float(b.float().abs().max()) == 0.0
 
 
 def test_operator_level_w8a8(dev):
@@ -339,3 +428,12 @@ def test_awq_loss_kernel(dev, dt, n):
         assert torch.isnan(ops.awq_loss(y[:0].to(dev), yh[:0].to(dev)))
         with pytest.raises(RuntimeError):
             ops.awq_loss(y.to(dev), yh[:-1].to(dev))
+
+
+def test_calculate_scale_offset_without_the_synchronising_check(dev):
+    mx = torch.tensor([[1.27], [float('inf')]], device=dev)
+    mn = torch.tensor([[-1.0], [0.0]], device=dev)
+    s, z = qutils.calculate_scale_offset(mx, mn, True, 'int8', check=False)       # no exception, no read-back
+    assert z is None and s[0, 0].item() == torch.tensor(1.27).div(127).item() and torch.isinf(s[1, 0])
+    with pytest.raises(RuntimeError, match="Param scale has invalid value"):
+        qutils.check_scale_offset(s, None)

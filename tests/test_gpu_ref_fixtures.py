@@ -4,7 +4,10 @@ exact-fraction known answers for 16-bit sources, groups and the cast-before-roun
 import pytest
 import torch
 
+import types
+
 from amct_amd import ops
+from amct_amd.deploy_op import HipQuantizationLinear, HipWeightQuantizedLinear
 from amct_amd.algorithm import awq as hawq
 from amct_amd.quantize_op import gptq as hgptq
 from amct_amd.quantize_op import smooth_quant_stats as hsq
@@ -143,3 +146,49 @@ def test_reference_gptq(dev, ref):
         frac = (diff > 0.51 * step).float().mean().item()
         assert frac <= 0.05, (idx, frac)
         assert float(diff.max()) <= 4.0 * step, (idx, float(diff.max()), step)
+
+
+def test_reference_weight_only_deploy_buffers(dev, ref):
+    """HipWeightQuantizedLinear built from the same calibrated fields as the reference's module: its buffers,
+    brought to the reference's layout, equal the registered buffers the reference wrote (the int4 word packing
+    itself lives in torch_npu: the fixture holds the unpacked [K, N] int32 codes)."""
+    for c in ref["weight_only_deploy"]:
+        qm = types.SimpleNamespace(weight=torch.nn.Parameter(c["weight"].to(dev), requires_grad=False),
+                                   bias=torch.nn.Parameter(c["bias"].to(dev), requires_grad=False),
+                                   wts_type=c["kind"], group_size=c["group"] or None, scale_w=c["scale_w"].to(dev),
+                                   offset_w=None if c["offset_w"] is None else c["offset_w"].to(dev), scale=None)
+        mod = HipWeightQuantizedLinear(qm)
+        want = c["buffers"]
+        qw, sw, ow = mod.reference_layout()
+        if c["kind"] == 'int4':
+            qw = ops.unpack_nibbles_to_i32_kn(mod.quantized_weight)
+        assert qw.dtype == want["quantized_weight"].dtype
+        assert torch.equal(qw.cpu(), want["quantized_weight"])
+        assert_bits_equal(sw, want["scale_w"], "scale_w")
+        if "offset_w" in want:
+            assert_bits_equal(ow, want["offset_w"], "offset_w")
+        else:
+            assert ow is None
+        assert torch.equal(mod.bias.cpu(), c["dep_bias"].float())
+        assert mod.group_size == c["dep_group_size"]
+
+
+def test_reference_w8a8_deploy_buffers(dev, ref):
+    """HipQuantizationLinear from the reference's calibrated SmoothQuant fields against the buffers its
+    NpuQuantizationLinear registered."""
+    for c in ref["smoothquant"]:
+        qm = types.SimpleNamespace(weight=torch.nn.Parameter(c["weight"].to(dev), requires_grad=False),
+                                   bias=torch.nn.Parameter(c["bias"].to(dev), requires_grad=False),
+                                   act_type='int8', wts_type='int8', scale_w=c["scale_w"].to(dev), offset_w=None,
+                                   scale_d=c["scale_d"].to(dev),
+                                   offset_d=None if c["offset_d"] is None else c["offset_d"].to(dev),
+                                   scale=c["smooth"].to(dev), group_size=None)
+        mod = HipQuantizationLinear(qm)
+        dep = c["deploy"]
+        assert torch.equal(mod.quantized_weight.cpu(), dep["quantized_weight"])
+        for k in ("act_scale", "act_offset", "deq_scale", "scale_factor"):
+            assert_bits_equal(getattr(mod, k), dep[k], k)
+        if "pertoken_scale" in dep:
+            assert_bits_equal(mod.pertoken_scale, dep["pertoken_scale"], "pertoken_scale")
+        want_b = c["deploy_bias"]
+        assert mod.bias.dtype == want_b.dtype and torch.equal(mod.bias.cpu(), want_b)
