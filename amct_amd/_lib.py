@@ -6,7 +6,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libamct_hip.so")
+# AMCT_HIP_LIB names another build of the same library (for comparing two builds on one machine)
+LIB_PATH = os.environ.get("AMCT_HIP_LIB") or os.path.join(_HERE, "lib", "libamct_hip.so")
 
 F32, F16, BF16 = 0, 1, 2
 SCOPE_AMCT, SCOPE_ABSMAX = 0, 1

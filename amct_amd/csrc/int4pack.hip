@@ -128,7 +128,11 @@ __global__ __launch_bounds__(kBlock) void int4_group_pack(PackArgs a) {
 // The factors of group u are computed by the lanes with lt % 4 == u and shared inside each quad by
 // DPP; the per-element division is the exact fma sequence when every group of the wave allows it.
 // ---------------------------------------------------------------------------
-template <int DT, int T, int NV, bool COL>
+// FULL: every block is complete (the group count is a multiple of the groups per block), every lane's vector exists
+// (group length = T * NV vectors) and the tensor is below 2 GiB: addresses are then one wave-uniform 64-bit base per
+// block plus 32-bit lane offsets and nothing is clamped or predicated, which removes about 90 of the 480 vector
+// instructions a wave spends on its 2048 elements.
+template <int DT, int T, int NV, bool COL, bool FULL = false>
 __global__ __launch_bounds__(kBlock) void int4_group_pack4(PackArgs a) {
     constexpr int U = 4;
     constexpr int VEC = Tr<DT>::VEC;
@@ -147,17 +151,31 @@ __global__ __launch_bounds__(kBlock) void int4_group_pack4(PackArgs a) {
     // group u of the team is u groups further, or the last group of the tensor if the team hangs over its end
     uint4 raw[U][NV];
     int64_t segc[U];
+    const uint32_t blk_bytes = (uint32_t)(TEAMS * U) * (uint32_t)a.seg_len * BYTES;      // input bytes of one block
+    const uint32_t lane_off = (uint32_t)(team * U) * ((uint32_t)a.seg_len * BYTES) + (uint32_t)lt * 16u;
+    if constexpr (FULL) {
+        const char* blk = reinterpret_cast<const char*>(a.w) + (int64_t)blockIdx.x * blk_bytes;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            segc[u] = seg0 + u;
+#pragma unroll
+            for (int v = 0; v < NV; ++v)
+                raw[u][v] = ldg16_nt(blk + (lane_off + (uint32_t)u * ((uint32_t)a.seg_len * BYTES) + (uint32_t)(v * T * 16)));
+        }
+    }
     const int64_t seg_first = seg0 < a.nseg ? seg0 : a.nseg - 1;
     const int64_t left = a.nseg - 1 - seg_first;                    // groups after the first one
     const int left32 = left < U ? (int)left : U - 1;
     const char* base = reinterpret_cast<const char*>(a.w) + seg_first * a.seg_len * BYTES;
     const uint32_t seg_bytes = (uint32_t)a.seg_len * BYTES;
+    if constexpr (!FULL) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-        const int uc = u < left32 ? u : left32;
-        segc[u] = seg_first + uc;
+        for (int u = 0; u < U; ++u) {
+            const int uc = u < left32 ? u : left32;
+            segc[u] = seg_first + uc;
 #pragma unroll
-        for (int v = 0; v < NV; ++v) raw[u][v] = ldg16_nt(base + (uint32_t)uc * seg_bytes + (uint32_t)vl[v] * 16u);
+            for (int v = 0; v < NV; ++v) raw[u][v] = ldg16_nt(base + (uint32_t)uc * seg_bytes + (uint32_t)vl[v] * 16u);
+        }
     }
     float x[U][NV][VEC];
 #pragma unroll
@@ -199,8 +217,8 @@ __global__ __launch_bounds__(kBlock) void int4_group_pack4(PackArgs a) {
     const Divisor dmy = divisor_of(f);
     const uint32_t big = max(__float_as_uint(mx_my) & 0x7FFFFFFFu, __float_as_uint(mn_my) & 0x7FFFFFFFu);
     const bool fast = wave_all(dmy.fast && big < 0x5D800000u);       // |x| < 2^60, finite
-    if (lt < 4 && seg0 + my < a.nseg) {
-        const int64_t sg = seg0 + my;
+    if (lt < 4 && (FULL || seg0 + my < a.nseg)) {
+        const int64_t sg = FULL ? (int64_t)blockIdx.x * (TEAMS * U) + (team * U + my) : seg0 + my;
         if (a.scales32) a.scales32[sg] = f.s;
         if (a.scales16) {
             reinterpret_cast<uint16_t*>(a.scales16)[sg] =
@@ -219,6 +237,12 @@ __global__ __launch_bounds__(kBlock) void int4_group_pack4(PackArgs a) {
 
     // codes u = q + 8 are gathered by exact fp32 arithmetic: sum (q_j + 8) * 16^j over 4 nibbles
     uint32_t word[U][NV];
+    // keeps each variant's arithmetic inside its own branch: without it the optimiser computes the first product of
+    // every division ahead of the four-way branch and holds 32 more registers live
+    auto pinned = [](float v) {
+        asm volatile("" : "+v"(v));
+        return v;
+    };
     auto encode = [&](auto fast_tag, auto asym_tag) {
         constexpr bool FAST = decltype(fast_tag)::value;
         constexpr bool ASYM = decltype(asym_tag)::value;
@@ -229,19 +253,22 @@ __global__ __launch_bounds__(kBlock) void int4_group_pack4(PackArgs a) {
                 float lo = 34952.0f, hi = 34952.0f;              // 8 * (1 + 16 + 256 + 4096)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const float q = quant_elem<DT, false, FAST, false>(x[u][v][j], dv[u], z[u], ASYM, -8.f, 7.f);
+                    const float q = quant_elem<DT, false, FAST, false>(pinned(x[u][v][j]), dv[u], z[u], ASYM, -8.f, 7.f);
                     lo = __builtin_fmaf(q, (float)(1 << (4 * j)), lo);
                 }
                 if constexpr (VEC == 8) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        const float q = quant_elem<DT, false, FAST, false>(x[u][v][4 + j], dv[u], z[u], ASYM, -8.f, 7.f);
+                        const float q = quant_elem<DT, false, FAST, false>(pinned(x[u][v][4 + j]), dv[u], z[u], ASYM, -8.f, 7.f);
                         hi = __builtin_fmaf(q, (float)(1 << (4 * j)), hi);
                     }
                     word[u][v] = (uint32_t)lo | ((uint32_t)hi << 16);
                 } else {
                     word[u][v] = (uint32_t)lo;
                 }
+                // one word at a time: left alone, the scheduler interleaves all 32 elements of a lane; bounded, the
+                // kernel needs fewer registers and runs 5 % faster (26.7 us against 28.1 us on W[14336,4096] bf16)
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
     };
@@ -249,6 +276,20 @@ __global__ __launch_bounds__(kBlock) void int4_group_pack4(PackArgs a) {
     else if (fast) encode(std::true_type{}, std::false_type{});
     else if (asym) encode(std::false_type{}, std::true_type{});
     else encode(std::false_type{}, std::false_type{});
+    if constexpr (FULL) {
+        // a 16-byte input vector becomes VEC / 2 output bytes: the output offsets are the input offsets / (2 * BYTES)
+        uint8_t* oblk = a.packed + (int64_t)blockIdx.x * (blk_bytes / (2 * BYTES));
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                const uint32_t o = (lane_off + (uint32_t)u * ((uint32_t)a.seg_len * BYTES) + (uint32_t)(v * T * 16)) / (2 * BYTES);
+                if constexpr (VEC == 8) stg4_nt(oblk + o, word[u][v]);
+                else *reinterpret_cast<uint16_t*>(oblk + o) = (uint16_t)word[u][v];
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
 #pragma unroll
@@ -333,7 +374,10 @@ template <int DT, int T, int NV>
 static void launch_pack4(const PackArgs& a, hipStream_t st) {
     const int64_t per_block = (int64_t)(kBlock / T) * 4;
     const int64_t nb = (a.nseg + per_block - 1) / per_block;
+    constexpr int BYTES = Tr<DT>::BYTES, VEC = Tr<DT>::VEC;
+    const bool full = a.nseg % per_block == 0 && a.seg_len == T * NV * VEC && a.nseg * a.seg_len * BYTES < (int64_t(1) << 31);
     if (a.col_mode != AMCT_COL_NONE) hipLaunchKernelGGL((int4_group_pack4<DT, T, NV, true>), dim3((unsigned)nb), dim3(kBlock), 0, st, a);
+    else if (full) hipLaunchKernelGGL((int4_group_pack4<DT, T, NV, false, true>), dim3((unsigned)nb), dim3(kBlock), 0, st, a);
     else hipLaunchKernelGGL((int4_group_pack4<DT, T, NV, false>), dim3((unsigned)nb), dim3(kBlock), 0, st, a);
 }
 
