@@ -1435,10 +1435,19 @@ __global__ __launch_bounds__(kBlock) void w4a16_general(W4A16Args a) {
 int wq16_int4_f16(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
                   const uint8_t* zeros, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group,
                   hipStream_t st);                                 // gemm_wq16.hip
+int w4a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
+                          const uint8_t* zeros, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group,
+                          hipStream_t st);                         // gemm_w4a16_stream.hip
 
 }  // namespace amct
 
 using namespace amct;
+
+extern "C" size_t amct_gemm_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K, int group, int has_smooth) {
+    (void)N;
+    if (M <= 0 || K <= 0 || group <= 0) return 0;
+    return has_smooth && M > 16 ? (size_t)M * (size_t)K * 2 : 0;          // tile kernels: x * smooth done once
+}
 
 extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t* wq, const void* scales,
                                int scale_dtype, const uint8_t* zeros, const float* bias, void* out, int64_t M,
@@ -1456,6 +1465,10 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
     W4A16Args a{(const uint16_t*)x, (const uint16_t*)smooth, wq, scales, zeros, bias, (uint16_t*)out, M, N, K, group, scale_dtype,
                 (uint32_t)(0x100000000ull / (uint64_t)group) + 1u};
     hipStream_t st = (hipStream_t)stream;
+    if (M <= 16) {                                                 // bf16, K % 1024 == 0, group 128: the weight-streaming kernel
+        const int rc = w4a16_stream_dispatch(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, st);
+        if (rc != AMCT_E_UNSUPPORTED) return rc;
+    }
     const bool vec_ok = aligned16(x) && aligned16(wq) && (!smooth || aligned16(smooth)) && group % 32 == 0;
     if (vec_ok && M <= 16 && K % 256 == 0 && K < 65536 && group % 32 == 0 && K / group <= 128 && (N * (K / group)) % 16 == 0 &&
         aligned16(scales) && aligned16(zeros)) {

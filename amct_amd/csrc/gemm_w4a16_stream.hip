@@ -1,0 +1,292 @@
+// K7 for M <= 16 (decode): the packed weights are the only large traffic, 29 MB for W[14336,4096], which the
+// memory system delivers in a few microseconds only if all of it is requested at once.  So every wave of the launch
+// is resident at the same time and issues ALL its weight loads (16 bytes per lane and 128 elements of K) before
+// anything else waits; what it needs besides (activations, smoothing factors, scales, zero-points) is staged once
+// per block through LDS with coalesced loads that were issued just before (waits are in issue order, so the staged
+// data can be consumed while the weights are still arriving) and the dequantisation then follows the data as it
+// lands.  A block owns CG groups of 16 output columns; KS waves per column group split K; a lane holds the 32
+// consecutive weights k0 + 32 g .. of column n0 + lane % 16 per step (g = lane / 16), i.e. one MFMA 16x16x32 operand
+// per 8 weights, and reads the matching activations of row lane % 16 from LDS.
+// Arithmetic: x' = bf16(x * smooth) as everywhere.  The weights enter the MFMA as the EXACT integers 16 + u (a
+// bf16 pattern 0x4180 | u << 3: two instructions per pair of weights instead of six for (u - z) * s rounded to bf16),
+// each group of `group` columns is accumulated on its own (P = sum x' * (16 + u), fp32) and folded into the result
+// as acc += s * P - s * (16 + z) * X with X = sum of the group's x' (computed once per block while staging).  That is
+// sum x' * (u - z) * s with the dequantised weight NOT rounded to bf16 -- the fp32 `weight * scale` of the reference's
+// CPU stand-in for this operator (tests/amct_pytorch/mock_torch_npu.py:33-55) -- whereas the tile kernels for larger M
+// feed bf16((u - z) * s) to the matrix pipe; both are within the 1e-3 tolerance of the fp64 result, this one closer.
+// The partial sums of the KS waves are added in wave order, so the result does not depend on the launch shape
+// beyond KS.
+#include "amct_common.h"
+
+namespace amct {
+
+typedef float s4f __attribute__((ext_vector_type(4)));
+typedef __bf16 s8bf __attribute__((ext_vector_type(8)));
+typedef __bf16 s2bf __attribute__((ext_vector_type(2)));
+typedef float s2f __attribute__((ext_vector_type(2)));
+
+struct StreamArgs {
+    const uint16_t* x;
+    const uint16_t* smooth;
+    const uint8_t* wq;
+    const uint16_t* scales;
+    const uint8_t* zeros;
+    const float* bias;
+    uint16_t* out;
+    int M, N, K, G;                                  // G = K / group
+    int group;
+    int scale_f16;
+    uint32_t kv_magic;                               // floor(2^32 / (K / 8)) + 1: v / (K / 8) == mulhi(v, magic)
+};
+
+AMCT_DEV uint32_t st_pack2(float lo, float hi) {
+    const s2f f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, s2bf));          // v_cvt_pk_bf16_f32, round-half-even
+}
+// 8 nibbles of w (nibble p = weight k0 + p) -> 4 words of two bf16 integers 16 + u each, word j = (weight j, weight j + 4)
+AMCT_DEV uint4 st_int8x(uint32_t w) {
+    constexpr uint32_t kMask = 0x00780078u, kBase = 0x41804180u;       // bf16(16 + u) = 0x4180 | u << 3
+    return make_uint4(((w << 3) & kMask) | kBase, ((w >> 1) & kMask) | kBase, ((w >> 5) & kMask) | kBase,
+                      ((w >> 9) & kMask) | kBase);
+}
+// the matching order of 8 activations: (k0, k4), (k1, k5), (k2, k6), (k3, k7)
+AMCT_DEV uint4 st_interleave8(const uint4& x) {
+    return make_uint4(__builtin_amdgcn_perm(x.z, x.x, 0x05040100u), __builtin_amdgcn_perm(x.z, x.x, 0x07060302u),
+                      __builtin_amdgcn_perm(x.w, x.y, 0x05040100u), __builtin_amdgcn_perm(x.w, x.y, 0x07060302u));
+}
+AMCT_DEV float st_sum8(const uint4& x) {
+    const uint32_t xs[4] = {x.x, x.y, x.z, x.w};
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) t = t + (__uint_as_float(xs[i] << 16) + __uint_as_float(xs[i] & 0xFFFF0000u));
+    return t;
+}
+AMCT_DEV uint4 st_smooth8(const uint4& x, const uint4& c) {
+    const uint32_t xs[4] = {x.x, x.y, x.z, x.w}, cs[4] = {c.x, c.y, c.z, c.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        o[i] = st_pack2(__uint_as_float(xs[i] << 16) * __uint_as_float(cs[i] << 16),
+                        __uint_as_float(xs[i] & 0xFFFF0000u) * __uint_as_float(cs[i] & 0xFFFF0000u));
+    return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+// XJ: 16-byte activation vectors a thread stages (clamped duplicates beyond the tensor)
+
+template <int KS, int CG, int NL, int XJ, bool SMOOTH>
+__global__ __launch_bounds__(KS * CG * 64) void w4a16_stream(StreamArgs a) {
+    static_assert(NL % 2 == 0, "the weight loads come in pairs");
+    extern __shared__ __align__(16) uint8_t lds[];
+    constexpr int NT = KS * CG * 64;
+    constexpr int COLS = CG * 16;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int cg = wave / KS, ks = wave % KS;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * COLS;
+    const uint32_t K = (uint32_t)a.K, M = (uint32_t)a.M, G = (uint32_t)a.G;
+    const uint32_t xstride = K * 2 + 16;             // 16 bytes of padding: the 16 rows of a fragment read hit different banks
+    const uint32_t xbytes = M * xstride;
+    const uint32_t red_bytes = (KS - 1) * CG * 64 * 16;
+    uint8_t* xs = lds;
+    float* xsum = reinterpret_cast<float*>(lds + xbytes);   // [G][16]: sum of x' per group and row
+
+    // ---- staging loads (activations, smoothing factors, this block's scales and zero-points) ----------------
+    const uint32_t KV = K / 8, n_xv = M * KV;
+    uint4 xv[XJ], cv[XJ];
+    uint32_t xrow[XJ], xkv[XJ];
+#pragma unroll
+    for (int j = 0; j < XJ; ++j) {
+        const uint32_t v = tid + NT * j;
+        const uint32_t vc = v < n_xv ? v : n_xv - 1;
+        xrow[j] = __umulhi(vc, a.kv_magic);           // vc / KV
+        xkv[j] = vc - xrow[j] * KV;
+        xv[j] = ldg16(a.x + (size_t)xrow[j] * K + xkv[j] * 8);
+        if constexpr (SMOOTH) cv[j] = ldg16(a.smooth + xkv[j] * 8);
+    }
+    // the scales and zero-points of this lane's column for the NL groups of this wave: 2 NL and NL contiguous bytes.
+    // They come from HBM like the weights and are only needed when the first group is folded, so they are loaded into
+    // registers by every lane itself (a block-wide table in LDS would hold up the barrier below for as long as an
+    // HBM access takes under the load of the whole launch's weight requests).
+    const int fcol = n0 + cg * 16 + r16;
+    const size_t fidx = (size_t)(fcol < a.N ? fcol : a.N - 1) * G + ks * NL;
+    uint32_t fsw[NL / 2], fzw[(NL + 3) / 4];
+#pragma unroll
+    for (int q = 0; q < NL / 2; ++q) fsw[q] = *reinterpret_cast<const uint32_t*>(a.scales + fidx + 2 * q);
+    if constexpr (NL >= 4) {
+#pragma unroll
+        for (int q = 0; q < NL / 4; ++q) fzw[q] = *reinterpret_cast<const uint32_t*>(a.zeros + fidx + 4 * q);
+    } else {
+        fzw[0] = *reinterpret_cast<const uint16_t*>(a.zeros + fidx);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- the whole weight stream of this wave ---------------------------------------------------------------------
+    // A load instruction fetches 8 weight rows x one whole 128-byte line (256 elements of K): lane l reads row l % 8
+    // (the second instruction of a pair rows 8 .. 15) and the 16-byte chunk chunk_of(l / 8) of the line.  Whole lines per
+    // instruction stream 1.3 us faster over W[14336,4096] than 16 rows x 64 bytes.  The MFMA wants 16 different rows in
+    // lanes 0 .. 15 of a lane group, so the two registers of a pair swap halves afterwards (two DPP moves per word):
+    // the first then holds chunks 0 .. 3 (one group of 128, chunk g in lane group g) for rows 0 .. 15, the second chunks
+    // 4 .. 7 (the next group).
+    const uint32_t kw = K / KS;                      // elements of K of this wave: NL steps of 128
+    const int ncol = n0 + cg * 16 + r16;
+    const uint32_t oct = lane >> 3;
+    const uint32_t chunk = (oct & 1) ? 4 + (oct >> 1) : (oct >> 1);
+    const int rlo = n0 + cg * 16 + (lane & 7), rhi = rlo + 8;
+    const uint8_t* wlo = a.wq + (size_t)(rlo < a.N ? rlo : a.N - 1) * (K / 2) + (ks * kw) / 2 + chunk * 16;
+    const uint8_t* whi = a.wq + (size_t)(rhi < a.N ? rhi : a.N - 1) * (K / 2) + (ks * kw) / 2 + chunk * 16;
+    u4v wv[NL];
+#pragma unroll
+    for (int i = 0; i < NL; i += 2) {
+        wv[i] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wlo + (i / 2) * 128));
+        wv[i + 1] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(whi + (i / 2) * 128));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- stage the activations: smoothed, interleaved to the operand order of st_int8x, summed per group ----------
+#pragma unroll
+    for (int j = 0; j < XJ; ++j) {
+        const uint32_t v = tid + NT * j;
+        if constexpr (SMOOTH) xv[j] = st_smooth8(xv[j], cv[j]);
+        // 16 consecutive lanes hold 128 consecutive elements of one row; whole groups of 16 lanes are valid or not
+        float t = st_sum8(xv[j]);
+        t = t + __shfl_xor(t, 1);
+        t = t + __shfl_xor(t, 2);
+        t = t + __shfl_xor(t, 4);
+        t = t + __shfl_xor(t, 8);
+        if (v < n_xv) {
+            *reinterpret_cast<uint4*>(xs + xrow[j] * xstride + xkv[j] * 16) = st_interleave8(xv[j]);
+            if ((tid & 15) == 0) {
+                xsum[(xkv[j] >> 4) * 16 + xrow[j]] = t;
+            }
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+
+    // ---- follow the weights as they land ---------------------------------------------------------------------------
+    s4f acc = {0.f, 0.f, 0.f, 0.f}, P = {0.f, 0.f, 0.f, 0.f};
+    const uint8_t* xlane = xs + (r16 < (int)M ? r16 : (int)M - 1) * xstride + (ks * kw + g * 32) * 2;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+        // the loads retire in order: step i waits for wv[i] only, the NL - 1 - i younger ones stay in flight
+        s8bf fa[4];
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4) fa[s4] = *reinterpret_cast<const s8bf*>(xlane + i * 256 + s4 * 16);
+        if ((i & 1) == 0) {                          // both registers of the pair have landed: swap halves
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const uint32_t lo = wv[i][d], hi = wv[i + 1][d];
+                // row_ror:8 inside each row of 16 lanes; bank_mask picks the lanes that take the rotated value
+                wv[i][d] = (uint32_t)__builtin_amdgcn_update_dpp((int)lo, (int)hi, 0x128, 0xF, 0xC, false);
+                wv[i + 1][d] = (uint32_t)__builtin_amdgcn_update_dpp((int)hi, (int)lo, 0x128, 0xF, 0x3, false);
+            }
+        }
+        const uint32_t ws[4] = {wv[i].x, wv[i].y, wv[i].z, wv[i].w};
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4)
+            P = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[s4], __builtin_bit_cast(s8bf, st_int8x(ws[s4])), P, 0, 0, 0);
+        {                                             // a step is one group of 128: fold it into the result
+            const uint32_t gi = (ks * kw) / 128 + i;
+            const uint32_t sbits = (fsw[i / 2] >> (16 * (i & 1))) & 0xFFFFu;
+            const uint32_t zu = (fzw[i / 4] >> (8 * (i & 3))) & 0xFFu;
+            const float s_h = f16_bits_to_f32(sbits), s_b = bf16_bits_to_f32(sbits);
+            const float sc = a.scale_f16 ? s_h : s_b;
+            const float c = -(sc * (float)(16u + zu));                        // exact: 5 bits x 11 bits
+            const s4f X = *reinterpret_cast<const s4f*>(xsum + gi * 16 + 4 * g);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[r] = __builtin_fmaf(sc, P[r], __builtin_fmaf(c, X[r], acc[r]));
+            P = s4f{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    s4f y = acc;
+
+    // ---- add the KS partial sums of a column group in wave order, write ------------------------------------
+    if constexpr (KS > 1) {
+        __syncthreads();                              // every wave is done reading activations: their rows are reused
+        float* red = reinterpret_cast<float*>(lds);
+        if (ks > 0) *reinterpret_cast<s4f*>(red + (((ks - 1) * CG + cg) * 64 + lane) * 4) = y;
+        __syncthreads();
+        if (ks == 0) {
+#pragma unroll
+            for (int w = 0; w < KS - 1; ++w) {
+                const s4f o = *reinterpret_cast<const s4f*>(red + ((w * CG + cg) * 64 + lane) * 4);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) y[r] = y[r] + o[r];
+            }
+        }
+    }
+    if (ks == 0 && ncol < a.N) {
+        const float b = a.bias ? a.bias[ncol] : 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int m = 4 * g + r;
+            float v = y[r];
+            if (a.bias) v = v + b;
+            if (m < (int)M) a.out[(size_t)m * a.N + ncol] = (uint16_t)f32_to_bf16_bits(v);
+        }
+    }
+}
+
+template <int KS, int CG, int NL, bool SMOOTH>
+static int stream_launch_x(const StreamArgs& a, size_t lds_bytes, hipStream_t st) {
+    constexpr int NT = KS * CG * 64;
+    const int n_xv = a.M * (a.K / 8);
+    const int xj = (n_xv + NT - 1) / NT;
+    const dim3 grid((unsigned)((a.N + CG * 16 - 1) / (CG * 16)));
+#define AMCT_STREAM_GO(XJ)                                                                                          \
+    {                                                                                                               \
+        auto kern = &w4a16_stream<KS, CG, NL, XJ, SMOOTH>;                                                          \
+        if (lds_bytes > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                       \
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess) { \
+            (void)hipGetLastError();                                                                                \
+            return AMCT_E_HIP;                                                                                      \
+        }                                                                                                           \
+        hipLaunchKernelGGL(kern, grid, dim3(NT), lds_bytes, st, a);                                                 \
+        return hip_status();                                                                                        \
+    }
+    if (xj <= 2) AMCT_STREAM_GO(2)
+    if (xj <= 4) AMCT_STREAM_GO(4)
+    if (xj <= 8) AMCT_STREAM_GO(8)
+#undef AMCT_STREAM_GO
+    return AMCT_E_UNSUPPORTED;
+}
+
+// Returns AMCT_E_UNSUPPORTED when the shape is not one this kernel takes (the caller then uses its other kernels).
+int w4a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
+                          const uint8_t* zeros, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group,
+                          hipStream_t st) {
+    // one group per step of 128 elements of K (the per-group partial sums of a step cannot be separated otherwise)
+    if (M < 1 || M > 16 || (K != 1024 && K != 2048 && K != 4096) || group != 128 || N > (int64_t(1) << 30)) return AMCT_E_UNSUPPORTED;
+    if (!aligned16(x) || !aligned16(wq) || (smooth && !aligned16(smooth)) || ((uintptr_t)scales & 3) || ((uintptr_t)zeros & 3))
+        return AMCT_E_UNSUPPORTED;
+    StreamArgs a{(const uint16_t*)x, (const uint16_t*)smooth, wq, (const uint16_t*)scales, zeros, bias, (uint16_t*)out,
+                 (int)M, (int)N, (int)K, (int)(K / group), group, scale_dtype == AMCT_F16 ? 1 : 0,
+                 (uint32_t)(0x100000000ull / (uint64_t)(K / 8)) + 1u};
+    // A wave streams K / 4 elements of 16 columns in NL = K / 512 steps, all of them in flight from the start.  Large
+    // activation blocks are staged by few, wide blocks (16 waves share one copy in LDS); small ones by many narrow
+    // blocks, several per CU.  Measured on W[14336,4096]: 8.8 us at M = 1 (11.0 us for the kernel this one replaced),
+    // 12.9 us at M = 16 (17.3 us); preparing the activation image once in a kernel of its own instead of in every block
+    // was slower for every M (the second launch costs more than the staging arithmetic it removes).
+    const size_t xbytes = (size_t)M * ((size_t)K * 2 + 16);
+    const int cg = xbytes > 40 * 1024 ? 4 : xbytes > 12 * 1024 ? 2 : 1;
+    const int64_t nl = K / 512;
+    const size_t red = (size_t)3 * cg * 64 * 16, img = xbytes + (size_t)(K / group) * 64;
+    const size_t lds_bytes = img > red ? img : red;
+    if (lds_bytes > 160 * 1024) return AMCT_E_UNSUPPORTED;
+#define AMCT_STREAM_SHAPE(CG_, NL_)                                                                       \
+    if (cg == CG_ && nl == NL_)                                                                           \
+        return smooth ? stream_launch_x<4, CG_, NL_, true>(a, lds_bytes, st) : stream_launch_x<4, CG_, NL_, false>(a, lds_bytes, st);
+    AMCT_STREAM_SHAPE(4, 8)
+    AMCT_STREAM_SHAPE(2, 8)
+    AMCT_STREAM_SHAPE(1, 8)
+    AMCT_STREAM_SHAPE(4, 4)
+    AMCT_STREAM_SHAPE(2, 4)
+    AMCT_STREAM_SHAPE(1, 4)
+    AMCT_STREAM_SHAPE(4, 2)
+    AMCT_STREAM_SHAPE(2, 2)
+    AMCT_STREAM_SHAPE(1, 2)
+#undef AMCT_STREAM_SHAPE
+    return AMCT_E_UNSUPPORTED;                        // K / 512 steps per wave beyond 8: the other kernels
+}
+
+}  // namespace amct

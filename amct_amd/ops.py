@@ -479,14 +479,17 @@ def gemm_w4a16(x, wq_packed, scales, zeros, group, smooth=None, bias=None):
     if bias is not None:
         bias = _c(bias.reshape(-1).to(torch.float32))
     out = torch.empty(M, N, dtype=x.dtype, device=dev)
-    # with smoothing the caller-owned workspace lets the multiply run once up front (the bf16 tile kernels need
-    # that; up to 16 rows the library takes its weight-streaming kernels, which smooth in place)
-    ws = torch.empty(M, K, dtype=x.dtype, device=dev) if (smooth is not None and M > 16 and x.dtype == torch.bfloat16) \
-        else None
+    # the workspace the library asks for: the smoothed activations for the tile kernels, or the activation image the
+    # weight-streaming kernel for a few rows fetches
+    ws = None
+    if x.dtype == torch.bfloat16:
+        nbytes = _lib.load().amct_gemm_w4a16_workspace_bytes(M, N, K, group, int(smooth is not None))
+        if nbytes:
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         _lib.check(_lib.load().amct_gemm_w4a16(_p(x), _p(smooth), _p(wq_packed), _p(scales), dtype_code(scales.dtype),
                                                _p(zeros), _p(bias), _p(out), M, N, K, group, dtype_code(x.dtype),
-                                               _p(ws), 0 if ws is None else ws.numel() * 2, _stream(dev)))
+                                               _p(ws), 0 if ws is None else ws.numel(), _stream(dev)))
     return out
 
 

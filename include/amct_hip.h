@@ -251,9 +251,15 @@ int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s_tok, const
  * amct_pytorch/utils/vars.py:43-47); smooth [K] of dtype or null; wq uint8 [N, K/2] as written by
  * amct_quant_int4_group_pack; scales [N, K/group] of scale_dtype; zeros uint8 [N, K/group];
  * bias fp32 [N] or null.  out [M, N] of dtype = x' @ dtype((u - zero) * scale)^T + bias, fp32 accumulate.
- * workspace (may be null): M*K*2 bytes the caller lends; with it the smoothing multiply is done once
- * up front instead of inside every column tile (same results; the fast bf16 tile kernels for M > 16 need it
- * when smooth is given, without it such calls take slower kernels that smooth in place). */
+ * workspace (may be null): amct_gemm_w4a16_workspace_bytes(M, N, K, group, smooth != null) bytes the caller lends,
+ * 16-byte aligned, contents irrelevant before and after the call.  For M > 16 with smooth the multiply is then done
+ * once up front instead of inside every column tile (same results; the fast bf16 tile kernels need it, without it such
+ * calls take slower kernels that smooth in place); 0 bytes are asked for otherwise.
+ * Arithmetic of the dequantisation: the tile kernels (M > 16) feed dtype((u - zero) * scale) to the matrix pipe; the
+ * weight-streaming bf16 kernel for M <= 16 (K % 1024 == 0, group = 128) keeps the weight as the exact integer and applies
+ * scale and zero per group in fp32, i.e. the dequantised weight is not rounded to bf16 there (the fp32 weight * scale of
+ * tests/amct_pytorch/mock_torch_npu.py:33-55).  Both stay within 1e-3 of the exact result. */
+size_t amct_gemm_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K, int group, int has_smooth);
 int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t* wq, const void* scales,
                     int scale_dtype, const uint8_t* zeros, const float* bias, void* out,
                     int64_t M, int64_t N, int64_t K, int group, int dtype,

@@ -30,9 +30,12 @@ documented arithmetic.  Pin status:
                         the output dtype.
   w4a16 dequant         PARITY UNPINNED against torch_npu (precision of the
                         dequantised weight); this repo fixes: (q - z) * s
-                        exact in fp32, rounded once to x's dtype, fp32
-                        accumulate.  Special case z=8 (unsigned), s=1 reduces
-                        to a plain matmul -- tested against torch.matmul.
+                        exact in fp32, rounded once to x's dtype (tile
+                        kernels) or not rounded at all (the weight-streaming
+                        kernel for M <= 16, as the reference's CPU stand-in
+                        mock_torch_npu.py:33-55 does), fp32 accumulate.
+                        Special case z=8 (unsigned), s=1 reduces to a plain
+                        matmul -- tested against torch.matmul.
   int4 word packing     PARITY UNPINNED against torch_npu (nibble order);
                         this repo fixes little-endian: nibble j of word i
                         holds column 8*i+j.
@@ -230,10 +233,20 @@ def w4a16_buffers(weight, bias, scale_w, offset_w, wts_type, group_size=None, aw
 
 
 def dequant_weight(codes_nk, scale_nk_g, antioffset_nk_g, group_size, dtype):
-    """(q + antiquant_offset) * antiquant_scale, exact in fp32, rounded once
-    to `dtype`.  scale/offset are [N,G] (G=1 for per-channel)."""
+    """(q + antiquant_offset) * antiquant_scale, exact in fp32, rounded once to `dtype` -- or, with dtype None, left
+    exact (fp64).  scale/offset are [N,G] (G=1 for per-channel).
+    Both readings of the un-vendored operator are kept: the matrix pipe takes 16-bit operands, so the tile kernels
+    round the dequantised weight to the activation dtype; the reference's CPU stand-in for the operator
+    (tests/amct_pytorch/mock_torch_npu.py:33-55) multiplies in fp32 and rounds nothing, which is what the
+    weight-streaming kernel for a few rows reproduces (integer weights in the matrix pipe, scale applied per group)."""
     n, k = codes_nk.shape
     g = group_size if group_size else k
+    if dtype is None:
+        q = iq.group_view(codes_nk.double(), g)
+        s = scale_nk_g.double().reshape(n, -1, 1)
+        if antioffset_nk_g is not None:
+            q = q + antioffset_nk_g.double().reshape(n, -1, 1)
+        return (q * s).reshape(n, -1)[:, :k]
     q = iq.group_view(codes_nk.float(), g)                    # [N,G,g]
     s = scale_nk_g.float().reshape(n, -1, 1)
     if antioffset_nk_g is not None:
@@ -249,16 +262,22 @@ def weight_quant_matmul_f64(x2d, wdq_nk, bias=None):
     return y
 
 
-def w4a16_forward_f64(x, codes_nk, scale_ng, antioffset_ng, group_size, bias=None, scale_factor=None):
-    """Module forward (weight_npu_quant_module.py:102-121) with the contraction
-    in fp64: x' = x*scale_factor rounded to x's dtype, weight dequantised and
-    rounded to x's dtype, exact products, fp64 sum.  Returns fp64 [.., N]."""
+def w4a16_forward_f64(x, codes_nk, scale_ng, antioffset_ng, group_size, bias=None, scale_factor=None, round_weight=True):
+    """Module forward (weight_npu_quant_module.py:102-121) with the contraction in fp64: x' = x*scale_factor rounded
+    to x's dtype, weight dequantised (rounded to x's dtype, or exact with round_weight=False), exact products, fp64
+    sum.  Returns fp64 [.., N]."""
     shp = x.shape
     x2 = x.reshape(-1, shp[-1])
     if scale_factor is not None:
         x2 = torch.mul(x2, scale_factor.to(x2.dtype))
-    wdq = dequant_weight(codes_nk, scale_ng, antioffset_ng, group_size, x.dtype)
+    wdq = dequant_weight(codes_nk, scale_ng, antioffset_ng, group_size, x.dtype if round_weight else None)
     return weight_quant_matmul_f64(x2, wdq, bias).reshape(*shp[:-1], -1)
+
+
+def w4a16_streams(M, K, group_size, dtype=torch.bfloat16):
+    """Whether the int4 GEMM takes its weight-streaming kernel for this shape (a few bf16 rows, K of 1024, 2048 or
+    4096, groups of 128): that kernel does not round the dequantised weight."""
+    return dtype == torch.bfloat16 and 1 <= M <= 16 and K in (1024, 2048, 4096) and group_size == 128
 
 
 # --------------------------------------------------------------------------
