@@ -26,18 +26,11 @@ PEAK_INT8_TOPS = 5000.0
 PEAK_BF16_TFLOPS = 2500.0
 
 # HBM bytes per launch as the hardware counted them (FETCH_SIZE + WRITE_SIZE, each scaled by what the same
-# counter reads for the plain copy kernel of known size).  A program cannot run the profiler around itself, so
-# these are constants of each kernel at its bench workload; the runs they come from and their commands are
-# kept in profiles/hbm_traffic_pmc_bench_workloads.txt and are refreshed when a kernel changes.
-MEASURED_TRAFFIC_BYTES = {
-    "int4_group_pack": 152270155,
-    "fakequant_int8": 134442394,
-    "mxfp8_quant": 101803014,
-    "hif8_encode": 100722479,
-    "w8a8_m2048": 254904953,
-    "w8a8_m16": 59904148,
-    "w4a16_m2048": 269965424,
-    "w4a16_m1": 36949937,
+# counter reads for the plain copy kernel of known size), with the kernel that was dispatched when they were
+# counted.  A program cannot run the profiler around itself, so these are constants of each kernel at its bench
+# workload; the runs they come from and their commands are kept in profiles/hbm_traffic_pmc_bench_workloads.txt.
+# A kernel that was changed and not counted again has no entry (reported as null).
+MEASURED_TRAFFIC = {
 }
 
 
@@ -46,6 +39,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--repeats", type=int, default=5, help="timed regions of --steps launches per kernel; the median is reported")
     ap.add_argument("--only", default="", help="comma list of kernel names (default: all)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     return ap.parse_args()
@@ -324,54 +318,114 @@ def spin_up(dev):
     torch.cuda.synchronize(dev)
 
 
-def time_case(case, steps, warmup, dev):
+def time_case(case, steps, warmup, dev, repeats):
+    """`repeats` timed regions of exactly `steps` launches each (device time by events on the launch stream, host
+    time around the same region); returns the median host time of a region, the median device time per launch and the latter for every region."""
     import torch
     for i in range(warmup):
         case.launch(i)
     torch.cuda.synchronize(dev)
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for i in range(steps):
-        case.launch(warmup + i)
-    e1.record()
-    torch.cuda.synchronize(dev)
-    wall = time.perf_counter() - t0
-    dev_ms = e0.elapsed_time(e1)
-    return wall, dev_ms / steps
+    walls, devs = [], []
+    idx = warmup
+    for _ in range(repeats):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for i in range(steps):
+            case.launch(idx + i)
+        e1.record()
+        torch.cuda.synchronize(dev)
+        walls.append(time.perf_counter() - t0)
+        devs.append(e0.elapsed_time(e1) / steps)
+        idx += steps
+    return sorted(walls)[len(walls) // 2], sorted(devs)[len(devs) // 2], devs
 
 
-def cpu_baseline():
-    """The oracle's restatement of the reference CPU path for the headline workload, on a bounded
-    row sample, all host cores torch gives us (capped at 16)."""
-    import torch
-    from amct_amd import workloads
-    from oracle import deploy as od
-    from oracle import int_quant as iq
-    cores = min(os.cpu_count() or 1, 16)
-    torch.set_num_threads(cores)
-    rows = 2048
-    w = workloads.c2_weight(rows, 4096)
-
-    def run():
-        s, z = iq.weight_scale_offset(w, 'group', False, 'int4', 128)
-        codes = iq.quant_codes(w, 'int4', s, z, 128).reshape(rows, -1)
-        packed = od.pack_nibbles_k(codes)
-        return packed, s.squeeze(-1).to(torch.float16), (z.squeeze(-1) + 8).to(torch.uint8)
+def _timed(run, budget_s, min_runs=3, max_runs=400):
     run()
     times = []
-    t_end = time.perf_counter() + 12.0
-    while len(times) < 5 or (time.perf_counter() < t_end and len(times) < 20):
+    t_end = time.perf_counter() + budget_s
+    while len(times) < min_runs or (time.perf_counter() < t_end and len(times) < max_runs):
         t0 = time.perf_counter()
         run()
         times.append(time.perf_counter() - t0)
     times.sort()
-    med = times[len(times) // 2]
-    work = rows * 4096 * 2 + rows * 4096 // 2 + rows * 32 * 3
-    return {"value": round(work / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-            "sample": "first {} of 14336 rows of the config-2 weight, median of {} runs, {:.1f} ms each".format(
-                rows, len(times), med * 1e3)}
+    return times[len(times) // 2], len(times)
+
+
+def cpu_baselines(names):
+    """The oracle's restatement of the reference's CPU path for each benchmark workload, timed on the host cores
+    torch gives us (capped at 16) on a bounded sample of the same synthetic input; about 25 s in total.  Returns
+    {kernel name: entry}; the entry of the headline kernel is also the line's top-level cpu_baseline."""
+    import torch
+    from amct_amd import workloads
+    from oracle import deploy as od
+    from oracle import hif8
+    from oracle import int_quant as iq
+    from oracle import mx
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    out = {}
+
+    def entry(name, work, unit, run, sample, budget=1.2):
+        if name not in names:
+            return
+        med, n = _timed(run, budget)
+        scale = 1e9 if unit == "GB/s" else 1e12
+        out[name] = {"value": round(work / med / scale, 4), "unit": unit, "cores": cores, "kind": "port",
+                     "sample": "{}; median of {} runs, {:.1f} ms each".format(sample, n, med * 1e3)}
+
+    rows = 2048
+    w2 = workloads.c2_weight(rows, 4096)
+
+    def k2():
+        s, z = iq.weight_scale_offset(w2, 'group', False, 'int4', 128)
+        codes = iq.quant_codes(w2, 'int4', s, z, 128).reshape(rows, -1)
+        return od.pack_nibbles_k(codes), s.squeeze(-1).to(torch.float16), (z.squeeze(-1) + 8).to(torch.uint8)
+    entry("int4_group_pack", rows * 4096 * 2 + rows * 4096 // 2 + rows * 32 * 3, "GB/s", k2,
+          "first 2048 of 14336 rows of the config-2 weight", 6.0)
+
+    w1 = workloads.c1_weight(1024, 4096)
+
+    def k1():
+        s, z = iq.weight_scale_offset(w1, 'channel', True, 'int8')
+        return iq.fake_quant(w1, 'int8', s, z)
+    entry("fakequant_int8", 1024 * 4096 * 8 + 1024 * 4, "GB/s", k1, "first 1024 of 4096 rows of the config-1 weight")
+
+    r3 = 512
+    x3 = workloads.c3_activations(r3, 4096)
+    n3 = r3 * 4096
+    entry("mxfp8_quant", n3 * 3 + n3 // 32, "GB/s", lambda: mx.mx_quant(x3, mx.E4M3), "first 512 of 8192 rows of the config-3 activations")
+    entry("mxfp4_quant", n3 * 2 + n3 // 2 + n3 // 32, "GB/s", lambda: mx.mx_quant(x3, mx.E2M1), "first 512 of 8192 rows of the config-3 activations")
+    el, sb = mx.mx_quant(x3, mx.E4M3)
+    entry("mxfp8_dequant", n3 * 3 + n3 // 32, "GB/s", lambda: mx.mx_dequant(el, sb, mx.E4M3, torch.bfloat16),
+          "first 512 of 8192 rows of the config-3 activations")
+    x3n = x3[:128].float().numpy()
+    entry("hif8_encode", 128 * 4096 * 3, "GB/s", lambda: hif8.encode_bruteforce(x3n), "first 128 of 8192 rows of the config-3 activations (nearest-code search)")
+    c3 = hif8.encode_bruteforce(x3n)
+    entry("hif8_decode", 128 * 4096 * 3, "GB/s", lambda: torch.from_numpy(hif8.decode(c3)).to(torch.bfloat16),
+          "first 128 of 8192 rows of the config-3 activations")
+    run_max, run_min = torch.full((1, 4096), -float("inf")), torch.full((1, 4096), float("inf"))
+    entry("col_minmax", n3 * 2 + 2 * 4096 * 4, "GB/s",
+          lambda: iq.channel_min_max_update(x3.float(), run_max, run_min), "first 512 of 8192 rows of the config-3 activations")
+
+    x4, wq4, sw4 = workloads.c4_w8a8(2048, 2048, 4096)
+    entry("act_quant_per_token", 2048 * 4096 * 3 + 2048 * 4, "GB/s", lambda: iq.dynamic_token_quant(x4), "the config-4 activations, whole")
+    xq4, st4 = iq.dynamic_token_quant(x4)
+    for name, m in (("w8a8_m2048", 256), ("w8a8_m16", 16)):
+        xs, ss = xq4[:m].contiguous(), st4.reshape(-1)[:m].contiguous()
+        entry(name, 2 * m * 2048 * 4096, "TOP/s", lambda xs=xs, ss=ss: od.quant_matmul(xs, wq4.t(), sw4, ss, None, torch.bfloat16),
+              "{} rows x the first 2048 of 14336 output channels of config 4".format(m))
+
+    x5, codes5, sc5, z5, sm5 = workloads.c5_w4a16(256, 2048, 4096)
+    signed5, anti5 = codes5.to(torch.int32) - 8, -(z5.to(torch.float32) - 8)
+    for name, m in (("w4a16_m2048", 256), ("w4a16_m16", 16), ("w4a16_m1", 1)):
+        xs = x5[:m].contiguous()
+        entry(name, 2 * m * 2048 * 4096, "TFLOP/s",
+              lambda xs=xs: od.w4a16_forward_f64(xs, signed5, sc5, anti5, 128, None, sm5.reshape(1, -1)).to(torch.bfloat16),
+              "{} rows x the first 2048 of 14336 output channels of config 5 (fp64 contraction of the checker)".format(m))
+    return out
 
 
 def main():
@@ -401,16 +455,19 @@ def run(args, dev, only):
     cases = build_cases(dev, only)
     torch.cuda.synchronize(dev)
     spin_up(dev)
+    repeats = max(1, args.repeats)
     results = {}
     head = None
     for c in cases:
-        wall, ms = time_case(c, args.steps, args.warmup, dev)
+        wall, ms, regions = time_case(c, args.steps, args.warmup, dev, repeats)
         rate = c.work / (ms * 1e-3) / 1e9 if c.bound == "hbm" else c.work / (ms * 1e-3) / 1e12
         peak = HBM_PEAK_GBS if c.bound == "hbm" else (PEAK_INT8_TOPS if c.bound == "mfma_i8" else PEAK_BF16_TFLOPS)
-        results[c.name] = {"desc": c.desc, "us_per_launch": round(ms * 1e3, 2), "achieved": round(rate, 1),
+        traffic = MEASURED_TRAFFIC.get(c.name)
+        results[c.name] = {"desc": c.desc, "us_per_launch": round(ms * 1e3, 2),
+                           "us_per_launch_by_region": [round(r * 1e3, 2) for r in regions], "achieved": round(rate, 1),
                            "unit": "GB/s" if c.bound == "hbm" else ("TOP/s" if c.bound == "mfma_i8" else "TFLOP/s"), "peak": peak,
-                           "frac": round(rate / peak, 4), "work_per_launch": c.work, "sets": c.nsets,
-                           "traffic": MEASURED_TRAFFIC_BYTES.get(c.name)}
+                           "frac": round(rate / peak, 4), "work_per_launch": c.work, "sets": c.nsets, "dtype": c.dtype,
+                           "traffic": traffic[1] if traffic else None, "traffic_kernel": traffic[0] if traffic else None}
         if c.name == "int4_group_pack":
             head = (c, wall, ms)
     # GEMM figures also as a fraction of what the register-only MFMA loop sustains on random operands
@@ -420,20 +477,26 @@ def run(args, dev, only):
             r["frac_of_yardstick"] = round(r["achieved"] / results[y]["achieved"], 4)
     c, wall, ms = head
     value = c.work * args.steps / wall / 1e9
+    traffic = MEASURED_TRAFFIC.get("int4_group_pack")
     line = {
         "metric": "quantize GB/s (% of HBM peak); W8A8 & W4A16 linear TOPS (% of MFMA peak)",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(wall / args.steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": c.dtype, "data": "synthetic",
-        "config": {"workload": c.desc, "rotating_sets": c.nsets},
+        "config": {"workload": c.desc, "rotating_sets": c.nsets, "input_dtype": "bf16",
+                   "timing": "median of {} regions of {} launches".format(repeats, args.steps)},
         "roofline": {"bound": "hbm", "achieved": round(c.work / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(c.work / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES["int4_group_pack"],
+                     "traffic": traffic[1] if traffic else None,
                      "kernel": "int4_group_pack", "bytes_per_launch": c.work},
         "kernels": results,
     }
     if not args.no_cpu:
-        line["cpu_baseline"] = cpu_baseline()
+        base = cpu_baselines(set(results) | {"int4_group_pack"})
+        line["cpu_baseline"] = base["int4_group_pack"]
+        for name, entry in base.items():
+            if name in results:
+                results[name]["cpu_baseline"] = entry
     return line
 
 

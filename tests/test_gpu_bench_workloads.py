@@ -1,0 +1,95 @@
+"""The tensors bench.py times (amct_amd.workloads, same seeds, same sizes) through the same entry points, against the
+oracle: the quantize kernels bit for bit on a row sample that covers every block position, config 4 as the chain
+dynamic per-token quantise -> W8A8 GEMM, config 5 with its SmoothQuant (alpha = 0.5) factor vector."""
+import pytest
+import torch
+
+from amct_amd import ops, workloads
+from oracle import deploy as od
+from oracle import int_quant as iq
+from oracle import mx
+from tests.util import assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+
+SAMPLE = [0, 1, 63, 64, 127, 128, 255, 256, 257, 511, 512, 1023, 1024, 1500, 2046, 2047]
+
+
+@pytest.fixture(scope="module")
+def c4():
+    return workloads.c4_w8a8()
+
+
+@pytest.fixture(scope="module")
+def c5():
+    return workloads.c5_w4a16(2048)
+
+
+@pytest.mark.parametrize("M", [2048, 16])
+def test_config4_dynamic_quant_then_w8a8_at_bench_size(dev, c4, M):
+    """X[M,4096] bf16 -> per-token int8 codes and scales (every row, bit for bit) -> GEMM against W[14336,4096] int8 with
+    the per-channel factors: accumulators and bf16 output of the sampled rows bit for bit, every column."""
+    x, wq, sw = c4
+    x = x[:M].contiguous()
+    xq, st = ops.act_quant_per_token_int8(x.to(dev))
+    want_q, want_s = iq.dynamic_token_quant(x)
+    assert_bits_equal(st, want_s, "per-token scales")
+    assert torch.equal(xq.cpu(), want_q), "per-token codes"
+    out, acc = ops.gemm_w8a8(xq, wq.to(dev), sw.to(dev), st, None, want_acc=True)
+    rows = [r for r in SAMPLE if r < M]
+    assert torch.equal(acc.cpu()[rows].to(torch.int64), od.int8_matmul_exact(want_q[rows], wq.t())), "accumulators"
+    assert_bits_equal(out.cpu()[rows], od.quant_matmul(want_q[rows], wq.t(), sw, want_s[rows], None, torch.bfloat16), "w8a8 out")
+
+
+@pytest.mark.parametrize("M", [2048, 16, 1])
+def test_config5_w4a16_with_smoothing_at_bench_size(dev, c5, M):
+    """x[M,4096] bf16 * smoothing vector, W[14336,4096] int4 g128 with fp16 scales: the sampled rows within 1e-3 of the
+    row's largest output (plus one bf16 ulp of the value) of the fp64 anchor, every column; with and without the
+    workspace the library takes the same kernels for these sizes or not, both must hold the tolerance."""
+    x, codes, scales, zeros, smooth_recip = c5
+    x = x[:M].contiguous()
+    packed = workloads.pack_nibbles(codes).to(dev)
+    out = ops.gemm_w4a16(x.to(dev), packed, scales.to(dev), zeros.to(dev), 128, smooth_recip.to(dev), None).cpu()
+    rows = [r for r in SAMPLE if r < M]
+    signed = codes.to(torch.int32) - 8
+    anti = -(zeros.to(torch.float32) - 8)
+    want = od.w4a16_forward_f64(x[rows], signed, scales, anti, 128, None, smooth_recip.reshape(1, -1),
+                                round_weight=not od.w4a16_streams(M, 4096, 128))
+    err = (out[rows].double() - want).abs()
+    tol = 1e-3 * want.abs().amax(dim=1, keepdim=True) + want.abs() * 2.0 ** -8
+    assert (err <= tol).all(), (err.max().item(), tol.min().item())
+
+
+def test_config2_int4_group_pack_at_bench_size(dev):
+    """W[14336,4096] bf16 (the headline workload): packed nibbles, fp16 scales and zero-points of a row sample that
+    covers the first, last and interior blocks bit for bit."""
+    w = workloads.c2_weight()
+    packed, scales, zeros, _ = ops.quant_int4_group_pack(w.to(dev), 128, scale_dtype=torch.float16)
+    rows = sorted(set(SAMPLE + [14335, 14334, 7168, 9999, 4095, 4096]))
+    ws = w[rows]
+    s, z = iq.weight_scale_offset(ws, 'group', False, 'int4', 128)
+    codes = iq.quant_codes(ws, 'int4', s, z, 128).reshape(len(rows), -1)
+    assert torch.equal(packed.cpu()[rows], od.pack_nibbles_k(codes)), "packed codes"
+    assert_bits_equal(scales.cpu()[rows], s.squeeze(-1).to(torch.float16), "scales")
+    assert torch.equal(zeros.cpu()[rows].to(torch.int32), (z.squeeze(-1) + 8).to(torch.int32)), "zero-points"
+
+
+def test_config1_int8_fakequant_at_bench_size(dev):
+    """W[4096,4096] fp32, int8 symmetric per-channel fake-quant: every element bit for bit."""
+    w = workloads.c1_weight()
+    s, z = iq.weight_scale_offset(w, 'channel', True, 'int8')
+    want = iq.fake_quant(w, 'int8', s, z)
+    dq, _, scale, _ = ops.fakequant_int(w.to(dev), 8, True)
+    assert_bits_equal(scale, s.reshape(-1), "per-channel scales")
+    assert_bits_equal(dq, want, "fake-quantised weight")
+
+
+@pytest.mark.parametrize("fmt", [mx.E4M3, mx.E2M1])
+def test_config3_mx_quant_at_bench_size(dev, fmt):
+    """X[8192,4096] bf16 -> MXFP8 / MXFP4: element codes and shared exponents of 1024 sampled rows bit for bit."""
+    x = workloads.c3_activations()
+    el, sb = ops.mx_quant(x.to(dev), fmt)
+    rows = torch.arange(0, 8192, 8)
+    want_el, want_sb = mx.mx_quant(x[rows], fmt)
+    assert torch.equal(el.cpu()[rows].reshape(-1), torch.as_tensor(want_el).reshape(-1)), "element codes"
+    assert torch.equal(sb.cpu()[rows].reshape(-1), torch.as_tensor(want_sb).reshape(-1)), "shared exponents"
