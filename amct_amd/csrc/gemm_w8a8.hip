@@ -9,8 +9,10 @@
 //                   256x192 tiles.
 //   tile kernel   : 128x128 block tile, 4 waves of 64x64, BK = 128 bytes, two register stages of
 //                   prefetch (shapes the large-tile kernel does not take).
-//   decode kernel : M <= 16: activations staged once per block in LDS, the weight streamed once straight
-//                   from HBM into MFMA operands (v_mfma_i32_16x16x64_i8), split-K across the waves.
+//   decode kernels: M <= 16: activations staged once per block in LDS, the weight streamed once straight
+//                   from HBM into MFMA operands (v_mfma_i32_16x16x64_i8), split-K across the waves; for K of 1024,
+//                   2048 or 4096 the variant in gemm_w8a8_stream.hip (all weight loads of the launch in flight at
+//                   once, whole 128-byte lines per load instruction).
 //   medium tiles  : 16 < M up to a few hundred rows: the large-tile body with 128x128 (4 waves) or 128x256 blocks and
 //                   three LDS stages, chosen so that all blocks of the launch run at once.
 //   skinny kernel : 16 < M <= 32 when K is not a multiple of 128 (and M <= 16 shapes the decode kernel does not
@@ -744,6 +746,10 @@ __global__ __launch_bounds__(kBlock) void w8a8_general(W8A8Args a) {
     w8a8_epilogue(a, m, n, acc);
 }
 
+int w8a8_stream_dispatch(const int8_t* xq, const int8_t* wq, const float* s_tok, const float* s_ch, const void* bias,
+                         int bias_kind, void* out, int32_t* acc_out, int64_t M, int64_t N, int64_t K, int out_dtype,
+                         hipStream_t st);
+
 }  // namespace amct
 
 using namespace amct;
@@ -762,6 +768,10 @@ extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s
     // operands below 4 GiB (32-bit lane offsets)
     const bool tile_ok = vec_ok && K % 128 == 0 && N % 8 == 0 && aligned16(out) && M * K < (int64_t(1) << 32) &&
                          N * K < (int64_t(1) << 32);
+    if (M <= 16) {                                              // weight-streaming kernel (K of 1024, 2048 or 4096)
+        const int rc = w8a8_stream_dispatch(xq, wq, s_tok, s_ch, bias, bias_kind, out, acc_out, M, N, K, out_dtype, st);
+        if (rc != AMCT_E_UNSUPPORTED) return rc;
+    }
     if (vec_ok && M <= 16 && K % 256 == 0 && (M <= 2 || !tile_ok)) {
         const int iters = (int)(K / 256);
         // measured: blocks of 2 or 4 waves, several per CU, stream best (one block's start-up and reduction

@@ -173,6 +173,159 @@ __global__ __launch_bounds__(kBlock) void mx_quant_k(const void* x, uint8_t* el,
     }
 }
 
+// ---- quantise, complete blocks of U * 256 vectors -------------------------------------------------
+// Same results as mx_quant_k; what differs is the instruction count (about 4.5 vector instructions per bf16 element
+// against 9.4, and no 64-bit address arithmetic).  The element cast is the hardware's scaled conversion
+// (v_cvt_scalef32_pk_{fp8,fp4}_{bf16,f32}: cast(value / scale), scale a power of two taken from the block
+// exponent), so nothing is multiplied.  Checked against the product form over every bf16 pattern and block
+// exponents from -126 to 125: the FP4 conversion saturates by itself, the FP8 one turns magnitudes above the
+// format's largest into NaN, hence the clamp to 448 * scale before it -- for bf16 input on the packed 16-bit
+// magnitudes (v_pk_min_u16; sign-magnitude order equals unsigned order), with the block maximum found the same
+// way (v_pk_max_u16).  Addresses are one wave-uniform base per block plus a 32-bit lane offset.
+// A wave that holds a block with an infinity, a NaN or a block exponent of zero (maximum below 2^(emax-126): the
+// scale is then a denormal) takes the general routine for all of its blocks.
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef unsigned short v2u16 __attribute__((ext_vector_type(2)));
+AMCT_DEV uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(v2u16, a), __builtin_bit_cast(v2u16, b)));
+}
+AMCT_DEV uint32_t pk_min_u16(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(v2u16, a), __builtin_bit_cast(v2u16, b)));
+}
+
+// general routine for one vector per lane (every lane of the wave calls it): returns the block byte, fills the
+// packed element codes (8, 4 or 2 bytes in w[0], w[1])
+template <int DT, int FMT>
+AMCT_DEV uint32_t mx_quant_vec_general(const uint4& raw, int scale_mode, uint32_t (&w)[2]) {
+    constexpr int VEC = Tr<DT>::VEC;
+    constexpr int T = 32 / VEC;
+    constexpr int EMAX = (FMT == kFmtE4M3) ? 8 : 2;
+    constexpr uint32_t FMAX_MAN = (FMT == kFmtE4M3) ? 0x600000u : 0x400000u;
+    float v[VEC];
+    unpack16<DT>(raw, v);
+    uint32_t amax = 0;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) amax = max(amax, __float_as_uint(v[j]) & 0x7FFFFFFFu);
+    amax = team_umax<T>(amax);
+    const bool has_nan = amax > 0x7F800000u;
+    int be = (int)(amax >> 23) - EMAX;
+    if (scale_mode == 1) be += ((amax & 0x7FFFFFu) > FMAX_MAN) ? 1 : 0;
+    be = has_nan ? 254 : min(max(be, 0), 254);
+    const int e = be - 127;
+    const int h = e >> 1;
+    const float f1 = __uint_as_float((uint32_t)(127 - h) << 23);
+    const float f2 = __uint_as_float((uint32_t)(127 - (e - h)) << 23);
+    w[0] = 0; w[1] = 0;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        const float tt = v[j] * f1 * f2;
+        if constexpr (FMT == kFmtE4M3) w[j / 4] |= sw_e4m3(tt) << (8 * (j % 4));
+        else w[0] |= sw_e2m1(tt) << (4 * j);
+    }
+    return has_nan ? 255u : (uint32_t)be;
+}
+
+template <int DT, int FMT, int U>
+__global__ __launch_bounds__(kBlock) void mx_quant_full(const void* x, uint8_t* el, uint8_t* e8, int scale_mode) {
+    constexpr int VEC = Tr<DT>::VEC;
+    constexpr int T = 32 / VEC;
+    constexpr int OB = (FMT == kFmtE4M3) ? VEC : VEC / 2;           // output bytes per vector
+    constexpr int EMAX = (FMT == kFmtE4M3) ? 8 : 2;
+    constexpr uint32_t FMAX_MAN = (FMT == kFmtE4M3) ? 0x600000u : 0x400000u;
+    constexpr uint32_t FMAX_BITS = (FMT == kFmtE4M3) ? 0x43E00000u : 0x40C00000u;
+    const uint32_t tid = threadIdx.x;
+    const int64_t v0 = (int64_t)blockIdx.x * (U * kBlock);
+    const char* xb = reinterpret_cast<const char*>(x) + v0 * 16;
+    uint8_t* eb = el + v0 * OB;
+    uint8_t* sb = e8 + v0 / T;
+    uint4 raw[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) raw[u] = ldg16_nt(xb + (uint32_t)((u * kBlock + tid) * 16));
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint32_t r[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+        uint32_t mag[4];
+        uint32_t amax;
+        if constexpr (DT == AMCT_BF16) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) mag[j] = r[j] & 0x7FFF7FFFu;
+            const uint32_t a = pk_max_u16(pk_max_u16(mag[0], mag[1]), pk_max_u16(mag[2], mag[3]));
+            amax = team_umax<T>(max(a & 0xFFFFu, a >> 16)) << 16;
+        } else {
+            float v[VEC];
+            unpack16<DT>(raw[u], v);
+            amax = 0;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) amax = max(amax, __float_as_uint(v[j]) & 0x7FFFFFFFu);
+            amax = team_umax<T>(amax);
+        }
+        int be = (int)(amax >> 23) - EMAX;
+        if (scale_mode == 1) be += ((amax & 0x7FFFFFu) > FMAX_MAN) ? 1 : 0;
+        const bool special = amax >= 0x7F800000u || (be <= 0 && amax != 0u);
+        uint32_t w[2] = {0u, 0u};
+        uint32_t byte;
+        if (__builtin_amdgcn_ballot_w64(special) != 0ull) {
+            byte = mx_quant_vec_general<DT, FMT>(raw[u], scale_mode, w);
+        } else {
+            byte = (uint32_t)max(be, 0);                          // be <= 254 - EMAX here; 0 only for an all-zero block
+            const uint32_t bs = (uint32_t)max(be, 1);
+            const float scale = __uint_as_float(bs << 23);
+            const uint32_t thr = FMAX_BITS + ((bs - 127u) << 23); // largest element magnitude times the scale
+            if constexpr (DT == AMCT_BF16) {
+                uint32_t q[4];
+                if constexpr (FMT == kFmtE4M3) {
+                    const uint32_t thr2 = (thr >> 16) * 0x10001u;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) q[j] = (r[j] & 0x80008000u) | pk_min_u16(mag[j], thr2);
+                    v2i16 o0 = {0, 0}, o1 = {0, 0};
+                    o0 = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(o0, __builtin_bit_cast(v2bf, q[0]), scale, false);
+                    o0 = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(o0, __builtin_bit_cast(v2bf, q[1]), scale, true);
+                    o1 = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(o1, __builtin_bit_cast(v2bf, q[2]), scale, false);
+                    o1 = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(o1, __builtin_bit_cast(v2bf, q[3]), scale, true);
+                    w[0] = __builtin_bit_cast(uint32_t, o0);
+                    w[1] = __builtin_bit_cast(uint32_t, o1);
+                } else {
+                    uint32_t o = 0;
+                    o = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(o, __builtin_bit_cast(v2bf, r[0]), scale, 0);
+                    o = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(o, __builtin_bit_cast(v2bf, r[1]), scale, 1);
+                    o = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(o, __builtin_bit_cast(v2bf, r[2]), scale, 2);
+                    o = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(o, __builtin_bit_cast(v2bf, r[3]), scale, 3);
+                    w[0] = o;
+                }
+            } else {
+                float v[VEC];
+                unpack16<DT>(raw[u], v);
+                const float lim = __uint_as_float(thr);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) v[j] = __builtin_amdgcn_fmed3f(v[j], -lim, lim);
+                if constexpr (FMT == kFmtE4M3) {
+#pragma unroll
+                    for (int j = 0; j < VEC / 4; ++j) {
+                        v2i16 o = {0, 0};
+                        o = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(o, v[4 * j], v[4 * j + 1], scale, false);
+                        o = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(o, v[4 * j + 2], v[4 * j + 3], scale, true);
+                        w[j] = __builtin_bit_cast(uint32_t, o);
+                    }
+                } else {
+                    uint32_t o = 0;
+                    o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, v[0], v[1], scale, 0);
+                    o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, v[2], v[3], scale, 1);
+                    if constexpr (VEC == 8) {
+                        o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, v[4], v[5], scale, 2);
+                        o = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(o, v[6], v[7], scale, 3);
+                    }
+                    w[0] = o;
+                }
+            }
+        }
+        const uint32_t idx = u * kBlock + tid;
+        if constexpr (OB == 8) stg8_nt(eb + idx * 8u, w[0], w[1]);
+        else if constexpr (OB == 4) stg4_nt(eb + idx * 4u, w[0]);
+        else *reinterpret_cast<uint16_t*>(eb + idx * 2u) = (uint16_t)w[0];
+        if ((tid & (T - 1)) == 0) sb[idx / T] = (uint8_t)byte;
+    }
+}
+
 // ---- dequantise -------------------------------------------------------------------------------
 // One lane produces one 16-byte output vector (VEC elements of the output dtype) per step, U steps in
 // flight.  Element codes are decoded by the hardware conversions (v_cvt_pk_f32_fp8, v_cvt_scalef32_pk_f32_fp4
@@ -236,9 +389,25 @@ __global__ __launch_bounds__(kBlock) void mx_dequant_k(const uint8_t* el, const 
     }
 }
 
+// Complete blocks of U * 256 vectors go to mx_quant_full; the rest (and everything, when the bit-manipulation cast is
+// asked for) to mx_quant_k.  Both give the same codes.
 template <int DT, int FMT>
 static int launch_quant(const void* x, uint8_t* el, uint8_t* e8, int64_t nvec, int scale_mode, bool hw, hipStream_t st) {
     constexpr int U = 4;
+    constexpr int VEC = Tr<DT>::VEC;
+    if (hw) {
+        const int64_t full = nvec / ((int64_t)kBlock * U);
+        if (full > 0) {
+            if (full > 0x7FFFFFFF) return AMCT_E_UNSUPPORTED;
+            hipLaunchKernelGGL((mx_quant_full<DT, FMT, U>), dim3((unsigned)full), dim3(kBlock), 0, st, x, el, e8, scale_mode);
+            const int64_t done = full * kBlock * U;
+            x = reinterpret_cast<const char*>(x) + done * 16;
+            el += done * (FMT == kFmtE4M3 ? VEC : VEC / 2);
+            e8 += done / (32 / VEC);
+            nvec -= done;
+            if (nvec == 0) return hip_status();
+        }
+    }
     const int64_t nb = (nvec + (int64_t)kBlock * U - 1) / ((int64_t)kBlock * U);
     if (hw) hipLaunchKernelGGL((mx_quant_k<DT, FMT, true, U>), dim3((unsigned)nb), dim3(kBlock), 0, st, x, el, e8, nvec, scale_mode);
     else hipLaunchKernelGGL((mx_quant_k<DT, FMT, false, U>), dim3((unsigned)nb), dim3(kBlock), 0, st, x, el, e8, nvec, scale_mode);

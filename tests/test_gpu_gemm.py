@@ -89,6 +89,23 @@ def test_w8a8_large_shapes_mixed_blocks(dev, M, N, K):
     assert_bits_equal(out, od.quant_matmul(xq, wq.t(), s_ch, s_tok, None, torch.bfloat16), "out bf16, no bias")
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 64, 1024), (16, 200, 2048), (9, 72, 1024), (5, 33, 2048), (16, 1000, 1024),
+                                   (13, 14336, 4096), (1, 14336, 2048), (3, 16, 4096), (16, 15, 1024), (2, 4104, 4096)])
+def test_w8a8_weight_streaming_kernel(dev, M, N, K):
+    """The kernel for a few rows (M <= 16, K of 1024/2048/4096): both block widths, ragged N, every epilogue variant
+    and output dtype; accumulators and outputs bit for bit."""
+    for per_token, bias_kind in ((True, 'float'), (False, 'int'), (True, None)):
+        xq, wq, s_ch, s_tok, b = w8a8_case(M, N, K, 150 + M, per_token, bias_kind)
+        want_acc = od.int8_matmul_exact(xq, wq.t())
+        if bias_kind == 'int':
+            want_acc = want_acc + b.to(torch.int64)
+        for odt in (torch.bfloat16, torch.float16, torch.float32):
+            out, acc = ops.gemm_w8a8(xq.to(dev), wq.to(dev), s_ch.to(dev), None if s_tok is None else s_tok.to(dev),
+                                     None if b is None else b.to(dev), out_dtype=odt, want_acc=True)
+            assert torch.equal(acc.cpu().to(torch.int64), want_acc), "accumulators"
+            assert_bits_equal(out, od.quant_matmul(xq, wq.t(), s_ch, s_tok, b, odt), "out %s" % odt)
+
+
 def w4a16_case(M, N, K, group, seed, sdt=torch.float16):
     g = torch.Generator().manual_seed(seed)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)
