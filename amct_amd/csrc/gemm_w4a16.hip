@@ -458,14 +458,18 @@ AMCT_DEV void gload_u8s(uint32_t& dst, const void* sbase, uint32_t voff) {
 }
 template <int N> AMCT_DEV void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory"); }
 
-template <int WM, int WN, int TI, int TJ, int STAGES>
+// STAGES: LDS stages of the activation tile (filled by direct-to-LDS loads; a third stage gives a load two steps to
+// land); SB: stages of the dequantised weight tile (written by the waves themselves one step ahead: two suffice)
+template <int WM, int WN, int TI, int TJ, int STAGES, int SB = STAGES>
 struct WideTile {
     static constexpr int kLM = 32 * TI * WM, kLN = 32 * TJ * WN, kWaves = WM * WN, kThreads = kWaves * 64;
-    static constexpr int kStageBytes = (kLM + kLN) * kWRow;
+    static constexpr int kABytes = kLM * kWRow, kBBytes = kLN * kWRow;     // one stage of each operand
+    static constexpr int kBBase = STAGES * kABytes;                        // the weight stages follow the activation stages
     static constexpr int kLW = kWaves / 2;                         // waves that issue the direct-to-LDS loads
     static constexpr int kNA = (kLM * kWRow / 1024) / kLW;         // activation pieces (8 rows x 128 B) per loading wave
     static constexpr int kEpi = kWaves * 16384;
-    static constexpr int kSmem = STAGES * kStageBytes > kEpi ? STAGES * kStageBytes : kEpi;
+    static constexpr int kRing = STAGES * kABytes + SB * kBBytes;
+    static constexpr int kSmem = kRing > kEpi ? kRing : kEpi;
     static constexpr int kQ = kThreads / kLN;                     // threads per weight row of the tile
     static constexpr int kBC = 8 / kQ;                             // 8-weight chunks a thread dequantises per step
     static_assert(kThreads == 2 * kLN || kThreads == 4 * kLN, "every thread dequantises a half or a quarter of a weight row of the tile per step");
@@ -473,13 +477,14 @@ struct WideTile {
     static_assert(kNA < 64, "vmcnt range");
 };
 
-template <bool SF16, int WM, int WN, int TI, int TJ, int STAGES>
+template <bool SF16, int WM, int WN, int TI, int TJ, int STAGES, int SB = STAGES>
 AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m0, const int64_t n0) {
-    using Sh = WideTile<WM, WN, TI, TJ, STAGES>;
-    constexpr int kLM = Sh::kLM, kStageBytes = Sh::kStageBytes, kWaves = Sh::kWaves, kLW = Sh::kLW, kNA = Sh::kNA;
+    using Sh = WideTile<WM, WN, TI, TJ, STAGES, SB>;
+    constexpr int kABytes = Sh::kABytes, kBBytes = Sh::kBBytes, kBBase = Sh::kBBase;
+    constexpr int kWaves = Sh::kWaves, kLW = Sh::kLW, kNA = Sh::kNA;
     constexpr int kNM = TI * TJ, kNR = TI + TJ;                    // MFMAs and fragment reads per k-slice
     constexpr int kRPM = (kNR + kNM - 1) / kNM;                    // fragment reads issued behind each MFMA
-    static_assert(STAGES == 2 || STAGES == 3, "2 or 3 stages");
+    static_assert((STAGES == 2 || STAGES == 3) && (SB == 2 || SB == 3) && SB <= STAGES, "2 or 3 stages");
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
@@ -507,7 +512,7 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
             const int st = step < last ? step : last;
 #pragma unroll
             for (int j = 0; j < kNA; ++j)
-                dma16s(lds0 + stg * kStageBytes + (lw * kNA + j) * 1024, a.x + (int64_t)st * kWK, goff[j]);
+                dma16s(lds0 + stg * kABytes + (lw * kNA + j) * 1024, a.x + (int64_t)st * kWK, goff[j]);
         }
     };
     // weight row of this thread: row tid/kQ of the tile, 8*kBC weights (4*kBC bytes) per step, which part from tid%kQ
@@ -518,7 +523,7 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
     const uint32_t soff = (uint32_t)(wrow * G * 2), zoff = (uint32_t)(wrow * G);
     int bdst[kBC];
 #pragma unroll
-    for (int c = 0; c < kBC; ++c) bdst[c] = kLM * kWRow + brow * kWRow + ((kBC * bpart + c) ^ swz(brow)) * 16;
+    for (int c = 0; c < kBC; ++c) bdst[c] = kBBase + brow * kWRow + ((kBC * bpart + c) ^ swz(brow)) * 16;
 
     typename std::conditional<kBC == 4, u4v, u2v>::type wreg[2];
     uint32_t sreg[2], zreg[2];
@@ -536,19 +541,21 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
         nzs = -((float)zreg[slot] * sc);
     };
     auto write_b = [&](int slot, int stg, int c) {                 // dequantise 8 weights into LDS
-        *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[c]) = dequant8(wreg[slot][c], sc, nzs);
+        *reinterpret_cast<uint4*>(smem + stg * kBBytes + bdst[c]) = dequant8(wreg[slot][c], sc, nzs);
     };
     // Wait until the weight loads of the previous iteration and the activation loads issued STAGES-1 iterations ago
-    // have landed and this wave's LDS operations are done.  An iteration issues its 3 weight loads first and then, in
-    // a loading wave, kNA direct-to-LDS loads; with three stages the latter may stay in flight, hence the
-    // wave-uniform choice of the count.  The slot's registers are tied to a statement behind the wait so that
+    // have landed and this wave's LDS operations are done.  An iteration issues its 3 weight loads in the middle of the
+    // step, as soon as their register slot has been dequantised (when the memory pipeline is idle: issued right after
+    // the barrier they queued behind the loading waves' burst and both waves of a SIMD stood still), and, in a loading
+    // wave, kNA direct-to-LDS loads right after the barrier.  The youngest weight loads may stay in flight, and with three
+    // stages the youngest activation loads too, hence the wave-uniform choice of the count.  The slot's registers are tied to a statement behind the wait so that
     // their uses (and any copies the register allocator makes) stay behind it.
     auto wait_older = [&]() {
         if constexpr (STAGES == 2) {
-            wait_vm<0>();
+            wait_vm<3>();
         } else {
-            if (loader) wait_vm<kNA>();
-            else wait_vm<0>();
+            if (loader) wait_vm<kNA + 3>();
+            else wait_vm<3>();
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     };
@@ -560,7 +567,7 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
         const int r = lane & 31;
         const int phys = (ks * 2 + (lane >> 5)) ^ swz(r);
         offA[ks] = (wm * 32 * TI + r) * kWRow + phys * 16;
-        offB[ks] = kLM * kWRow + (wn * 32 * TJ + r) * kWRow + phys * 16;
+        offB[ks] = kBBase + (wn * 32 * TJ + r) * kWRow + phys * 16;
     }
     v16f acc[TI][TJ];
 #pragma unroll
@@ -571,11 +578,12 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     // fragment q in the order the MFMAs need them: A0, B0, B1, .., A1, A2, ..
-    auto read_one = [&](int stg, int ks, int q, v8bf (&fa)[TI], v8bf (&fb)[TJ]) {
-        const uint8_t* st = smem + stg * kStageBytes;
-        if (q == 0) fa[0] = *reinterpret_cast<const v8bf*>(st + offA[ks]);
-        else if (q <= TJ) fb[q - 1] = *reinterpret_cast<const v8bf*>(st + offB[ks] + (q - 1) * 32 * kWRow);
-        else fa[q - TJ] = *reinterpret_cast<const v8bf*>(st + offA[ks] + (q - TJ) * 32 * kWRow);
+    auto read_one = [&](int sa, int sb, int ks, int q, v8bf (&fa)[TI], v8bf (&fb)[TJ]) {
+        const uint8_t* pa = smem + sa * kABytes;
+        const uint8_t* pb = smem + sb * kBBytes;
+        if (q == 0) fa[0] = *reinterpret_cast<const v8bf*>(pa + offA[ks]);
+        else if (q <= TJ) fb[q - 1] = *reinterpret_cast<const v8bf*>(pb + offB[ks] + (q - 1) * 32 * kWRow);
+        else fa[q - TJ] = *reinterpret_cast<const v8bf*>(pa + offA[ks] + (q - TJ) * 32 * kWRow);
     };
     auto mfma_one = [&](int m, const v8bf (&fa)[TI], const v8bf (&fb)[TJ]) {
         const int i = m / TJ, j = m % TJ;
@@ -601,21 +609,23 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 #pragma unroll
-    for (int q = 0; q < kNR; ++q) read_one(0, 0, q, fa[0], fb[0]);
+    for (int q = 0; q < kNR; ++q) read_one(0, 0, 0, q, fa[0], fb[0]);
 
     // iteration s (LDS stage cur, the next one nxt; register slot SL holds B(s+1), landed; the other slot B(s+2)):
     //   k-slices 0, 1 : MFMAs, fragment reads of the next slice, dequantisation of B(s+1) into stage nxt
+    //   loads         : B(s+3) into slot SL (its old content is in LDS now)
     //   k-slice 2     : MFMAs, fragment reads of slice 3
     //   wait (A(s+1) and B(s+2) have landed; own LDS operations done), barrier: stage cur is free, nxt complete
-    //   loads         : B(s+3) into slot SL, A(s+STAGES) into stage cur (loading waves)
+    //   loads         : A(s+STAGES) into stage cur (loading waves)
     //   k-slice 3     : MFMAs, fragment reads of slice 0 of stage nxt
-    int cur = 0, nxt = 1;
+    int cur = 0, nxt = 1;                                           // activation stages
+    int curb = 0, nxtb = 1;                                         // weight stages
 #define AMCT_WSLICE_DQ(CUR, NXT, SL, KS)                                                 \
     {                                                                                  \
         __builtin_amdgcn_sched_barrier(0);                                             \
         _Pragma("unroll") for (int m_ = 0; m_ < kNM; ++m_) mfma_one(m_, fa[(KS) & 1], fb[(KS) & 1]); \
-        _Pragma("unroll") for (int q_ = 0; q_ < kNR; ++q_) read_one(CUR, (KS) + 1, q_, fa[((KS) + 1) & 1], fb[((KS) + 1) & 1]); \
-        _Pragma("unroll") for (int c_ = 0; c_ < kBC / 2; ++c_) write_b(SL, NXT, (kBC / 2) * (KS) + c_); \
+        _Pragma("unroll") for (int q_ = 0; q_ < kNR; ++q_) read_one(CUR, curb, (KS) + 1, q_, fa[((KS) + 1) & 1], fb[((KS) + 1) & 1]); \
+        _Pragma("unroll") for (int c_ = 0; c_ < kBC / 2; ++c_) write_b(SL, nxtb, (kBC / 2) * (KS) + c_); \
         _Pragma("unroll") for (int g_ = 0; g_ < kNM; ++g_) {                           \
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                      /* 1 MFMA */ \
             __builtin_amdgcn_sched_group_barrier(0x002, (14 * kBC + kNM - 1) / kNM, 0); /* VALU */ \
@@ -623,13 +633,13 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
         }                                                                              \
         __builtin_amdgcn_sched_barrier(0);                                             \
     }
-#define AMCT_WSLICE_PIN(STG, KSREAD, KS)                                               \
+#define AMCT_WSLICE_PIN(STG, STGB, KSREAD, KS)                                         \
     {                                                                                  \
         _Pragma("unroll") for (int m_ = 0; m_ < kNM; ++m_) {                           \
             mfma_one(m_, fa[(KS) & 1], fb[(KS) & 1]);                                  \
             __builtin_amdgcn_sched_barrier(0);                                         \
             _Pragma("unroll") for (int q_ = m_ * kRPM; q_ < (m_ + 1) * kRPM && q_ < kNR; ++q_) { \
-                read_one(STG, KSREAD, q_, fa[((KS) + 1) & 1], fb[((KS) + 1) & 1]);     \
+                read_one(STG, STGB, KSREAD, q_, fa[((KS) + 1) & 1], fb[((KS) + 1) & 1]); \
                 __builtin_amdgcn_sched_barrier(0);                                     \
             }                                                                          \
         }                                                                              \
@@ -640,17 +650,20 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
         factors(SL);                                                                   \
         AMCT_WSLICE_DQ(cur, nxt, SL, 0)                                                \
         AMCT_WSLICE_DQ(cur, nxt, SL, 1)                                                \
-        AMCT_WSLICE_PIN(cur, 3, 2)                                                     \
+        issue_b(SL, (step) + 3);                                                       \
+        __builtin_amdgcn_sched_barrier(0);                                             \
+        AMCT_WSLICE_PIN(cur, curb, 3, 2)                                               \
         wait_older();                                                                  \
         __builtin_amdgcn_s_barrier();                                                  \
         asm volatile("" ::: "memory");                                                 \
         __builtin_amdgcn_sched_barrier(0);                                             \
-        issue_b(SL, (step) + 3);                                                       \
         dma_a(cur, (step) + STAGES);                                                   \
         __builtin_amdgcn_sched_barrier(0);                                             \
-        AMCT_WSLICE_PIN(nxt, 0, 3)                                                     \
+        AMCT_WSLICE_PIN(nxt, nxtb, 0, 3)                                               \
         cur = nxt;                                                                     \
         nxt = nxt + 1 == STAGES ? 0 : nxt + 1;                                         \
+        curb = nxtb;                                                                   \
+        nxtb = nxtb + 1 == SB ? 0 : nxtb + 1;                                          \
     }
     for (int step = 0; step < nsteps; step += 2) {                  // K % 128 == 0: an even number of steps
         AMCT_WITER(1, step)
@@ -701,11 +714,11 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
 }
 
 // blockIdx.x: column tile, blockIdx.y: row tile
-template <bool SF16, int WM, int WN, int TI, int TJ, int STAGES>
+template <bool SF16, int WM, int WN, int TI, int TJ, int STAGES, int SB = STAGES>
 __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM * WN / 4, WM * WN / 4))) void w4a16_tile_wide(W4A16Args a) {
-    using Sh = WideTile<WM, WN, TI, TJ, STAGES>;
+    using Sh = WideTile<WM, WN, TI, TJ, STAGES, SB>;
     __shared__ __attribute__((aligned(1024))) uint8_t smem[Sh::kSmem];
-    w4a16_wide_body<SF16, WM, WN, TI, TJ, STAGES>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
+    w4a16_wide_body<SF16, WM, WN, TI, TJ, STAGES, SB>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
 }
 
 // ---------------------------------------------------------------------------

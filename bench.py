@@ -83,6 +83,17 @@ def build_cases(dev, only):
             assert rc == 0, rc
         cases.append(Case("copy", "hbm", 2 * nbytes, "B", launch, nsc, "u8", "plain copy of 128 MiB (yardstick)"))
 
+    # ---- launch floor: a copy of 4 KiB, i.e. what one launch costs back to back whatever the kernel does -------------
+    if want("launch_floor"):
+        sf = torch.zeros(4096, dtype=torch.uint8, device=dev)
+        df = torch.zeros(4096, dtype=torch.uint8, device=dev)
+
+        def launch(i, sf=sf, df=df):
+            rc = lib.amct_copy_bytes(sf.data_ptr(), df.data_ptr(), 4096, st)
+            assert rc == 0, rc
+        cases.append(Case("launch_floor", "hbm", 8192, "B", launch, 1, "u8",
+                          "copy of 4 KiB: the time one launch takes back to back (yardstick for the launch-bound kernels)"))
+
     # ---- K2 (headline): int4 asym g128 quant + pack, W[14336,4096] bf16 -------------------------
     if want("int4_group_pack"):
         w = workloads.c2_weight()
@@ -248,6 +259,28 @@ def build_cases(dev, only):
             cases.append(Case(yname, bound, ops_out.value, "OP", launch, 1, ydesc,
                               "register-only %s MFMA loop on every CU, pseudo-random operands (yardstick: what the "
                               "matrix pipe sustains under the power limit on such data)" % ydesc))
+
+    # ---- the vendor library's GEMMs at the same shape (hipBLASLt through torch), as yardsticks of what tuned kernels
+    # reach on this part and these operands: a plain bf16 x bf16 Linear (no dequantisation) and a plain int8 x int8
+    # product (no rescale epilogue).  They are not part of the product.
+    if want("lib_gemm_bf16"):
+        xl = workloads.c5_w4a16(2048, 64, 4096)[0].to(dev)
+        gl = torch.Generator().manual_seed(1021)
+        wl = [(torch.randn(14336, 4096, generator=gl) * 0.02).to(torch.bfloat16).to(dev) for _ in range(4)]
+
+        def launch(i, xl=xl, wl=wl):
+            torch.nn.functional.linear(xl, wl[i % len(wl)])
+        cases.append(Case("lib_gemm_bf16", "mfma_bf16", 2 * 2048 * 14336 * 4096, "flop", launch, 4, "bf16",
+                          "torch.nn.functional.linear bf16 x bf16, M=2048 N=14336 K=4096 (vendor library yardstick)"))
+    if want("lib_gemm_i8"):
+        x6l, wq6l, _ = workloads.c4_w8a8()
+        xql = ops.act_quant_per_token_int8(x6l.to(dev))[0]
+        wql = [wq6l.to(dev).t()] + [wq6l.to(dev).clone().t() for _ in range(3)]
+
+        def launch(i, xql=xql, wql=wql):
+            torch._int_mm(xql, wql[i % len(wql)])
+        cases.append(Case("lib_gemm_i8", "mfma_i8", 2 * 2048 * 14336 * 4096, "op", launch, 4, "int8",
+                          "torch._int_mm int8 x int8 -> int32, M=2048 N=14336 K=4096 (vendor library yardstick)"))
 
     # ---- K6: W8A8 Linear, W[14336,4096] int8 ----------------------------------------------------------
     if want("w8a8_m2048") or want("w8a8_m16"):
@@ -475,6 +508,9 @@ def run(args, dev, only):
         y = {"TOP/s": "mfma_i8_yardstick", "TFLOP/s": "mfma_bf16_yardstick"}.get(r["unit"])
         if y and y in results and name != y:
             r["frac_of_yardstick"] = round(r["achieved"] / results[y]["achieved"], 4)
+        lib = {"TOP/s": "lib_gemm_i8", "TFLOP/s": "lib_gemm_bf16"}.get(r["unit"])
+        if lib and lib in results and not name.startswith(("lib_gemm", "mfma_")):
+            r["vs_vendor_library"] = round(r["achieved"] / results[lib]["achieved"], 4)
     c, wall, ms = head
     value = c.work * args.steps / wall / 1e9
     traffic = MEASURED_TRAFFIC.get("int4_group_pack")
