@@ -31,6 +31,20 @@ PEAK_BF16_TFLOPS = 2500.0
 # workload; the runs they come from and their commands are kept in profiles/hbm_traffic_pmc_bench_workloads.txt.
 # A kernel that was changed and not counted again has no entry (reported as null).
 MEASURED_TRAFFIC = {
+    "int4_group_pack": ("int4_group_pack4<2, 16, 1, false, true>", 148551685),
+    "fakequant_int8": ("fq_fused<0, 256, 4, 1, false, false>", 134440825),
+    "mxfp8_quant": ("mx_quant_full<2, 0, 4>", 101801445),
+    "mxfp4_quant": ("mx_quant_full<2, 1, 4>", 85023231),
+    "mxfp8_dequant": ("mx_dequant_k<2, 0, 4>", 101755184),
+    "hif8_encode": ("hif8_encode_k<2, 4>", 100729581),
+    "hif8_decode": ("hif8_decode_k<2, 4>", 100747659),
+    "act_quant_per_token": ("act_quant_token<2, 2>", 25292715),
+    "col_minmax": ("col_partial_k<2, false> + col_final_k", 69345307),
+    "w8a8_m2048": ("w8a8_tile_mix<2, 2, 128>", 254984145),
+    "w8a8_m16": ("w8a8_stream<2, 4, 4, 16, 4>", 59796000),
+    "w4a16_m2048": ("smooth_rows + w4a16_tile_wide<true, 2, 4, 4, 2, 2, 2>", 303591087),
+    "w4a16_m16": ("w4a16_stream<4, 4, 8, 8, true>", 32474218),
+    "w4a16_m1": ("w4a16_stream<4, 1, 8, 2, true>", 31011237),
 }
 
 
