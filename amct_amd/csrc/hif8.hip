@@ -153,6 +153,68 @@ __global__ __launch_bounds__(kBlock) void hif8_encode_k(const void* x, uint8_t* 
     }
 }
 
+// complete chunks of U * 256 vectors only: one wave-uniform base per chunk, 32-bit lane offsets, nothing clamped or
+// predicated (the remainder goes to hif8_encode_k)
+template <int DT, int U>
+__global__ __launch_bounds__(kBlock) void hif8_encode_full(const void* x, uint8_t* y, int64_t nchunks, int saturate) {
+    constexpr int VEC = Tr<DT>::VEC;
+    __shared__ Hif8Tables tbl;
+    const uint32_t tid = threadIdx.x;
+    hif8_build_tables(tbl, (int)tid, kBlock, saturate != 0);
+    __syncthreads();
+    for (int64_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
+        const char* xb = reinterpret_cast<const char*>(x) + c * (U * kBlock * 16);
+        uint8_t* yb = y + c * (U * kBlock * VEC);
+        uint4 raw[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) raw[u] = ldg16_nt(xb + (u * kBlock + tid) * 16u);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            float v[VEC];
+            unpack16<DT>(raw[u], v);
+            uint32_t w[VEC / 4];
+#pragma unroll
+            for (int j = 0; j < VEC / 4; ++j)
+                w[j] = hif8_enc_lut(tbl, v[4 * j]) | (hif8_enc_lut(tbl, v[4 * j + 1]) << 8) |
+                       (hif8_enc_lut(tbl, v[4 * j + 2]) << 16) | (hif8_enc_lut(tbl, v[4 * j + 3]) << 24);
+            uint32_t* p = reinterpret_cast<uint32_t*>(yb + (u * kBlock + tid) * (uint32_t)VEC);
+            if constexpr (VEC == 8) stg8_nt(p, w[0], w[1]);
+            else stg4_nt(p, w[0]);
+        }
+    }
+}
+
+template <int DT, int U>
+__global__ __launch_bounds__(kBlock) void hif8_decode_full(const uint8_t* x, void* y, int64_t nchunks) {
+    constexpr int VEC = Tr<DT>::VEC;
+    __shared__ float tbl[256];
+    const uint32_t tid = threadIdx.x;
+    tbl[tid] = hif8_dec(tid);
+    __syncthreads();
+    for (int64_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
+        const uint8_t* xb = x + c * (U * kBlock * VEC);
+        char* yb = reinterpret_cast<char*>(y) + c * (U * kBlock * 16);
+        uint32_t w[U][2];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            w[u][1] = 0;
+            if constexpr (VEC == 8) {
+                const u2v r = __builtin_nontemporal_load(reinterpret_cast<const u2v*>(xb + (u * kBlock + tid) * 8u));
+                w[u][0] = r.x; w[u][1] = r.y;
+            } else {
+                w[u][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(xb + (u * kBlock + tid) * 4u));
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            float out[VEC];
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) out[j] = tbl[(w[u][j / 4] >> (8 * (j % 4))) & 0xFFu];
+            stg16_nt(yb + (u * kBlock + tid) * 16u, pack16<DT>(out));
+        }
+    }
+}
+
 // decode through a 256-entry table in LDS built by the block itself; U vectors per lane in flight
 template <int DT, int U>
 __global__ __launch_bounds__(kBlock) void hif8_decode_k(const uint8_t* x, void* y, int64_t nvec, int64_t n) {
@@ -204,11 +266,19 @@ extern "C" int amct_hif8_encode(const void* x, uint8_t* y, int64_t n, int dtype,
     hipStream_t st = (hipStream_t)stream;
 #define AMCT_HE(DT)                                                                                              \
     {                                                                                                            \
-        const int64_t nvec = n / Tr<DT>::VEC;                                                                    \
-        int64_t nb = (nvec + (int64_t)kBlock * U - 1) / ((int64_t)kBlock * U);                                   \
-        if (nb == 0) nb = 1;                                                                                     \
-        if (nb > 2048) nb = 2048; /* blocks loop over chunks: the table build is paid 8 times per CU at most */ \
-        hipLaunchKernelGGL((hif8_encode_k<DT, U>), dim3((unsigned)nb), dim3(kBlock), 0, st, x, y, nvec, n, saturate); \
+        constexpr int64_t per = (int64_t)kBlock * U * Tr<DT>::VEC;      /* elements of a complete chunk */       \
+        const int64_t full = n / per;                                                                            \
+        if (full > 0) {                                                                                          \
+            /* blocks loop over chunks: the table build is paid 8 times per CU at most */                        \
+            hipLaunchKernelGGL((hif8_encode_full<DT, U>), dim3((unsigned)(full > 2048 ? 2048 : full)), dim3(kBlock), 0, st, x, y, full, saturate); \
+            x = reinterpret_cast<const char*>(x) + full * per * Tr<DT>::BYTES;                                   \
+            y += full * per;                                                                                     \
+            n -= full * per;                                                                                     \
+        }                                                                                                        \
+        if (n > 0) {                                                                                             \
+            const int64_t nvec = n / Tr<DT>::VEC;                                                                \
+            hipLaunchKernelGGL((hif8_encode_k<DT, U>), dim3(1), dim3(kBlock), 0, st, x, y, nvec, n, saturate);   \
+        }                                                                                                        \
     }
     switch (dtype) {
         case AMCT_F32: AMCT_HE(AMCT_F32) break;
@@ -227,11 +297,18 @@ extern "C" int amct_hif8_decode(const uint8_t* x, void* y, int64_t n, int dtype,
     hipStream_t st = (hipStream_t)stream;
 #define AMCT_HD(DT)                                                                                   \
     {                                                                                                 \
-        const int64_t nvec = n / Tr<DT>::VEC;                                                         \
-        int64_t nb = (nvec + (int64_t)kBlock * 4 - 1) / ((int64_t)kBlock * 4);                        \
-        if (nb == 0) nb = 1;                                                                          \
-        if (nb > 4096) nb = 4096;                                                                     \
-        hipLaunchKernelGGL((hif8_decode_k<DT, 4>), dim3((unsigned)nb), dim3(kBlock), 0, st, x, y, nvec, n); \
+        constexpr int64_t per = (int64_t)kBlock * 4 * Tr<DT>::VEC;                                    \
+        const int64_t full = n / per;                                                                 \
+        if (full > 0) {                                                                               \
+            hipLaunchKernelGGL((hif8_decode_full<DT, 4>), dim3((unsigned)(full > 4096 ? 4096 : full)), dim3(kBlock), 0, st, x, y, full); \
+            x += full * per;                                                                          \
+            y = reinterpret_cast<char*>(y) + full * per * Tr<DT>::BYTES;                              \
+            n -= full * per;                                                                          \
+        }                                                                                             \
+        if (n > 0) {                                                                                  \
+            const int64_t nvec = n / Tr<DT>::VEC;                                                     \
+            hipLaunchKernelGGL((hif8_decode_k<DT, 4>), dim3(1), dim3(kBlock), 0, st, x, y, nvec, n);  \
+        }                                                                                             \
     }
     switch (dtype) {
         case AMCT_F32: AMCT_HD(AMCT_F32) break;

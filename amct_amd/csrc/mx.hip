@@ -391,6 +391,61 @@ __global__ __launch_bounds__(kBlock) void mx_dequant_k(const uint8_t* el, const 
 
 // Complete blocks of U * 256 vectors go to mx_quant_full; the rest (and everything, when the bit-manipulation cast is
 // asked for) to mx_quant_k.  Both give the same codes.
+// complete blocks of U * 256 output vectors: one wave-uniform base per block, 32-bit lane offsets, nothing clamped
+template <int DT, int FMT, int U>
+__global__ __launch_bounds__(kBlock) void mx_dequant_full(const uint8_t* el, const uint8_t* e8, void* y) {
+    constexpr int VEC = Tr<DT>::VEC;
+    constexpr int T = 32 / VEC;
+    constexpr int EB = FMT == kFmtE4M3 ? VEC : VEC / 2;         // element bytes per output vector
+    const uint32_t tid = threadIdx.x;
+    const int64_t v0 = (int64_t)blockIdx.x * (U * kBlock);
+    const uint8_t* eb = el + v0 * EB;
+    const uint8_t* sbp = e8 + v0 / T;
+    char* yb = reinterpret_cast<char*>(y) + v0 * 16;
+    uint32_t w[U][2];
+    uint32_t sb[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint32_t idx = u * kBlock + tid;
+        sb[u] = sbp[idx / T];
+        w[u][1] = 0;
+        if constexpr (EB == 8) {
+            const u2v r = __builtin_nontemporal_load(reinterpret_cast<const u2v*>(eb + idx * 8u));
+            w[u][0] = r.x; w[u][1] = r.y;
+        } else if constexpr (EB == 4) {
+            w[u][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(eb + idx * 4u));
+        } else {
+            w[u][0] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(eb + idx * 2u));
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const float sc = e8m0_to_f32(sb[u]);
+        float out[VEC];
+        if constexpr (FMT == kFmtE4M3) {
+#pragma unroll
+            for (int j = 0; j < VEC / 2; ++j) {
+                const v2f p = (j & 1) ? __builtin_amdgcn_cvt_pk_f32_fp8((int)w[u][j / 2], true)
+                                      : __builtin_amdgcn_cvt_pk_f32_fp8((int)w[u][j / 2], false);
+                out[2 * j] = p.x * sc;
+                out[2 * j + 1] = p.y * sc;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < VEC / 2; ++j) {
+                v2f p;
+                if (j == 0) p = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[u][0], 1.0f, 0);
+                else if (j == 1) p = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[u][0], 1.0f, 1);
+                else if (j == 2) p = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[u][0], 1.0f, 2);
+                else p = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[u][0], 1.0f, 3);
+                out[2 * j] = p.x * sc;
+                out[2 * j + 1] = p.y * sc;
+            }
+        }
+        stg16_nt(yb + (u * kBlock + tid) * 16u, pack16<DT>(out));
+    }
+}
+
 template <int DT, int FMT>
 static int launch_quant(const void* x, uint8_t* el, uint8_t* e8, int64_t nvec, int scale_mode, bool hw, hipStream_t st) {
     constexpr int U = 4;
@@ -417,8 +472,20 @@ static int launch_quant(const void* x, uint8_t* el, uint8_t* e8, int64_t nvec, i
 template <int DT, int FMT>
 static int launch_dequant(const uint8_t* el, const uint8_t* e8, void* y, int64_t nvec, hipStream_t st) {
     constexpr int U = 4;
+    constexpr int VEC = Tr<DT>::VEC;
+    const int64_t full = nvec / ((int64_t)kBlock * U);
+    if (full > 0) {
+        if (full > 0x7FFFFFFF) return AMCT_E_UNSUPPORTED;
+        hipLaunchKernelGGL((mx_dequant_full<DT, FMT, U>), dim3((unsigned)full), dim3(kBlock), 0, st, el, e8, y);
+        const int64_t done = full * kBlock * U;
+        el += done * (FMT == kFmtE4M3 ? VEC : VEC / 2);
+        e8 += done / (32 / VEC);
+        y = reinterpret_cast<char*>(y) + done * 16;
+        nvec -= done;
+        if (nvec == 0) return hip_status();
+    }
     int64_t nb = (nvec + (int64_t)kBlock * U - 1) / ((int64_t)kBlock * U);
-    if (nb > 4096) nb = 4096;                                     // blocks loop over chunks; the table is built once per block
+    if (nb > 4096) nb = 4096;                                     // blocks loop over chunks
     hipLaunchKernelGGL((mx_dequant_k<DT, FMT, U>), dim3((unsigned)nb), dim3(kBlock), 0, st, el, e8, y, nvec);
     return hip_status();
 }
