@@ -130,8 +130,8 @@ __global__ __launch_bounds__(kBlock) void int4_group_pack(PackArgs a) {
 // ---------------------------------------------------------------------------
 // FULL: every block is complete (the group count is a multiple of the groups per block), every lane's vector exists
 // (group length = T * NV vectors) and the tensor is below 2 GiB: addresses are then one wave-uniform 64-bit base per
-// block plus 32-bit lane offsets and nothing is clamped or predicated, which removes about 90 of the 480 vector
-// instructions a wave spends on its 2048 elements.
+// block plus 32-bit lane offsets and nothing is clamped or predicated, which removes 70 of the 560 vector
+// instructions a wave executes for its 2048 elements (counted by the hardware).
 template <int DT, int T, int NV, bool COL, bool FULL = false>
 __global__ __launch_bounds__(kBlock) void int4_group_pack4(PackArgs a) {
     constexpr int U = 4;
