@@ -281,6 +281,34 @@ def w4a16_streams(M, K, group_size, dtype=torch.bfloat16):
 
 
 # --------------------------------------------------------------------------
+# the reference's CPU stand-ins for the two matmul operators, as the timed CPU baseline of bench.py
+# --------------------------------------------------------------------------
+def cpu_standin_quant_matmul_f32(xq, wq_nk, scale, pertoken_scale=None, bias=None, output_dtype=torch.bfloat16):
+    """What the reference's tests run for npu_quant_matmul when no NPU is present
+    (tests/amct_pytorch/mock_torch_npu.py:58-67): operands upcast to fp32, one fp32 F.linear, the per-channel factor
+    (plus the per-token factor, which the stand-in leaves out), cast.  fp32 accumulation is NOT exact at K = 4096,
+    so this is a speed baseline only, never a checker."""
+    out = torch.nn.functional.linear(xq.to(torch.float32), wq_nk.to(torch.float32), None)
+    out *= scale.reshape(1, -1)
+    if pertoken_scale is not None:
+        out *= pertoken_scale.reshape(-1, 1)
+    if bias is not None:
+        out += bias.to(torch.float32)
+    return out.to(output_dtype)
+
+
+def cpu_standin_weight_quant_matmul_f32(x, codes_nk, scale_ng, antioffset_ng, group_size, bias=None, scale_factor=None):
+    """mock_torch_npu.py:33-55 with the group-wise factors the operator takes: x * scale_factor in x's dtype
+    (weight_npu_quant_module.py:113-114), fp32 dequantise, fp32 F.linear, cast to x's dtype.  Speed baseline only."""
+    x2 = x.reshape(-1, x.shape[-1])
+    if scale_factor is not None:
+        x2 = torch.mul(x2, scale_factor.to(x2.dtype))
+    wdq = dequant_weight(codes_nk, scale_ng, antioffset_ng, group_size, torch.float32)
+    out = torch.nn.functional.linear(x2.float(), wdq, None if bias is None else bias.float())
+    return out.to(x.dtype)
+
+
+# --------------------------------------------------------------------------
 # interchange formats of the checkpoint converter
 # (amct_pytorch/experimental/quantization/DeepSeekV3.2/deploy.py)
 # --------------------------------------------------------------------------
