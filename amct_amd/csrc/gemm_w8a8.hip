@@ -1,12 +1,14 @@
 // K6: W8A8 Linear.  out[m,n] = cast(fp32(sum_k xq[m,k]*wq[n,k] + ibias[n]) * s_ch[n] * s_tok[m] + fbias[n])
 // Reference call site: amct_pytorch/deploy_op/npu_quantization_linear.py:100-102.
 //
-// Both operands are K-contiguous, which is the natural operand order of the gfx950 int8 MFMA
-// (v_mfma_i32_32x32x32_i8: lane l supplies 16 consecutive k-bytes of row l%32, k-half l/32).
+// Both operands are K-contiguous, which is the natural operand order of the gfx950 int8 MFMAs
+// (v_mfma_i32_32x32x32_i8: lane l supplies 16 consecutive k-bytes of row l%32, k-half l/32;
+//  v_mfma_i32_16x16x64_i8: row l%16, k-quarter l/16).
 //   large tiles   : 256x256 block tile, 8 waves of 128x64, LDS stages of 128 bytes of K filled by direct
 //                   global->LDS loads, fragment reads software-pipelined against the MFMAs in a pinned
 //                   issue order; when the tile count does not fill the CUs evenly, one launch mixes in
-//                   256x192 tiles.
+//                   256x192 tiles.  With K a multiple of 128 the 16x16x64 form runs (w8a8_dma_body16), else the
+//                   32x32x32 form with 64-byte rows (w8a8_dma_body).
 //   tile kernel   : 128x128 block tile, 4 waves of 64x64, BK = 128 bytes, two register stages of
 //                   prefetch (shapes the large-tile kernel does not take).
 //   decode kernels: M <= 16: activations staged once per block in LDS, the weight streamed once straight
@@ -464,6 +466,242 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
     }
 }
 
+template <int ODT, int WM, int WN, int TI, int TJ, int STAGES>
+AMCT_DEV void w8a8_dma_body16(const W8A8Args& a, int8_t* smem, const int64_t m0, const int64_t n0) {
+    constexpr int LK = 128;
+    using Sh = DmaTile<WM, WN, TI, TJ, STAGES, LK>;
+    constexpr int kLM = Sh::kLM, kLN = Sh::kLN, kRP = Sh::kRP, kNA = Sh::kNA, kNB = Sh::kNB, kPPW = Sh::kPPW;
+    constexpr int kLStageBytes = Sh::kLStageBytes, kWaves = Sh::kWaves, kLW = Sh::kLW;
+    constexpr int kCH = LK / 16;                                    // 16-byte chunks per row
+    constexpr int kKS = LK / 32;                                    // MFMA k-slices per stage
+    static_assert(LK == 64 || LK == 128, "row length");
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const int nsteps = (int)(a.K / LK);
+    const int last = nsteps - 1;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t*)smem;
+    // Rows are LK bytes, unpadded (a direct-to-LDS load writes the 64 lanes' 16-byte pieces to 1024 contiguous
+    // bytes); 16-byte chunk c of row r lives at chunk position c ^ swz(r), which spreads the 16 rows that one
+    // phase of a 16-byte fragment read touches over all banks.
+    auto swz = [](int r) { return LK == 64 ? (r >> 2) & 3 : (r >> 1) & 7; };
+
+    // this wave's 1 KiB pieces of a stage: kNA pieces of A rows, then kNB pieces of B rows.  A load is addressed
+    // as (operand base + LK * step) in SGPRs plus a constant 32-bit byte offset per lane and piece (the host
+    // admits only operands below 4 GiB to this kernel).
+    const bool loader = wave >= kWaves - kLW;                       // the last kLW waves: one per SIMD when kLW = 4
+    const int lw = loader ? wave - (kWaves - kLW) : 0;
+    uint32_t goff[kPPW];
+    {
+        const int rin = lane / kCH;                                 // row inside the piece
+        const int pc = lane % kCH;                                  // physical chunk this lane fills
+#pragma unroll
+        for (int j = 0; j < kPPW; ++j) {
+            int64_t r;
+            int lr;                                                 // row inside the operand's LDS tile
+            if (j < kNA) {
+                lr = (lw * kNA + j) * kRP + rin;
+                r = m0 + lr < a.M ? m0 + lr : a.M - 1;
+            } else {
+                // a wave beyond the last piece fetches the last piece again: same bytes to the same place
+                const int pb = lw * kNB + (j - kNA) < kLN / kRP ? lw * kNB + (j - kNA) : kLN / kRP - 1;
+                lr = pb * kRP + rin;
+                r = n0 + lr < a.N ? n0 + lr : a.N - 1;
+            }
+            goff[j] = (uint32_t)(r * a.K + (pc ^ swz(lr)) * 16);
+        }
+    }
+    auto dma_one = [&](int stg, int step, int j) {
+        if (j < kNA) {
+            dma16s(lds0 + stg * kLStageBytes + (lw * kNA + j) * 1024, a.xq + (int64_t)step * LK, goff[j]);
+        } else {
+            const int pb = lw * kNB + (j - kNA) < kLN / kRP ? lw * kNB + (j - kNA) : kLN / kRP - 1;
+            dma16s(lds0 + stg * kLStageBytes + kLM * LK + pb * 1024, a.wq + (int64_t)step * LK, goff[j]);
+        }
+    };
+    auto dma_stage = [&](int stage, int step) {
+        if (loader) {
+#pragma unroll
+            for (int j = 0; j < kPPW; ++j) dma_one(stage, step, j);
+        }
+    };
+
+    // A stage holds two k-slices of 64 bytes; each is done in two units (the upper and the lower half of the wave's
+    // 16-row tiles), so a stage is four units u = 2 * slice + half, as many as the 32x32x32 form has k-slices.
+    // Fragment of unit u: lane reads row (tile base + lane % 16), logical chunk 4 * slice + lane / 16.
+    constexpr int TA = TI;                                          // 16-row tiles per unit
+    constexpr int TB = 2 * TJ;                                      // 16-column tiles of the wave
+    int offA[4], offB[2];
+    {
+        const int r = lane & 15;
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            offA[u] = (wm * 32 * TI + (u & 1) * 16 * TA + r) * LK + ((4 * (u >> 1) + (lane >> 4)) ^ swz(r)) * 16;
+#pragma unroll
+        for (int sl = 0; sl < 2; ++sl)
+            offB[sl] = kLM * LK + (wn * 32 * TJ + r) * LK + ((4 * sl + (lane >> 4)) ^ swz(r)) * 16;
+    }
+
+    v4i acc[2 * TI][TB];
+#pragma unroll
+    for (int i = 0; i < 2 * TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TB; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s) dma_stage(s, s < last ? s : last);
+
+    // The schedule of w8a8_dma_body with units in the place of its k-slices: while the MFMAs of a unit run, the fragments
+    // of the next one are read (TA row fragments, plus the TB column fragments when the next unit starts a slice); before
+    // the last unit of a stage the waves meet, the refill loads follow, and the last unit reads the first fragments of the
+    // next stage.  Row fragments alternate between two buffers per unit, column fragments per slice.
+    constexpr int kNM = TA * TB;                                    // MFMAs per unit
+    constexpr int kNRmax = TA + TB;
+    constexpr int kGap = kNM / kNRmax;                              // one fragment read behind every kGap-th MFMA
+    static_assert(kGap >= 1, "fewer MFMAs than fragment reads per unit");
+    v4i fa[2][TA], fb[2][TB];
+    auto read_one = [&](int stg, int u, int q) {                    // u, q: compile-time in every use
+        const int8_t* st = smem + stg * kLStageBytes;
+        if (q < TA) fa[u & 1][q] = *reinterpret_cast<const v4i*>(st + offA[u] + q * 16 * LK);
+        else if ((u & 1) == 0 && q < TA + TB) fb[(u >> 1) & 1][q - TA] = *reinterpret_cast<const v4i*>(st + offB[u >> 1] + (q - TA) * 16 * LK);
+    };
+    auto mfma_one = [&](int u, int m) {
+        const int i = m / TB, j = m % TB;
+        acc[(u & 1) * TA + i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[u & 1][i], fb[(u >> 1) & 1][j], acc[(u & 1) * TA + i][j], 0, 0, 0);
+    };
+    wait_dma_lds<(STAGES - 2) * kPPW>();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    dma_stage(STAGES - 1, STAGES - 1 < last ? STAGES - 1 : last);
+#pragma unroll
+    for (int q = 0; q < kNRmax; ++q) read_one(0, 0, q);
+    int stage = 0;
+    for (int step = 0; step < nsteps; ++step) {
+        const int next = stage + 1 == STAGES ? 0 : stage + 1;
+        const int refill = step + STAGES < last ? step + STAGES : last;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < 3; ++u) {
+#pragma unroll
+            for (int m = 0; m < kNM; ++m) {
+                mfma_one(u, m);
+                __builtin_amdgcn_sched_barrier(0);
+                if (m % kGap == 0 && m / kGap < kNRmax) {
+                    read_one(stage, u + 1, m / kGap);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+        wait_dma_lds<(STAGES - 2) * kPPW>();
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        dma_stage(stage, refill);                                   // loading waves only
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int m = 0; m < kNM; ++m) {
+            mfma_one(3, m);
+            __builtin_amdgcn_sched_barrier(0);
+            if (m % kGap == 0 && m / kGap < kNRmax) {
+                read_one(next, 0, m / kGap);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        stage = next;
+    }
+    // all loads landed and every wave is done with the stages before LDS is reused
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+
+    // epilogue: fp32(acc + ibias) * s_ch * s_tok + fbias, narrowed, transposed through a per-wave LDS
+    // patch of 32 rows x 32*TJ columns, stored as 16-byte pieces of full rows.  Branch-free per element:
+    // absent factors are replaced by their neutral elements (x * 1.0f and x + (-0.0f) return x bit for bit),
+    // the row factors of the wave come from a small LDS table, every LDS address is base + immediate.
+    constexpr int ES = (ODT == AMCT_F32) ? 4 : 2;                   // bytes per output element
+    constexpr int kPW = 32 * TJ;                                   // patch width in columns
+    constexpr int kPatchRow = kPW * ES + 16;                       // padded patch row
+    constexpr int CPR = kPW * ES / 16;                             // 16-byte chunks per patch row
+    constexpr int kTokOff = 16384 - 512;                           // 32*TI <= 128 row factors behind the patch
+    static_assert(32 * kPatchRow <= kTokOff && (32 * CPR) % 64 == 0 && TI <= 4,
+                  "patch and row factors must fit the wave's 16 KiB; the patch must split into wave-wide reads");
+    int8_t* patch = smem + wave * 16384;
+    float* tokl = reinterpret_cast<float*>(patch + kTokOff);
+    float sc[TB], fb2[TB];
+    int32_t ib[TB];
+#pragma unroll
+    for (int j = 0; j < TB; ++j) {
+        const int64_t n = n0 + wn * kPW + j * 16 + (lane & 15);
+        const int64_t nc = n < a.N ? n : a.N - 1;
+        sc[j] = a.s_ch[nc];
+        ib[j] = a.bias_kind == 1 ? reinterpret_cast<const int32_t*>(a.bias)[nc] : 0;
+        fb2[j] = a.bias_kind == 2 ? reinterpret_cast<const float*>(a.bias)[nc] : -0.0f;
+    }
+#pragma unroll
+    for (int t = lane; t < 32 * TI; t += 64) {
+        const int64_t m = m0 + wm * 32 * TI + t;
+        tokl[t] = a.s_tok ? a.s_tok[m < a.M ? m : a.M - 1] : 1.0f;
+    }
+    // accumulator tile (t, j), register r: row 16 t + 4 (lane / 16) + r, column 16 j + lane % 16 of the wave tile
+    if (a.acc_out) {                                                // accumulators on request (tests): plain stores
+#pragma unroll
+        for (int t = 0; t < 2 * TI; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int j = 0; j < TB; ++j) {
+                    const int64_t m = m0 + wm * 32 * TI + t * 16 + 4 * (lane >> 4) + r;
+                    const int64_t n = n0 + wn * kPW + j * 16 + (lane & 15);
+                    if (m < a.M && n < a.N) a.acc_out[m * a.N + n] = acc[t][j][r] + ib[j];
+                }
+    }
+    const int q4 = 4 * (lane >> 4);
+    int8_t* wbase = patch + q4 * kPatchRow + (lane & 15) * ES;      // this lane's element of patch row q4
+    const int8_t* rbase = patch + (lane / CPR) * kPatchRow + (lane % CPR) * 16;
+    constexpr int RPI = 64 / CPR;                                   // patch rows per wave-wide read when CPR divides 64
+#pragma unroll
+    for (int i = 0; i < TI; ++i) {                                  // 32 rows of the wave tile per pass: tiles 2 i and 2 i + 1
+        const int64_t mbase = m0 + wm * 32 * TI + i * 32;
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+            const float4 t4 = *reinterpret_cast<const float4*>(tokl + i * 32 + 16 * hh + q4);
+            const float tks[4] = {t4.x, t4.y, t4.z, t4.w};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+#pragma unroll
+                for (int j = 0; j < TB; ++j) {
+                    float f = (float)(acc[2 * i + hh][j][r] + ib[j]) * sc[j];
+                    f = f * tks[r];
+                    f = f + fb2[j];
+                    int8_t* dst = wbase + (16 * hh + r) * kPatchRow + j * 16 * ES;
+                    if constexpr (ODT == AMCT_F32) *reinterpret_cast<float*>(dst) = f;
+                    else if constexpr (ODT == AMCT_BF16) *reinterpret_cast<uint16_t*>(dst) = (uint16_t)f32_to_bf16_bits(f);
+                    else *reinterpret_cast<uint16_t*>(dst) = (uint16_t)f32_to_f16_bits(f);
+                }
+            }
+        }
+        // LDS operations of one wave complete in order: the reads below see the writes above
+#pragma unroll
+        for (int it = 0; it < 32 * CPR / 64; ++it) {
+            int prow, chunk;
+            uint4 v;
+            if constexpr (64 % CPR == 0) {
+                prow = it * RPI + lane / CPR;
+                chunk = lane % CPR;
+                v = *reinterpret_cast<const uint4*>(rbase + it * RPI * kPatchRow);
+            } else {
+                const int idx = it * 64 + lane;                    // 16-byte chunk of the patch, row-major
+                prow = idx / CPR;
+                chunk = idx % CPR;
+                v = *reinterpret_cast<const uint4*>(patch + prow * kPatchRow + chunk * 16);
+            }
+            const int64_t m = mbase + prow;
+            const int64_t n = n0 + wn * kPW + chunk * (16 / ES);
+            if (m < a.M && n < a.N) stg16_nt(reinterpret_cast<char*>(a.out) + (m * a.N + n) * ES, v);
+        }
+    }
+}
+
 template <int ODT, int WM, int WN, int STAGES, int LK>
 __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void w8a8_tile_dma(W8A8Args a) {
     using Sh = DmaTile<WM, WN, 4, 2, STAGES, LK>;
@@ -483,6 +721,29 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int s = b - p.big;
         w8a8_dma_body<ODT, 4, 2, 2, 3, STAGES, LK>(a, smem, (int64_t)(s / p.nsmall) * 256,
                                                    (int64_t)p.nbig * 256 + (int64_t)(s % p.nsmall) * 192);
+    }
+}
+
+// the same two launches on v_mfma_i32_16x16x64_i8 (K a multiple of 128)
+template <int ODT>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void w8a8_tile_dma16(W8A8Args a) {
+    using Sh = DmaTile<2, 4, 4, 2, 2, 128>;
+    __shared__ __attribute__((aligned(1024))) int8_t smem[Sh::kSmem];
+    w8a8_dma_body16<ODT, 2, 4, 4, 2, 2>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
+}
+
+template <int ODT>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void w8a8_tile_mix16(W8A8Args a, MixPlan p) {
+    using Big = DmaTile<2, 4, 4, 2, 2, 128>;
+    using Small = DmaTile<4, 2, 2, 3, 2, 128>;
+    __shared__ __attribute__((aligned(1024))) int8_t smem[Big::kSmem > Small::kSmem ? Big::kSmem : Small::kSmem];
+    const int b = blockIdx.x;
+    if (b < p.big) {
+        w8a8_dma_body16<ODT, 2, 4, 4, 2, 2>(a, smem, (int64_t)(b / p.nbig) * 256, (int64_t)(b % p.nbig) * 256);
+    } else {
+        const int s = b - p.big;
+        w8a8_dma_body16<ODT, 4, 2, 2, 3, 2>(a, smem, (int64_t)(s / p.nsmall) * 256,
+                                            (int64_t)p.nbig * 256 + (int64_t)(s % p.nsmall) * 192);
     }
 }
 
@@ -835,14 +1096,20 @@ extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s
         // 128-byte LDS rows and 2 stages when K allows (whole cache lines per load, one barrier per 128 bytes of K:
         // 7 % faster), else 64-byte rows and 4 stages
         const bool wide = K % 128 == 0;
+        // Under the part's power limit v_mfma_i32_16x16x64_i8 sustains more than v_mfma_i32_32x32x32_i8 on non-constant
+        // operands (register-only loops: 3.74 against 3.24 POP/s; with the large tile's fragment reads interleaved 3.8
+        // against 3.4), at equal LDS traffic per wave tile: 98 against 105 us on M = 2048, N = 14336, K = 4096.
+        constexpr bool mi16 = true;
 #define AMCT_LAUNCH_DMA(ODT)                                                                                        \
     {                                                                                                               \
         if (plan.nbig >= 0) {                                                                                       \
             const dim3 g1((unsigned)(plan.big + plan.mtiles * plan.nsmall));                                        \
-            if (wide) hipLaunchKernelGGL((w8a8_tile_mix<ODT, 2, 128>), g1, dim3(512), 0, st, a, plan);              \
+            if (wide && mi16) hipLaunchKernelGGL((w8a8_tile_mix16<ODT>), g1, dim3(512), 0, st, a, plan);            \
+            else if (wide) hipLaunchKernelGGL((w8a8_tile_mix<ODT, 2, 128>), g1, dim3(512), 0, st, a, plan);         \
             else hipLaunchKernelGGL((w8a8_tile_mix<ODT, 4, 64>), g1, dim3(512), 0, st, a, plan);                    \
         } else {                                                                                                    \
-            if (wide) hipLaunchKernelGGL((w8a8_tile_dma<ODT, 2, 4, 2, 128>), grid, dim3(512), 0, st, a);            \
+            if (wide && mi16) hipLaunchKernelGGL((w8a8_tile_dma16<ODT>), grid, dim3(512), 0, st, a);                \
+            else if (wide) hipLaunchKernelGGL((w8a8_tile_dma<ODT, 2, 4, 2, 128>), grid, dim3(512), 0, st, a);       \
             else hipLaunchKernelGGL((w8a8_tile_dma<ODT, 2, 4, 4, 64>), grid, dim3(512), 0, st, a);                  \
         }                                                                                                           \
     }
