@@ -713,12 +713,288 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
     }
 }
 
+template <bool SF16, int WM, int WN, int TI, int TJ, int STAGES, int SB = STAGES>
+AMCT_DEV void w4a16_wide_body16(const W4A16Args& a, uint8_t* smem, const int64_t m0, const int64_t n0) {
+    using Sh = WideTile<WM, WN, TI, TJ, STAGES, SB>;
+    constexpr int kABytes = Sh::kABytes, kBBytes = Sh::kBBytes, kBBase = Sh::kBBase;
+    constexpr int kWaves = Sh::kWaves, kLW = Sh::kLW, kNA = Sh::kNA;
+    // v_mfma_f32_16x16x32_bf16: a stage (64 elements of K) is two k-slices of 32; each is done in two units (the upper
+    // and the lower half of the wave's 16-row tiles), so a stage is four units u = 2 * slice + half, as many as the
+    // 32x32x16 form has k-slices, and the schedule below is that form's with units in the place of slices.
+    constexpr int TA = TI;                                         // 16-row tiles per unit
+    constexpr int TB = 2 * TJ;                                     // 16-column tiles of the wave
+    constexpr int kNM = TA * TB;                                   // MFMAs per unit
+    constexpr int kDqGap = kNM / (4 * (Sh::kBC / 2));              // a dequantisation piece behind every kDqGap-th MFMA
+    static_assert(kDqGap >= 1 && Sh::kBC >= 2, "a dequantising unit takes kBC / 2 chunks of four pieces");
+    static_assert(TA >= 2 && TA * 2 >= TB, "the unit must have room for its fragment reads");
+    static_assert((STAGES == 2 || STAGES == 3) && (SB == 2 || SB == 3) && SB <= STAGES, "2 or 3 stages");
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const int nsteps = (int)(a.K / kWK);
+    const int last = nsteps - 1;
+    const uint32_t G = (uint32_t)(a.K / a.group);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
+    auto swz = [](int r) { return (r >> 1) & 7; };
+
+    // activation pieces (8 rows x 128 B) of the loading waves
+    const bool loader = wave >= kWaves - kLW;
+    const int lw = loader ? wave - (kWaves - kLW) : 0;
+    uint32_t goff[kNA];
+    {
+        const int rin = lane >> 3, pc = lane & 7;
+#pragma unroll
+        for (int j = 0; j < kNA; ++j) {
+            const int lr = (lw * kNA + j) * 8 + rin;
+            const int64_t r = m0 + lr < a.M ? m0 + lr : a.M - 1;
+            goff[j] = (uint32_t)((r * a.K + (pc ^ swz(lr)) * 8) * 2);
+        }
+    }
+    auto dma_a = [&](int stg, int step) {
+        if (loader) {
+            const int st = step < last ? step : last;
+#pragma unroll
+            for (int j = 0; j < kNA; ++j)
+                dma16s(lds0 + stg * kABytes + (lw * kNA + j) * 1024, a.x + (int64_t)st * kWK, goff[j]);
+        }
+    };
+    // weight row of this thread: row tid/kQ of the tile, 8*kBC weights (4*kBC bytes) per step, which part from tid%kQ
+    constexpr int kQ = Sh::kQ, kBC = Sh::kBC;
+    const int brow = tid / kQ, bpart = tid % kQ;
+    const int64_t wrow = (n0 + brow < a.N) ? n0 + brow : a.N - 1;
+    const uint32_t woff = (uint32_t)(wrow * (a.K / 2) + bpart * (4 * kBC));
+    const uint32_t soff = (uint32_t)(wrow * G * 2), zoff = (uint32_t)(wrow * G);
+    int bdst[kBC];
+#pragma unroll
+    for (int c = 0; c < kBC; ++c) bdst[c] = kBBase + brow * kWRow + ((kBC * bpart + c) ^ swz(brow)) * 16;
+
+    typename std::conditional<kBC == 4, u4v, u2v>::type wreg[2];
+    uint32_t sreg[2], zreg[2];
+    auto issue_b = [&](int slot, int step) {                       // the weight loads of K-step `step`
+        const int st = step < last ? step : last;
+        const uint32_t k = (uint32_t)st * kWK;
+        const uint32_t gi = __umulhi(k, a.group_magic);             // k / group (k, group < 2^16); group % 64 == 0
+        gload16s(wreg[slot], a.wq + k / 2, woff);
+        gload_u16s(sreg[slot], reinterpret_cast<const uint8_t*>(a.scales) + gi * 2, soff);
+        gload_u8s(zreg[slot], a.zeros + gi, zoff);
+    };
+    float sc = 0.f, nzs = 0.f;
+    auto factors = [&](int slot) {
+        sc = SF16 ? f16_bits_to_f32(sreg[slot]) : bf16_bits_to_f32(sreg[slot]);
+        nzs = -((float)zreg[slot] * sc);
+    };
+    auto write_b = [&](int slot, int stg, int c) {                 // dequantise 8 weights into LDS
+        *reinterpret_cast<uint4*>(smem + stg * kBBytes + bdst[c]) = dequant8(wreg[slot][c], sc, nzs);
+    };
+    // Wait until the weight loads of the previous iteration and the activation loads issued STAGES-1 iterations ago
+    // have landed and this wave's LDS operations are done.  An iteration issues its 3 weight loads in the middle of the
+    // step, as soon as their register slot has been dequantised (when the memory pipeline is idle: issued right after
+    // the barrier they queued behind the loading waves' burst and both waves of a SIMD stood still), and, in a loading
+    // wave, kNA direct-to-LDS loads right after the barrier.  The youngest weight loads may stay in flight, and with three
+    // stages the youngest activation loads too, hence the wave-uniform choice of the count.  The slot's registers are tied to a statement behind the wait so that
+    // their uses (and any copies the register allocator makes) stay behind it.
+    auto wait_older = [&]() {
+        if constexpr (STAGES == 2) {
+            wait_vm<3>();
+        } else {
+            if (loader) wait_vm<kNA + 3>();
+            else wait_vm<3>();
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+#define AMCT_TIE_SLOT(slot) asm volatile("" : "+v"(wreg[slot]), "+v"(sreg[slot]), "+v"(zreg[slot]) : : "memory")
+
+    // fragment of unit u: lane reads row (tile base + lane % 16), logical chunk 4 * slice + lane / 16
+    int offA[4], offB[2];
+    {
+        const int r = lane & 15;
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            offA[u] = (wm * 32 * TI + (u & 1) * 16 * TA + r) * kWRow + ((4 * (u >> 1) + (lane >> 4)) ^ swz(r)) * 16;
+#pragma unroll
+        for (int sl = 0; sl < 2; ++sl)
+            offB[sl] = kBBase + (wn * 32 * TJ + r) * kWRow + ((4 * sl + (lane >> 4)) ^ swz(r)) * 16;
+    }
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    v4f acc[2 * TI][TB];
+#pragma unroll
+    for (int i = 0; i < 2 * TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TB; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    // Row fragments live in ONE set of registers: a unit walks its MFMAs row tile by row tile, and the fragment of a row
+    // tile is loaded again (for the next unit) right behind the last MFMA that used it.  Column fragments are used by
+    // every row tile of both units of a slice, so they alternate between two sets per slice.
+    v8bf fa[TA], fb[2][TB];
+    auto read_a = [&](int sa, int u, int i) {                       // u, i: compile-time in every use
+        fa[i] = *reinterpret_cast<const v8bf*>(smem + sa * kABytes + offA[u] + i * 16 * kWRow);
+    };
+    auto read_b = [&](int sb, int sl, int j) {
+        fb[sl & 1][j] = *reinterpret_cast<const v8bf*>(smem + sb * kBBytes + offB[sl] + j * 16 * kWRow);
+    };
+    auto mfma_one = [&](int u, int m) {
+        const int i = m / TB, j = m % TB;
+        acc[(u & 1) * TA + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fb[(u >> 1) & 1][j], acc[(u & 1) * TA + i][j], 0, 0, 0);
+    };
+    // dequantisation of 8 weights in four pieces of two, so that the pieces can sit between MFMAs
+    uint32_t dq_lo = 0, dq_hi = 0, dq_o[4];
+    auto dq_piece = [&](int slot, int c, int bb) {                  // c, bb: compile-time
+        if (bb == 0) {
+            dq_lo = wreg[slot][c] & 0x0F0F0F0Fu;                   // elements 0, 2, 4, 6 in bytes 0 .. 3
+            dq_hi = (wreg[slot][c] >> 4) & 0x0F0F0F0Fu;            // elements 1, 3, 5, 7
+            asm("" : "+v"(dq_lo));                                  // keeps the byte conversions below as v_cvt_f32_ubyteN
+            asm("" : "+v"(dq_hi));
+        }
+        const float e0 = (float)((dq_lo >> (8 * bb)) & 0xFFu);
+        const float e1 = (float)((dq_hi >> (8 * bb)) & 0xFFu);
+        dq_o[bb] = pack_bf16x2(__builtin_fmaf(e0, sc, nzs), __builtin_fmaf(e1, sc, nzs));
+    };
+    auto dq_write = [&](int stg, int c) {
+        *reinterpret_cast<uint4*>(smem + stg * kBBytes + bdst[c]) = make_uint4(dq_o[0], dq_o[1], dq_o[2], dq_o[3]);
+    };
+
+    // prologue: B(0), B(1) and A(0 .. STAGES-2); once B(0) is dequantised into stage 0 its slot takes B(2), and
+    // A(STAGES-1) follows (weights first, as in the loop)
+    issue_b(0, 0);
+    issue_b(1, 1);
+#pragma unroll
+    for (int j = 0; j < STAGES - 1; ++j) dma_a(j, j);
+    wait_vm<0>();
+    AMCT_TIE_SLOT(0);
+    AMCT_TIE_SLOT(1);
+    factors(0);
+#pragma unroll
+    for (int c = 0; c < kBC; ++c) write_b(0, 0, c);
+    issue_b(0, 2);
+    dma_a(STAGES - 1, STAGES - 1);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int q = 0; q < TA; ++q) read_a(0, 0, q);
+#pragma unroll
+    for (int q = 0; q < TB; ++q) read_b(0, 0, q);
+
+    // iteration s (LDS stage cur, the next one nxt; register slot SL holds B(s+1), landed; the other slot B(s+2)):
+    //   k-slices 0, 1 : MFMAs, fragment reads of the next slice, dequantisation of B(s+1) into stage nxt
+    //   loads         : B(s+3) into slot SL (its old content is in LDS now)
+    //   k-slice 2     : MFMAs, fragment reads of slice 3
+    //   wait (A(s+1) and B(s+2) have landed; own LDS operations done), barrier: stage cur is free, nxt complete
+    //   loads         : A(s+STAGES) into stage cur (loading waves)
+    //   k-slice 3     : MFMAs, fragment reads of slice 0 of stage nxt
+    int cur = 0, nxt = 1;                                           // activation stages
+    int curb = 0, nxtb = 1;                                         // weight stages
+    // one unit, every instruction in its place: MFMA m; behind the last MFMA of a row tile the reload of its fragment for
+    // unit UN (stage SA); when UN starts a slice, its column fragments (stage SBR) behind the second MFMA of each row
+    // tile; in a dequantising unit a piece of two weights behind every second MFMA and the 16-byte LDS write of a chunk
+    // behind its last piece
+#define AMCT_WUNIT(U, UN, SA, SBR, DQ, SL)                                             \
+    {                                                                                  \
+        _Pragma("unroll") for (int m_ = 0; m_ < kNM; ++m_) {                           \
+            mfma_one((U), m_);                                                         \
+            __builtin_amdgcn_sched_barrier(0);                                         \
+            if (m_ % TB == TB - 1) {                                                   \
+                read_a((SA), (UN), m_ / TB);                                           \
+                __builtin_amdgcn_sched_barrier(0);                                     \
+            }                                                                          \
+            if (((UN) & 1) == 0 && m_ % TA == 1 && m_ / TA < TB) {                     \
+                read_b((SBR), (UN) >> 1, m_ / TA);                                     \
+                __builtin_amdgcn_sched_barrier(0);                                     \
+            }                                                                          \
+            if ((DQ) && m_ % kDqGap == 0 && m_ / kDqGap < 4 * (kBC / 2)) {             \
+                dq_piece((SL), (kBC / 2) * (U) + (m_ / kDqGap) / 4, (m_ / kDqGap) % 4); \
+                __builtin_amdgcn_sched_barrier(0);                                     \
+                if ((m_ / kDqGap) % 4 == 3) {                                          \
+                    dq_write(nxtb, (kBC / 2) * (U) + (m_ / kDqGap) / 4);               \
+                    __builtin_amdgcn_sched_barrier(0);                                 \
+                }                                                                      \
+            }                                                                          \
+        }                                                                              \
+    }
+#define AMCT_WITER(SL, step)                                                           \
+    {                                                                                  \
+        AMCT_TIE_SLOT(SL);                                                             \
+        factors(SL);                                                                   \
+        __builtin_amdgcn_sched_barrier(0);                                             \
+        AMCT_WUNIT(0, 1, cur, curb, true, SL)                                          \
+        AMCT_WUNIT(1, 2, cur, curb, true, SL)                                          \
+        issue_b(SL, (step) + 3);                                                       \
+        __builtin_amdgcn_sched_barrier(0);                                             \
+        AMCT_WUNIT(2, 3, cur, curb, false, SL)                                         \
+        wait_older();                                                                  \
+        __builtin_amdgcn_s_barrier();                                                  \
+        asm volatile("" ::: "memory");                                                 \
+        __builtin_amdgcn_sched_barrier(0);                                             \
+        dma_a(cur, (step) + STAGES);                                                   \
+        __builtin_amdgcn_sched_barrier(0);                                             \
+        AMCT_WUNIT(3, 0, nxt, nxtb, false, SL)                                         \
+        cur = nxt;                                                                     \
+        nxt = nxt + 1 == STAGES ? 0 : nxt + 1;                                         \
+        curb = nxtb;                                                                   \
+        nxtb = nxtb + 1 == SB ? 0 : nxtb + 1;                                          \
+    }
+    for (int step = 0; step < nsteps; step += 2) {                  // K % 128 == 0: an even number of steps
+        AMCT_WITER(1, step)
+        AMCT_WITER(0, step + 1)
+    }
+#undef AMCT_WITER
+#undef AMCT_WUNIT
+#undef AMCT_TIE_SLOT
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+
+    // epilogue: + bias (or + (-0.0f), which returns the value bit for bit), narrow to bf16, transpose through a
+    // per-wave LDS patch of 32 rows x 32*TJ columns, 16-byte stores of full rows
+    constexpr int kPW = 32 * TJ;                                   // patch width in columns
+    constexpr int kPatchRow = kPW * 2 + 16;
+    constexpr int CPR = kPW * 2 / 16;                              // 16-byte chunks per patch row
+    static_assert(32 * kPatchRow <= 16384 && (32 * CPR) % 64 == 0, "patch");
+    uint8_t* patch = smem + wave * 16384;
+    // accumulator tile (t, j), register r: row 16 t + 4 (lane / 16) + r, column 16 j + lane % 16 of the wave tile
+    float bs[TB];
+#pragma unroll
+    for (int j = 0; j < TB; ++j) {
+        const int64_t n = n0 + wn * kPW + j * 16 + (lane & 15);
+        bs[j] = a.bias ? a.bias[n < a.N ? n : a.N - 1] : -0.0f;
+    }
+    uint8_t* wbase = patch + 4 * (lane >> 4) * kPatchRow + (lane & 15) * 2;
+#pragma unroll
+    for (int i = 0; i < TI; ++i) {                                  // 32 rows of the wave tile per pass: tiles 2 i and 2 i + 1
+        const int64_t mbase = m0 + wm * 32 * TI + i * 32;
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int j = 0; j < TB; ++j)
+                    *reinterpret_cast<uint16_t*>(wbase + (16 * hh + r) * kPatchRow + j * 32) =
+                        (uint16_t)f32_to_bf16_bits(acc[2 * i + hh][j][r] + bs[j]);
+#pragma unroll
+        for (int it = 0; it < 32 * CPR / 64; ++it) {
+            const int idx = it * 64 + lane;                        // 16-byte chunk of the patch, row-major
+            const int prow = idx / CPR, chunk = idx % CPR;
+            const uint4 v = *reinterpret_cast<const uint4*>(patch + prow * kPatchRow + chunk * 16);
+            const int64_t m = mbase + prow;
+            const int64_t n = n0 + wn * kPW + chunk * 8;
+            if (m < a.M && n < a.N) stg16_nt(reinterpret_cast<char*>(a.out) + (m * a.N + n) * 2, v);
+        }
+    }
+}
+
 // blockIdx.x: column tile, blockIdx.y: row tile
 template <bool SF16, int WM, int WN, int TI, int TJ, int STAGES, int SB = STAGES>
 __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM * WN / 4, WM * WN / 4))) void w4a16_tile_wide(W4A16Args a) {
     using Sh = WideTile<WM, WN, TI, TJ, STAGES, SB>;
     __shared__ __attribute__((aligned(1024))) uint8_t smem[Sh::kSmem];
     w4a16_wide_body<SF16, WM, WN, TI, TJ, STAGES, SB>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
+}
+
+template <bool SF16, int WM, int WN, int TI, int TJ, int STAGES, int SB = STAGES>
+__global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM * WN / 4, WM * WN / 4))) void w4a16_tile_wide16(W4A16Args a) {
+    using Sh = WideTile<WM, WN, TI, TJ, STAGES, SB>;
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[Sh::kSmem];
+    w4a16_wide_body16<SF16, WM, WN, TI, TJ, STAGES, SB>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
 }
 
 // ---------------------------------------------------------------------------
@@ -1568,6 +1844,10 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
             else if (cus > 0 && mt * nt128 <= cus) shape = 1;
             else if (cus > 0 && (mt * nt256 <= cus || M < 256)) shape = 2;
             if (mt > 65535) return AMCT_E_UNSUPPORTED;
+            // 256x256 tiles run on v_mfma_f32_16x16x32_bf16: under the part's power limit it sustains more than the
+            // 32x32x16 form on non-constant operands (register-only loops: 1.81 - 1.97 against 1.67 - 1.81 PFLOP/s) at equal
+            // LDS traffic per wave tile: 217.5 against 225.2 us on M = 2048, N = 14336, K = 4096 (pre-pass included).
+            constexpr bool mi16 = true;
 #define AMCT_LAUNCH_WIDE(SF)                                                                                           \
     {                                                                                                                  \
         if (shape == 3 && K % 256 == 0 && G <= kSpecMaxG) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3, 1, 1>), dim3((unsigned)nt64, 1), dim3(kSpecThreads), 0, st, a); \
@@ -1578,6 +1858,7 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
         else if (shape == 1) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 2, 2, 3>), dim3((unsigned)nt128, (unsigned)mt), dim3(256), 0, st, a); \
         else if (shape == 2 && M > 256 && (M + 255) / 256 * nt128 <= cus) hipLaunchKernelGGL((w4a16_tile_wide<SF, 4, 2, 2, 2, 3>), dim3((unsigned)nt128, (unsigned)((M + 255) / 256)), dim3(512), 0, st, a); \
         else if (shape == 2) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 4, 2, 2, 3>), dim3((unsigned)nt256, (unsigned)mt), dim3(512), 0, st, a); \
+        else if (mi16) hipLaunchKernelGGL((w4a16_tile_wide16<SF, 2, 4, 4, 2, 2>), grid, dim3(kQThreads), 0, st, a);    \
         else hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 4, 4, 2, 2>), grid, dim3(kQThreads), 0, st, a);                \
     }
             if (scale_dtype == AMCT_F16) AMCT_LAUNCH_WIDE(true)
