@@ -24,11 +24,37 @@ FLAGS = [
 ]
 
 
+# Kernels whose s_waitcnt vmcnt values are counted by hand (inline-asm loads with a fixed number of operations per
+# iteration): a register spill would add scratch loads and stores to that count and make them read registers before
+# their data has landed.  The build refuses such a kernel instead of shipping it.
+NO_SPILL = ("w8a8_tile_", "w4a16_tile_")
+
+
+def _spilling_kernels(remarks):
+    """Names of NO_SPILL kernels for which the compiler reports spilled vector registers or scratch memory."""
+    bad, name = [], None
+    for line in remarks.splitlines():
+        if "Function Name:" in line:
+            name = line.split("Function Name:")[1].split("[")[0].strip()
+        elif name and any(k in name for k in NO_SPILL):
+            for key in ("VGPRs Spill:", "ScratchSize [bytes/lane]:"):
+                if key in line and int(line.split(key)[1].split("[")[0].strip()) != 0:
+                    bad.append("{} ({} {})".format(name, key, line.split(key)[1].split("[")[0].strip()))
+    return sorted(set(bad))
+
+
 def _compile(src):
     obj = os.path.join(OBJDIR, os.path.basename(src)[:-4] + ".o")
-    cmd = [HIPCC] + FLAGS + ["-c", src, "-o", obj]
+    check = os.path.basename(src).startswith("gemm_")
+    cmd = [HIPCC] + FLAGS + (["-Rpass-analysis=kernel-resource-usage"] if check else []) + ["-c", src, "-o", obj]
     p = subprocess.run(cmd, capture_output=True, text=True)
-    return src, obj, p.returncode, p.stdout + p.stderr
+    out = p.stdout + p.stderr
+    if check and p.returncode == 0:
+        bad = _spilling_kernels(out)
+        if bad:
+            return src, obj, 1, "kernels with hand-counted waits must not spill:\n  " + "\n  ".join(bad)
+        out = "\n".join(l for l in out.splitlines() if "remark:" not in l and "__launch_bounds__" not in l and not l.strip().startswith(("|", "^")))
+    return src, obj, p.returncode, out
 
 
 def build_library(verbose=True, jobs=8):
