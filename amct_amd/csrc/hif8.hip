@@ -10,8 +10,8 @@
 
 namespace amct {
 
-AMCT_DEV uint32_t hif8_enc(float x, bool saturate) {
-    const uint32_t u = __float_as_uint(x);
+// u: the fp32 bit pattern.  Integer arithmetic only, so the compiler can also evaluate it (the table below).
+__host__ __device__ constexpr uint32_t hif8_enc_bits(uint32_t u, bool saturate) {
     const uint32_t sign = (u >> 24) & 0x80u;
     const uint32_t a = u & 0x7FFFFFFFu;
     if (a > 0x7F800000u) return 0x80u;
@@ -39,6 +39,20 @@ AMCT_DEV uint32_t hif8_enc(float x, bool saturate) {
     if (a2 <= 7) return sign | 0x40u | (es << 4) | ((uint32_t)(a2 & 3) << 2) | ((r >> 21) & 3u);
     return sign | 0x60u | (es << 4) | ((uint32_t)(a2 & 7) << 1) | ((r >> 22) & 1u);
 }
+AMCT_DEV uint32_t hif8_enc(float x, bool saturate) { return hif8_enc_bits(__float_as_uint(x), saturate); }
+
+// The code of a bf16 value depends on its sign, its exponent and the first four bits of its mantissa only (at most
+// three are kept and ties go away from zero, so the first dropped bit decides the rounding) -- except for exponent 255,
+// where the last three bits tell a NaN from an infinity.  Table of the 8192 values with the last three bits zero, for
+// overflow to infinity [0] and to the largest finite value [1], computed by the compiler.
+struct Hif8Bf16Table {
+    uint8_t code[2][8192];
+    constexpr Hif8Bf16Table() : code{} {
+        for (int s = 0; s < 2; ++s)
+            for (uint32_t i = 0; i < 8192u; ++i) code[s][i] = (uint8_t)hif8_enc_bits(i << 19, s != 0);
+    }
+};
+__device__ const Hif8Bf16Table kHif8Bf16{};
 
 AMCT_DEV float hif8_dec(uint32_t c) {
     const uint32_t b = c & 0x7Fu;
@@ -184,33 +198,112 @@ __global__ __launch_bounds__(kBlock) void hif8_encode_full(const void* x, uint8_
     }
 }
 
-template <int DT, int U>
-__global__ __launch_bounds__(kBlock) void hif8_decode_full(const uint8_t* x, void* y, int64_t nchunks) {
+// bf16 input, complete chunks of U * BLK vectors: one look-up per element in the block's copy of the 8 KB table
+// above (index = the first 13 bits of the value), four codes merged by one byte permute.  A wave that holds an infinity
+// or a NaN (a magnitude of 0x7F80 or more in any lane, found with packed 16-bit maxima) encodes its vectors by the
+// arithmetic routine instead.  The next chunk's loads are issued before this one is encoded.
+typedef unsigned short h2u16 __attribute__((ext_vector_type(2)));
+AMCT_DEV uint32_t hif8_pk_max_u16(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(h2u16, a), __builtin_bit_cast(h2u16, b)));
+}
+// the two codes of a word of two bf16 values, zero-extended to 16 bits each
+AMCT_DEV uint32_t hif8_lut2(const uint8_t* tbl, uint32_t w) {
+    h2u16 p;
+    p.x = tbl[__builtin_amdgcn_ubfe(w, 3, 13)];
+    p.y = tbl[w >> 19];
+    return __builtin_bit_cast(uint32_t, p);
+}
+
+template <int BLK, int U>
+__global__ __launch_bounds__(BLK) void hif8_encode_bf16_lut(const void* x, uint8_t* y, int64_t nchunks, int saturate) {
+    __shared__ __align__(16) uint8_t tbl[8192];
+    const uint32_t tid = threadIdx.x;
+    {
+        const uint4* src = reinterpret_cast<const uint4*>(kHif8Bf16.code[saturate ? 1 : 0]);
+        for (uint32_t i = tid; i < 512u; i += BLK) reinterpret_cast<uint4*>(tbl)[i] = src[i];
+    }
+    uint4 nxt[U];
+    if ((int64_t)blockIdx.x < nchunks) {
+        const char* xb = reinterpret_cast<const char*>(x) + (int64_t)blockIdx.x * (U * BLK * 16);
+#pragma unroll
+        for (int u = 0; u < U; ++u) nxt[u] = ldg16_nt(xb + (u * BLK + tid) * 16u);
+    }
+    __syncthreads();
+    for (int64_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
+        uint8_t* yb = y + c * (U * BLK * 8);
+        uint4 raw[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) raw[u] = nxt[u];
+        if (c + gridDim.x < nchunks) {
+            const char* xb = reinterpret_cast<const char*>(x) + (c + gridDim.x) * (U * BLK * 16);
+#pragma unroll
+            for (int u = 0; u < U; ++u) nxt[u] = ldg16_nt(xb + (u * BLK + tid) * 16u);
+        }
+        uint32_t m = 0;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            m = hif8_pk_max_u16(m, hif8_pk_max_u16(hif8_pk_max_u16(raw[u].x & 0x7FFF7FFFu, raw[u].y & 0x7FFF7FFFu),
+                                                   hif8_pk_max_u16(raw[u].z & 0x7FFF7FFFu, raw[u].w & 0x7FFF7FFFu)));
+        }
+        const bool special = (m & 0xFFFFu) >= 0x7F80u || m >= 0x7F800000u;
+        if (__builtin_amdgcn_ballot_w64(special) == 0) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const uint32_t w0 = __builtin_amdgcn_perm(hif8_lut2(tbl, raw[u].y), hif8_lut2(tbl, raw[u].x), 0x06040200u);
+                const uint32_t w1 = __builtin_amdgcn_perm(hif8_lut2(tbl, raw[u].w), hif8_lut2(tbl, raw[u].z), 0x06040200u);
+                stg8_nt(yb + (u * BLK + tid) * 8u, w0, w1);
+            }
+        } else {
+#pragma unroll                                       // (a rolled loop would index raw[] at run time: 64 KB of LDS)
+            for (int u = 0; u < U; ++u) {
+                float v[8];
+                unpack16<AMCT_BF16>(raw[u], v);
+                uint32_t w[2];
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    w[j] = hif8_enc(v[4 * j], saturate != 0) | (hif8_enc(v[4 * j + 1], saturate != 0) << 8) |
+                           (hif8_enc(v[4 * j + 2], saturate != 0) << 16) | (hif8_enc(v[4 * j + 3], saturate != 0) << 24);
+                stg8_nt(yb + (u * BLK + tid) * 8u, w[0], w[1]);
+            }
+        }
+    }
+}
+
+// complete chunks of U * BLK vectors; the next chunk's codes are loaded before this one's are looked up
+template <int DT, int BLK, int U>
+__global__ __launch_bounds__(BLK) void hif8_decode_full(const uint8_t* x, void* y, int64_t nchunks) {
     constexpr int VEC = Tr<DT>::VEC;
     __shared__ float tbl[256];
     const uint32_t tid = threadIdx.x;
-    tbl[tid] = hif8_dec(tid);
+    if (tid < 256u) tbl[tid] = hif8_dec(tid);
     __syncthreads();
-    for (int64_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
-        const uint8_t* xb = x + c * (U * kBlock * VEC);
-        char* yb = reinterpret_cast<char*>(y) + c * (U * kBlock * 16);
-        uint32_t w[U][2];
+    auto load = [&](int64_t c, uint32_t (&w)[U][2]) {
+        const uint8_t* xb = x + c * (U * BLK * VEC);
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             w[u][1] = 0;
             if constexpr (VEC == 8) {
-                const u2v r = __builtin_nontemporal_load(reinterpret_cast<const u2v*>(xb + (u * kBlock + tid) * 8u));
+                const u2v r = __builtin_nontemporal_load(reinterpret_cast<const u2v*>(xb + (u * BLK + tid) * 8u));
                 w[u][0] = r.x; w[u][1] = r.y;
             } else {
-                w[u][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(xb + (u * kBlock + tid) * 4u));
+                w[u][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(xb + (u * BLK + tid) * 4u));
             }
         }
+    };
+    uint32_t nxt[U][2];
+    if ((int64_t)blockIdx.x < nchunks) load(blockIdx.x, nxt);
+    for (int64_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
+        char* yb = reinterpret_cast<char*>(y) + c * (U * BLK * 16);
+        uint32_t w[U][2];
+#pragma unroll
+        for (int u = 0; u < U; ++u) { w[u][0] = nxt[u][0]; w[u][1] = nxt[u][1]; }
+        if (c + gridDim.x < nchunks) load(c + gridDim.x, nxt);
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             float out[VEC];
 #pragma unroll
             for (int j = 0; j < VEC; ++j) out[j] = tbl[(w[u][j / 4] >> (8 * (j % 4))) & 0xFFu];
-            stg16_nt(yb + (u * kBlock + tid) * 16u, pack16<DT>(out));
+            stg16_nt(yb + (u * BLK + tid) * 16u, pack16<DT>(out));
         }
     }
 }
@@ -254,6 +347,12 @@ __global__ __launch_bounds__(kBlock) void hif8_decode_k(const uint8_t* x, void* 
     }
 }
 
+// Launch shapes, measured on X[8192,4096] bf16: encoder 1024 threads x 1 vector, two blocks per CU, 17.3 us (512 x 4:
+// 17.6; the two-table kernel 18.5); decoder 256 threads x 8 vectors, four blocks per CU, 17.3 us (256 x 4 with one
+// chunk per block and no look-ahead 18.9; 1024 x 4: 19.5).
+constexpr int kHif8LutBlock = 1024, kHif8LutU = 1, kHif8LutBlocksPerCu = 2;
+constexpr int kHif8DecBlock = 256, kHif8DecU = 8, kHif8DecBlocksPerCu = 4;
+
 }  // namespace amct
 
 using namespace amct;
@@ -280,6 +379,19 @@ extern "C" int amct_hif8_encode(const void* x, uint8_t* y, int64_t n, int dtype,
             hipLaunchKernelGGL((hif8_encode_k<DT, U>), dim3(1), dim3(kBlock), 0, st, x, y, nvec, n, saturate);   \
         }                                                                                                        \
     }
+    if (dtype == AMCT_BF16) {
+        constexpr int BLK = kHif8LutBlock, UL = kHif8LutU;
+        constexpr int64_t per = (int64_t)BLK * UL * 8;
+        const int64_t full = n / per;
+        if (full > 0) {
+            const int64_t cap = (int64_t)kHif8LutBlocksPerCu * 256;
+            hipLaunchKernelGGL((hif8_encode_bf16_lut<BLK, UL>), dim3((unsigned)(full > cap ? cap : full)), dim3(BLK), 0, st, x, y, full, saturate);
+            x = reinterpret_cast<const char*>(x) + full * per * 2;
+            y += full * per;
+            n -= full * per;
+        }
+        if (n == 0) return hip_status();
+    }
     switch (dtype) {
         case AMCT_F32: AMCT_HE(AMCT_F32) break;
         case AMCT_F16: AMCT_HE(AMCT_F16) break;
@@ -297,10 +409,10 @@ extern "C" int amct_hif8_decode(const uint8_t* x, void* y, int64_t n, int dtype,
     hipStream_t st = (hipStream_t)stream;
 #define AMCT_HD(DT)                                                                                   \
     {                                                                                                 \
-        constexpr int64_t per = (int64_t)kBlock * 4 * Tr<DT>::VEC;                                    \
-        const int64_t full = n / per;                                                                 \
+        constexpr int64_t per = (int64_t)kHif8DecBlock * kHif8DecU * Tr<DT>::VEC;                     \
+        const int64_t full = n / per, cap = (int64_t)kHif8DecBlocksPerCu * 256;                       \
         if (full > 0) {                                                                               \
-            hipLaunchKernelGGL((hif8_decode_full<DT, 4>), dim3((unsigned)(full > 4096 ? 4096 : full)), dim3(kBlock), 0, st, x, y, full); \
+            hipLaunchKernelGGL((hif8_decode_full<DT, kHif8DecBlock, kHif8DecU>), dim3((unsigned)(full > cap ? cap : full)), dim3(kHif8DecBlock), 0, st, x, y, full); \
             x += full * per;                                                                          \
             y = reinterpret_cast<char*>(y) + full * per * Tr<DT>::BYTES;                              \
             n -= full * per;                                                                          \

@@ -142,3 +142,32 @@ def test_hif8_config3(dev):
     # odd element counts take the scalar tail
     y = x.reshape(-1)[:1003].contiguous()
     assert np.array_equal(ops.hif8_encode(y.to(dev)).cpu().numpy(), hif8.encode_bruteforce(y.float().numpy()))
+
+
+@pytest.mark.parametrize("sat", [False, True])
+def test_hif8_bf16_specials_among_ordinary_values(dev, sat):
+    """A bf16 tensor of many chunks (so that blocks loop) plus a ragged remainder, with infinities, NaNs of every kind
+    (payload in the last three mantissa bits only included), signed zeros, values around the overflow threshold and
+    below the smallest code scattered among ordinary values: waves with and without a special value take different
+    routines and must agree with the brute-force encoder everywhere; decode then returns to the table values."""
+    g = torch.Generator().manual_seed(29)
+    n = 1024 * 8 * 300 + 8 * 77 + 5
+    x = (torch.randn(n, generator=g) * torch.exp2(torch.randint(-26, 17, (n,), generator=g).float())).to(torch.bfloat16)
+    bits = x.view(torch.int16).clone()
+    special = torch.tensor([0x7F80, 0xFF80, 0x7FC0, 0xFFC0, 0x7F81, 0xFF87, 0x7FFF, 0x0000, 0x8000, 0x0001, 0x8001,
+                            0x4700, 0x4720, 0x4740, 0xC720, 0x3400, 0x33C0, 0xB400, 0x3380], dtype=torch.int32).to(torch.int16)
+    where = torch.randperm(n, generator=g)[: 4000]
+    bits[where] = special[torch.arange(where.numel()) % special.numel()]
+    # leave a long stretch without any special value, so that whole waves take the table routine
+    bits[1024 * 8 * 100: 1024 * 8 * 200] = x.view(torch.int16)[1024 * 8 * 100: 1024 * 8 * 200]
+    x = bits.view(torch.bfloat16)
+    got = ops.hif8_encode(x.to(dev), sat)
+    want = hif8.encode_bruteforce(x.float().numpy(), sat)
+    bad = np.nonzero(got.cpu().numpy() != want)[0]
+    assert bad.size == 0, (sat, bad[:5], x[bad[:5].tolist()], got.cpu().numpy()[bad[:5]], want[bad[:5]])
+    for dtype in (torch.bfloat16, torch.float16, torch.float32):
+        d = ops.hif8_decode(got, dtype).cpu()
+        ref = torch.from_numpy(hif8.decode(want)).to(dtype)
+        nan = torch.isnan(ref)
+        assert torch.equal(torch.isnan(d), nan)
+        assert_bits_equal(torch.where(nan, torch.zeros_like(d), d), torch.where(nan, torch.zeros_like(ref), ref), "decode")
