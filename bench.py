@@ -297,7 +297,8 @@ def build_cases(dev, only):
                           "torch._int_mm int8 x int8 -> int32, M=2048 N=14336 K=4096 (vendor library yardstick)"))
 
     # ---- K6: W8A8 Linear, W[14336,4096] int8 ----------------------------------------------------------
-    if want("w8a8_m2048") or want("w8a8_m16"):
+    chain = {"w8a8_dynamic_m2048": 2048, "w8a8_dynamic_m16": 16}
+    if want("w8a8_m2048") or want("w8a8_m16") or any(want(n) for n in chain):
         x6, wq6, sw6 = workloads.c4_w8a8()
         N6, K6 = wq6.shape
         nw = 6                                           # 6 x 58.7 MB of weights rotate through HBM
@@ -320,6 +321,31 @@ def build_cases(dev, only):
             else:
                 cases.append(Case(name, "hbm", N6 * K6 + M6 * K6 + M6 * N6 * 2 + N6 * 4 + M6 * 4, "B", launch, nw, "int8",
                                   "W8A8 Linear M=%d (decode): weight streaming (config 4)" % M6))
+
+        # config 4 as the deployed module runs it with dynamic activation quantisation: K3 (per-token scales and codes
+        # of the bf16 activations) and K6 back to back on one stream, two launches per step.  (Quantising inside the
+        # GEMM would repeat K3's arithmetic in every one of the 56 / 224 blocks that share a row.)
+        for name, M6 in chain.items():
+            if not want(name):
+                continue
+            xb6 = x6[:M6].contiguous().to(dev)
+            xq6 = torch.empty(M6, K6, dtype=torch.int8, device=dev)
+            st6 = torch.empty(M6, dtype=torch.float32, device=dev)
+            outs = [torch.empty(M6, N6, dtype=torch.bfloat16, device=dev) for _ in range(nw)]
+
+            def launch(i, xb6=xb6, xq6=xq6, st6=st6, outs=outs, M6=M6, wqs=wqs, swd=swd, N6=N6, K6=K6):
+                j = i % len(wqs)
+                rc = lib.amct_act_quant_per_token_int8(xb6.data_ptr(), None, xq6.data_ptr(), st6.data_ptr(), M6, K6, 0, _lib.BF16, st)
+                assert rc == 0, rc
+                rc = lib.amct_gemm_w8a8(xq6.data_ptr(), wqs[j].data_ptr(), st6.data_ptr(), swd.data_ptr(), None, 0,
+                                        outs[j].data_ptr(), None, M6, N6, K6, _lib.BF16, st)
+                assert rc == 0, rc
+            if M6 >= 256:
+                cases.append(Case(name, "mfma_i8", 2 * M6 * N6 * K6, "op", launch, nw, "int8",
+                                  "dynamic per-token quantise + W8A8 Linear, M=%d, two launches (config 4 as deployed)" % M6))
+            else:
+                cases.append(Case(name, "hbm", N6 * K6 + M6 * K6 * 2 + M6 * N6 * 2 + N6 * 4, "B", launch, nw, "int8",
+                                  "dynamic per-token quantise + W8A8 Linear, M=%d (decode), two launches" % M6))
 
     # ---- K7: W4A16 Linear, W[14336,4096] int4 g128 ------------------------------------------------------
     if want("w4a16_m2048") or want("w4a16_m16") or want("w4a16_m1"):
