@@ -30,6 +30,8 @@ SIGNATURES = {
     "amct_mfma_yardstick": (_I, [_I, _I, _I, _P, _P, _P]),
     "amct_minmax": (_I, [_P, _P, _P, _L, _L, _I, _I, _P]),
     "amct_gptq_block": (_I, [_P, _L, _P, _L, _P, _L, _P, _P, _L, _P, _L, _I, _I, _I, _P]),
+    "amct_hessian_update_workspace_bytes": (ctypes.c_size_t, [_L, _L]),
+    "amct_hessian_update": (_I, [_P, _P, _L, _L, ctypes.c_float, ctypes.c_float, _I, _P, ctypes.c_size_t, _P]),
     "amct_fp8_block_dequant": (_I, [_P, _P, _P, _L, _L, _I, _I, _P]),
     "amct_pack_int4_pairs_n": (_I, [_P, _P, _L, _L, _P]),
     "amct_scale_f32_to_u64": (_I, [_P, _P, _L, _P]),

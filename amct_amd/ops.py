@@ -124,6 +124,25 @@ def awq_loss(y, yhat):
     return loss
 
 
+def hessian_update(hessian, x, beta, alpha):
+    """hessian [C,C] fp32 <- beta * hessian + alpha * x^T x in place, x [tokens, C] bf16|f16 (gptq_module.py:176-181).
+    beta == 0 does not read hessian."""
+    dev = _dev(hessian, x)
+    _need(hessian.dim() == 2 and hessian.shape[0] == hessian.shape[1] and hessian.dtype == torch.float32 and
+          hessian.is_contiguous(), "hessian_update: the Hessian must be a contiguous square fp32 matrix")
+    _need(x.dim() == 2 and x.shape[1] == hessian.shape[0], "hessian_update: x must be [tokens, {}]".format(hessian.shape[0]))
+    _need(x.dtype in (torch.bfloat16, torch.float16), "hessian_update: 16-bit activations only")
+    x = _c(x)
+    lib = _lib.load()
+    tokens, cols = x.shape
+    nbytes = lib.amct_hessian_update_workspace_bytes(tokens, cols)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(lib.amct_hessian_update(_p(hessian), _p(x), tokens, cols, float(beta), float(alpha), dtype_code(x.dtype),
+                                           _p(ws), ws.numel(), _stream(dev)))
+    return hessian
+
+
 def scale_offset(vmax, vmin, bits, symmetric, scope_rule=SCOPE_AMCT, bad=None):
     """Elementwise (max, min) -> (scale fp32, offset int32 | None), same shape as the inputs."""
     dev = _dev(vmax, vmin, bad)

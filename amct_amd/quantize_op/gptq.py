@@ -16,13 +16,25 @@ def update_hessian(hessian, nsamples, input_data, columns):
     if len(input_data.shape) == 2:
         input_data = input_data.unsqueeze(0)
     batch_size = input_data.shape[0]
-    x = input_data.reshape((-1, input_data.shape[-1])).t()
-    if hessian is None:
-        hessian = torch.zeros((columns, columns), device=x.device)
-    hessian = hessian * (nsamples / (nsamples + batch_size))
-    nsamples += batch_size
-    x = math.sqrt(2 / nsamples) * x.float()
-    hessian = hessian + x.matmul(x.t())
+    rows = input_data.reshape((-1, input_data.shape[-1]))
+    if rows.is_cuda and rows.dtype in (torch.bfloat16, torch.float16):
+        # the matrix-pipe kernel: one pass over the lower triangle of H, the product of the 16-bit values exact in fp32
+        if hessian is None:
+            hessian = torch.empty((columns, columns), dtype=torch.float32, device=rows.device)
+            beta = 0.0
+        else:
+            beta = nsamples / (nsamples + batch_size)
+        nsamples += batch_size
+        hessian = ops.hessian_update(hessian, rows, beta, 2 / nsamples)
+    else:
+        # fp32 activations keep the fp32 product
+        x = rows.t()
+        if hessian is None:
+            hessian = torch.zeros((columns, columns), device=x.device)
+        hessian = hessian * (nsamples / (nsamples + batch_size))
+        nsamples += batch_size
+        x = math.sqrt(2 / nsamples) * x.float()
+        hessian = hessian + x.matmul(x.t())
     if not torch.isfinite(hessian).all():
         raise RuntimeError("hessian matrix has invalid value, inf or nan.")
     return hessian, nsamples

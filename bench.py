@@ -375,6 +375,36 @@ def build_cases(dev, only):
             else:
                 cases.append(Case(name, "hbm", wbytes + M7 * K7 * 2 + M7 * N7 * 2, "B", launch, nw7, "bf16",
                                   "W4A16 Linear M=%d (decode): weight streaming (config 5)" % M7))
+    # ---- GPTQ Hessian accumulation: H[4096,4096] fp32 <- beta H + alpha X^T X, X[2048,4096] bf16 ------------------
+    # (after everything else: it heats the part like the GEMMs do).  Work = the multiply-adds of the lower triangle
+    # with its diagonal, which is what a symmetric update needs; the library path beside it is the reference's
+    # sequence on the device (scale H, scale x in fp32, fp32 matmul, add).
+    if want("gptq_hessian_update") or want("lib_hessian_update_fp32"):
+        import math
+        Th, Ch = 2048, 4096
+        gh = torch.Generator().manual_seed(1031)
+        xh = [torch.randn(Th, Ch, generator=gh).to(torch.bfloat16).to(dev) for _ in range(4)]
+        hh = [torch.zeros(Ch, Ch, dtype=torch.float32, device=dev) for _ in range(4)]
+        wsh = torch.empty(lib.amct_hessian_update_workspace_bytes(Th, Ch), dtype=torch.uint8, device=dev)
+        work = 2 * Th * Ch * (Ch + 1) // 2
+        if want("gptq_hessian_update"):
+            def launch(i, xh=xh, hh=hh, wsh=wsh, Th=Th, Ch=Ch):
+                j = i % len(xh)
+                rc = lib.amct_hessian_update(hh[j].data_ptr(), xh[j].data_ptr(), Th, Ch, 0.5, 2.0 / 4096, _lib.BF16,
+                                             wsh.data_ptr(), wsh.numel(), st)
+                assert rc == 0, rc
+            cases.append(Case("gptq_hessian_update", "mfma_bf16", work, "flop", launch, 4, "bf16",
+                              "GPTQ Hessian update H[4096,4096] += X^T X, X[2048,4096] bf16 (transpose + symmetric MFMA kernel; "
+                              "flops of the lower triangle)"))
+        if want("lib_hessian_update_fp32"):
+            def launch(i, xh=xh, hh=hh):
+                j = i % len(xh)
+                hh[j].mul_(0.5)
+                xs = math.sqrt(2.0 / 4096) * xh[j].float().t()
+                hh[j].add_(xs.matmul(xs.t()))
+            cases.append(Case("lib_hessian_update_fp32", "mfma_bf16", work, "flop", launch, 4, "f32",
+                              "the same update as the reference writes it, on the device with library calls (fp32 matmul); "
+                              "same flop count as above for comparison"))
     return cases
 
 
@@ -556,8 +586,12 @@ def run(args, dev, only):
         if y and y in results and name != y:
             r["frac_of_yardstick"] = round(r["achieved"] / results[y]["achieved"], 4)
         lib = {"TOP/s": "lib_gemm_i8", "TFLOP/s": "lib_gemm_bf16"}.get(r["unit"])
-        if lib and lib in results and not name.startswith(("lib_gemm", "mfma_")):
+        if lib and lib in results and not name.startswith(("lib_gemm", "mfma_", "lib_hessian", "gptq_hessian")):
             r["vs_vendor_library"] = round(r["achieved"] / results[lib]["achieved"], 4)
+    if "gptq_hessian_update" in results and "lib_hessian_update_fp32" in results:
+        results["gptq_hessian_update"]["vs_vendor_library"] = round(
+            results["lib_hessian_update_fp32"]["us_per_launch"] / results["gptq_hessian_update"]["us_per_launch"], 4)
+        results["gptq_hessian_update"].pop("frac_of_yardstick", None)
     c, wall, ms = head
     value = c.work * args.steps / wall / 1e9
     traffic = MEASURED_TRAFFIC.get("int4_group_pack")

@@ -292,6 +292,20 @@ int amct_gptq_block(float* w, int64_t ld_w, float* err_out, int64_t ld_e, const 
                     const float* scale, const int32_t* offset, int64_t scale_stride, const int32_t* gidx,
                     int64_t rows, int count, int qmin, int qmax, amct_stream_t stream);
 
+/* ---- GPTQ Hessian accumulation --------------------------------------------------------------
+ * The update of amct_pytorch/quantize_op/gptq_module.py:176-181 for 16-bit calibration activations:
+ *   hessian *= n / (n + b);  x = sqrt(2 / (n + b)) * x.float();  hessian += x.t() @ x      (x [tokens, cols])
+ * as hessian <- beta * hessian + alpha * (x^T x) with beta = n / (n + b), alpha = 2 / (n + b): the products of two
+ * 16-bit values are exact in fp32 and are summed in fp32 on the matrix pipe, alpha is applied to the sum (the reference
+ * scales every element by sqrt(alpha) first: the results agree to fp32 rounding, not bit for bit).  hessian fp32
+ * [cols, cols], symmetric: only its lower triangle is read, both triangles are written; beta == 0 reads nothing, so the
+ * first call may pass uninitialised memory.  x of dtype AMCT_BF16 or AMCT_F16 (fp32 activations: AMCT_E_UNSUPPORTED,
+ * the caller keeps its fp32 product).  workspace: amct_hessian_update_workspace_bytes(tokens, cols) bytes, 16-byte
+ * aligned (x transposed and padded to whole tiles), contents irrelevant before and after the call. */
+size_t amct_hessian_update_workspace_bytes(int64_t tokens, int64_t cols);
+int amct_hessian_update(float* hessian, const void* x, int64_t tokens, int64_t cols, float beta, float alpha,
+                        int dtype, void* workspace, size_t workspace_bytes, amct_stream_t stream);
+
 /* ---- interchange formats of the checkpoint converter ---------------------------------------
  * (amct_pytorch/experimental/quantization/DeepSeekV3.2/deploy.py)
  * amct_fp8_block_dequant: weight_dequant :48-92.  w E4M3FN codes [rows, cols], scale fp32

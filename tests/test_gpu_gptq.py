@@ -106,3 +106,55 @@ def test_gptq_whole_routine(dev, strategy, group, sym):
     plain = iq.fake_quant(w, 'int4', ws, wz, group)
     plain_err = ((x @ w.float().t()) - (x @ plain.float().t())).pow(2).mean()
     assert float(got_err) < float(plain_err)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("tokens,cols", [(256, 128), (1, 64), (63, 200), (65, 136), (1000, 520), (2048, 1024), (300, 4104), (77, 100), (130, 1099)])
+def test_hessian_update_kernel(dev, dtype, tokens, cols):
+    """H <- beta H + alpha X^T X (gptq_module.py:176-181) on the matrix pipe.  Small integers make every product
+    and sum exact in fp32, so the first call (beta = 0, H full of NaN beforehand: it must not be read) and a second,
+    accumulating call are compared bit for bit with an integer matmul; random activations are compared with the fp64
+    product at the fp32 rounding of a sum of that many terms.  Ragged tokens and columns; H comes out exactly symmetric."""
+    from amct_amd import ops
+    g = torch.Generator().manual_seed(tokens * 31 + cols)
+    xi = torch.randint(-4, 5, (tokens, cols), generator=g)
+    h = torch.full((cols, cols), float('nan'), dtype=torch.float32, device=dev)
+    ops.hessian_update(h, xi.to(dtype).to(dev), 0.0, 1.0)
+    want = (xi.double().t() @ xi.double())
+    assert_bits_equal(h, want.float() + 0.0, "first call, integers")     # (+ 0.0: a sum that starts at +0 never ends at -0)
+    xj = torch.randint(-4, 5, (max(tokens // 2, 1), cols), generator=g)
+    ops.hessian_update(h, xj.to(dtype).to(dev), 0.5, 2.0)            # powers of two: still exact
+    want = 0.5 * want + 2.0 * (xj.double().t() @ xj.double())
+    assert_bits_equal(h, want.float() + 0.0, "second call, integers")
+    x = torch.randn(tokens, cols, generator=g).to(dtype)
+    h0 = torch.randn(cols, cols, generator=g)
+    h0 = (h0 + h0.t()).contiguous()
+    hd = h0.clone().to(dev)
+    beta, alpha = 0.75, 2.0 / (tokens + 7)
+    ops.hessian_update(hd, x.to(dev), beta, alpha)
+    ref = beta * h0.double() + alpha * (x.double().t() @ x.double())
+    mag = beta * h0.double().abs() + alpha * (x.double().abs().t() @ x.double().abs())
+    err = (hd.cpu().double() - ref).abs()
+    assert (err <= 2.0 ** -20 * mag + 1e-30).all(), float((err / (mag + 1e-30)).max())
+    assert torch.equal(hd, hd.t()), "symmetry"
+
+
+def test_update_hessian_on_16_bit_activations(dev):
+    """quantize_op.gptq.update_hessian with bf16 activations on the device takes the kernel; against the oracle's
+    restatement of the reference (fp32 product of the scaled activations) within the rounding of the two orders of
+    operations."""
+    torch.manual_seed(5)
+    k = 384
+    x = (torch.randn(640, k) * (1 + 3 * (torch.arange(k) % 17 == 0))).to(torch.bfloat16)
+    hess, ns = og.update_hessian(None, 0, x[:256], k)
+    hess, ns = og.update_hessian(hess, ns, x[256:].reshape(3, 128, k), k)
+    dh, dn = gptq.update_hessian(None, 0, x[:256].to(dev), k)
+    dh, dn = gptq.update_hessian(dh, dn, x[256:].reshape(3, 128, k).to(dev), k)
+    assert dn == ns and dh.dtype == torch.float32
+    torch.testing.assert_close(dh.cpu(), hess, rtol=1e-4, atol=1e-4)
+    # both are fp32 sums in different orders; against the same recurrence in fp64 the kernel is the closer one or as close
+    xd = x.double()
+    exact = (2 / 1) * (xd[:256].t() @ xd[:256]) * (1 / 1)            # first call: nsamples 0 -> 1
+    exact = exact * (1 / 4) + (2 / 4) * (xd[256:].t() @ xd[256:])    # second call: batch of 3, nsamples 1 -> 4
+    mine, theirs = (dh.cpu().double() - exact).abs().max(), (hess.double() - exact).abs().max()
+    assert float(mine) <= 1.5 * float(theirs) + 1e-6, (float(mine), float(theirs))
