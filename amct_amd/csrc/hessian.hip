@@ -8,8 +8,9 @@
 //
 // Two kernels.  hess_transpose_k writes X^T, zero-padded to whole tiles, into the caller's workspace ([Cp, Tp], K
 // contiguous), so that both MFMA operands are rows of one matrix.  hess_syrk_k owns one 128 x 128 tile of the lower
-// triangle: 4 waves of 64 x 64 (2 x 2 MFMA 32x32x16), 64 tokens per step, two LDS stages (16-byte chunks of a row
-// swizzled by the row so that fragment reads spread over the banks), one barrier per step.  The epilogue reads the
+// triangle: 4 waves of 64 x 64 (2 x 2 MFMA 32x32x16), 64 tokens per step, one LDS stage (16-byte chunks of a row
+// swizzled by the row so that fragment reads spread over the banks; the next step waits in registers), two barriers
+// per step.  The epilogue reads the
 // tile of H, applies beta and alpha, writes the tile and -- through LDS, as whole 256-byte rows -- its mirror image, so H
 // stays exactly symmetric and only its lower triangle is ever read.
 #include "amct_common.h"
@@ -96,8 +97,9 @@ AMCT_DEV h16f hs_mfma(const uint4& a, const uint4& b, const h16f& c) {
 }
 
 template <bool F16>
-__global__ __launch_bounds__(kBlock, 2) void hess_syrk_k(SyrkArgs a) {
-    // two stages x two operands x 128 rows x 128 bytes = 64 KB; the epilogue reuses it as four 64 x 64 fp32 patches
+__global__ __launch_bounds__(kBlock, 3) void hess_syrk_k(SyrkArgs a) {
+    // one stage: two operands x 128 rows x 128 bytes = 32 KB (the next step waits in registers); the epilogue reuses it as
+    // four 64 x 32 fp32 patches.  Three blocks fit a CU.
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -136,8 +138,10 @@ __global__ __launch_bounds__(kBlock, 2) void hess_syrk_k(SyrkArgs a) {
     const uint8_t* ga = reinterpret_cast<const uint8_t*>(a.xt) + ((i0 + ld_row) * a.Tp) * 2 + ld_chunk * 16;
     const uint8_t* gb = reinterpret_cast<const uint8_t*>(a.xt) + ((j0 + ld_row) * a.Tp) * 2 + ld_chunk * 16;
     const int64_t row_step = 32 * a.Tp * 2;          // bytes between the repeats
-    const uint32_t st_off = (uint32_t)ld_row * 128u + (uint32_t)((ld_chunk ^ (ld_row & 7)) * 16);   // (ld_row + 32 r) & 7 == ld_row & 7
-    constexpr uint32_t kTileBytes = kHsTile * 128, kStageBytes = 2 * kTileBytes;
+    // chunk c of row r sits at c ^ ((r >> 1) & 7): LDS has 64 banks of 4 bytes, two 128-byte rows cover them once, so 16
+    // lanes reading the same logical chunk of 16 consecutive rows meet in no bank
+    const uint32_t st_off = (uint32_t)ld_row * 128u + (uint32_t)((ld_chunk ^ ((ld_row >> 1) & 7)) * 16);   // rows 32 apart: same swizzle
+    constexpr uint32_t kTileBytes = kHsTile * 128;
 
     // fragments: lane l holds row l % 32 of a 32-row tile, chunk 2 * slice + l / 32 of the step's 128 bytes
     const int fr = lane & 31, fh = lane >> 5;
@@ -148,7 +152,7 @@ __global__ __launch_bounds__(kBlock, 2) void hess_syrk_k(SyrkArgs a) {
         fa_off[m] = ra * 128u;
         fb_off[m] = rb * 128u + kTileBytes;
     }
-    const uint32_t fsw = (uint32_t)(fr & 7);         // rows of a fragment: (64 w + 32 m + fr) & 7 == fr & 7
+    const uint32_t fsw = (uint32_t)((fr >> 1) & 7);  // rows of a fragment are 64 w + 32 m + fr: the swizzle depends on fr only
 
     h16f acc[2][2];
 #pragma unroll
@@ -173,9 +177,9 @@ __global__ __launch_bounds__(kBlock, 2) void hess_syrk_k(SyrkArgs a) {
         rb2 = *reinterpret_cast<const uint4*>(gb + 2 * row_step + so);                    \
         rb3 = *reinterpret_cast<const uint4*>(gb + 3 * row_step + so);                    \
     }
-#define AMCT_HS_LSTORE(STAGE)                                                             \
+#define AMCT_HS_LSTORE()                                                                  \
     {                                                                                     \
-        uint8_t* base = lds + (STAGE) * kStageBytes + st_off;                             \
+        uint8_t* base = lds + st_off;                                                     \
         *reinterpret_cast<uint4*>(base) = ra0;                                            \
         *reinterpret_cast<uint4*>(base + 32 * 128) = ra1;                                 \
         *reinterpret_cast<uint4*>(base + 64 * 128) = ra2;                                 \
@@ -186,11 +190,11 @@ __global__ __launch_bounds__(kBlock, 2) void hess_syrk_k(SyrkArgs a) {
         *reinterpret_cast<uint4*>(base + kTileBytes + 96 * 128) = rb3;                    \
     }
     AMCT_HS_GLOAD(0)
-    AMCT_HS_LSTORE(0)
+    AMCT_HS_LSTORE()
     __syncthreads();
     for (int s = 0; s < steps; ++s) {
         if (s + 1 < steps) AMCT_HS_GLOAD(s + 1)      // in flight during this step's MFMAs
-        const uint8_t* st = lds + (s & 1) * kStageBytes;
+        const uint8_t* st = lds;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             const uint32_t ch = ((uint32_t)(2 * ks + fh) ^ fsw) * 16u;
@@ -205,55 +209,62 @@ __global__ __launch_bounds__(kBlock, 2) void hess_syrk_k(SyrkArgs a) {
 #pragma unroll
                 for (int n = 0; n < 2; ++n) acc[m][n] = hs_mfma<F16>(fa[m], fb[n], acc[m][n]);
         }
-        if (s + 1 < steps) AMCT_HS_LSTORE((s + 1) & 1)   // the other stage: everyone left it at the last barrier
-        __syncthreads();
+        __syncthreads();                             // everyone has read this step's tiles
+        if (s + 1 < steps) {
+            AMCT_HS_LSTORE()
+            __syncthreads();
+        }
     }
 #undef AMCT_HS_GLOAD
 #undef AMCT_HS_LSTORE
 
     // ---- epilogue -------------------------------------------------------------------------------------------
     // acc[m][n][r]: row 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32 of the 32 x 32 tile (m, n) of this wave
+    // Addresses: one block-uniform base per wave plus 32-bit lane offsets (cols < 2^22 is checked by the host), so an
+    // address costs one register and the compiler keeps none of them alive in 64 bits.
     const bool have = a.beta != 0.f;
-    float* patch = reinterpret_cast<float*>(lds) + wave * (64 * 64);          // 16 KB per wave (after the last barrier)
-    const int64_t gi0 = i0 + wi * 64 + 4 * fh, gj0 = j0 + wj * 64 + fr;       // + m * 32 + 8 (r / 4) + r % 4, + n * 32
-    // all of the tile's old values first (64 independent loads in flight; one at a time, each behind the store
-    // before it, they cost 64 trips to memory), then the arithmetic and the stores
-    h16f old[2][2];
+    float* patch = reinterpret_cast<float*>(lds) + wave * (64 * 32);          // 8 KB per wave (after the last barrier)
+    const uint32_t C32 = (uint32_t)a.C;
+    const int64_t wi0 = i0 + wi * 64, wj0 = j0 + wj * 64;                     // the wave's first row and column
+    float* hw = a.h + wi0 * a.C + wj0;                                        // H[wi0][wj0]
+    float* hm = a.h + wj0 * a.C + wi0;                                        // its mirror image H[wj0][wi0]
+    const int rows_left = (int)min((int64_t)64, a.C - wi0), cols_left = (int)min((int64_t)64, a.C - wj0);   // may be <= 0
+    const uint32_t lane_off = (uint32_t)(4 * fh) * C32 + (uint32_t)fr;
 #pragma unroll
-    for (int m = 0; m < 2; ++m)
+    for (int n = 0; n < 2; ++n) {                    // the wave's columns 32 n .. 32 n + 31
+        const bool col_ok = n * 32 + fr < cols_left;
+        // all of the half's old values first (32 independent loads in flight; one at a time, each behind the store
+        // before it, they cost a trip to memory each), then the arithmetic and the stores
+        h16f old[2];
 #pragma unroll
-        for (int n = 0; n < 2; ++n)
+        for (int m = 0; m < 2; ++m)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int64_t gi = gi0 + m * 32 + 8 * (r / 4) + (r % 4), gj = gj0 + n * 32;
-                old[m][n][r] = (have && gi < a.C && gj < a.C) ? __builtin_nontemporal_load(a.h + gi * a.C + gj) : 0.f;
+                const int row = m * 32 + 8 * (r / 4) + (r % 4);               // + 4 fh
+                const uint32_t idx = lane_off + (uint32_t)row * C32 + (uint32_t)(n * 32);
+                old[m][r] = (have && col_ok && row + 4 * fh < rows_left) ? __builtin_nontemporal_load(hw + idx) : 0.f;
             }
 #pragma unroll
-    for (int m = 0; m < 2; ++m) {
-#pragma unroll
-        for (int n = 0; n < 2; ++n) {
+        for (int m = 0; m < 2; ++m) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int lr = m * 32 + 8 * (r / 4) + 4 * fh + (r % 4), lc = n * 32 + fr;      // inside the wave's 64 x 64
-                const int64_t gi = gi0 + m * 32 + 8 * (r / 4) + (r % 4), gj = gj0 + n * 32;
+                const int row = m * 32 + 8 * (r / 4) + (r % 4);
+                const int lr = row + 4 * fh;                                  // row inside the wave's 64 x 64
+                const uint32_t idx = lane_off + (uint32_t)row * C32 + (uint32_t)(n * 32);
                 float v = a.alpha * acc[m][n][r];
-                if (have) v = old[m][n][r] * a.beta + v;
-                if (gi < a.C && gj < a.C) a.h[gi * a.C + gj] = v;
-                patch[lr * 64 + (lc ^ (lr & 31))] = v;
+                if (have) v = old[m][r] * a.beta + v;
+                if (col_ok && lr < rows_left) hw[idx] = v;
+                patch[lr * 32 + (fr ^ (lr & 31))] = v;
             }
         }
-    }
-    if (diag) return;                                // the tile on the diagonal is its own mirror image
-    // mirror image: H[gj][gi] = H[gi][gj]; lane = row lr of the patch, one column lc per instruction, so a wave
-    // writes 64 consecutive floats of row gj.  (The patch is the wave's own: no barrier.)
-    {
+        if (diag) continue;                          // the tile on the diagonal is its own mirror image
+        // mirror image: H[gj][gi] = H[gi][gj]; lane = row lr of the patch, one column per instruction, so the wave
+        // writes 64 consecutive floats of a row of H.  (The patch is the wave's own: no barrier.)
         const int lr = lane;
-        const int64_t gi = i0 + wi * 64 + lr;
 #pragma unroll 8
-        for (int lc = 0; lc < 64; ++lc) {
-            const int64_t gj = j0 + wj * 64 + lc;
-            const float v = patch[lr * 64 + (lc ^ (lr & 31))];
-            if (gi < a.C && gj < a.C) a.h[gj * a.C + gi] = v;
+        for (int lc = 0; lc < 32; ++lc) {
+            const float v = patch[lr * 32 + (lc ^ (lr & 31))];
+            if (lr < rows_left && n * 32 + lc < cols_left) hm[(uint32_t)(n * 32 + lc) * C32 + (uint32_t)lr] = v;
         }
     }
 }
@@ -276,7 +287,7 @@ extern "C" int amct_hessian_update(float* hessian, const void* x, int64_t tokens
     if (tokens != 0 && !x) return AMCT_E_BADARG;
     const int64_t Cp = hs_round_up(cols, kHsTile), Tp = hs_round_up(tokens > 0 ? tokens : 1, kHsK);
     const int64_t nb = Cp / kHsTile;
-    if (nb * (nb + 1) / 2 > 0x7FFFFFFF || nb > 30000) return AMCT_E_TOO_LARGE;
+    if (cols >= (int64_t(1) << 22)) return AMCT_E_TOO_LARGE;                  // 32-bit offsets inside a tile, block ids
     if (!workspace || workspace_bytes < (size_t)Cp * (size_t)Tp * 2) return AMCT_E_BADARG;
     if (!aligned16(workspace) || (reinterpret_cast<uintptr_t>(hessian) & 3u) != 0 || (reinterpret_cast<uintptr_t>(x) & 1u) != 0)
         return AMCT_E_ALIGN;
@@ -289,7 +300,7 @@ extern "C" int amct_hessian_update(float* hessian, const void* x, int64_t tokens
                            reinterpret_cast<const uint16_t*>(x), reinterpret_cast<uint16_t*>(workspace), tokens, cols, Tp);
     const int64_t ntiles = nb * (nb + 1) / 2, per_die = (ntiles + 7) / 8;
     SyrkArgs a{reinterpret_cast<const uint16_t*>(workspace), hessian, cols, Tp, (int)nb, (int)per_die, ntiles, beta, alpha};
-    constexpr size_t lds_bytes = 2 * 2 * kHsTile * 128;                       // 64 KB
+    constexpr size_t lds_bytes = 2 * kHsTile * 128;                           // 32 KB
     const dim3 grid((unsigned)(8 * per_die));
     if (dtype == AMCT_F16) hipLaunchKernelGGL((hess_syrk_k<true>), grid, dim3(kBlock), lds_bytes, st, a);
     else hipLaunchKernelGGL((hess_syrk_k<false>), grid, dim3(kBlock), lds_bytes, st, a);
