@@ -93,3 +93,43 @@ def test_config3_mx_quant_at_bench_size(dev, fmt):
     want_el, want_sb = mx.mx_quant(x[rows], fmt)
     assert torch.equal(el.cpu()[rows].reshape(-1), torch.as_tensor(want_el).reshape(-1)), "element codes"
     assert torch.equal(sb.cpu()[rows].reshape(-1), torch.as_tensor(want_sb).reshape(-1)), "shared exponents"
+
+
+def test_decode_step_captured_in_a_graph(dev, c4, c5):
+    """The library allocates nothing and records no memory-set nodes, so a decode step -- dynamic per-token quantise ->
+    W8A8 Linear, and the W4A16 Linear with smoothing, M = 16 -- can be captured in a HIP graph as it is.  Every replay,
+    with new activations written into the captured input and eager work of the same kernels between the replays, gives
+    the eager results bit for bit."""
+    x, wq, sw = c4
+    x5, codes, scales, zeros, smooth_recip = c5
+    wqd, swd = wq.to(dev), sw.to(dev)
+    packed = workloads.pack_nibbles(codes).to(dev)
+    scd, zd, smd = scales.to(dev), zeros.to(dev), smooth_recip.to(dev)
+    xin = x[:16].contiguous().to(dev)
+    xin5 = x5[:16].contiguous().to(dev)
+
+    def step():
+        xq, st = ops.act_quant_per_token_int8(xin)
+        return ops.gemm_w8a8(xq, wqd, swd, st, None), ops.gemm_w4a16(xin5, packed, scd, zd, 128, smd, None)
+
+    step()                                                          # first-call set-up outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream(dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            g8, g4 = step()
+    torch.cuda.current_stream(dev).wait_stream(side)
+    torch.cuda.synchronize()
+    for rep in range(4):
+        lo = 16 * (rep + 1)
+        xin.copy_(x[lo:lo + 16].to(dev))
+        xin5.copy_(x5[lo:lo + 16].to(dev))
+        graph.replay()
+        torch.cuda.synchronize()
+        got8, got4 = g8.clone(), g4.clone()
+        want8, want4 = step()                                       # eager, same inputs: also the work between replays
+        torch.cuda.synchronize()
+        assert_bits_equal(got8, want8, "W8A8 decode step, replay %d" % rep)
+        assert_bits_equal(got4, want4, "W4A16 decode step, replay %d" % rep)
