@@ -33,11 +33,11 @@ PEAK_BF16_TFLOPS = 2500.0
 MEASURED_TRAFFIC = {
     "int4_group_pack": ("int4_group_pack4<2, 16, 1, false, true>", 148551685),
     "fakequant_int8": ("fq_fused<0, 256, 4, 1, false, false>", 134440825),
-    "mxfp8_quant": ("mx_quant_full<2, 0, 4>", 101801445),
-    "mxfp4_quant": ("mx_quant_full<2, 1, 4>", 85023231),
-    "mxfp8_dequant": ("mx_dequant_k<2, 0, 4>", 101755184),
-    "hif8_encode": ("hif8_encode_k<2, 4>", 100729581),
-    "hif8_decode": ("hif8_decode_k<2, 4>", 100747659),
+    "mxfp8_quant": ("mx_quant_full<2, 0, 2>", 101751472),
+    "mxfp4_quant": ("mx_quant_full<2, 1, 2>", 84973719),
+    "mxfp8_dequant": ("mx_dequant_full<2, 0, 8>", 101830190),
+    "hif8_encode": ("hif8_encode_bf16_lut<1024, 1>", 100773601),
+    "hif8_decode": ("hif8_decode_full<2, 256, 8>", 100748936),
     "act_quant_per_token": ("act_quant_token<2, 2>", 25292715),
     "col_minmax": ("col_partial_k<2, false> + col_final_k", 69345307),
     "w8a8_m2048": ("w8a8_tile_mix16<2>", 254747636),
