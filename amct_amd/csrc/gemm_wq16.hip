@@ -449,6 +449,12 @@ int wq16_int4_f16(const void* x, const void* smooth, const uint8_t* wq, const vo
 
 }  // namespace amct
 
+namespace amct {
+int w8a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
+                          const uint8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group,
+                          int dtype, hipStream_t st);      // gemm_w8a16_stream.hip
+}
+
 using namespace amct;
 
 extern "C" int amct_gemm_w8a16(const void* x, const void* smooth, const int8_t* wq, const void* scales, int scale_dtype,
@@ -464,5 +470,10 @@ extern "C" int amct_gemm_w8a16(const void* x, const void* smooth, const int8_t* 
              reinterpret_cast<const uint8_t*>(offsets), bias, (uint16_t*)out, M, N, K, group, scale_dtype,
              (uint32_t)(0x100000000ull / (uint64_t)group) + 1u};
     hipStream_t st = (hipStream_t)stream;
+    if (M <= 16) {                                   // K of 1024 / 2048 / 4096, groups of 128 .. K: the weight-streaming kernel
+        const int rc = w8a16_stream_dispatch(x, smooth, reinterpret_cast<const uint8_t*>(wq), scales, scale_dtype,
+                                             reinterpret_cast<const uint8_t*>(offsets), bias, out, M, N, K, group, dtype, st);
+        if (rc != AMCT_E_UNSUPPORTED) return rc;
+    }
     return dtype == AMCT_BF16 ? wq16_dispatch<8, AMCT_BF16>(a, st) : wq16_dispatch<8, AMCT_F16>(a, st);
 }

@@ -375,6 +375,23 @@ def build_cases(dev, only):
             else:
                 cases.append(Case(name, "hbm", wbytes + M7 * K7 * 2 + M7 * N7 * 2, "B", launch, nw7, "bf16",
                                   "W4A16 Linear M=%d (decode): weight streaming (config 5)" % M7))
+    # ---- int8 weight-only Linear (W8A16), W[14336,4096] int8 per-channel, bf16 activations, M = 16 ------------------
+    if want("w8a16_m16"):
+        x9 = workloads.c5_w4a16(2048)[0][:16].contiguous().to(dev)
+        g9 = torch.Generator().manual_seed(1033)
+        N9, K9 = 14336, 4096
+        w9 = dev_copies(torch.randint(-128, 128, (N9, K9), generator=g9, dtype=torch.int16).to(torch.int8), 6)
+        s9 = (1e-3 + 9e-3 * torch.rand(N9, 1, generator=g9)).to(torch.bfloat16).to(dev)
+        outs9 = [torch.empty(16, N9, dtype=torch.bfloat16, device=dev) for _ in range(6)]
+
+        def launch(i, x9=x9, w9=w9, s9=s9, outs9=outs9, N9=N9, K9=K9):
+            j = i % len(w9)
+            rc = lib.amct_gemm_w8a16(x9.data_ptr(), None, w9[j].data_ptr(), s9.data_ptr(), _lib.BF16, None, None,
+                                     outs9[j].data_ptr(), 16, N9, K9, K9, _lib.BF16, st)
+            assert rc == 0, rc
+        cases.append(Case("w8a16_m16", "hbm", N9 * K9 + 16 * K9 * 2 + 16 * N9 * 2 + N9 * 2, "B", launch, 6, "bf16",
+                          "int8 weight-only Linear M=16 N=14336 K=4096, per-channel scales, bf16 activations (decode): weight streaming"))
+
     # ---- GPTQ Hessian accumulation: H[4096,4096] fp32 <- beta H + alpha X^T X, X[2048,4096] bf16 ------------------
     # (after everything else: it heats the part like the GEMMs do).  Work = the multiply-adds of the lower triangle
     # with its diagonal, which is what a symmetric update needs; the library path beside it is the reference's

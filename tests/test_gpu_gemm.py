@@ -199,6 +199,51 @@ def test_w4a16_weight_streaming_kernel(dev, M, N, K):
     assert_bits_equal(out, want.to(torch.bfloat16), "integer special case")
 
 
+def w8a16_case(M, N, K, group, seed, dtype, sdt, sym):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, K, generator=g).to(dtype)
+    codes = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int16).to(torch.int8)
+    scales = (1e-3 + 9e-3 * torch.rand(N, K // group, generator=g)).to(sdt)
+    offsets = None if sym else torch.randint(-128, 128, (N, K // group), generator=g, dtype=torch.int16).to(torch.int8)
+    smooth = (0.5 + torch.rand(K, generator=g)).to(dtype)
+    bias = torch.randn(N, generator=g)
+    return x, codes, scales, offsets, smooth, bias
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K,group", [(1, 64, 1024, 128), (16, 200, 2048, 256), (9, 72, 1024, 1024), (5, 33, 2048, 128),
+                                         (16, 1000, 4096, 4096), (13, 14336, 4096, 128), (1, 14336, 4096, 4096),
+                                         (3, 16, 4096, 512), (16, 15, 1024, 512), (2, 300, 4096, 2048), (16, 520, 4096, 1024)])
+def test_w8a16_weight_streaming_kernel(dev, dtype, M, N, K, group):
+    """The int8 weight-only kernel for a few rows (M <= 16, K of 1024/2048/4096, groups of 128, 256, ... up to K, i.e.
+    per-channel factors too): every block width, ragged N, both activation and factor dtypes, symmetric and with
+    offsets, with and without smoothing and bias, against the fp64 anchor whose dequantised weight is not rounded; then
+    the integer special case (scale 1, small integer activations), where the result is an integer matmul bit for bit."""
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    for sdt, sym in ((torch.float16, False), (torch.bfloat16, True)):
+        x, codes, scales, offsets, smooth, bias = w8a16_case(M, N, K, group, 150 + M, dtype, sdt, sym)
+        for sm, b in ((None, None), (smooth, bias)):
+            out = ops.gemm_w8a16(x.to(dev), codes.to(dev), scales.to(dev), None if offsets is None else offsets.to(dev), group,
+                                 None if sm is None else sm.to(dev), None if b is None else b.to(dev))
+            assert out.dtype == dtype
+            want = od.w4a16_forward_f64(x, codes.to(torch.int32), scales, None if offsets is None else -offsets.float(), group, b,
+                                        None if sm is None else sm.reshape(1, -1), round_weight=False)
+            err = (out.cpu().double() - want).abs()
+            # exact weights, fp32 accumulation of x' * (q + 128) and of the correction term: 2e-5 of the row's largest
+            # output plus half an ulp of the value
+            tol = 2e-5 * want.abs().amax(dim=1, keepdim=True) + want.abs() * ulp
+            assert (err <= tol).all(), (float((err / tol).max()), sdt, sym, sm is not None)
+    g = torch.Generator().manual_seed(151)
+    xi = torch.randint(-4, 5, (M, K), generator=g).to(dtype)
+    wi = torch.randint(-7, 8, (N, K), generator=g, dtype=torch.int16).to(torch.int8)
+    zi = torch.randint(-3, 4, (N, K // group), generator=g, dtype=torch.int16).to(torch.int8)
+    ones = torch.ones(N, K // group, dtype=torch.float16)
+    out = ops.gemm_w8a16(xi.to(dev), wi.to(dev), ones.to(dev), zi.to(dev), group)
+    want = torch.matmul(xi.double(), (wi.double() - zi.double().repeat_interleave(group, dim=1)).t())
+    # every partial sum is an integer below 2^24, so the kernel's fp32 result is exact and its one rounding is torch's
+    assert_bits_equal(out, want.to(dtype), "integer special case")
+
+
 def test_w4a16_reduces_to_plain_matmul(dev):
     """zero = 8 (code 0 in signed terms), scale = 1: the kernel is a bf16 GEMM against integer
     weights, checked against torch.matmul."""
