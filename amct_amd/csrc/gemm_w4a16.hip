@@ -1726,7 +1726,7 @@ int wq16_int4_f16(const void* x, const void* smooth, const uint8_t* wq, const vo
                   hipStream_t st);                                 // gemm_wq16.hip
 int w4a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
                           const uint8_t* zeros, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group,
-                          hipStream_t st);                         // gemm_w4a16_stream.hip
+                          int dtype, hipStream_t st);              // gemm_w4a16_stream.hip
 
 }  // namespace amct
 
@@ -1748,14 +1748,21 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
     if (dtype != AMCT_BF16 && dtype != AMCT_F16) return AMCT_E_UNSUPPORTED;
     if (K % group != 0 || K % 2 != 0) return AMCT_E_ALIGN;
     if (M == 0) return AMCT_OK;
-    // fp16 activations: the kernels shared with the int8-weight path (gemm_wq16.hip), which smooth in the tile
-    if (dtype == AMCT_F16)
+    // fp16 activations: a few rows take the weight-streaming kernel like bf16 ones; otherwise the kernels shared with
+    // the int8-weight path (gemm_wq16.hip), which smooth in the tile
+    if (dtype == AMCT_F16) {
+        if (M <= 16) {
+            const int rc = w4a16_stream_dispatch(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, dtype,
+                                                 (hipStream_t)stream);
+            if (rc != AMCT_E_UNSUPPORTED) return rc;
+        }
         return wq16_int4_f16(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, (hipStream_t)stream);
+    }
     W4A16Args a{(const uint16_t*)x, (const uint16_t*)smooth, wq, scales, zeros, bias, (uint16_t*)out, M, N, K, group, scale_dtype,
                 (uint32_t)(0x100000000ull / (uint64_t)group) + 1u};
     hipStream_t st = (hipStream_t)stream;
     if (M <= 16) {                                                 // bf16, K % 1024 == 0, group 128: the weight-streaming kernel
-        const int rc = w4a16_stream_dispatch(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, st);
+        const int rc = w4a16_stream_dispatch(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, dtype, st);
         if (rc != AMCT_E_UNSUPPORTED) return rc;
     }
     const bool vec_ok = aligned16(x) && aligned16(wq) && (!smooth || aligned16(smooth)) && group % 32 == 0;

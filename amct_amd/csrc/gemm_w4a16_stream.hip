@@ -39,41 +39,68 @@ struct StreamArgs {
     uint32_t kv_magic;                               // floor(2^32 / (K / 8)) + 1: v / (K / 8) == mulhi(v, magic)
 };
 
-AMCT_DEV uint32_t st_pack2(float lo, float hi) {
-    const s2f f = {lo, hi};
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, s2bf));          // v_cvt_pk_bf16_f32, round-half-even
-}
-// 8 nibbles of w (nibble p = weight k0 + p) -> 4 words of two bf16 integers 16 + u each, word j = (weight j, weight j + 4)
-AMCT_DEV uint4 st_int8x(uint32_t w) {
-    constexpr uint32_t kMask = 0x00780078u, kBase = 0x41804180u;       // bf16(16 + u) = 0x4180 | u << 3
-    return make_uint4(((w << 3) & kMask) | kBase, ((w >> 1) & kMask) | kBase, ((w >> 5) & kMask) | kBase,
-                      ((w >> 9) & kMask) | kBase);
-}
+typedef _Float16 s8h __attribute__((ext_vector_type(8)));
+
+// what differs between the two activation types: the pack, the unpack, the bit pattern of the integer 16 + u, the MFMA
+template <int DT> struct StAct;
+template <> struct StAct<AMCT_BF16> {
+    static AMCT_DEV uint32_t pack2(float lo, float hi) {
+        const s2f f = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, s2bf));      // v_cvt_pk_bf16_f32, round-half-even
+    }
+    static AMCT_DEV float lo(uint32_t w) { return __uint_as_float(w << 16); }
+    static AMCT_DEV float hi(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
+    // 8 nibbles of w (nibble p = weight k0 + p) -> 4 words of two integers 16 + u each, word j = (weight j, weight j + 4)
+    static AMCT_DEV uint4 int8x(uint32_t w) {
+        constexpr uint32_t kMask = 0x00780078u, kBase = 0x41804180u;   // bf16(16 + u) = 0x4180 | u << 3
+        return make_uint4(((w << 3) & kMask) | kBase, ((w >> 1) & kMask) | kBase, ((w >> 5) & kMask) | kBase,
+                          ((w >> 9) & kMask) | kBase);
+    }
+    static AMCT_DEV s4f mfma(const uint4& a, const uint4& b, s4f c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(s8bf, a), __builtin_bit_cast(s8bf, b), c, 0, 0, 0);
+    }
+    static AMCT_DEV uint32_t out_bits(float v) { return f32_to_bf16_bits(v); }
+};
+template <> struct StAct<AMCT_F16> {
+    static AMCT_DEV uint32_t pack2(float lo, float hi) { return f32_to_f16_bits(lo) | (f32_to_f16_bits(hi) << 16); }
+    static AMCT_DEV float lo(uint32_t w) { return f16_bits_to_f32(w & 0xFFFFu); }
+    static AMCT_DEV float hi(uint32_t w) { return f16_bits_to_f32(w >> 16); }
+    static AMCT_DEV uint4 int8x(uint32_t w) {
+        constexpr uint32_t kMask = 0x03C003C0u, kBase = 0x4C004C00u;   // f16(16 + u) = 0x4C00 | u << 6
+        return make_uint4(((w << 6) & kMask) | kBase, ((w << 2) & kMask) | kBase, ((w >> 2) & kMask) | kBase,
+                          ((w >> 6) & kMask) | kBase);
+    }
+    static AMCT_DEV s4f mfma(const uint4& a, const uint4& b, s4f c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(s8h, a), __builtin_bit_cast(s8h, b), c, 0, 0, 0);
+    }
+    static AMCT_DEV uint32_t out_bits(float v) { return f32_to_f16_bits(v); }
+};
 // the matching order of 8 activations: (k0, k4), (k1, k5), (k2, k6), (k3, k7)
 AMCT_DEV uint4 st_interleave8(const uint4& x) {
     return make_uint4(__builtin_amdgcn_perm(x.z, x.x, 0x05040100u), __builtin_amdgcn_perm(x.z, x.x, 0x07060302u),
                       __builtin_amdgcn_perm(x.w, x.y, 0x05040100u), __builtin_amdgcn_perm(x.w, x.y, 0x07060302u));
 }
+template <int DT>
 AMCT_DEV float st_sum8(const uint4& x) {
     const uint32_t xs[4] = {x.x, x.y, x.z, x.w};
     float t = 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) t = t + (__uint_as_float(xs[i] << 16) + __uint_as_float(xs[i] & 0xFFFF0000u));
+    for (int i = 0; i < 4; ++i) t = t + (StAct<DT>::lo(xs[i]) + StAct<DT>::hi(xs[i]));
     return t;
 }
+template <int DT>
 AMCT_DEV uint4 st_smooth8(const uint4& x, const uint4& c) {
     const uint32_t xs[4] = {x.x, x.y, x.z, x.w}, cs[4] = {c.x, c.y, c.z, c.w};
     uint32_t o[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-        o[i] = st_pack2(__uint_as_float(xs[i] << 16) * __uint_as_float(cs[i] << 16),
-                        __uint_as_float(xs[i] & 0xFFFF0000u) * __uint_as_float(cs[i] & 0xFFFF0000u));
+        o[i] = StAct<DT>::pack2(StAct<DT>::lo(xs[i]) * StAct<DT>::lo(cs[i]), StAct<DT>::hi(xs[i]) * StAct<DT>::hi(cs[i]));
     return make_uint4(o[0], o[1], o[2], o[3]);
 }
 
 // XJ: 16-byte activation vectors a thread stages (clamped duplicates beyond the tensor)
 
-template <int KS, int CG, int NL, int XJ, bool SMOOTH>
+template <int DT, int KS, int CG, int NL, int XJ, bool SMOOTH>
 __global__ __launch_bounds__(KS * CG * 64) void w4a16_stream(StreamArgs a) {
     static_assert(NL % 2 == 0, "the weight loads come in pairs");
     extern __shared__ __align__(16) uint8_t lds[];
@@ -146,9 +173,9 @@ __global__ __launch_bounds__(KS * CG * 64) void w4a16_stream(StreamArgs a) {
 #pragma unroll
     for (int j = 0; j < XJ; ++j) {
         const uint32_t v = tid + NT * j;
-        if constexpr (SMOOTH) xv[j] = st_smooth8(xv[j], cv[j]);
+        if constexpr (SMOOTH) xv[j] = st_smooth8<DT>(xv[j], cv[j]);
         // 16 consecutive lanes hold 128 consecutive elements of one row; whole groups of 16 lanes are valid or not
-        float t = st_sum8(xv[j]);
+        float t = st_sum8<DT>(xv[j]);
         t = t + __shfl_xor(t, 1);
         t = t + __shfl_xor(t, 2);
         t = t + __shfl_xor(t, 4);
@@ -169,9 +196,9 @@ __global__ __launch_bounds__(KS * CG * 64) void w4a16_stream(StreamArgs a) {
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
         // the loads retire in order: step i waits for wv[i] only, the NL - 1 - i younger ones stay in flight
-        s8bf fa[4];
+        uint4 fa[4];
 #pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4) fa[s4] = *reinterpret_cast<const s8bf*>(xlane + i * 256 + s4 * 16);
+        for (int s4 = 0; s4 < 4; ++s4) fa[s4] = *reinterpret_cast<const uint4*>(xlane + i * 256 + s4 * 16);
         if ((i & 1) == 0) {                          // both registers of the pair have landed: swap halves
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
@@ -184,7 +211,7 @@ __global__ __launch_bounds__(KS * CG * 64) void w4a16_stream(StreamArgs a) {
         const uint32_t ws[4] = {wv[i].x, wv[i].y, wv[i].z, wv[i].w};
 #pragma unroll
         for (int s4 = 0; s4 < 4; ++s4)
-            P = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[s4], __builtin_bit_cast(s8bf, st_int8x(ws[s4])), P, 0, 0, 0);
+            P = StAct<DT>::mfma(fa[s4], StAct<DT>::int8x(ws[s4]), P);
         {                                             // a step is one group of 128: fold it into the result
             const uint32_t gi = (ks * kw) / 128 + i;
             const uint32_t sbits = (fsw[i / 2] >> (16 * (i & 1))) & 0xFFFFu;
@@ -222,12 +249,12 @@ __global__ __launch_bounds__(KS * CG * 64) void w4a16_stream(StreamArgs a) {
             const int m = 4 * g + r;
             float v = y[r];
             if (a.bias) v = v + b;
-            if (m < (int)M) a.out[(size_t)m * a.N + ncol] = (uint16_t)f32_to_bf16_bits(v);
+            if (m < (int)M) a.out[(size_t)m * a.N + ncol] = (uint16_t)StAct<DT>::out_bits(v);
         }
     }
 }
 
-template <int KS, int CG, int NL, bool SMOOTH>
+template <int DT, int KS, int CG, int NL, bool SMOOTH>
 static int stream_launch_x(const StreamArgs& a, size_t lds_bytes, hipStream_t st) {
     constexpr int NT = KS * CG * 64;
     const int n_xv = a.M * (a.K / 8);
@@ -235,7 +262,7 @@ static int stream_launch_x(const StreamArgs& a, size_t lds_bytes, hipStream_t st
     const dim3 grid((unsigned)((a.N + CG * 16 - 1) / (CG * 16)));
 #define AMCT_STREAM_GO(XJ)                                                                                          \
     {                                                                                                               \
-        auto kern = &w4a16_stream<KS, CG, NL, XJ, SMOOTH>;                                                          \
+        auto kern = &w4a16_stream<DT, KS, CG, NL, XJ, SMOOTH>;                                                          \
         if (lds_bytes > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                       \
                                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess) { \
             (void)hipGetLastError();                                                                                \
@@ -254,7 +281,7 @@ static int stream_launch_x(const StreamArgs& a, size_t lds_bytes, hipStream_t st
 // Returns AMCT_E_UNSUPPORTED when the shape is not one this kernel takes (the caller then uses its other kernels).
 int w4a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
                           const uint8_t* zeros, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group,
-                          hipStream_t st) {
+                          int dtype, hipStream_t st) {
     // one group per step of 128 elements of K (the per-group partial sums of a step cannot be separated otherwise)
     if (M < 1 || M > 16 || (K != 1024 && K != 2048 && K != 4096) || group != 128 || N > (int64_t(1) << 30)) return AMCT_E_UNSUPPORTED;
     if (!aligned16(x) || !aligned16(wq) || (smooth && !aligned16(smooth)) || ((uintptr_t)scales & 3) || ((uintptr_t)zeros & 3))
@@ -274,8 +301,13 @@ int w4a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, 
     const size_t lds_bytes = img > red ? img : red;
     if (lds_bytes > 160 * 1024) return AMCT_E_UNSUPPORTED;
 #define AMCT_STREAM_SHAPE(CG_, NL_)                                                                       \
-    if (cg == CG_ && nl == NL_)                                                                           \
-        return smooth ? stream_launch_x<4, CG_, NL_, true>(a, lds_bytes, st) : stream_launch_x<4, CG_, NL_, false>(a, lds_bytes, st);
+    if (cg == CG_ && nl == NL_) {                                                                         \
+        if (dtype == AMCT_F16)                                                                            \
+            return smooth ? stream_launch_x<AMCT_F16, 4, CG_, NL_, true>(a, lds_bytes, st)                \
+                          : stream_launch_x<AMCT_F16, 4, CG_, NL_, false>(a, lds_bytes, st);              \
+        return smooth ? stream_launch_x<AMCT_BF16, 4, CG_, NL_, true>(a, lds_bytes, st)                   \
+                      : stream_launch_x<AMCT_BF16, 4, CG_, NL_, false>(a, lds_bytes, st);                 \
+    }
     AMCT_STREAM_SHAPE(4, 8)
     AMCT_STREAM_SHAPE(2, 8)
     AMCT_STREAM_SHAPE(1, 8)

@@ -256,7 +256,7 @@ int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s_tok, const
  * once up front instead of inside every column tile (same results; the fast bf16 tile kernels need it, without it such
  * calls take slower kernels that smooth in place); 0 bytes are asked for otherwise.
  * Arithmetic of the dequantisation: the tile kernels (M > 16) feed dtype((u - zero) * scale) to the matrix pipe; the
- * weight-streaming bf16 kernel for M <= 16 (K % 1024 == 0, group = 128) keeps the weight as the exact integer and applies
+ * weight-streaming kernel for M <= 16 (bf16 or fp16, K of 1024 / 2048 / 4096, group = 128) keeps the weight as the exact integer and applies
  * scale and zero per group in fp32, i.e. the dequantised weight is not rounded to bf16 there (the fp32 weight * scale of
  * tests/amct_pytorch/mock_torch_npu.py:33-55).  Both stay within 1e-3 of the exact result. */
 size_t amct_gemm_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K, int group, int has_smooth);

@@ -275,9 +275,9 @@ def w4a16_forward_f64(x, codes_nk, scale_ng, antioffset_ng, group_size, bias=Non
 
 
 def w4a16_streams(M, K, group_size, dtype=torch.bfloat16):
-    """Whether the int4 GEMM takes its weight-streaming kernel for this shape (a few bf16 rows, K of 1024, 2048 or
-    4096, groups of 128): that kernel does not round the dequantised weight."""
-    return dtype == torch.bfloat16 and 1 <= M <= 16 and K in (1024, 2048, 4096) and group_size == 128
+    """Whether the int4 GEMM takes its weight-streaming kernel for this shape (a few rows of bf16 or fp16 activations, K
+    of 1024, 2048 or 4096, groups of 128): that kernel does not round the dequantised weight."""
+    return dtype in (torch.bfloat16, torch.float16) and 1 <= M <= 16 and K in (1024, 2048, 4096) and group_size == 128
 
 
 # --------------------------------------------------------------------------

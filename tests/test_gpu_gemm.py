@@ -124,7 +124,7 @@ def w4a16_oracle(x, codes, scales, zeros, group, smooth, bias, rows=None):
     anti = -(zeros.to(torch.float32) - 8)
     m = x.shape[0] if rows is None else rows
     return od.w4a16_forward_f64(x, signed, scales, anti, group, bias, None if smooth is None else smooth.reshape(1, -1),
-                                round_weight=not od.w4a16_streams(m, x.shape[1], group))
+                                round_weight=not od.w4a16_streams(m, x.shape[1], group, x.dtype))
 
 
 @pytest.mark.parametrize("M,N,K,group", [(300, 1000, 256, 64), (256, 448, 128, 128), (2048, 14336, 256, 128), (2000, 14328, 128, 64),
@@ -173,30 +173,34 @@ def test_w4a16_vs_oracle(dev, M, N, K, group, sdt):
 
 @pytest.mark.parametrize("M,N,K", [(1, 64, 1024), (16, 200, 2048), (9, 72, 1024), (5, 33, 2048), (16, 1000, 1024),
                                    (13, 14336, 4096), (1, 14336, 2048), (3, 16, 4096), (16, 15, 1024)])
-def test_w4a16_weight_streaming_kernel(dev, M, N, K):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_w4a16_weight_streaming_kernel(dev, M, N, K, dtype):
     """The kernel for a few rows (M <= 16, K of 1024/2048/4096, groups of 128): every block width, ragged N, both factor
     dtypes, with and without smoothing, against the fp64 anchor whose dequantised weight is not rounded; then the
     integer special case (scale 1, small integer activations), where both readings of the dequantisation give the same
     bits as an integer matmul."""
-    assert od.w4a16_streams(M, K, 128)
+    assert od.w4a16_streams(M, K, 128, dtype)
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
     for sdt in (torch.float16, torch.bfloat16):
         x, codes, scales, zeros, smooth, bias = w4a16_case(M, N, K, 128, 140 + M, sdt)
+        x, smooth = x.to(dtype), smooth.to(dtype)
         packed = workloads.pack_nibbles(codes).to(dev)
         for sm, b in ((None, None), (smooth, bias)):
             out = ops.gemm_w4a16(x.to(dev), packed, scales.to(dev), zeros.to(dev), 128,
                                  None if sm is None else sm.to(dev), None if b is None else b.to(dev))
             want = w4a16_oracle(x, codes, scales, zeros, 128, sm, b)
             err = (out.cpu().double() - want).abs()
-            # exact weights, fp32 accumulation: half a bf16 ulp of the value plus 1e-5 of the row's largest output
-            tol = 1e-5 * want.abs().amax(dim=1, keepdim=True) + want.abs() * 2.0 ** -8
+            # exact weights, fp32 accumulation: half an ulp of the value plus 1e-5 of the row's largest output
+            tol = 1e-5 * want.abs().amax(dim=1, keepdim=True) + want.abs() * ulp
             assert (err <= tol).all(), (err.max().item(), tol.min().item())
+            assert out.dtype == dtype
     g = torch.Generator().manual_seed(141)
-    xi = torch.randint(-4, 5, (M, K), generator=g).to(torch.bfloat16)
+    xi = torch.randint(-4, 5, (M, K), generator=g).to(dtype)
     ones = torch.ones(N, K // 128, dtype=torch.float16)
     out = ops.gemm_w4a16(xi.to(dev), packed, ones.to(dev), zeros.to(dev), 128)
     wi = codes.float() - zeros.float().repeat_interleave(128, dim=1)
     want = torch.matmul(xi.double(), wi.double().t())                # integers below 2^24: exact in the kernel's fp32 too
-    assert_bits_equal(out, want.to(torch.bfloat16), "integer special case")
+    assert_bits_equal(out, want.to(dtype), "integer special case")
 
 
 def w8a16_case(M, N, K, group, seed, dtype, sdt, sym):
