@@ -51,7 +51,16 @@ AMCT_DEV uint32_t pack_bf16x2(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, v2bf));
 }
 
-// 8 nibbles of `w` (element j in bits 4j..4j+3) -> 8 bf16 of (u - z) * s, as 4 packed dwords
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+// the same for fp16: one v_cvt_pk_f16_f32
+AMCT_DEV uint32_t pack_f16x2(float lo, float hi) {
+    const v2f f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, v2h));
+}
+template <bool AF16> AMCT_DEV uint32_t pack_act2(float lo, float hi) { return AF16 ? pack_f16x2(lo, hi) : pack_bf16x2(lo, hi); }
+
+// 8 nibbles of `w` (element j in bits 4j..4j+3) -> 8 values of (u - z) * s in the activation type, as 4 packed dwords
+template <bool AF16 = false>
 AMCT_DEV uint4 dequant8(uint32_t w, float s, float nzs) {
     uint32_t lo = w & 0x0F0F0F0Fu;                  // elements 0,2,4,6 in bytes 0..3
     uint32_t hi = (w >> 4) & 0x0F0F0F0Fu;           // elements 1,3,5,7
@@ -64,7 +73,7 @@ AMCT_DEV uint4 dequant8(uint32_t w, float s, float nzs) {
     for (int b = 0; b < 4; ++b) {
         const float e0 = (float)((lo >> (8 * b)) & 0xFFu);
         const float e1 = (float)((hi >> (8 * b)) & 0xFFu);
-        o[b] = pack_bf16x2(__builtin_fmaf(e0, s, nzs), __builtin_fmaf(e1, s, nzs));
+        o[b] = pack_act2<AF16>(__builtin_fmaf(e0, s, nzs), __builtin_fmaf(e1, s, nzs));
     }
     return make_uint4(o[0], o[1], o[2], o[3]);
 }
@@ -713,7 +722,7 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
     }
 }
 
-template <bool SF16, int WM, int WN, int TI, int TJ, int STAGES, int SB = STAGES>
+template <bool SF16, int WM, int WN, int TI, int TJ, int STAGES, int SB = STAGES, bool AF16 = false>
 AMCT_DEV void w4a16_wide_body16(const W4A16Args& a, uint8_t* smem, const int64_t m0, const int64_t n0) {
     using Sh = WideTile<WM, WN, TI, TJ, STAGES, SB>;
     constexpr int kABytes = Sh::kABytes, kBBytes = Sh::kBBytes, kBBase = Sh::kBBase;
@@ -784,7 +793,7 @@ AMCT_DEV void w4a16_wide_body16(const W4A16Args& a, uint8_t* smem, const int64_t
         nzs = -((float)zreg[slot] * sc);
     };
     auto write_b = [&](int slot, int stg, int c) {                 // dequantise 8 weights into LDS
-        *reinterpret_cast<uint4*>(smem + stg * kBBytes + bdst[c]) = dequant8(wreg[slot][c], sc, nzs);
+        *reinterpret_cast<uint4*>(smem + stg * kBBytes + bdst[c]) = dequant8<AF16>(wreg[slot][c], sc, nzs);
     };
     // Wait until the weight loads of the previous iteration and the activation loads issued STAGES-1 iterations ago
     // have landed and this wave's LDS operations are done.  An iteration issues its 3 weight loads in the middle of the
@@ -834,7 +843,13 @@ AMCT_DEV void w4a16_wide_body16(const W4A16Args& a, uint8_t* smem, const int64_t
     };
     auto mfma_one = [&](int u, int m) {
         const int i = m / TB, j = m % TB;
-        acc[(u & 1) * TA + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fb[(u >> 1) & 1][j], acc[(u & 1) * TA + i][j], 0, 0, 0);
+        if constexpr (AF16) {
+            typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+            acc[(u & 1) * TA + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, fa[i]), __builtin_bit_cast(v8h, fb[(u >> 1) & 1][j]),
+                                                                          acc[(u & 1) * TA + i][j], 0, 0, 0);
+        } else {
+            acc[(u & 1) * TA + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fb[(u >> 1) & 1][j], acc[(u & 1) * TA + i][j], 0, 0, 0);
+        }
     };
     // dequantisation of 8 weights in four pieces of two, so that the pieces can sit between MFMAs
     uint32_t dq_lo = 0, dq_hi = 0, dq_o[4];
@@ -847,7 +862,7 @@ AMCT_DEV void w4a16_wide_body16(const W4A16Args& a, uint8_t* smem, const int64_t
         }
         const float e0 = (float)((dq_lo >> (8 * bb)) & 0xFFu);
         const float e1 = (float)((dq_hi >> (8 * bb)) & 0xFFu);
-        dq_o[bb] = pack_bf16x2(__builtin_fmaf(e0, sc, nzs), __builtin_fmaf(e1, sc, nzs));
+        dq_o[bb] = pack_act2<AF16>(__builtin_fmaf(e0, sc, nzs), __builtin_fmaf(e1, sc, nzs));
     };
     auto dq_write = [&](int stg, int c) {
         *reinterpret_cast<uint4*>(smem + stg * kBBytes + bdst[c]) = make_uint4(dq_o[0], dq_o[1], dq_o[2], dq_o[3]);
@@ -969,7 +984,7 @@ AMCT_DEV void w4a16_wide_body16(const W4A16Args& a, uint8_t* smem, const int64_t
 #pragma unroll
                 for (int j = 0; j < TB; ++j)
                     *reinterpret_cast<uint16_t*>(wbase + (16 * hh + r) * kPatchRow + j * 32) =
-                        (uint16_t)f32_to_bf16_bits(acc[2 * i + hh][j][r] + bs[j]);
+                        (uint16_t)(AF16 ? f32_to_f16_bits(acc[2 * i + hh][j][r] + bs[j]) : f32_to_bf16_bits(acc[2 * i + hh][j][r] + bs[j]));
 #pragma unroll
         for (int it = 0; it < 32 * CPR / 64; ++it) {
             const int idx = it * 64 + lane;                        // 16-byte chunk of the patch, row-major
@@ -990,11 +1005,11 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM
     w4a16_wide_body<SF16, WM, WN, TI, TJ, STAGES, SB>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
 }
 
-template <bool SF16, int WM, int WN, int TI, int TJ, int STAGES, int SB = STAGES>
+template <bool SF16, int WM, int WN, int TI, int TJ, int STAGES, int SB = STAGES, bool AF16 = false>
 __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM * WN / 4, WM * WN / 4))) void w4a16_tile_wide16(W4A16Args a) {
     using Sh = WideTile<WM, WN, TI, TJ, STAGES, SB>;
     __shared__ __attribute__((aligned(1024))) uint8_t smem[Sh::kSmem];
-    w4a16_wide_body16<SF16, WM, WN, TI, TJ, STAGES, SB>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
+    w4a16_wide_body16<SF16, WM, WN, TI, TJ, STAGES, SB, AF16>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
 }
 
 // ---------------------------------------------------------------------------
@@ -1325,6 +1340,20 @@ __global__ __launch_bounds__(kBlock) void smooth_rows(const uint16_t* x, const u
     for (int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += stride) {
         const uint4 c = ldg16(smooth + (v % kvec) * 8);
         stg16(y + v * 8, smooth8(ldg16_nt(x + v * 8), c));
+    }
+}
+// the same for fp16 activations: x' = fp16(x * smooth[k])
+__global__ __launch_bounds__(kBlock) void smooth_rows_f16(const uint16_t* x, const uint16_t* smooth, uint16_t* y, int64_t nvec, int kvec) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += stride) {
+        const uint4 c = ldg16(smooth + (v % kvec) * 8), xv = ldg16_nt(x + v * 8);
+        const uint32_t xs[4] = {xv.x, xv.y, xv.z, xv.w}, cs[4] = {c.x, c.y, c.z, c.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            o[i] = pack_f16x2(f16_bits_to_f32(xs[i] & 0xFFFFu) * f16_bits_to_f32(cs[i] & 0xFFFFu),
+                              f16_bits_to_f32(xs[i] >> 16) * f16_bits_to_f32(cs[i] >> 16));
+        stg16(y + v * 8, make_uint4(o[0], o[1], o[2], o[3]));
     }
 }
 
@@ -1755,6 +1784,35 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
             const int rc = w4a16_stream_dispatch(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, dtype,
                                                  (hipStream_t)stream);
             if (rc != AMCT_E_UNSUPPORTED) return rc;
+        }
+        // many rows: the 256x256 tile kernel with fp16 operands (the same body: the dequantised weight and the smoothed
+        // activations are rounded to fp16 instead of bf16, one v_cvt_pk_f16_f32 per pair, and the MFMA is the f16 one);
+        // the same conditions as for bf16 below, and the caller's workspace when the activations are to be smoothed
+        {
+            hipStream_t st = (hipStream_t)stream;
+            const int64_t cus = current_cu_count();
+            const int64_t mt = (M + 127) / 128, nt256 = (N + 255) / 256, G = K / group;
+            const bool ok = aligned16(x) && aligned16(wq) && (!smooth || aligned16(smooth)) && aligned16(out) && K % 128 == 0 &&
+                            K < 65536 && N % 8 == 0 && group % 64 == 0 && M * K * 2 < (int64_t(1) << 32) &&
+                            N * (K / 2) < (int64_t(1) << 32) && N * G * 2 < (int64_t(1) << 32) && M >= 256 && cus > 0 &&
+                            mt * nt256 > cus && (M + kQM - 1) / kQM <= 65535 &&
+                            (!smooth || (workspace && workspace_bytes >= (size_t)(M * K * 2) && aligned16(workspace)));
+            if (ok) {
+                W4A16Args a{(const uint16_t*)x, (const uint16_t*)smooth, wq, scales, zeros, bias, (uint16_t*)out, M, N, K, group,
+                            scale_dtype, (uint32_t)(0x100000000ull / (uint64_t)group) + 1u};
+                if (smooth) {
+                    const int64_t nvec = M * K / 8;
+                    int64_t nb = (nvec + kBlock - 1) / kBlock;
+                    if (nb > 16384) nb = 16384;
+                    hipLaunchKernelGGL(smooth_rows_f16, dim3((unsigned)nb), dim3(kBlock), 0, st, a.x, a.smooth, (uint16_t*)workspace, nvec, (int)(K / 8));
+                    a.x = (const uint16_t*)workspace;
+                    a.smooth = nullptr;
+                }
+                const dim3 grid((unsigned)((N + kQN - 1) / kQN), (unsigned)((M + kQM - 1) / kQM));
+                if (scale_dtype == AMCT_F16) hipLaunchKernelGGL((w4a16_tile_wide16<true, 2, 4, 4, 2, 2, 2, true>), grid, dim3(kQThreads), 0, st, a);
+                else hipLaunchKernelGGL((w4a16_tile_wide16<false, 2, 4, 4, 2, 2, 2, true>), grid, dim3(kQThreads), 0, st, a);
+                return hip_status();
+            }
         }
         return wq16_int4_f16(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, (hipStream_t)stream);
     }

@@ -501,10 +501,9 @@ def gemm_w4a16(x, wq_packed, scales, zeros, group, smooth=None, bias=None):
     # the workspace the library asks for: the smoothed activations for the tile kernels, or the activation image the
     # weight-streaming kernel for a few rows fetches
     ws = None
-    if x.dtype == torch.bfloat16:
-        nbytes = _lib.load().amct_gemm_w4a16_workspace_bytes(M, N, K, group, int(smooth is not None))
-        if nbytes:
-            ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    nbytes = _lib.load().amct_gemm_w4a16_workspace_bytes(M, N, K, group, int(smooth is not None))
+    if nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         _lib.check(_lib.load().amct_gemm_w4a16(_p(x), _p(smooth), _p(wq_packed), _p(scales), dtype_code(scales.dtype),
                                                _p(zeros), _p(bias), _p(out), M, N, K, group, dtype_code(x.dtype),

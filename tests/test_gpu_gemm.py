@@ -312,6 +312,29 @@ def test_gemms_at_the_benchmark_size(dev, M):
         assert (err <= tol).all(), (M, sm is not None, err.max().item())
 
 
+@pytest.mark.parametrize("M", [2048, 520])
+def test_w4a16_fp16_at_the_benchmark_size(dev, M):
+    """fp16 activations at N = 14336, K = 4096: many rows take the 256x256 tile kernel with fp16 operands (with the lent
+    workspace when the activations are smoothed, which ops.gemm_w4a16 lends), fewer the shared 128x128 kernel; sampled
+    rows within 1e-3 of the row's largest output (plus half an fp16 ulp of the value) of the fp64 anchor whose
+    dequantised weight is rounded to fp16, every column; both factor dtypes."""
+    N, K, grp = 14336, 4096, 128
+    rows = [r for r in FULL_ROWS if r < M]
+    for sdt in (torch.float16, torch.bfloat16):
+        x, codes, scales, zeros, smooth, bias = w4a16_case(M, N, K, grp, 313, sdt)
+        x, smooth = x.to(torch.float16), smooth.to(torch.float16)
+        packed = workloads.pack_nibbles(codes).to(dev)
+        for sm in (None, smooth):
+            out = ops.gemm_w4a16(x.to(dev), packed, scales.to(dev), zeros.to(dev), grp, None if sm is None else sm.to(dev),
+                                 bias.to(dev))
+            assert out.dtype == torch.float16
+            out = out.cpu()[rows]
+            want = w4a16_oracle(x[rows], codes, scales, zeros, grp, sm, bias, rows=M)
+            err = (out.double() - want).abs()
+            tol = 1e-3 * want.abs().amax(dim=1, keepdim=True) + want.abs() * 2.0 ** -11
+            assert (err <= tol).all(), (M, sdt, sm is not None, float((err / tol).max()))
+
+
 @pytest.mark.parametrize("seed", [1, 2])
 def test_gemm_random_shapes(dev, seed):
     """Seeded random (M, N, K, group, scale dtype, smoothing) over the values at which the libraries switch kernels and
