@@ -486,7 +486,7 @@ struct WideTile {
     static_assert(kNA < 64, "vmcnt range");
 };
 
-template <bool SF16, int WM, int WN, int TI, int TJ, int STAGES, int SB = STAGES>
+template <bool SF16, int WM, int WN, int TI, int TJ, int STAGES, int SB = STAGES, bool AF16 = false>
 AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m0, const int64_t n0) {
     using Sh = WideTile<WM, WN, TI, TJ, STAGES, SB>;
     constexpr int kABytes = Sh::kABytes, kBBytes = Sh::kBBytes, kBBase = Sh::kBBase;
@@ -550,7 +550,7 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
         nzs = -((float)zreg[slot] * sc);
     };
     auto write_b = [&](int slot, int stg, int c) {                 // dequantise 8 weights into LDS
-        *reinterpret_cast<uint4*>(smem + stg * kBBytes + bdst[c]) = dequant8(wreg[slot][c], sc, nzs);
+        *reinterpret_cast<uint4*>(smem + stg * kBBytes + bdst[c]) = dequant8<AF16>(wreg[slot][c], sc, nzs);
     };
     // Wait until the weight loads of the previous iteration and the activation loads issued STAGES-1 iterations ago
     // have landed and this wave's LDS operations are done.  An iteration issues its 3 weight loads in the middle of the
@@ -596,7 +596,12 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
     };
     auto mfma_one = [&](int m, const v8bf (&fa)[TI], const v8bf (&fb)[TJ]) {
         const int i = m / TJ, j = m % TJ;
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        if constexpr (AF16) {
+            typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, fa[i]), __builtin_bit_cast(v8h, fb[j]), acc[i][j], 0, 0, 0);
+        } else {
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
     };
 
     // prologue: B(0), B(1) and A(0 .. STAGES-2); once B(0) is dequantised into stage 0 its slot takes B(2), and
@@ -708,7 +713,7 @@ AMCT_DEV void w4a16_wide_body(const W4A16Args& a, uint8_t* smem, const int64_t m
             const int prow0 = 8 * (r >> 2) + (r & 3);
 #pragma unroll
             for (int j = 0; j < TJ; ++j)
-                *reinterpret_cast<uint16_t*>(wbase + prow0 * kPatchRow + j * 64) = (uint16_t)f32_to_bf16_bits(acc[i][j][r] + bs[j]);
+                *reinterpret_cast<uint16_t*>(wbase + prow0 * kPatchRow + j * 64) = (uint16_t)(AF16 ? f32_to_f16_bits(acc[i][j][r] + bs[j]) : f32_to_bf16_bits(acc[i][j][r] + bs[j]));
         }
 #pragma unroll
         for (int it = 0; it < 32 * CPR / 64; ++it) {
@@ -998,11 +1003,11 @@ AMCT_DEV void w4a16_wide_body16(const W4A16Args& a, uint8_t* smem, const int64_t
 }
 
 // blockIdx.x: column tile, blockIdx.y: row tile
-template <bool SF16, int WM, int WN, int TI, int TJ, int STAGES, int SB = STAGES>
+template <bool SF16, int WM, int WN, int TI, int TJ, int STAGES, int SB = STAGES, bool AF16 = false>
 __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM * WN / 4, WM * WN / 4))) void w4a16_tile_wide(W4A16Args a) {
     using Sh = WideTile<WM, WN, TI, TJ, STAGES, SB>;
     __shared__ __attribute__((aligned(1024))) uint8_t smem[Sh::kSmem];
-    w4a16_wide_body<SF16, WM, WN, TI, TJ, STAGES, SB>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
+    w4a16_wide_body<SF16, WM, WN, TI, TJ, STAGES, SB, AF16>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
 }
 
 template <bool SF16, int WM, int WN, int TI, int TJ, int STAGES, int SB = STAGES, bool AF16 = false>
@@ -1785,18 +1790,18 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
                                                  (hipStream_t)stream);
             if (rc != AMCT_E_UNSUPPORTED) return rc;
         }
-        // many rows: the 256x256 tile kernel with fp16 operands (the same body: the dequantised weight and the smoothed
-        // activations are rounded to fp16 instead of bf16, one v_cvt_pk_f16_f32 per pair, and the MFMA is the f16 one);
-        // the same conditions as for bf16 below, and the caller's workspace when the activations are to be smoothed
+        // more than 64 rows: the tile kernels with fp16 operands (the same bodies: the dequantised weight and the smoothed
+        // activations are rounded to fp16 instead of bf16, one v_cvt_pk_f16_f32 per pair, and the MFMAs are the f16 ones);
+        // the same conditions and block shapes as for bf16 below (without the kernels with specialised waves), and the
+        // caller's workspace when the activations are to be smoothed
         {
             hipStream_t st = (hipStream_t)stream;
             const int64_t cus = current_cu_count();
-            const int64_t mt = (M + 127) / 128, nt256 = (N + 255) / 256, G = K / group;
+            const int64_t mt = (M + 127) / 128, nt64 = (N + 63) / 64, nt128 = (N + 127) / 128, nt256 = (N + 255) / 256, G = K / group;
             const bool ok = aligned16(x) && aligned16(wq) && (!smooth || aligned16(smooth)) && aligned16(out) && K % 128 == 0 &&
                             K < 65536 && N % 8 == 0 && group % 64 == 0 && M * K * 2 < (int64_t(1) << 32) &&
-                            N * (K / 2) < (int64_t(1) << 32) && N * G * 2 < (int64_t(1) << 32) && M >= 256 && cus > 0 &&
-                            mt * nt256 > cus && (M + kQM - 1) / kQM <= 65535 &&
-                            (!smooth || (workspace && workspace_bytes >= (size_t)(M * K * 2) && aligned16(workspace)));
+                            N * (K / 2) < (int64_t(1) << 32) && N * G * 2 < (int64_t(1) << 32) && M > 64 && cus > 0 &&
+                            mt <= 65535 && (!smooth || (workspace && workspace_bytes >= (size_t)(M * K * 2) && aligned16(workspace)));
             if (ok) {
                 W4A16Args a{(const uint16_t*)x, (const uint16_t*)smooth, wq, scales, zeros, bias, (uint16_t*)out, M, N, K, group,
                             scale_dtype, (uint32_t)(0x100000000ull / (uint64_t)group) + 1u};
@@ -1808,9 +1813,22 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
                     a.x = (const uint16_t*)workspace;
                     a.smooth = nullptr;
                 }
+                int shape = 0;
+                if (mt * nt64 <= cus) shape = 4;
+                else if (mt * nt128 <= cus) shape = 1;
+                else if (mt * nt256 <= cus || M < 256) shape = 2;
                 const dim3 grid((unsigned)((N + kQN - 1) / kQN), (unsigned)((M + kQM - 1) / kQM));
-                if (scale_dtype == AMCT_F16) hipLaunchKernelGGL((w4a16_tile_wide16<true, 2, 4, 4, 2, 2, 2, true>), grid, dim3(kQThreads), 0, st, a);
-                else hipLaunchKernelGGL((w4a16_tile_wide16<false, 2, 4, 4, 2, 2, 2, true>), grid, dim3(kQThreads), 0, st, a);
+#define AMCT_LAUNCH_WIDE_F16(SF)                                                                                       \
+    {                                                                                                                  \
+        if (shape == 4) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 2, 1, 3, 3, true>), dim3((unsigned)nt64, (unsigned)mt), dim3(256), 0, st, a); \
+        else if (shape == 1) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 2, 2, 3, 3, true>), dim3((unsigned)nt128, (unsigned)mt), dim3(256), 0, st, a); \
+        else if (shape == 2 && M > 256 && (M + 255) / 256 * nt128 <= cus) hipLaunchKernelGGL((w4a16_tile_wide<SF, 4, 2, 2, 2, 3, 3, true>), dim3((unsigned)nt128, (unsigned)((M + 255) / 256)), dim3(512), 0, st, a); \
+        else if (shape == 2) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 4, 2, 2, 3, 3, true>), dim3((unsigned)nt256, (unsigned)mt), dim3(512), 0, st, a); \
+        else hipLaunchKernelGGL((w4a16_tile_wide16<SF, 2, 4, 4, 2, 2, 2, true>), grid, dim3(kQThreads), 0, st, a);     \
+    }
+                if (scale_dtype == AMCT_F16) AMCT_LAUNCH_WIDE_F16(true)
+                else AMCT_LAUNCH_WIDE_F16(false)
+#undef AMCT_LAUNCH_WIDE_F16
                 return hip_status();
             }
         }

@@ -312,13 +312,14 @@ def test_gemms_at_the_benchmark_size(dev, M):
         assert (err <= tol).all(), (M, sm is not None, err.max().item())
 
 
-@pytest.mark.parametrize("M", [2048, 520])
-def test_w4a16_fp16_at_the_benchmark_size(dev, M):
-    """fp16 activations at N = 14336, K = 4096: many rows take the 256x256 tile kernel with fp16 operands (with the lent
-    workspace when the activations are smoothed, which ops.gemm_w4a16 lends), fewer the shared 128x128 kernel; sampled
-    rows within 1e-3 of the row's largest output (plus half an fp16 ulp of the value) of the fp64 anchor whose
-    dequantised weight is rounded to fp16, every column; both factor dtypes."""
-    N, K, grp = 14336, 4096, 128
+@pytest.mark.parametrize("M,N,K", [(2048, 14336, 4096), (520, 14336, 4096), (300, 14336, 4096), (130, 14336, 4096),
+                                   (70, 14336, 4096), (200, 20000, 1024), (65, 72, 128)])
+def test_w4a16_fp16_at_the_benchmark_size(dev, M, N, K):
+    """fp16 activations, more than 64 rows: the tile kernels with fp16 operands, every block shape the dispatch knows
+    (256x256, 256x128, 128x256, 128x128, 128x64), with the lent workspace when the activations are smoothed (which
+    ops.gemm_w4a16 lends); sampled rows within 1e-3 of the row's largest output (plus half an fp16 ulp of the value) of
+    the fp64 anchor whose dequantised weight is rounded to fp16, every column; both factor dtypes."""
+    grp = 128
     rows = [r for r in FULL_ROWS if r < M]
     for sdt in (torch.float16, torch.bfloat16):
         x, codes, scales, zeros, smooth, bias = w4a16_case(M, N, K, grp, 313, sdt)
