@@ -1362,6 +1362,26 @@ __global__ __launch_bounds__(kBlock) void smooth_rows_f16(const uint16_t* x, con
     }
 }
 
+// The whole weight dequantised once, dt((u - z) * s) as the tile kernels compute it per block, 32 weights (16 bytes of
+// nibbles, one group: group % 32 == 0) per thread and step: for so many rows that dequantising inside every row tile
+// costs more than writing and re-reading the 16-bit weight (the product is then the plain 16-bit GEMM on the large
+// tiles of the W8A8 kernel, gemm_w8a8.hip: gemm16_tiles).
+template <bool AF16>
+__global__ __launch_bounds__(kBlock) void w4_dequant_rows(W4A16Args a, uint16_t* wdq, int64_t nvec) {   // nvec = N * K / 32
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    const int64_t G = a.K / a.group;
+    for (int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += stride) {
+        const int64_t e = v * 32, row = e / a.K, k = e - row * a.K;
+        const int64_t gi = row * G + k / a.group;
+        const float s = load_scale(a, gi), nzs = -((float)a.zeros[gi] * s);
+        const uint4 w = ldg16_nt(a.wq + e / 2);
+        stg16(wdq + e, dequant8<AF16>(w.x, s, nzs));
+        stg16(wdq + e + 8, dequant8<AF16>(w.y, s, nzs));
+        stg16(wdq + e + 16, dequant8<AF16>(w.z, s, nzs));
+        stg16(wdq + e + 24, dequant8<AF16>(w.w, s, nzs));
+    }
+}
+
 // ---------------------------------------------------------------------------
 // decode kernel (M <= 16 * MT, K % 128 == 0, group % 32 == 0): weight streaming.
 // A block owns 64 output columns; its waves split K in runs of 128 (one iteration = 4 MFMA k-slots of
@@ -1762,13 +1782,59 @@ int w4a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, 
                           const uint8_t* zeros, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group,
                           int dtype, hipStream_t st);              // gemm_w4a16_stream.hip
 
+int gemm16_tiles(const void* x, const void* w, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int dtype,
+                 hipStream_t st);                                  // gemm_w8a8.hip
+
+// From this many rows on, dequantising the weight once into a lent workspace and running the plain 16-bit GEMM beats
+// dequantising inside every row tile.  Measured on W[14336,4096] with smoothing, fused kernel / two passes: M = 1024
+// 130 / 141 us, 1536 214 / 209, 2048 221 / 217, 3072 332 / 331, 4096 445 / 393: the weight pass costs 35 us, a row of
+// the plain GEMM 0.083 us against 0.107 us for the fused kernel.
+constexpr int64_t kTwoPassFrom = 3584;
+
+static size_t two_pass_workspace(int64_t M, int64_t N, int64_t K, int group, int has_smooth) {
+    if (M < kTwoPassFrom || K % 64 != 0 || N % 8 != 0 || group % 32 != 0 || K % group != 0 || N * K * 2 >= (int64_t(1) << 32) ||
+        M * K * 2 >= (int64_t(1) << 32))
+        return 0;
+    return (size_t)N * (size_t)K * 2 + (has_smooth ? (size_t)M * (size_t)K * 2 : 0);
+}
+
+// dequantise, smooth, multiply; AMCT_E_UNSUPPORTED when the shape or the workspace does not allow it
+static int two_pass(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype, const uint8_t* zeros,
+                    const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group, int dtype, void* workspace,
+                    size_t workspace_bytes, hipStream_t st) {
+    const size_t need = two_pass_workspace(M, N, K, group, smooth != nullptr);
+    if (!need || !workspace || workspace_bytes < need || !aligned16(workspace) || !aligned16(x) || !aligned16(wq) || !aligned16(out) ||
+        (smooth && !aligned16(smooth)))
+        return AMCT_E_UNSUPPORTED;
+    W4A16Args a{(const uint16_t*)x, (const uint16_t*)smooth, wq, scales, zeros, bias, (uint16_t*)out, M, N, K, group, scale_dtype,
+                (uint32_t)(0x100000000ull / (uint64_t)group) + 1u};
+    uint16_t* wdq = reinterpret_cast<uint16_t*>(workspace);
+    uint16_t* xs = wdq + (size_t)N * (size_t)K;
+    const int64_t nvec_w = N * K / 32;
+    int64_t nb = (nvec_w + kBlock - 1) / kBlock;
+    if (nb > 8192) nb = 8192;
+    if (dtype == AMCT_F16) hipLaunchKernelGGL((w4_dequant_rows<true>), dim3((unsigned)nb), dim3(kBlock), 0, st, a, wdq, nvec_w);
+    else hipLaunchKernelGGL((w4_dequant_rows<false>), dim3((unsigned)nb), dim3(kBlock), 0, st, a, wdq, nvec_w);
+    const void* xa = x;
+    if (smooth) {
+        const int64_t nvec = M * K / 8;
+        int64_t nbs = (nvec + kBlock - 1) / kBlock;
+        if (nbs > 16384) nbs = 16384;
+        if (dtype == AMCT_F16) hipLaunchKernelGGL(smooth_rows_f16, dim3((unsigned)nbs), dim3(kBlock), 0, st, a.x, a.smooth, xs, nvec, (int)(K / 8));
+        else hipLaunchKernelGGL(smooth_rows, dim3((unsigned)nbs), dim3(kBlock), 0, st, a.x, a.smooth, xs, nvec, (int)(K / 8));
+        xa = xs;
+    }
+    return gemm16_tiles(xa, wdq, bias, out, M, N, K, dtype, st);
+}
+
 }  // namespace amct
 
 using namespace amct;
 
 extern "C" size_t amct_gemm_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K, int group, int has_smooth) {
-    (void)N;
-    if (M <= 0 || K <= 0 || group <= 0) return 0;
+    if (M <= 0 || N <= 0 || K <= 0 || group <= 0) return 0;
+    const size_t two = two_pass_workspace(M, N, K, group, has_smooth);    // many rows: the dequantised weight as well
+    if (two) return two;
     return has_smooth && M > 16 ? (size_t)M * (size_t)K * 2 : 0;          // tile kernels: x * smooth done once
 }
 
@@ -1788,6 +1854,11 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
         if (M <= 16) {
             const int rc = w4a16_stream_dispatch(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, dtype,
                                                  (hipStream_t)stream);
+            if (rc != AMCT_E_UNSUPPORTED) return rc;
+        }
+        if (M >= kTwoPassFrom) {
+            const int rc = two_pass(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, dtype, workspace,
+                                    workspace_bytes, (hipStream_t)stream);
             if (rc != AMCT_E_UNSUPPORTED) return rc;
         }
         // more than 64 rows: the tile kernels with fp16 operands (the same bodies: the dequantised weight and the smoothed
@@ -1839,6 +1910,11 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
     hipStream_t st = (hipStream_t)stream;
     if (M <= 16) {                                                 // bf16, K % 1024 == 0, group 128: the weight-streaming kernel
         const int rc = w4a16_stream_dispatch(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, dtype, st);
+        if (rc != AMCT_E_UNSUPPORTED) return rc;
+    }
+    if (M >= kTwoPassFrom) {                                       // many rows and a workspace for the dequantised weight
+        const int rc = two_pass(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, dtype, workspace,
+                                workspace_bytes, st);
         if (rc != AMCT_E_UNSUPPORTED) return rc;
     }
     const bool vec_ok = aligned16(x) && aligned16(wq) && (!smooth || aligned16(smooth)) && group % 32 == 0;

@@ -21,6 +21,8 @@
 //                   take): as above with the activations read from L2 per MFMA.
 //   general kernel: any shape, one output per thread.
 #include "amct_common.h"
+
+#include <type_traits>
 #include "gemm_plan.h"
 
 namespace amct {
@@ -466,7 +468,10 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
     }
 }
 
-template <int ODT, int WM, int WN, int TI, int TJ, int STAGES>
+// MODE 0: int8 operands (v_mfma_i32_16x16x64_i8).  MODE 1 / 2: bf16 / fp16 operands with fp32 accumulation
+// (v_mfma_f32_16x16x32_bf16 / _f16): the same 64 bytes of K per row and MFMA and the same fragment layout in bytes, so
+// the body is that of the int8 kernel with a.K counted in BYTES of a row; s_ch and s_tok are null then (factor 1).
+template <int ODT, int WM, int WN, int TI, int TJ, int STAGES, int MODE = 0>
 AMCT_DEV void w8a8_dma_body16(const W8A8Args& a, int8_t* smem, const int64_t m0, const int64_t n0) {
     constexpr int LK = 128;
     using Sh = DmaTile<WM, WN, TI, TJ, STAGES, LK>;
@@ -542,11 +547,16 @@ AMCT_DEV void w8a8_dma_body16(const W8A8Args& a, int8_t* smem, const int64_t m0,
             offB[sl] = kLM * LK + (wn * 32 * TJ + r) * LK + ((4 * sl + (lane >> 4)) ^ swz(r)) * 16;
     }
 
-    v4i acc[2 * TI][TB];
+    typedef float v4fa __attribute__((ext_vector_type(4)));
+    typedef typename std::conditional<MODE == 0, v4i, v4fa>::type acc_t;
+    acc_t acc[2 * TI][TB];
 #pragma unroll
     for (int i = 0; i < 2 * TI; ++i)
 #pragma unroll
-        for (int j = 0; j < TB; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+        for (int j = 0; j < TB; ++j) {
+            if constexpr (MODE == 0) acc[i][j] = v4i{0, 0, 0, 0};
+            else acc[i][j] = v4fa{0.f, 0.f, 0.f, 0.f};
+        }
 
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s) dma_stage(s, s < last ? s : last);
@@ -567,7 +577,17 @@ AMCT_DEV void w8a8_dma_body16(const W8A8Args& a, int8_t* smem, const int64_t m0,
     };
     auto mfma_one = [&](int u, int m) {
         const int i = m / TB, j = m % TB;
-        acc[(u & 1) * TA + i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[u & 1][i], fb[(u >> 1) & 1][j], acc[(u & 1) * TA + i][j], 0, 0, 0);
+        if constexpr (MODE == 0) {
+            acc[(u & 1) * TA + i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[u & 1][i], fb[(u >> 1) & 1][j], acc[(u & 1) * TA + i][j], 0, 0, 0);
+        } else if constexpr (MODE == 1) {
+            typedef __bf16 v8bfm __attribute__((ext_vector_type(8)));
+            acc[(u & 1) * TA + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bfm, fa[u & 1][i]), __builtin_bit_cast(v8bfm, fb[(u >> 1) & 1][j]),
+                                                                           acc[(u & 1) * TA + i][j], 0, 0, 0);
+        } else {
+            typedef _Float16 v8hm __attribute__((ext_vector_type(8)));
+            acc[(u & 1) * TA + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8hm, fa[u & 1][i]), __builtin_bit_cast(v8hm, fb[(u >> 1) & 1][j]),
+                                                                          acc[(u & 1) * TA + i][j], 0, 0, 0);
+        }
     };
     wait_dma_lds<(STAGES - 2) * kPPW>();
     __builtin_amdgcn_s_barrier();
@@ -633,7 +653,7 @@ AMCT_DEV void w8a8_dma_body16(const W8A8Args& a, int8_t* smem, const int64_t m0,
     for (int j = 0; j < TB; ++j) {
         const int64_t n = n0 + wn * kPW + j * 16 + (lane & 15);
         const int64_t nc = n < a.N ? n : a.N - 1;
-        sc[j] = a.s_ch[nc];
+        sc[j] = a.s_ch ? a.s_ch[nc] : 1.0f;
         ib[j] = a.bias_kind == 1 ? reinterpret_cast<const int32_t*>(a.bias)[nc] : 0;
         fb2[j] = a.bias_kind == 2 ? reinterpret_cast<const float*>(a.bias)[nc] : -0.0f;
     }
@@ -643,7 +663,7 @@ AMCT_DEV void w8a8_dma_body16(const W8A8Args& a, int8_t* smem, const int64_t m0,
         tokl[t] = a.s_tok ? a.s_tok[m < a.M ? m : a.M - 1] : 1.0f;
     }
     // accumulator tile (t, j), register r: row 16 t + 4 (lane / 16) + r, column 16 j + lane % 16 of the wave tile
-    if (a.acc_out) {                                                // accumulators on request (tests): plain stores
+    if constexpr (MODE == 0) if (a.acc_out) {                       // accumulators on request (tests): plain stores
 #pragma unroll
         for (int t = 0; t < 2 * TI; ++t)
 #pragma unroll
@@ -670,7 +690,9 @@ AMCT_DEV void w8a8_dma_body16(const W8A8Args& a, int8_t* smem, const int64_t m0,
             for (int r = 0; r < 4; ++r) {
 #pragma unroll
                 for (int j = 0; j < TB; ++j) {
-                    float f = (float)(acc[2 * i + hh][j][r] + ib[j]) * sc[j];
+                    float f;
+                    if constexpr (MODE == 0) f = (float)(acc[2 * i + hh][j][r] + ib[j]) * sc[j];
+                    else f = acc[2 * i + hh][j][r] * sc[j];
                     f = f * tks[r];
                     f = f + fb2[j];
                     int8_t* dst = wbase + (16 * hh + r) * kPatchRow + j * 16 * ES;
@@ -725,24 +747,24 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 }
 
 // the same two launches on v_mfma_i32_16x16x64_i8 (K a multiple of 128)
-template <int ODT>
+template <int ODT, int MODE = 0>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void w8a8_tile_dma16(W8A8Args a) {
     using Sh = DmaTile<2, 4, 4, 2, 2, 128>;
     __shared__ __attribute__((aligned(1024))) int8_t smem[Sh::kSmem];
-    w8a8_dma_body16<ODT, 2, 4, 4, 2, 2>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
+    w8a8_dma_body16<ODT, 2, 4, 4, 2, 2, MODE>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
 }
 
-template <int ODT>
+template <int ODT, int MODE = 0>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void w8a8_tile_mix16(W8A8Args a, MixPlan p) {
     using Big = DmaTile<2, 4, 4, 2, 2, 128>;
     using Small = DmaTile<4, 2, 2, 3, 2, 128>;
     __shared__ __attribute__((aligned(1024))) int8_t smem[Big::kSmem > Small::kSmem ? Big::kSmem : Small::kSmem];
     const int b = blockIdx.x;
     if (b < p.big) {
-        w8a8_dma_body16<ODT, 2, 4, 4, 2, 2>(a, smem, (int64_t)(b / p.nbig) * 256, (int64_t)(b % p.nbig) * 256);
+        w8a8_dma_body16<ODT, 2, 4, 4, 2, 2, MODE>(a, smem, (int64_t)(b / p.nbig) * 256, (int64_t)(b % p.nbig) * 256);
     } else {
         const int s = b - p.big;
-        w8a8_dma_body16<ODT, 4, 2, 2, 3, 2>(a, smem, (int64_t)(s / p.nsmall) * 256,
+        w8a8_dma_body16<ODT, 4, 2, 2, 3, 2, MODE>(a, smem, (int64_t)(s / p.nsmall) * 256,
                                             (int64_t)p.nbig * 256 + (int64_t)(s % p.nsmall) * 192);
     }
 }
@@ -1010,6 +1032,33 @@ __global__ __launch_bounds__(kBlock) void w8a8_general(W8A8Args a) {
 int w8a8_stream_dispatch(const int8_t* xq, const int8_t* wq, const float* s_tok, const float* s_ch, const void* bias,
                          int bias_kind, void* out, int32_t* acc_out, int64_t M, int64_t N, int64_t K, int out_dtype,
                          hipStream_t st);
+
+// out [M, N] of dtype = x [M, K] @ w [N, K]^T + bias (fp32 [N] or null), fp32 accumulation, both operands of dtype (bf16 or
+// fp16), K contiguous: the 256x256 / 256x192 tiles of the W8A8 kernel on the 16-bit MFMAs.  Returns AMCT_E_UNSUPPORTED
+// for shapes the tiles do not take (fewer than 256 rows, K not a multiple of 64, N not a multiple of 8, unaligned or
+// 4 GiB operands).  Used by the int8 weight-only Linear, which dequantises its weight into a workspace first.
+int gemm16_tiles(const void* x, const void* w, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int dtype,
+                 hipStream_t st) {
+    const int64_t Kb = K * 2;                                       // bytes of a row
+    if (dtype != AMCT_BF16 && dtype != AMCT_F16) return AMCT_E_UNSUPPORTED;
+    if (M < 256 || Kb % 128 != 0 || N % 8 != 0 || !aligned16(x) || !aligned16(w) || !aligned16(out) ||
+        M * Kb >= (int64_t(1) << 32) || N * Kb >= (int64_t(1) << 32))
+        return AMCT_E_UNSUPPORTED;
+    const dim3 grid((unsigned)((N + 255) / 256), (unsigned)((M + 255) / 256));
+    if (grid.y > 65535) return AMCT_E_UNSUPPORTED;
+    W8A8Args a{reinterpret_cast<const int8_t*>(x), reinterpret_cast<const int8_t*>(w), nullptr, nullptr, bias, out, nullptr,
+               M, N, Kb, bias ? 2 : 0, dtype};
+    const MixPlan plan = plan_mix(M, N, current_cu_count());
+    if (plan.nbig >= 0) {
+        const dim3 g1((unsigned)(plan.big + plan.mtiles * plan.nsmall));
+        if (dtype == AMCT_BF16) hipLaunchKernelGGL((w8a8_tile_mix16<AMCT_BF16, 1>), g1, dim3(512), 0, st, a, plan);
+        else hipLaunchKernelGGL((w8a8_tile_mix16<AMCT_F16, 2>), g1, dim3(512), 0, st, a, plan);
+    } else {
+        if (dtype == AMCT_BF16) hipLaunchKernelGGL((w8a8_tile_dma16<AMCT_BF16, 1>), grid, dim3(512), 0, st, a);
+        else hipLaunchKernelGGL((w8a8_tile_dma16<AMCT_F16, 2>), grid, dim3(512), 0, st, a);
+    }
+    return hip_status();
+}
 
 }  // namespace amct
 

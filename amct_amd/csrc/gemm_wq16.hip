@@ -450,6 +450,42 @@ int wq16_int4_f16(const void* x, const void* smooth, const uint8_t* wq, const vo
 }  // namespace amct
 
 namespace amct {
+
+// ---------------------------------------------------------------------------
+// int8 weights, many rows: the weight is dequantised once into the caller's workspace, dt((q - offset) * scale) as the
+// tile kernel above computes it per block, and the product is the plain 16-bit GEMM on the 256x256 tiles of the W8A8
+// kernel (gemm_w8a8.hip: gemm16_tiles); the activations are smoothed into the workspace first when asked for.
+// ---------------------------------------------------------------------------
+template <int DT>
+__global__ __launch_bounds__(kBlock) void w8_dequant_rows(WqArgs a, uint16_t* wdq, int64_t nvec) {   // nvec = N * K / 16
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    const int64_t G = a.K / a.group;
+    for (int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += stride) {
+        const int64_t e = v * 16, row = e / a.K, k = e - row * a.K;          // 16 weights of one row and one group
+        const int64_t gi = row * G + k / a.group;
+        const float s = wq_scale(a, gi), nzs = -(wq_zero<8>(a, gi) * s);
+        const uint4 w = ldg16_nt(a.wq + e);
+        stg16(wdq + e, dq8_int8<DT>(w.x, w.y, s, nzs));
+        stg16(wdq + e + 8, dq8_int8<DT>(w.z, w.w, s, nzs));
+    }
+}
+template <int DT>
+__global__ __launch_bounds__(kBlock) void smooth_rows_dt(const uint16_t* x, const uint16_t* smooth, uint16_t* y, int64_t nvec, int kvec) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += stride)
+        stg16(y + v * 8, smooth8_dt<DT>(ldg16_nt(x + v * 8), ldg16(smooth + (v % kvec) * 8)));
+}
+
+int gemm16_tiles(const void* x, const void* w, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int dtype,
+                 hipStream_t st);                           // gemm_w8a8.hip
+
+static size_t w8a16_tiles_workspace(int64_t M, int64_t N, int64_t K, int group, int has_smooth) {
+    if (M < 256 || N <= 0 || K <= 0 || group <= 0 || K % 64 != 0 || K % 16 != 0 || group % 16 != 0 || K % group != 0 || N % 8 != 0 ||
+        N * K * 2 >= (int64_t(1) << 32) || M * K * 2 >= (int64_t(1) << 32))
+        return 0;
+    return (size_t)N * (size_t)K * 2 + (has_smooth ? (size_t)M * (size_t)K * 2 : 0);
+}
+
 int w8a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
                           const uint8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group,
                           int dtype, hipStream_t st);      // gemm_w8a16_stream.hip
@@ -457,9 +493,19 @@ int w8a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, 
 
 using namespace amct;
 
+extern "C" size_t amct_gemm_w8a16_workspace_bytes(int64_t M, int64_t N, int64_t K, int group, int has_smooth) {
+    return w8a16_tiles_workspace(M, N, K, group, has_smooth);
+}
+
 extern "C" int amct_gemm_w8a16(const void* x, const void* smooth, const int8_t* wq, const void* scales, int scale_dtype,
                                const int8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K,
                                int group, int dtype, amct_stream_t stream) {
+    return amct_gemm_w8a16_ws(x, smooth, wq, scales, scale_dtype, offsets, bias, out, M, N, K, group, dtype, nullptr, 0, stream);
+}
+
+extern "C" int amct_gemm_w8a16_ws(const void* x, const void* smooth, const int8_t* wq, const void* scales, int scale_dtype,
+                                  const int8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K,
+                                  int group, int dtype, void* workspace, size_t workspace_bytes, amct_stream_t stream) {
     if (M < 0 || N <= 0 || K <= 0 || group <= 0) return AMCT_E_BADARG;
     if (M != 0 && (!x || !wq || !scales || !out)) return AMCT_E_BADARG;
     if (scale_dtype != AMCT_F16 && scale_dtype != AMCT_BF16) return AMCT_E_BADARG;
@@ -474,6 +520,30 @@ extern "C" int amct_gemm_w8a16(const void* x, const void* smooth, const int8_t* 
         const int rc = w8a16_stream_dispatch(x, smooth, reinterpret_cast<const uint8_t*>(wq), scales, scale_dtype,
                                              reinterpret_cast<const uint8_t*>(offsets), bias, out, M, N, K, group, dtype, st);
         if (rc != AMCT_E_UNSUPPORTED) return rc;
+    }
+    // many rows and a lent workspace: dequantise once, then the plain 16-bit GEMM on the large tiles
+    const size_t need = w8a16_tiles_workspace(M, N, K, group, smooth != nullptr);
+    if (need && workspace && workspace_bytes >= need && aligned16(workspace) && aligned16(x) && aligned16(wq) && aligned16(out) &&
+        (!smooth || aligned16(smooth)) && (reinterpret_cast<uintptr_t>(scales) & 1u) == 0) {
+        uint16_t* wdq = reinterpret_cast<uint16_t*>(workspace);
+        uint16_t* xs = wdq + (size_t)N * (size_t)K;
+        const int64_t nvec_w = N * K / 16;
+        int64_t nb = (nvec_w + kBlock - 1) / kBlock;
+        if (nb > 8192) nb = 8192;
+        if (dtype == AMCT_BF16) hipLaunchKernelGGL((w8_dequant_rows<AMCT_BF16>), dim3((unsigned)nb), dim3(kBlock), 0, st, a, wdq, nvec_w);
+        else hipLaunchKernelGGL((w8_dequant_rows<AMCT_F16>), dim3((unsigned)nb), dim3(kBlock), 0, st, a, wdq, nvec_w);
+        const void* xa = x;
+        if (smooth) {
+            const int64_t nvec = M * K / 8;
+            int64_t nbs = (nvec + kBlock - 1) / kBlock;
+            if (nbs > 16384) nbs = 16384;
+            if (dtype == AMCT_BF16) hipLaunchKernelGGL((smooth_rows_dt<AMCT_BF16>), dim3((unsigned)nbs), dim3(kBlock), 0, st, a.x, a.smooth, xs, nvec, (int)(K / 8));
+            else hipLaunchKernelGGL((smooth_rows_dt<AMCT_F16>), dim3((unsigned)nbs), dim3(kBlock), 0, st, a.x, a.smooth, xs, nvec, (int)(K / 8));
+            xa = xs;
+        }
+        const int rc = gemm16_tiles(xa, wdq, bias, out, M, N, K, dtype, st);
+        if (rc != AMCT_E_UNSUPPORTED) return rc;
+        // (the two preparatory kernels above only wrote the workspace: the call below starts from the caller's operands)
     }
     return dtype == AMCT_BF16 ? wq16_dispatch<8, AMCT_BF16>(a, st) : wq16_dispatch<8, AMCT_F16>(a, st);
 }

@@ -525,8 +525,13 @@ def gemm_w8a16(x, wq_nk, scales, offsets, group, smooth=None, bias=None):
     if bias is not None:
         bias = _c(bias.reshape(-1).to(torch.float32))
     out = torch.empty(M, N, dtype=x.dtype, device=dev)
+    # the workspace the library asks for: from 256 rows on, the dequantised weight (and the smoothed activations)
+    ws = None
+    nbytes = _lib.load().amct_gemm_w8a16_workspace_bytes(M, N, K, group, int(smooth is not None))
+    if nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
-        _lib.check(_lib.load().amct_gemm_w8a16(_p(x), _p(smooth), _p(wq_nk), _p(scales), dtype_code(scales.dtype),
-                                               _p(offsets), _p(bias), _p(out), M, N, K, group, dtype_code(x.dtype),
-                                               _stream(dev)))
+        _lib.check(_lib.load().amct_gemm_w8a16_ws(_p(x), _p(smooth), _p(wq_nk), _p(scales), dtype_code(scales.dtype),
+                                                  _p(offsets), _p(bias), _p(out), M, N, K, group, dtype_code(x.dtype),
+                                                  _p(ws), 0 if ws is None else ws.numel(), _stream(dev)))
     return out

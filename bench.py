@@ -392,6 +392,28 @@ def build_cases(dev, only):
         cases.append(Case("w8a16_m16", "hbm", N9 * K9 + 16 * K9 * 2 + 16 * N9 * 2 + N9 * 2, "B", launch, 6, "bf16",
                           "int8 weight-only Linear M=16 N=14336 K=4096, per-channel scales, bf16 activations (decode): weight streaming"))
 
+    # ---- the same operator at M = 2048: dequantise the weight once into the lent workspace, then the 16-bit GEMM on the
+    # large tiles (three launches with smoothing)
+    if want("w8a16_m2048"):
+        x10 = workloads.c5_w4a16(2048)[0].contiguous().to(dev)
+        sm10 = workloads.c5_w4a16(2048)[4].to(dev)
+        g10 = torch.Generator().manual_seed(1033)
+        N10, K10 = 14336, 4096
+        w10 = dev_copies(torch.randint(-128, 128, (N10, K10), generator=g10, dtype=torch.int16).to(torch.int8), 6)
+        s10 = (1e-3 + 9e-3 * torch.rand(N10, K10 // 128, generator=g10)).to(torch.float16).to(dev)
+        z10 = torch.randint(-128, 128, (N10, K10 // 128), generator=g10, dtype=torch.int16).to(torch.int8).to(dev)
+        outs10 = [torch.empty(2048, N10, dtype=torch.bfloat16, device=dev) for _ in range(6)]
+        ws10 = torch.empty(lib.amct_gemm_w8a16_workspace_bytes(2048, N10, K10, 128, 1), dtype=torch.uint8, device=dev)
+
+        def launch(i, x10=x10, sm10=sm10, w10=w10, s10=s10, z10=z10, outs10=outs10, ws10=ws10, N10=N10, K10=K10):
+            j = i % len(w10)
+            rc = lib.amct_gemm_w8a16_ws(x10.data_ptr(), sm10.data_ptr(), w10[j].data_ptr(), s10.data_ptr(), _lib.F16, z10.data_ptr(),
+                                        None, outs10[j].data_ptr(), 2048, N10, K10, 128, _lib.BF16, ws10.data_ptr(), ws10.numel(), st)
+            assert rc == 0, rc
+        cases.append(Case("w8a16_m2048", "mfma_bf16", 2 * 2048 * N10 * K10, "flop", launch, 6, "bf16",
+                          "int8 weight-only Linear M=2048 N=14336 K=4096, group-128 scales and offsets, smoothing: dequantise "
+                          "into the workspace + smoothing pre-pass + 16-bit GEMM on the 256x256 tiles"))
+
     # ---- GPTQ Hessian accumulation: H[4096,4096] fp32 <- beta H + alpha X^T X, X[2048,4096] bf16 ------------------
     # (after everything else: it heats the part like the GEMMs do).  Work = the multiply-adds of the lower triangle
     # with its diagonal, which is what a symmetric update needs; the library path beside it is the reference's

@@ -254,7 +254,10 @@ int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s_tok, const
  * workspace (may be null): amct_gemm_w4a16_workspace_bytes(M, N, K, group, smooth != null) bytes the caller lends,
  * 16-byte aligned, contents irrelevant before and after the call.  For M > 16 with smooth the multiply is then done
  * once up front instead of inside every column tile (same results; the fast bf16 tile kernels need it, without it such
- * calls take slower kernels that smooth in place); 0 bytes are asked for otherwise.
+ * calls take slower kernels that smooth in place).  From M = 3584 on the query also asks for N * K * 2 bytes: the weight
+ * is then dequantised once into the workspace and the product runs as a plain 16-bit GEMM, which beats dequantising inside
+ * every row tile from there on (same arithmetic; a smaller workspace keeps the fused kernels).  0 bytes are asked for
+ * otherwise; a null or smaller workspace is never an error.
  * Arithmetic of the dequantisation: the tile kernels (M > 16) feed dtype((u - zero) * scale) to the matrix pipe; the
  * weight-streaming kernel for M <= 16 (bf16 or fp16, K of 1024 / 2048 / 4096, group = 128) keeps the weight as the exact integer and applies
  * scale and zero per group in fp32, i.e. the dequantised weight is not rounded to bf16 there (the fp32 weight * scale of
@@ -280,6 +283,16 @@ int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t* wq, const 
 int amct_gemm_w8a16(const void* x, const void* smooth, const int8_t* wq, const void* scales, int scale_dtype,
                     const int8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K,
                     int group, int dtype, amct_stream_t stream);
+/* The same with a workspace (may be null): amct_gemm_w8a16_workspace_bytes(M, N, K, group, smooth != null) bytes the
+ * caller lends, 16-byte aligned, contents irrelevant before and after the call.  From M = 256 on the weight is then
+ * dequantised once into it (N * K * 2 bytes; the smoothed activations follow), and the product runs as a plain 16-bit
+ * GEMM on the 256x256 tiles of the W8A8 kernel: the same arithmetic as the tile kernel without workspace (the
+ * dequantised weight rounded to dtype, fp32 accumulation), about three times as fast.  0 bytes are asked for when the
+ * shape does not take that path; a null or smaller workspace is never an error. */
+size_t amct_gemm_w8a16_workspace_bytes(int64_t M, int64_t N, int64_t K, int group, int has_smooth);
+int amct_gemm_w8a16_ws(const void* x, const void* smooth, const int8_t* wq, const void* scales, int scale_dtype,
+                       const int8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group,
+                       int dtype, void* workspace, size_t workspace_bytes, amct_stream_t stream);
 
 /* ---- GPTQ inner block ------------------------------------------------------------------------
  * The column loop of amct_pytorch/quantize_op/gptq_module.py:128-151 for one block of count <= 128 columns,

@@ -248,6 +248,40 @@ def test_w8a16_weight_streaming_kernel(dev, dtype, M, N, K, group):
     assert_bits_equal(out, want.to(dtype), "integer special case")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K,group", [(2048, 14336, 4096, 128), (256, 264, 64, 64), (300, 1000, 320, 32), (513, 2056, 1024, 1024),
+                                         (1000, 4104, 192, 64)])
+def test_w8a16_many_rows_through_the_workspace(dev, dtype, M, N, K, group):
+    """Int8 weight-only Linear from 256 rows on: with the workspace the library asks for, the weight is dequantised once
+    and the product is the plain 16-bit GEMM on the large tiles (uniform and mixed tile launches, ragged M and N, K of
+    one and of many steps); without it the shared 128x128 kernel runs.  Both compute dt((q - offset) * scale) and
+    accumulate the exact products in fp32: sampled rows within 1e-3 of the row's largest output (plus half an ulp) of
+    the fp64 anchor, and the two within that of each other; small integers give an integer matmul bit for bit."""
+    from amct_amd import _lib
+    lib = _lib.load()
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    rows = [r for r in FULL_ROWS if r < M]
+    assert lib.amct_gemm_w8a16_workspace_bytes(M, N, K, group, 1) == N * K * 2 + M * K * 2
+    for sdt, sym in ((torch.float16, False), (torch.bfloat16, True)):
+        x, codes, scales, offsets, smooth, bias = w8a16_case(M, N, K, group, 170 + M % 97, dtype, sdt, sym)
+        for sm, b in ((None, None), (smooth, bias)):
+            out = ops.gemm_w8a16(x.to(dev), codes.to(dev), scales.to(dev), None if offsets is None else offsets.to(dev), group,
+                                 None if sm is None else sm.to(dev), None if b is None else b.to(dev)).cpu()[rows]
+            want = od.w4a16_forward_f64(x[rows], codes.to(torch.int32), scales, None if offsets is None else -offsets.float(), group,
+                                        b, None if sm is None else sm.reshape(1, -1), round_weight=True)
+            err = (out.double() - want).abs()
+            tol = 1e-3 * want.abs().amax(dim=1, keepdim=True) + want.abs() * ulp
+            assert (err <= tol).all(), (float((err / tol).max()), sdt, sym, sm is not None)
+    g = torch.Generator().manual_seed(171)
+    xi = torch.randint(-4, 5, (M, K), generator=g).to(dtype)
+    wi = torch.randint(-7, 8, (N, K), generator=g, dtype=torch.int16).to(torch.int8)
+    zi = torch.randint(-3, 4, (N, K // group), generator=g, dtype=torch.int16).to(torch.int8)
+    ones = torch.ones(N, K // group, dtype=torch.float16)
+    out = ops.gemm_w8a16(xi.to(dev), wi.to(dev), ones.to(dev), zi.to(dev), group)
+    want = torch.matmul(xi[rows].double(), (wi.double() - zi.double().repeat_interleave(group, dim=1)).t())
+    assert_bits_equal(out.cpu()[rows], want.to(dtype), "integer special case")
+
+
 def test_w4a16_reduces_to_plain_matmul(dev):
     """zero = 8 (code 0 in signed terms), scale = 1: the kernel is a bf16 GEMM against integer
     weights, checked against torch.matmul."""
@@ -334,6 +368,41 @@ def test_w4a16_fp16_at_the_benchmark_size(dev, M, N, K):
             err = (out.double() - want).abs()
             tol = 1e-3 * want.abs().amax(dim=1, keepdim=True) + want.abs() * 2.0 ** -11
             assert (err <= tol).all(), (M, sdt, sm is not None, float((err / tol).max()))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K,group", [(3584, 1000, 320, 32), (4100, 264, 64, 64)])
+def test_w4a16_very_many_rows_dequantise_once(dev, dtype, M, N, K, group):
+    """From 3584 rows on, with the workspace the library asks for (the 16-bit weight and the smoothed activations), the
+    int4 weight is dequantised once and the product is the plain 16-bit GEMM on the large tiles; with the smaller
+    workspace of the fused kernels those run.  Same arithmetic (dt((u - z) * s), exact products, fp32 accumulation):
+    sampled rows of both within the tolerance of the fp64 anchor; small integers bit for bit."""
+    from amct_amd import _lib
+    lib = _lib.load()
+    assert lib.amct_gemm_w4a16_workspace_bytes(M, N, K, group, 1) == N * K * 2 + M * K * 2
+    assert lib.amct_gemm_w4a16_workspace_bytes(M, N, K, group, 0) == N * K * 2
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    rows = FULL_ROWS + [M - 1, M - 2, 3583]
+    x, codes, scales, zeros, smooth, bias = w4a16_case(M, N, K, group, 333, torch.float16)
+    x, smooth = x.to(dtype), smooth.to(dtype)
+    xd, packed, sd, zd, smd, bd = x.to(dev), workloads.pack_nibbles(codes).to(dev), scales.to(dev), zeros.to(dev), smooth.to(dev), bias.to(dev)
+    want = w4a16_oracle(x[rows], codes, scales, zeros, group, smooth, bias, rows=M)
+    tol = 1e-3 * want.abs().amax(dim=1, keepdim=True) + want.abs() * ulp
+    st = torch.cuda.current_stream(dev).cuda_stream
+    for nbytes in (N * K * 2 + M * K * 2, M * K * 2):
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        out = torch.empty(M, N, dtype=dtype, device=dev)
+        _lib.check(lib.amct_gemm_w4a16(xd.data_ptr(), smd.data_ptr(), packed.data_ptr(), sd.data_ptr(), _lib.F16, zd.data_ptr(),
+                                       bd.data_ptr(), out.data_ptr(), M, N, K, group, _lib.BF16 if dtype == torch.bfloat16 else _lib.F16,
+                                       ws.data_ptr(), ws.numel(), st))
+        err = (out.cpu()[rows].double() - want).abs()
+        assert (err <= tol).all(), (nbytes, float((err / tol).max()))
+    g = torch.Generator().manual_seed(334)
+    xi = torch.randint(-4, 5, (M, K), generator=g).to(dtype)
+    ones = torch.ones(N, K // group, dtype=torch.float16)
+    out = ops.gemm_w4a16(xi.to(dev), packed, ones.to(dev), zd, group)
+    wi = codes.float() - zeros.float().repeat_interleave(group, dim=1)
+    assert_bits_equal(out.cpu()[rows], torch.matmul(xi[rows].double(), wi.double().t()).to(dtype), "integer special case")
 
 
 @pytest.mark.parametrize("seed", [1, 2])
