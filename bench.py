@@ -40,11 +40,11 @@ MEASURED_TRAFFIC = {
     "hif8_decode": ("hif8_decode_full<2, 256, 8>", 100748936),
     "act_quant_per_token": ("act_quant_token<2, 2>", 25292715),
     "col_minmax": ("col_partial_k<2, false> + col_final_k", 69345307),
-    "w8a8_m2048": ("w8a8_tile_mix16<2>", 254747636),
+    "w8a8_m2048": ("w8a8_tile_mix16<2, 0>", 255069388),
     "w8a8_m16": ("w8a8_stream<2, 4, 4, 16, 4>", 59796000),
-    "w4a16_m2048": ("smooth_rows + w4a16_tile_wide16<true, 2, 4, 4, 2, 2, 2>", 303587625),
-    "w4a16_m16": ("w4a16_stream<4, 4, 8, 8, true>", 32474218),
-    "w4a16_m1": ("w4a16_stream<4, 1, 8, 2, true>", 31011237),
+    "w4a16_m2048": ("smooth_rows + w4a16_tile_wide16<true, 2, 4, 4, 2, 2, 2, false>", 303572868),
+    "w4a16_m16": ("w4a16_stream<2, 4, 4, 8, 8, true>", 32474218),
+    "w4a16_m1": ("w4a16_stream<2, 4, 1, 8, 2, true>", 31011237),
 }
 
 
