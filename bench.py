@@ -3,7 +3,7 @@
 
 `python bench.py --gpus 1 --steps K --warmup W` prints ONE JSON line.  A step is one pass of
 the headline kernel over one batch of synthetic input already resident in HBM: INT4 asymmetric
-group-128 quantise + pack of a bf16 weight [14336, 4096] (BASELINE config 2).  The line also
+group-128 quantise + pack of a bf16 weight [14336, 4096] (benchmark configuration 2).  The line also
 carries, under "kernels", the same measurement for every other kernel of the path, the roofline
 of the headline kernel, and the CPU oracle timed on the host cores on a bounded sample.
 

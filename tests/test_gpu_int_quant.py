@@ -261,7 +261,7 @@ def test_fp32_halfway_points(dev):
 
 
 def test_config1_full_size(dev):
-    """BASELINE config 1: W[4096,4096] fp32 N(0,0.02), int8 symmetric per channel."""
+    """Benchmark configuration 1: W[4096,4096] fp32 N(0,0.02), int8 symmetric per channel."""
     from amct_amd import workloads
     w = workloads.c1_weight()
     dq, codes, s, _ = ops.fakequant_int(w.to(dev), 8, True, codes_kind=ops.CODES_I8)
