@@ -78,7 +78,7 @@ def test_mx_dequant_all_codes(dev, fmt, dtype):
 
 
 def test_mx_config3_roundtrip(dev):
-    """BASELINE config 3 at full size: oracle parity on a row sample, idempotence on all of it."""
+    """Benchmark configuration 3 at full size: oracle parity on a row sample, idempotence on all of it."""
     x = workloads.c3_activations()
     xd = x.to(dev)
     rows = torch.arange(0, 8192, 61)

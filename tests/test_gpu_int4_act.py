@@ -39,7 +39,7 @@ def test_int4_group_pack(dev, dtype, shape, group, sym):
 
 
 def test_config2_slice(dev):
-    """BASELINE config 2 (outliers, bf16, g=128) on the first 1024 rows vs the oracle."""
+    """Benchmark configuration 2 (outliers, bf16, g=128) on the first 1024 rows vs the oracle."""
     w = workloads.c2_weight(1024, 4096)
     packed, s16, zeros, s32 = ops.quant_int4_group_pack(w.to(dev), 128, False, torch.float16, want_scales32=True)
     op, os16, oz, os32 = oracle_pack(w, 128, False, torch.float16)
