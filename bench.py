@@ -574,6 +574,31 @@ def cpu_baselines(names):
             entry(name, 2 * m * 14336 * 4096, "TFLOP/s",
                   lambda xs=xs: od.cpu_standin_weight_quant_matmul_f32(xs, signed5, sc5, anti5, 128, None, sm5.reshape(1, -1)),
                   "{} of the rows of config 5, all 14336 output channels, fp32 dequantise + F.linear as the reference's CPU stand-in".format(m))
+    if "gptq_hessian_update" in names:
+        from oracle import gptq as og
+        th, ch = 512, 4096
+        xh = torch.randn(th, ch, generator=torch.Generator().manual_seed(1031)).to(torch.bfloat16)
+        hh = [None]
+
+        def hess():
+            hh[0], _ = og.update_hessian(hh[0], 4, xh, ch)
+        entry("gptq_hessian_update", 2 * th * ch * (ch + 1) // 2, "TFLOP/s", hess,
+              "512 of the 2048 tokens, all 4096 columns: the reference's update (scale, fp32 matmul, add) on the host; "
+              "flops of the lower triangle as for the kernel")
+    if any(n in names for n in ("w8a16_m2048", "w8a16_m16")):
+        g9 = torch.Generator().manual_seed(1033)
+        w9 = torch.randint(-128, 128, (14336, 4096), generator=g9, dtype=torch.int16).to(torch.int32)
+        s9 = (1e-3 + 9e-3 * torch.rand(14336, 32, generator=g9)).to(torch.float16)
+        z9 = torch.randint(-128, 128, (14336, 32), generator=g9, dtype=torch.int16).float()
+        x9 = workloads.c5_w4a16(256, 64, 4096)[0]
+        for name, m in (("w8a16_m2048", 256), ("w8a16_m16", 16)):
+            if name not in names:
+                continue
+            xs = x9[:m].contiguous()
+            entry(name, 2 * m * 14336 * 4096, "TFLOP/s",
+                  lambda xs=xs: od.cpu_standin_weight_quant_matmul_f32(xs, w9, s9, -z9, 128, None, None),
+                  "{} rows, all 14336 output channels of an int8 weight with group-128 factors, fp32 dequantise + F.linear as the "
+                  "reference's CPU stand-in".format(m))
     return out
 
 
