@@ -216,8 +216,9 @@ struct DmaTile {
     static constexpr int kPPW = kNA + kNB;
     static constexpr int kEpiBytes = kWaves * 16384;
     static constexpr int kSmem = STAGES * kLStageBytes > kEpiBytes ? STAGES * kLStageBytes : kEpiBytes;
+    static constexpr int kSmemFac = kSmem + 3 * 256 * 4;           // with the epilogue's factor table behind it
     static_assert((kLM / kRP) % kLW == 0, "the A pieces must divide evenly among the loading waves");
-    static_assert(kSmem <= 160 * 1024, "LDS");
+    static_assert(kSmemFac <= 160 * 1024, "LDS");
 };
 
 template <int ODT, int WM, int WN, int TI, int TJ, int STAGES, int LK>
@@ -300,6 +301,32 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s) dma_stage(s, s < last ? s : last);
 
+    // The factors of the epilogue (per column: s_ch and the float bias; per row: s_tok; absent ones replaced by their
+    // neutral elements) are fetched now, one or two per thread, and parked in an LDS table behind the stages: read at the
+    // end of the tile they would cost a round trip to memory with nothing to hide it.  An integer bias is where the
+    // accumulators start (its loads wait together with the first stage's), so the epilogue never sees it.
+    static_assert(kLN + kLM <= kWaves * 64 && kLN <= 256 && kLM <= 256, "one factor per thread");
+    float fac0 = 1.0f, fac1 = -0.0f;
+    if (tid < kLN) {
+        const int64_t n = n0 + tid < a.N ? n0 + tid : a.N - 1;
+        if (a.s_ch) fac0 = a.s_ch[n];
+        if (a.bias_kind == 2) fac1 = reinterpret_cast<const float*>(a.bias)[n];
+    } else if (tid - kLN < kLM) {
+        const int64_t m = m0 + (tid - kLN) < a.M ? m0 + (tid - kLN) : a.M - 1;
+        if (a.s_tok) fac0 = a.s_tok[m];
+    }
+    if (a.bias_kind == 1) {
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+            const int64_t n = n0 + wn * 32 * TJ + j * 32 + (lane & 31);
+            const int32_t b = reinterpret_cast<const int32_t*>(a.bias)[n < a.N ? n : a.N - 1];
+#pragma unroll
+            for (int i = 0; i < TI; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = b;
+        }
+    }
+
     // Software pipeline over k-slices of 32 bytes: while the MFMAs of one slice run, the fragments of the next
     // slice are read from LDS.  Before the last slice of a stage the waves meet: every wave then holds that
     // slice's fragments in registers (lgkmcnt(0)), so the stage is free for the loads of step s + STAGES, and
@@ -329,6 +356,13 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
     };
     v4i fa[2][TI], fb[2][TJ];
     wait_dma_lds<(STAGES - 2) * kPPW>();
+    float* ftab = reinterpret_cast<float*>(smem + Sh::kSmem);       // [0, 256) s_ch, [256, 512) float bias, [512, 768) s_tok
+    if (tid < kLN) {
+        ftab[tid] = fac0;
+        ftab[256 + tid] = fac1;
+    } else if (tid - kLN < kLM) {
+        ftab[512 + tid - kLN] = fac0;
+    }
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     dma_stage(STAGES - 1, STAGES - 1 < last ? STAGES - 1 : last);
@@ -379,33 +413,23 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 
-    // epilogue: fp32(acc + ibias) * s_ch * s_tok + fbias, narrowed, transposed through a per-wave LDS
+    // epilogue: fp32(acc, integer bias included) * s_ch * s_tok + fbias, narrowed, transposed through a per-wave LDS
     // patch of 32 rows x 32*TJ columns, stored as 16-byte pieces of full rows.  Branch-free per element:
     // absent factors are replaced by their neutral elements (x * 1.0f and x + (-0.0f) return x bit for bit),
-    // the row factors of the wave come from a small LDS table, every LDS address is base + immediate.
+    // the factors come from the block's LDS table, every LDS address is base + immediate.
     constexpr int ES = (ODT == AMCT_F32) ? 4 : 2;                   // bytes per output element
     constexpr int kPW = 32 * TJ;                                   // patch width in columns
     constexpr int kPatchRow = kPW * ES + 16;                       // padded patch row
     constexpr int CPR = kPW * ES / 16;                             // 16-byte chunks per patch row
-    constexpr int kTokOff = 16384 - 512;                           // 32*TI <= 128 row factors behind the patch
-    static_assert(32 * kPatchRow <= kTokOff && (32 * CPR) % 64 == 0 && TI <= 4,
-                  "patch and row factors must fit the wave's 16 KiB; the patch must split into wave-wide reads");
+    static_assert(32 * kPatchRow <= 16384 && (32 * CPR) % 64 == 0 && TI <= 4,
+                  "the patch must fit the wave's 16 KiB and split into wave-wide reads");
     int8_t* patch = smem + wave * 16384;
-    float* tokl = reinterpret_cast<float*>(patch + kTokOff);
+    const float* tokl = ftab + 512 + wm * 32 * TI;                  // the row factors of this wave
     float sc[TJ], fb2[TJ];
-    int32_t ib[TJ];
 #pragma unroll
     for (int j = 0; j < TJ; ++j) {
-        const int64_t n = n0 + wn * kPW + j * 32 + (lane & 31);
-        const int64_t nc = n < a.N ? n : a.N - 1;
-        sc[j] = a.s_ch[nc];
-        ib[j] = a.bias_kind == 1 ? reinterpret_cast<const int32_t*>(a.bias)[nc] : 0;
-        fb2[j] = a.bias_kind == 2 ? reinterpret_cast<const float*>(a.bias)[nc] : -0.0f;
-    }
-#pragma unroll
-    for (int t = lane; t < 32 * TI; t += 64) {
-        const int64_t m = m0 + wm * 32 * TI + t;
-        tokl[t] = a.s_tok ? a.s_tok[m < a.M ? m : a.M - 1] : 1.0f;
+        sc[j] = ftab[wn * kPW + j * 32 + (lane & 31)];
+        fb2[j] = ftab[256 + wn * kPW + j * 32 + (lane & 31)];
     }
     if (a.acc_out) {                                                // accumulators on request (tests): plain stores
 #pragma unroll
@@ -416,7 +440,7 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
                 for (int j = 0; j < TJ; ++j) {
                     const int64_t m = m0 + wm * 32 * TI + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                     const int64_t n = n0 + wn * kPW + j * 32 + (lane & 31);
-                    if (m < a.M && n < a.N) a.acc_out[m * a.N + n] = acc[i][j][r] + ib[j];
+                    if (m < a.M && n < a.N) a.acc_out[m * a.N + n] = acc[i][j][r];
                 }
     }
     const int h4 = 4 * (lane >> 5);
@@ -437,7 +461,7 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
             const int prow0 = 8 * (r >> 2) + (r & 3);               // patch row minus h4
 #pragma unroll
             for (int j = 0; j < TJ; ++j) {
-                float f = (float)(acc[i][j][r] + ib[j]) * sc[j];
+                float f = (float)acc[i][j][r] * sc[j];
                 f = f * tks[r];
                 f = f + fb2[j];
                 int8_t* dst = wbase + prow0 * kPatchRow + j * 32 * ES;
@@ -467,6 +491,9 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
         }
     }
 }
+
+constexpr int kFacOff = 128 * 1024;                                 // the epilogue's factor table behind the LDS stages
+constexpr int kFacBytes = 3 * 256 * 4;
 
 // MODE 0: int8 operands (v_mfma_i32_16x16x64_i8).  MODE 1 / 2: bf16 / fp16 operands with fp32 accumulation
 // (v_mfma_f32_16x16x32_bf16 / _f16): the same 64 bytes of K per row and MFMA and the same fragment layout in bytes, so
@@ -561,6 +588,36 @@ AMCT_DEV void w8a8_dma_body16(const W8A8Args& a, int8_t* smem, const int64_t m0,
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s) dma_stage(s, s < last ? s : last);
 
+    // The factors of the epilogue (per column: s_ch and the float bias; per row: s_tok; absent ones replaced by their
+    // neutral elements) are fetched now, one or two per thread, and parked in an LDS table behind the stages: read at the
+    // end of the tile they would cost a round trip to memory with nothing to hide it.
+    float fac0 = 1.0f, fac1 = -0.0f;
+    if (tid < kLN) {
+        const int64_t n = n0 + tid < a.N ? n0 + tid : a.N - 1;
+        if (a.s_ch) fac0 = a.s_ch[n];
+        if (a.bias_kind == 2) fac1 = reinterpret_cast<const float*>(a.bias)[n];
+    } else if (tid - kLN < kLM) {
+        const int64_t m = m0 + (tid - kLN) < a.M ? m0 + (tid - kLN) : a.M - 1;
+        if (a.s_tok) fac0 = a.s_tok[m];
+    }
+    // The weight fragment is the MFMA's first operand, so a lane's four accumulator registers of tile (t, j) are four
+    // ADJACENT COLUMNS 16 j + 4 (lane / 16) + r of row 16 t + lane % 16 of the wave tile: the epilogue converts them in pairs
+    // and moves them with one LDS write.  An integer bias is where the accumulators start (its loads wait together with
+    // the first stage's), so the epilogue never sees it.
+    if constexpr (MODE == 0) {
+        if (a.bias_kind == 1) {
+#pragma unroll
+            for (int j = 0; j < TB; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int64_t n = n0 + wn * 32 * TJ + j * 16 + 4 * (lane >> 4) + r;
+                    const int32_t b = reinterpret_cast<const int32_t*>(a.bias)[n < a.N ? n : a.N - 1];
+#pragma unroll
+                    for (int i = 0; i < 2 * TI; ++i) acc[i][j][r] = b;
+                }
+        }
+    }
+
     // The schedule of w8a8_dma_body with units in the place of its k-slices: while the MFMAs of a unit run, the fragments
     // of the next one are read (TA row fragments, plus the TB column fragments when the next unit starts a slice); before
     // the last unit of a stage the waves meet, the refill loads follow, and the last unit reads the first fragments of the
@@ -578,18 +635,27 @@ AMCT_DEV void w8a8_dma_body16(const W8A8Args& a, int8_t* smem, const int64_t m0,
     auto mfma_one = [&](int u, int m) {
         const int i = m / TB, j = m % TB;
         if constexpr (MODE == 0) {
-            acc[(u & 1) * TA + i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[u & 1][i], fb[(u >> 1) & 1][j], acc[(u & 1) * TA + i][j], 0, 0, 0);
+            acc[(u & 1) * TA + i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[(u >> 1) & 1][j], fa[u & 1][i], acc[(u & 1) * TA + i][j], 0, 0, 0);
         } else if constexpr (MODE == 1) {
             typedef __bf16 v8bfm __attribute__((ext_vector_type(8)));
-            acc[(u & 1) * TA + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bfm, fa[u & 1][i]), __builtin_bit_cast(v8bfm, fb[(u >> 1) & 1][j]),
+            acc[(u & 1) * TA + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bfm, fb[(u >> 1) & 1][j]), __builtin_bit_cast(v8bfm, fa[u & 1][i]),
                                                                            acc[(u & 1) * TA + i][j], 0, 0, 0);
         } else {
             typedef _Float16 v8hm __attribute__((ext_vector_type(8)));
-            acc[(u & 1) * TA + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8hm, fa[u & 1][i]), __builtin_bit_cast(v8hm, fb[(u >> 1) & 1][j]),
+            acc[(u & 1) * TA + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8hm, fb[(u >> 1) & 1][j]), __builtin_bit_cast(v8hm, fa[u & 1][i]),
                                                                           acc[(u & 1) * TA + i][j], 0, 0, 0);
         }
     };
     wait_dma_lds<(STAGES - 2) * kPPW>();
+    {
+        float* ftab = reinterpret_cast<float*>(smem + kFacOff);     // [0, 256) s_ch, [256, 512) float bias, [512, 768) s_tok
+        if (tid < kLN) {
+            ftab[tid] = fac0;
+            ftab[256 + tid] = fac1;
+        } else if (tid - kLN < kLM) {
+            ftab[512 + tid - kLN] = fac0;
+        }
+    }
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     dma_stage(STAGES - 1, STAGES - 1 < last ? STAGES - 1 : last);
@@ -634,49 +700,44 @@ AMCT_DEV void w8a8_dma_body16(const W8A8Args& a, int8_t* smem, const int64_t m0,
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 
-    // epilogue: fp32(acc + ibias) * s_ch * s_tok + fbias, narrowed, transposed through a per-wave LDS
-    // patch of 32 rows x 32*TJ columns, stored as 16-byte pieces of full rows.  Branch-free per element:
-    // absent factors are replaced by their neutral elements (x * 1.0f and x + (-0.0f) return x bit for bit),
-    // the row factors of the wave come from a small LDS table, every LDS address is base + immediate.
+    // epilogue: fp32(acc, integer bias included) * s_ch * s_tok + fbias, narrowed, through a per-wave LDS patch of 32 rows x
+    // 32*TJ columns, stored as 16-byte pieces of full rows.  Branch-free per element: absent factors are replaced by
+    // their neutral elements (x * 1.0f and x + (-0.0f) return x bit for bit).  A lane holds the factors of its 4 TB
+    // columns and of its 2 TI rows in registers.
     constexpr int ES = (ODT == AMCT_F32) ? 4 : 2;                   // bytes per output element
     constexpr int kPW = 32 * TJ;                                   // patch width in columns
     constexpr int kPatchRow = kPW * ES + 16;                       // padded patch row
     constexpr int CPR = kPW * ES / 16;                             // 16-byte chunks per patch row
-    constexpr int kTokOff = 16384 - 512;                           // 32*TI <= 128 row factors behind the patch
-    static_assert(32 * kPatchRow <= kTokOff && (32 * CPR) % 64 == 0 && TI <= 4,
-                  "patch and row factors must fit the wave's 16 KiB; the patch must split into wave-wide reads");
+    static_assert(32 * kPatchRow <= 16384 && (32 * CPR) % 64 == 0 && TI <= 4,
+                  "the patch must fit the wave's 16 KiB and split into wave-wide reads");
     int8_t* patch = smem + wave * 16384;
-    float* tokl = reinterpret_cast<float*>(patch + kTokOff);
-    float sc[TB], fb2[TB];
-    int32_t ib[TB];
+    const int q4 = 4 * (lane >> 4);
+    float sc[TB][4], fb2[TB][4], tks[2 * TI];
+    {
+        const float* ftab = reinterpret_cast<const float*>(smem + kFacOff);
 #pragma unroll
-    for (int j = 0; j < TB; ++j) {
-        const int64_t n = n0 + wn * kPW + j * 16 + (lane & 15);
-        const int64_t nc = n < a.N ? n : a.N - 1;
-        sc[j] = a.s_ch ? a.s_ch[nc] : 1.0f;
-        ib[j] = a.bias_kind == 1 ? reinterpret_cast<const int32_t*>(a.bias)[nc] : 0;
-        fb2[j] = a.bias_kind == 2 ? reinterpret_cast<const float*>(a.bias)[nc] : -0.0f;
-    }
+        for (int j = 0; j < TB; ++j) {
+            const float4 s4 = *reinterpret_cast<const float4*>(ftab + wn * kPW + j * 16 + q4);
+            const float4 b4 = *reinterpret_cast<const float4*>(ftab + 256 + wn * kPW + j * 16 + q4);
+            sc[j][0] = s4.x, sc[j][1] = s4.y, sc[j][2] = s4.z, sc[j][3] = s4.w;
+            fb2[j][0] = b4.x, fb2[j][1] = b4.y, fb2[j][2] = b4.z, fb2[j][3] = b4.w;
+        }
 #pragma unroll
-    for (int t = lane; t < 32 * TI; t += 64) {
-        const int64_t m = m0 + wm * 32 * TI + t;
-        tokl[t] = a.s_tok ? a.s_tok[m < a.M ? m : a.M - 1] : 1.0f;
+        for (int t = 0; t < 2 * TI; ++t) tks[t] = ftab[512 + wm * 32 * TI + t * 16 + (lane & 15)];
     }
-    // accumulator tile (t, j), register r: row 16 t + 4 (lane / 16) + r, column 16 j + lane % 16 of the wave tile
     if constexpr (MODE == 0) if (a.acc_out) {                       // accumulators on request (tests): plain stores
 #pragma unroll
         for (int t = 0; t < 2 * TI; ++t)
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
+            for (int j = 0; j < TB; ++j)
 #pragma unroll
-                for (int j = 0; j < TB; ++j) {
-                    const int64_t m = m0 + wm * 32 * TI + t * 16 + 4 * (lane >> 4) + r;
-                    const int64_t n = n0 + wn * kPW + j * 16 + (lane & 15);
-                    if (m < a.M && n < a.N) a.acc_out[m * a.N + n] = acc[t][j][r] + ib[j];
+                for (int r = 0; r < 4; ++r) {
+                    const int64_t m = m0 + wm * 32 * TI + t * 16 + (lane & 15);
+                    const int64_t n = n0 + wn * kPW + j * 16 + q4 + r;
+                    if (m < a.M && n < a.N) a.acc_out[m * a.N + n] = acc[t][j][r];
                 }
     }
-    const int q4 = 4 * (lane >> 4);
-    int8_t* wbase = patch + q4 * kPatchRow + (lane & 15) * ES;      // this lane's element of patch row q4
+    int8_t* wbase = patch + (lane & 15) * kPatchRow + q4 * ES;      // this lane's first element of patch row lane % 16
     const int8_t* rbase = patch + (lane / CPR) * kPatchRow + (lane % CPR) * 16;
     constexpr int RPI = 64 / CPR;                                   // patch rows per wave-wide read when CPR divides 64
 #pragma unroll
@@ -684,21 +745,35 @@ AMCT_DEV void w8a8_dma_body16(const W8A8Args& a, int8_t* smem, const int64_t m0,
         const int64_t mbase = m0 + wm * 32 * TI + i * 32;
 #pragma unroll
         for (int hh = 0; hh < 2; ++hh) {
-            const float4 t4 = *reinterpret_cast<const float4*>(tokl + i * 32 + 16 * hh + q4);
-            const float tks[4] = {t4.x, t4.y, t4.z, t4.w};
+            const int t = 2 * i + hh;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
+            for (int j = 0; j < TB; ++j) {
+                float f[4];
 #pragma unroll
-                for (int j = 0; j < TB; ++j) {
-                    float f;
-                    if constexpr (MODE == 0) f = (float)(acc[2 * i + hh][j][r] + ib[j]) * sc[j];
-                    else f = acc[2 * i + hh][j][r] * sc[j];
-                    f = f * tks[r];
-                    f = f + fb2[j];
-                    int8_t* dst = wbase + (16 * hh + r) * kPatchRow + j * 16 * ES;
-                    if constexpr (ODT == AMCT_F32) *reinterpret_cast<float*>(dst) = f;
-                    else if constexpr (ODT == AMCT_BF16) *reinterpret_cast<uint16_t*>(dst) = (uint16_t)f32_to_bf16_bits(f);
-                    else *reinterpret_cast<uint16_t*>(dst) = (uint16_t)f32_to_f16_bits(f);
+                for (int r = 0; r < 4; ++r) {
+                    f[r] = (float)acc[t][j][r] * sc[j][r];
+                    f[r] = f[r] * tks[t];
+                    f[r] = f[r] + fb2[j][r];
+                }
+                int8_t* dst = wbase + 16 * hh * kPatchRow + j * 16 * ES;
+                if constexpr (ODT == AMCT_F32) {
+                    *reinterpret_cast<float4*>(dst) = make_float4(f[0], f[1], f[2], f[3]);
+                } else {
+                    // one packed conversion per pair; the empty asm keeps it a conversion of the rounded fp32 sum
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) asm("" : "+v"(f[r]));
+                    typedef float v2fe __attribute__((ext_vector_type(2)));
+                    uint2 w;
+                    if constexpr (ODT == AMCT_BF16) {
+                        typedef __bf16 v2be __attribute__((ext_vector_type(2)));
+                        w.x = __builtin_bit_cast(uint32_t, __builtin_convertvector((v2fe{f[0], f[1]}), v2be));
+                        w.y = __builtin_bit_cast(uint32_t, __builtin_convertvector((v2fe{f[2], f[3]}), v2be));
+                    } else {
+                        typedef _Float16 v2he __attribute__((ext_vector_type(2)));
+                        w.x = __builtin_bit_cast(uint32_t, __builtin_convertvector((v2fe{f[0], f[1]}), v2he));
+                        w.y = __builtin_bit_cast(uint32_t, __builtin_convertvector((v2fe{f[2], f[3]}), v2he));
+                    }
+                    *reinterpret_cast<uint2*>(dst) = w;
                 }
             }
         }
@@ -727,7 +802,7 @@ AMCT_DEV void w8a8_dma_body16(const W8A8Args& a, int8_t* smem, const int64_t m0,
 template <int ODT, int WM, int WN, int STAGES, int LK>
 __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void w8a8_tile_dma(W8A8Args a) {
     using Sh = DmaTile<WM, WN, 4, 2, STAGES, LK>;
-    __shared__ __attribute__((aligned(1024))) int8_t smem[Sh::kSmem];
+    __shared__ __attribute__((aligned(1024))) int8_t smem[Sh::kSmemFac];
     w8a8_dma_body<ODT, WM, WN, 4, 2, STAGES, LK>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
 }
 
@@ -735,7 +810,8 @@ template <int ODT, int STAGES, int LK>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void w8a8_tile_mix(W8A8Args a, MixPlan p) {
     using Big = DmaTile<2, 4, 4, 2, STAGES, LK>;
     using Small = DmaTile<4, 2, 2, 3, STAGES, LK>;
-    __shared__ __attribute__((aligned(1024))) int8_t smem[Big::kSmem > Small::kSmem ? Big::kSmem : Small::kSmem];
+    static_assert(Big::kSmem == Small::kSmem, "one place for the factor table");
+    __shared__ __attribute__((aligned(1024))) int8_t smem[Big::kSmemFac];
     const int b = blockIdx.x;
     if (b < p.big) {
         w8a8_dma_body<ODT, 2, 4, 4, 2, STAGES, LK>(a, smem, (int64_t)(b / p.nbig) * 256, (int64_t)(b % p.nbig) * 256);
@@ -750,7 +826,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 template <int ODT, int MODE = 0>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void w8a8_tile_dma16(W8A8Args a) {
     using Sh = DmaTile<2, 4, 4, 2, 2, 128>;
-    __shared__ __attribute__((aligned(1024))) int8_t smem[Sh::kSmem];
+    static_assert(Sh::kSmem <= kFacOff, "the factor table lies behind the stages");
+    __shared__ __attribute__((aligned(1024))) int8_t smem[kFacOff + kFacBytes];
     w8a8_dma_body16<ODT, 2, 4, 4, 2, 2, MODE>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
 }
 
@@ -758,7 +835,8 @@ template <int ODT, int MODE = 0>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void w8a8_tile_mix16(W8A8Args a, MixPlan p) {
     using Big = DmaTile<2, 4, 4, 2, 2, 128>;
     using Small = DmaTile<4, 2, 2, 3, 2, 128>;
-    __shared__ __attribute__((aligned(1024))) int8_t smem[Big::kSmem > Small::kSmem ? Big::kSmem : Small::kSmem];
+    static_assert(Big::kSmem <= kFacOff && Small::kSmem <= kFacOff, "the factor table lies behind the stages");
+    __shared__ __attribute__((aligned(1024))) int8_t smem[kFacOff + kFacBytes];
     const int b = blockIdx.x;
     if (b < p.big) {
         w8a8_dma_body16<ODT, 2, 4, 4, 2, 2, MODE>(a, smem, (int64_t)(b / p.nbig) * 256, (int64_t)(b % p.nbig) * 256);
@@ -773,7 +851,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 template <int ODT, int WM, int WN, int TI, int TJ, int STAGES, int LK>
 __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM * WN / 4, WM * WN / 4))) void w8a8_tile_shape(W8A8Args a) {
     using Sh = DmaTile<WM, WN, TI, TJ, STAGES, LK>;
-    __shared__ __attribute__((aligned(1024))) int8_t smem[Sh::kSmem];
+    __shared__ __attribute__((aligned(1024))) int8_t smem[Sh::kSmemFac];
     w8a8_dma_body<ODT, WM, WN, TI, TJ, STAGES, LK>(a, smem, (int64_t)blockIdx.y * Sh::kLM, (int64_t)blockIdx.x * Sh::kLN);
 }
 
