@@ -1339,18 +1339,21 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
 }
 
 // x' = bf16(x * smooth[k]) over the whole activation matrix (K % 8 == 0): used when the caller lends a
-// workspace, so that the multiply is done once instead of once per column tile
-__global__ __launch_bounds__(kBlock) void smooth_rows(const uint16_t* x, const uint16_t* smooth, uint16_t* y, int64_t nvec, int kvec) {
-    const int64_t stride = (int64_t)gridDim.x * kBlock;
-    for (int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += stride) {
+// workspace, so that the multiply is done once instead of once per column tile.  Block `block` of `nblocks`.
+AMCT_DEV void smooth_rows_body(const uint16_t* x, const uint16_t* smooth, uint16_t* y, int64_t nvec, int kvec, unsigned block, unsigned nblocks) {
+    const int64_t stride = (int64_t)nblocks * kBlock;
+    for (int64_t v = (int64_t)block * kBlock + threadIdx.x; v < nvec; v += stride) {
         const uint4 c = ldg16(smooth + (v % kvec) * 8);
         stg16(y + v * 8, smooth8(ldg16_nt(x + v * 8), c));
     }
 }
+__global__ __launch_bounds__(kBlock) void smooth_rows(const uint16_t* x, const uint16_t* smooth, uint16_t* y, int64_t nvec, int kvec) {
+    smooth_rows_body(x, smooth, y, nvec, kvec, blockIdx.x, gridDim.x);
+}
 // the same for fp16 activations: x' = fp16(x * smooth[k])
-__global__ __launch_bounds__(kBlock) void smooth_rows_f16(const uint16_t* x, const uint16_t* smooth, uint16_t* y, int64_t nvec, int kvec) {
-    const int64_t stride = (int64_t)gridDim.x * kBlock;
-    for (int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += stride) {
+AMCT_DEV void smooth_rows_f16_body(const uint16_t* x, const uint16_t* smooth, uint16_t* y, int64_t nvec, int kvec, unsigned block, unsigned nblocks) {
+    const int64_t stride = (int64_t)nblocks * kBlock;
+    for (int64_t v = (int64_t)block * kBlock + threadIdx.x; v < nvec; v += stride) {
         const uint4 c = ldg16(smooth + (v % kvec) * 8), xv = ldg16_nt(x + v * 8);
         const uint32_t xs[4] = {xv.x, xv.y, xv.z, xv.w}, cs[4] = {c.x, c.y, c.z, c.w};
         uint32_t o[4];
@@ -1361,24 +1364,48 @@ __global__ __launch_bounds__(kBlock) void smooth_rows_f16(const uint16_t* x, con
         stg16(y + v * 8, make_uint4(o[0], o[1], o[2], o[3]));
     }
 }
+__global__ __launch_bounds__(kBlock) void smooth_rows_f16(const uint16_t* x, const uint16_t* smooth, uint16_t* y, int64_t nvec, int kvec) {
+    smooth_rows_f16_body(x, smooth, y, nvec, kvec, blockIdx.x, gridDim.x);
+}
 
-// The whole weight dequantised once, dt((u - z) * s) as the tile kernels compute it per block, 32 weights (16 bytes of
-// nibbles, one group: group % 32 == 0) per thread and step: for so many rows that dequantising inside every row tile
-// costs more than writing and re-reading the 16-bit weight (the product is then the plain 16-bit GEMM on the large
-// tiles of the W8A8 kernel, gemm_w8a8.hip: gemm16_tiles).
+// The whole weight dequantised once, dt((u - z) * s) as the tile kernels compute it per block: for so many rows that
+// dequantising inside every row tile costs more than writing and re-reading the 16-bit weight (the product is then the
+// plain 16-bit GEMM on the large tiles of the W8A8 kernel, gemm_w8a8.hip: gemm16_tiles).  A thread takes 8 weights at a
+// time (4 bytes of nibbles in, 16 bytes out), the threads of a block walk along a row: a wave reads 256 and writes 1024
+// contiguous bytes per step.  group % 8 == 0, so the 8 weights share a group.
+#ifndef AMCT_DQ_ROWS
+#define AMCT_DQ_ROWS 4
+#endif
+constexpr int kDqRows = AMCT_DQ_ROWS;                               // rows of the weight per block, their loads in flight together
+// The first `wblocks` blocks of the launch dequantise (kDqRows rows each); the others, if any, smooth the activations
+// into `xs` (two independent passes in one launch: the short one runs beside the long one).
 template <bool AF16>
-__global__ __launch_bounds__(kBlock) void w4_dequant_rows(W4A16Args a, uint16_t* wdq, int64_t nvec) {   // nvec = N * K / 32
-    const int64_t stride = (int64_t)gridDim.x * kBlock;
-    const int64_t G = a.K / a.group;
-    for (int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += stride) {
-        const int64_t e = v * 32, row = e / a.K, k = e - row * a.K;
-        const int64_t gi = row * G + k / a.group;
-        const float s = load_scale(a, gi), nzs = -((float)a.zeros[gi] * s);
-        const uint4 w = ldg16_nt(a.wq + e / 2);
-        stg16(wdq + e, dequant8<AF16>(w.x, s, nzs));
-        stg16(wdq + e + 8, dequant8<AF16>(w.y, s, nzs));
-        stg16(wdq + e + 16, dequant8<AF16>(w.z, s, nzs));
-        stg16(wdq + e + 24, dequant8<AF16>(w.w, s, nzs));
+__global__ __launch_bounds__(kBlock) void w4_dequant_rows(W4A16Args a, uint16_t* wdq, uint16_t* xs, unsigned wblocks) {
+    if (blockIdx.x >= wblocks) {
+        const int64_t nvec = a.M * a.K / 8;
+        if constexpr (AF16) smooth_rows_f16_body(a.x, a.smooth, xs, nvec, (int)(a.K / 8), blockIdx.x - wblocks, gridDim.x - wblocks);
+        else smooth_rows_body(a.x, a.smooth, xs, nvec, (int)(a.K / 8), blockIdx.x - wblocks, gridDim.x - wblocks);
+        return;
+    }
+    const uint32_t kv = (uint32_t)(a.K >> 3), G = (uint32_t)(a.K / a.group);
+    const bool small_k = a.K < 65536;                               // k / group by the multiply-high then
+    const int64_t row0 = (int64_t)blockIdx.x * kDqRows;
+    for (uint32_t v = threadIdx.x; v < kv; v += kBlock) {
+        const uint32_t k = v * 8;
+        const uint32_t g = small_k ? __umulhi(k, a.group_magic) : k / (uint32_t)a.group;
+        uint32_t w[kDqRows];
+        float sc[kDqRows], nzs[kDqRows];
+#pragma unroll
+        for (int r = 0; r < kDqRows; ++r) {
+            const int64_t row = row0 + r < a.N ? row0 + r : a.N - 1;
+            const int64_t gi = row * G + g;
+            w[r] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(a.wq + row * (a.K >> 1)) + v);
+            sc[r] = load_scale(a, gi);
+            nzs[r] = -((float)a.zeros[gi] * sc[r]);
+        }
+#pragma unroll
+        for (int r = 0; r < kDqRows; ++r)
+            if (row0 + r < a.N) stg16(wdq + (row0 + r) * a.K + k, dequant8<AF16>(w[r], sc[r], nzs[r]));
     }
 }
 
@@ -1787,9 +1814,10 @@ int gemm16_tiles(const void* x, const void* w, const float* bias, void* out, int
 
 // From this many rows on, dequantising the weight once into a lent workspace and running the plain 16-bit GEMM beats
 // dequantising inside every row tile.  Measured on W[14336,4096] with smoothing, fused kernel / two passes: M = 1024
-// 130 / 141 us, 1536 214 / 209, 2048 221 / 217, 3072 332 / 331, 4096 445 / 393: the weight pass costs 35 us, a row of
-// the plain GEMM 0.083 us against 0.107 us for the fused kernel.
-constexpr int64_t kTwoPassFrom = 3584;
+// 132 / 132 us, 1088 209 / 187, 1280 209 / 188, 1536 214 / 206, 2048 222 / 209, 3072 333 / 321, 4096 439 / 384: the
+// weight pass costs 26 us, a row of the plain GEMM 0.083 us against 0.107 us for the fused kernel, and up to 1024 rows
+// the fused kernel's tiles fit the CUs in one round.
+constexpr int64_t kTwoPassFrom = 1025;
 
 static size_t two_pass_workspace(int64_t M, int64_t N, int64_t K, int group, int has_smooth) {
     if (M < kTwoPassFrom || K % 64 != 0 || N % 8 != 0 || group % 32 != 0 || K % group != 0 || N * K * 2 >= (int64_t(1) << 32) ||
@@ -1810,20 +1838,17 @@ static int two_pass(const void* x, const void* smooth, const uint8_t* wq, const 
                 (uint32_t)(0x100000000ull / (uint64_t)group) + 1u};
     uint16_t* wdq = reinterpret_cast<uint16_t*>(workspace);
     uint16_t* xs = wdq + (size_t)N * (size_t)K;
-    const int64_t nvec_w = N * K / 32;
-    int64_t nb = (nvec_w + kBlock - 1) / kBlock;
-    if (nb > 8192) nb = 8192;
-    if (dtype == AMCT_F16) hipLaunchKernelGGL((w4_dequant_rows<true>), dim3((unsigned)nb), dim3(kBlock), 0, st, a, wdq, nvec_w);
-    else hipLaunchKernelGGL((w4_dequant_rows<false>), dim3((unsigned)nb), dim3(kBlock), 0, st, a, wdq, nvec_w);
-    const void* xa = x;
-    if (smooth) {
-        const int64_t nvec = M * K / 8;
-        int64_t nbs = (nvec + kBlock - 1) / kBlock;
-        if (nbs > 16384) nbs = 16384;
-        if (dtype == AMCT_F16) hipLaunchKernelGGL(smooth_rows_f16, dim3((unsigned)nbs), dim3(kBlock), 0, st, a.x, a.smooth, xs, nvec, (int)(K / 8));
-        else hipLaunchKernelGGL(smooth_rows, dim3((unsigned)nbs), dim3(kBlock), 0, st, a.x, a.smooth, xs, nvec, (int)(K / 8));
-        xa = xs;
+    const int64_t wblocks = (N + kDqRows - 1) / kDqRows;
+    int64_t sblocks = 0;
+    if (smooth) {                                                   // about 4 vectors of 16 bytes per thread
+        sblocks = (M * K / 8 + 4 * kBlock - 1) / (4 * kBlock);
+        if (sblocks > 16384) sblocks = 16384;
     }
+    if (wblocks + sblocks > 0x7FFFFFFF) return AMCT_E_UNSUPPORTED;
+    const dim3 grid((unsigned)(wblocks + sblocks));
+    if (dtype == AMCT_F16) hipLaunchKernelGGL((w4_dequant_rows<true>), grid, dim3(kBlock), 0, st, a, wdq, xs, (unsigned)wblocks);
+    else hipLaunchKernelGGL((w4_dequant_rows<false>), grid, dim3(kBlock), 0, st, a, wdq, xs, (unsigned)wblocks);
+    const void* xa = smooth ? (const void*)xs : x;
     return gemm16_tiles(xa, wdq, bias, out, M, N, K, dtype, st);
 }
 

@@ -456,24 +456,43 @@ namespace amct {
 // tile kernel above computes it per block, and the product is the plain 16-bit GEMM on the 256x256 tiles of the W8A8
 // kernel (gemm_w8a8.hip: gemm16_tiles); the activations are smoothed into the workspace first when asked for.
 // ---------------------------------------------------------------------------
+// A thread takes 8 weights at a time (8 bytes in, 16 bytes out; group % 8 == 0, so they share a group), the threads of
+// a block walk along kW8Rows rows at once: a wave reads 512 and writes 1024 contiguous bytes per row and step.  The
+// first `wblocks` blocks of the launch dequantise; the others, if any, smooth the activations into `xs` (two independent
+// passes in one launch: the short one runs beside the long one).
+constexpr int kW8Rows = 4;
 template <int DT>
-__global__ __launch_bounds__(kBlock) void w8_dequant_rows(WqArgs a, uint16_t* wdq, int64_t nvec) {   // nvec = N * K / 16
-    const int64_t stride = (int64_t)gridDim.x * kBlock;
-    const int64_t G = a.K / a.group;
-    for (int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += stride) {
-        const int64_t e = v * 16, row = e / a.K, k = e - row * a.K;          // 16 weights of one row and one group
-        const int64_t gi = row * G + k / a.group;
-        const float s = wq_scale(a, gi), nzs = -(wq_zero<8>(a, gi) * s);
-        const uint4 w = ldg16_nt(a.wq + e);
-        stg16(wdq + e, dq8_int8<DT>(w.x, w.y, s, nzs));
-        stg16(wdq + e + 8, dq8_int8<DT>(w.z, w.w, s, nzs));
-    }
+AMCT_DEV void smooth_rows_dt_body(const uint16_t* x, const uint16_t* smooth, uint16_t* y, int64_t nvec, int kvec, unsigned block, unsigned nblocks) {
+    const int64_t stride = (int64_t)nblocks * kBlock;
+    for (int64_t v = (int64_t)block * kBlock + threadIdx.x; v < nvec; v += stride)
+        stg16(y + v * 8, smooth8_dt<DT>(ldg16_nt(x + v * 8), ldg16(smooth + (v % kvec) * 8)));
 }
 template <int DT>
-__global__ __launch_bounds__(kBlock) void smooth_rows_dt(const uint16_t* x, const uint16_t* smooth, uint16_t* y, int64_t nvec, int kvec) {
-    const int64_t stride = (int64_t)gridDim.x * kBlock;
-    for (int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += stride)
-        stg16(y + v * 8, smooth8_dt<DT>(ldg16_nt(x + v * 8), ldg16(smooth + (v % kvec) * 8)));
+__global__ __launch_bounds__(kBlock) void w8_dequant_rows(WqArgs a, uint16_t* wdq, uint16_t* xs, unsigned wblocks) {
+    if (blockIdx.x >= wblocks) {
+        smooth_rows_dt_body<DT>(a.x, a.smooth, xs, a.M * a.K / 8, (int)(a.K / 8), blockIdx.x - wblocks, gridDim.x - wblocks);
+        return;
+    }
+    const uint32_t kv = (uint32_t)(a.K >> 3), G = (uint32_t)(a.K / a.group);
+    const bool small_k = a.K < 65536;                               // k / group by the multiply-high then
+    const int64_t row0 = (int64_t)blockIdx.x * kW8Rows;
+    for (uint32_t v = threadIdx.x; v < kv; v += kBlock) {
+        const uint32_t k = v * 8;
+        const uint32_t g = small_k ? __umulhi(k, a.group_magic) : k / (uint32_t)a.group;
+        u2v w[kW8Rows];
+        float sc[kW8Rows], nzs[kW8Rows];
+#pragma unroll
+        for (int r = 0; r < kW8Rows; ++r) {
+            const int64_t row = row0 + r < a.N ? row0 + r : a.N - 1;
+            const int64_t gi = row * G + g;
+            w[r] = __builtin_nontemporal_load(reinterpret_cast<const u2v*>(a.wq + row * a.K) + v);
+            sc[r] = wq_scale(a, gi);
+            nzs[r] = -(wq_zero<8>(a, gi) * sc[r]);
+        }
+#pragma unroll
+        for (int r = 0; r < kW8Rows; ++r)
+            if (row0 + r < a.N) stg16(wdq + (row0 + r) * a.K + k, dq8_int8<DT>(w[r].x, w[r].y, sc[r], nzs[r]));
+    }
 }
 
 int gemm16_tiles(const void* x, const void* w, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int dtype,
@@ -527,20 +546,16 @@ extern "C" int amct_gemm_w8a16_ws(const void* x, const void* smooth, const int8_
         (!smooth || aligned16(smooth)) && (reinterpret_cast<uintptr_t>(scales) & 1u) == 0) {
         uint16_t* wdq = reinterpret_cast<uint16_t*>(workspace);
         uint16_t* xs = wdq + (size_t)N * (size_t)K;
-        const int64_t nvec_w = N * K / 16;
-        int64_t nb = (nvec_w + kBlock - 1) / kBlock;
-        if (nb > 8192) nb = 8192;
-        if (dtype == AMCT_BF16) hipLaunchKernelGGL((w8_dequant_rows<AMCT_BF16>), dim3((unsigned)nb), dim3(kBlock), 0, st, a, wdq, nvec_w);
-        else hipLaunchKernelGGL((w8_dequant_rows<AMCT_F16>), dim3((unsigned)nb), dim3(kBlock), 0, st, a, wdq, nvec_w);
-        const void* xa = x;
-        if (smooth) {
-            const int64_t nvec = M * K / 8;
-            int64_t nbs = (nvec + kBlock - 1) / kBlock;
-            if (nbs > 16384) nbs = 16384;
-            if (dtype == AMCT_BF16) hipLaunchKernelGGL((smooth_rows_dt<AMCT_BF16>), dim3((unsigned)nbs), dim3(kBlock), 0, st, a.x, a.smooth, xs, nvec, (int)(K / 8));
-            else hipLaunchKernelGGL((smooth_rows_dt<AMCT_F16>), dim3((unsigned)nbs), dim3(kBlock), 0, st, a.x, a.smooth, xs, nvec, (int)(K / 8));
-            xa = xs;
+        const int64_t wblocks = (N + kW8Rows - 1) / kW8Rows;
+        int64_t sblocks = 0;
+        if (smooth) {                                               // about 4 vectors of 16 bytes per thread
+            sblocks = (M * K / 8 + 4 * kBlock - 1) / (4 * kBlock);
+            if (sblocks > 16384) sblocks = 16384;
         }
+        const dim3 grid((unsigned)(wblocks + sblocks));             // N * K < 2^31 (workspace check): far below the grid limit
+        if (dtype == AMCT_BF16) hipLaunchKernelGGL((w8_dequant_rows<AMCT_BF16>), grid, dim3(kBlock), 0, st, a, wdq, xs, (unsigned)wblocks);
+        else hipLaunchKernelGGL((w8_dequant_rows<AMCT_F16>), grid, dim3(kBlock), 0, st, a, wdq, xs, (unsigned)wblocks);
+        const void* xa = smooth ? (const void*)xs : x;
         const int rc = gemm16_tiles(xa, wdq, bias, out, M, N, K, dtype, st);
         if (rc != AMCT_E_UNSUPPORTED) return rc;
         // (the two preparatory kernels above only wrote the workspace: the call below starts from the caller's operands)

@@ -254,7 +254,7 @@ int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s_tok, const
  * workspace (may be null): amct_gemm_w4a16_workspace_bytes(M, N, K, group, smooth != null) bytes the caller lends,
  * 16-byte aligned, contents irrelevant before and after the call.  For M > 16 with smooth the multiply is then done
  * once up front instead of inside every column tile (same results; the fast bf16 tile kernels need it, without it such
- * calls take slower kernels that smooth in place).  From M = 3584 on the query also asks for N * K * 2 bytes: the weight
+ * calls take slower kernels that smooth in place).  From M = 1025 on the query also asks for N * K * 2 bytes: the weight
  * is then dequantised once into the workspace and the product runs as a plain 16-bit GEMM, which beats dequantising inside
  * every row tile from there on (same arithmetic; a smaller workspace keeps the fused kernels).  0 bytes are asked for
  * otherwise; a null or smaller workspace is never an error.
