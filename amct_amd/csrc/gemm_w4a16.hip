@@ -1030,7 +1030,7 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM
 // ---------------------------------------------------------------------------
 // Tile (64*TI) x (64*TJ): 2 x 2 matrix waves of (32*TI) x (32*TJ) and 8 data-movement waves (512 / (64*TJ) threads per
 // weight row of the tile); 128x128 as described above, 64x64 and 128x64 for small M (8 weights per thread and step).
-template <bool SF16, int STAGES, int TI = 2, int TJ = 2, int kD = 4>
+template <bool SF16, int STAGES, int TI = 2, int TJ = 2, int kD = 4, bool AF16 = false>
 __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) void w4a16_tile_spec(W4A16Args a) {
     constexpr int kLM = 64 * TI, kLN = 64 * TJ, WN = 2;
     constexpr int kThreads = kSpecThreads;
@@ -1126,9 +1126,9 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
             __builtin_amdgcn_sched_barrier(0);                      // keeps the read in front of the writes
             const float sc = SF16 ? f16_bits_to_f32(e & 0xFFFFu) : bf16_bits_to_f32(e & 0xFFFFu);
             const float nzs = -((float)(e >> 16) * sc);
-            *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[0]) = dequant8((uint32_t)wreg[slot], sc, nzs);
+            *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[0]) = dequant8<AF16>((uint32_t)wreg[slot], sc, nzs);
             if constexpr (kBC == 2)
-                *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[1]) = dequant8((uint32_t)((uint64_t)wreg[slot] >> 32), sc, nzs);
+                *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[1]) = dequant8<AF16>((uint32_t)((uint64_t)wreg[slot] >> 32), sc, nzs);
         };
 #define AMCT_TIE_SLOT(slot) asm volatile("" : "+v"(wreg[slot]) : : "memory")
         // prologue: B(0 .. kD-1) into their slots and A(0 .. STAGES-2); everything lands; B(0), B(1) are dequantised into
@@ -1208,7 +1208,12 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
     };
     auto mfma_one = [&](int m, const v8bf (&fa)[TI], const v8bf (&fb)[TJ]) {
         const int i = m / TJ, j = m % TJ;
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        if constexpr (AF16) {
+            typedef _Float16 v8hs __attribute__((ext_vector_type(8)));
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8hs, fa[i]), __builtin_bit_cast(v8hs, fb[j]), acc[i][j], 0, 0, 0);
+        } else {
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
     };
     // One fragment buffer per k-slice: a 64x64 wave tile has only 4 MFMAs per slice, fewer cycles than an LDS read
     // takes, so the reads of slices 1..3 of a step are all issued behind the MFMAs of slice 0 (the stage is complete
@@ -1306,7 +1311,7 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 
-    // epilogue (matrix waves only): + bias (or + (-0.0f)), narrow to bf16, transpose through a per-wave LDS patch
+    // epilogue (matrix waves only): + bias (or + (-0.0f)), narrow to the activation type, transpose through a per-wave LDS patch
     constexpr int kPW = 32 * TJ, kPatchRow = kPW * 2 + 16, CPR = kPW * 2 / 16;
     uint8_t* patch = smem + wave * 16384;
     float bs[TJ];
@@ -1324,7 +1329,7 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
             const int prow0 = 8 * (r >> 2) + (r & 3);
 #pragma unroll
             for (int j = 0; j < TJ; ++j)
-                *reinterpret_cast<uint16_t*>(wbase + prow0 * kPatchRow + j * 64) = (uint16_t)f32_to_bf16_bits(acc[i][j][r] + bs[j]);
+                *reinterpret_cast<uint16_t*>(wbase + prow0 * kPatchRow + j * 64) = (uint16_t)(AF16 ? f32_to_f16_bits(acc[i][j][r] + bs[j]) : f32_to_bf16_bits(acc[i][j][r] + bs[j]));
         }
 #pragma unroll
         for (int it = 0; it < 32 * CPR / 64; ++it) {
@@ -1886,17 +1891,18 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
                                     workspace_bytes, (hipStream_t)stream);
             if (rc != AMCT_E_UNSUPPORTED) return rc;
         }
-        // more than 64 rows: the tile kernels with fp16 operands (the same bodies: the dequantised weight and the smoothed
+        // more than 16 rows: the tile kernels with fp16 operands (the same bodies: the dequantised weight and the smoothed
         // activations are rounded to fp16 instead of bf16, one v_cvt_pk_f16_f32 per pair, and the MFMAs are the f16 ones);
-        // the same conditions and block shapes as for bf16 below (without the kernels with specialised waves), and the
-        // caller's workspace when the activations are to be smoothed
+        // the same conditions and block shapes as for bf16 below (up to 64 rows only the kernels with specialised waves,
+        // i.e. K % 256 == 0), and the caller's workspace when the activations are to be smoothed
         {
             hipStream_t st = (hipStream_t)stream;
             const int64_t cus = current_cu_count();
             const int64_t mt = (M + 127) / 128, nt64 = (N + 63) / 64, nt128 = (N + 127) / 128, nt256 = (N + 255) / 256, G = K / group;
             const bool ok = aligned16(x) && aligned16(wq) && (!smooth || aligned16(smooth)) && aligned16(out) && K % 128 == 0 &&
                             K < 65536 && N % 8 == 0 && group % 64 == 0 && M * K * 2 < (int64_t(1) << 32) &&
-                            N * (K / 2) < (int64_t(1) << 32) && N * G * 2 < (int64_t(1) << 32) && M > 64 && cus > 0 &&
+                            N * (K / 2) < (int64_t(1) << 32) && N * G * 2 < (int64_t(1) << 32) && cus > 0 &&
+                            (M > 64 || (M > 16 && K % 256 == 0 && G <= kSpecMaxG)) &&   // few rows: only the kernels with specialised waves
                             mt <= 65535 && (!smooth || (workspace && workspace_bytes >= (size_t)(M * K * 2) && aligned16(workspace)));
             if (ok) {
                 W4A16Args a{(const uint16_t*)x, (const uint16_t*)smooth, wq, scales, zeros, bias, (uint16_t*)out, M, N, K, group,
@@ -1910,13 +1916,19 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
                     a.smooth = nullptr;
                 }
                 int shape = 0;
-                if (mt * nt64 <= cus) shape = 4;
+                if (M <= 64 && nt64 <= cus) shape = 3;
+                else if (mt * nt64 <= cus) shape = 4;
                 else if (mt * nt128 <= cus) shape = 1;
                 else if (mt * nt256 <= cus || M < 256) shape = 2;
+                const bool spec = K % 256 == 0 && G <= kSpecMaxG;   // 4 matrix + 8 data-movement waves, as for bf16
                 const dim3 grid((unsigned)((N + kQN - 1) / kQN), (unsigned)((M + kQM - 1) / kQM));
 #define AMCT_LAUNCH_WIDE_F16(SF)                                                                                       \
     {                                                                                                                  \
-        if (shape == 4) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 2, 1, 3, 3, true>), dim3((unsigned)nt64, (unsigned)mt), dim3(256), 0, st, a); \
+        if (shape == 3 && spec) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3, 1, 1, 4, true>), dim3((unsigned)nt64, 1), dim3(kSpecThreads), 0, st, a); \
+        else if (shape == 4 && spec) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3, 2, 1, 4, true>), dim3((unsigned)nt64, (unsigned)mt), dim3(kSpecThreads), 0, st, a); \
+        else if (shape == 1 && spec) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3, 2, 2, 4, true>), dim3((unsigned)nt128, (unsigned)mt), dim3(kSpecThreads), 0, st, a); \
+        else if (shape == 3) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 1, 1, 3, 3, true>), dim3((unsigned)nt64, 1), dim3(256), 0, st, a); \
+        else if (shape == 4) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 2, 1, 3, 3, true>), dim3((unsigned)nt64, (unsigned)mt), dim3(256), 0, st, a); \
         else if (shape == 1) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 2, 2, 2, 3, 3, true>), dim3((unsigned)nt128, (unsigned)mt), dim3(256), 0, st, a); \
         else if (shape == 2 && M > 256 && (M + 255) / 256 * nt128 <= cus) hipLaunchKernelGGL((w4a16_tile_wide<SF, 4, 2, 2, 2, 3, 3, true>), dim3((unsigned)nt128, (unsigned)((M + 255) / 256)), dim3(512), 0, st, a); \
         else if (shape == 2) hipLaunchKernelGGL((w4a16_tile_wide<SF, 2, 4, 2, 2, 3, 3, true>), dim3((unsigned)nt256, (unsigned)mt), dim3(512), 0, st, a); \

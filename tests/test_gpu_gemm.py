@@ -347,12 +347,14 @@ def test_gemms_at_the_benchmark_size(dev, M):
 
 
 @pytest.mark.parametrize("M,N,K", [(2048, 14336, 4096), (520, 14336, 4096), (300, 14336, 4096), (130, 14336, 4096),
-                                   (70, 14336, 4096), (200, 20000, 1024), (65, 72, 128)])
+                                   (70, 14336, 4096), (200, 20000, 1024), (65, 72, 128), (17, 14336, 4096), (40, 14336, 4096),
+                                   (64, 520, 1024), (33, 200, 512), (100, 1000, 768), (128, 20000, 256), (24, 72, 128)])
 def test_w4a16_fp16_at_the_benchmark_size(dev, M, N, K):
-    """fp16 activations, more than 64 rows: the tile kernels with fp16 operands, every block shape the dispatch knows
-    (256x256, 256x128, 128x256, 128x128, 128x64), with the lent workspace when the activations are smoothed (which
-    ops.gemm_w4a16 lends); sampled rows within 1e-3 of the row's largest output (plus half an fp16 ulp of the value) of
-    the fp64 anchor whose dequantised weight is rounded to fp16, every column; both factor dtypes."""
+    """fp16 activations, more than 16 rows: the tile kernels with fp16 operands, every block shape the dispatch knows
+    (256x256, 256x128, 128x256, 128x128, 128x64, 64x64; with specialised waves when K is a multiple of 256, the only
+    tile kernels up to 64 rows; the dequantise-once form from 1025 rows on), with the lent workspace when the activations
+    are smoothed (which ops.gemm_w4a16 lends); sampled rows within 1e-3 of the row's largest output (plus half an fp16
+    ulp of the value) of the fp64 anchor whose dequantised weight is rounded to fp16, every column; both factor dtypes."""
     grp = 128
     rows = [r for r in FULL_ROWS if r < M]
     for sdt in (torch.float16, torch.bfloat16):
