@@ -59,6 +59,22 @@ AMCT_DEV uint32_t pack_f16x2(float lo, float hi) {
 }
 template <bool AF16> AMCT_DEV uint32_t pack_act2(float lo, float hi) { return AF16 ? pack_f16x2(lo, hi) : pack_bf16x2(lo, hi); }
 
+// 8 signed bytes (two words) -> 8 values of (q - offset) * s in the activation type: the bytes as q + 128 (one
+// v_cvt_f32_ubyteN each), z = offset + 128, one fma(u, s, -z s) per weight, as the other int8 weight-only kernels do
+template <bool AF16>
+AMCT_DEV uint4 dequant8_i8(uint32_t w0, uint32_t w1, float s, float nzs) {
+    w0 ^= 0x80808080u;
+    w1 ^= 0x80808080u;
+    asm("" : "+v"(w0), "+v"(w1));
+    float e[8];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        e[b] = __builtin_fmaf((float)((w0 >> (8 * b)) & 0xFFu), s, nzs);
+        e[4 + b] = __builtin_fmaf((float)((w1 >> (8 * b)) & 0xFFu), s, nzs);
+    }
+    return make_uint4(pack_act2<AF16>(e[0], e[1]), pack_act2<AF16>(e[2], e[3]), pack_act2<AF16>(e[4], e[5]), pack_act2<AF16>(e[6], e[7]));
+}
+
 // 8 nibbles of `w` (element j in bits 4j..4j+3) -> 8 values of (u - z) * s in the activation type, as 4 packed dwords
 template <bool AF16 = false>
 AMCT_DEV uint4 dequant8(uint32_t w, float s, float nzs) {
@@ -1030,7 +1046,9 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(WM
 // ---------------------------------------------------------------------------
 // Tile (64*TI) x (64*TJ): 2 x 2 matrix waves of (32*TI) x (32*TJ) and 8 data-movement waves (512 / (64*TJ) threads per
 // weight row of the tile); 128x128 as described above, 64x64 and 128x64 for small M (8 weights per thread and step).
-template <bool SF16, int STAGES, int TI = 2, int TJ = 2, int kD = 4, bool AF16 = false>
+// WBITS = 8: the weight is int8 [N, K] (a.wq), a.zeros the int8 offsets or null; everything but the weight loads (twice the
+// bytes per thread and step) and the dequantisation is the int4 kernel.
+template <bool SF16, int STAGES, int TI = 2, int TJ = 2, int kD = 4, bool AF16 = false, int WBITS = 4>
 __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) void w4a16_tile_spec(W4A16Args a) {
     constexpr int kLM = 64 * TI, kLN = 64 * TJ, WN = 2;
     constexpr int kThreads = kSpecThreads;
@@ -1067,7 +1085,8 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
         for (int j = 0; j < kIt; ++j) {
             const uint32_t g = g0 + j * kTPR < G ? g0 + j * kTPR : G - 1;
             sb[j] = reinterpret_cast<const uint16_t*>(a.scales)[wr * G + g];
-            zb[j] = a.zeros[wr * G + g];
+            if constexpr (WBITS == 4) zb[j] = a.zeros[wr * G + g];
+            else zb[j] = a.zeros ? (uint32_t)((int)reinterpret_cast<const int8_t*>(a.zeros)[wr * G + g] + 128) : 128u;
         }
 #pragma unroll
         for (int j = 0; j < kIt; ++j)
@@ -1098,20 +1117,25 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
         // weight row ptid/kPPR of the tile, 8*kBC weights (4*kBC bytes) per step, which part from ptid%kPPR
         const int brow = ptid / kPPR, bq = ptid % kPPR;
         const int64_t wrow = (n0 + brow < a.N) ? n0 + brow : a.N - 1;
-        const uint32_t woff = (uint32_t)(wrow * (a.K / 2) + bq * (4 * kBC));
+        constexpr int kWB = WBITS == 4 ? 4 : 8;                     // bytes of 8 weights
+        const uint32_t woff = (uint32_t)(wrow * (a.K * kWB / 8) + bq * (kWB * kBC));
         const uint32_t* const trow = tab + brow * (kSpecMaxG + 1);
         int bdst[kBC];
 #pragma unroll
         for (int c = 0; c < kBC; ++c) bdst[c] = kLM * kWRow + brow * kWRow + ((kBC * bq + c) ^ swz(brow)) * 16;
         // The weights stream from HBM and a step of this small tile is shorter than that latency, so the packed
         // weights of a step are fetched kD steps ahead into kD register slots (the loop is unrolled by kD).
-        typename std::conditional<kBC == 2, uint64_t, uint32_t>::type wreg[kD];
+        typedef unsigned int wq4 __attribute__((ext_vector_type(4)));
+        typename std::conditional<kWB * kBC == 16, wq4, typename std::conditional<kWB * kBC == 8, uint64_t, uint32_t>::type>::type wreg[kD];
         auto issue_b = [&](int slot, int step) {
             const int st = step < last ? step : last;
-            if constexpr (kBC == 2)
-                asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(wreg[slot]) : "v"(woff), "s"(a.wq + (uint32_t)st * (kWK / 2)) : "memory");
+            const uint8_t* src = a.wq + (uint32_t)st * (kWK * kWB / 8);
+            if constexpr (kWB * kBC == 16)
+                asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(wreg[slot]) : "v"(woff), "s"(src) : "memory");
+            else if constexpr (kWB * kBC == 8)
+                asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(wreg[slot]) : "v"(woff), "s"(src) : "memory");
             else
-                asm volatile("global_load_dword %0, %1, %2" : "=v"(wreg[slot]) : "v"(woff), "s"(a.wq + (uint32_t)st * (kWK / 2)) : "memory");
+                asm volatile("global_load_dword %0, %1, %2" : "=v"(wreg[slot]) : "v"(woff), "s"(src) : "memory");
         };
         // the factors of a step are read from the table one iteration before they are used (enext): the LDS latency
         // would otherwise head the chain table read -> arithmetic -> LDS write -> barrier that bounds a step
@@ -1126,9 +1150,17 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
             __builtin_amdgcn_sched_barrier(0);                      // keeps the read in front of the writes
             const float sc = SF16 ? f16_bits_to_f32(e & 0xFFFFu) : bf16_bits_to_f32(e & 0xFFFFu);
             const float nzs = -((float)(e >> 16) * sc);
-            *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[0]) = dequant8<AF16>((uint32_t)wreg[slot], sc, nzs);
-            if constexpr (kBC == 2)
-                *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[1]) = dequant8<AF16>((uint32_t)((uint64_t)wreg[slot] >> 32), sc, nzs);
+            if constexpr (WBITS == 4) {
+                *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[0]) = dequant8<AF16>((uint32_t)wreg[slot], sc, nzs);
+                if constexpr (kBC == 2)
+                    *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[1]) = dequant8<AF16>((uint32_t)((uint64_t)wreg[slot] >> 32), sc, nzs);
+            } else if constexpr (kBC == 2) {
+                *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[0]) = dequant8_i8<AF16>(wreg[slot].x, wreg[slot].y, sc, nzs);
+                *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[1]) = dequant8_i8<AF16>(wreg[slot].z, wreg[slot].w, sc, nzs);
+            } else {
+                *reinterpret_cast<uint4*>(smem + stg * kStageBytes + bdst[0]) =
+                    dequant8_i8<AF16>((uint32_t)wreg[slot], (uint32_t)((uint64_t)wreg[slot] >> 32), sc, nzs);
+            }
         };
 #define AMCT_TIE_SLOT(slot) asm volatile("" : "+v"(wreg[slot]) : : "memory")
         // prologue: B(0 .. kD-1) into their slots and A(0 .. STAGES-2); everything lands; B(0), B(1) are dequantised into
@@ -1855,6 +1887,50 @@ static int two_pass(const void* x, const void* smooth, const uint8_t* wq, const 
     else hipLaunchKernelGGL((w4_dequant_rows<false>), grid, dim3(kBlock), 0, st, a, wdq, xs, (unsigned)wblocks);
     const void* xa = smooth ? (const void*)xs : x;
     return gemm16_tiles(xa, wdq, bias, out, M, N, K, dtype, st);
+}
+
+// The int8 weight-only Linear (gemm_wq16.hip) on the kernels with specialised waves: 17 rows and more, while the blocks
+// of the launch fit the CUs in one round (up to 256 rows on W[14336, 4096]); K a multiple of 256, groups a multiple of 64,
+// at most kSpecMaxG of them.  With `smooth` the activations go through the pre-pass into `workspace` (M * K * 2 bytes)
+// first.  AMCT_E_UNSUPPORTED when the shape or the workspace does not allow it (nothing has been launched then).
+int w8a16_spec_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
+                        const uint8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group, int dtype,
+                        void* workspace, size_t workspace_bytes, hipStream_t st) {
+    const int64_t G = K / group, cus = current_cu_count();
+    if (M <= 16 || cus <= 0 || K % 256 != 0 || K >= 65536 || G > kSpecMaxG || group % 64 != 0 || N % 8 != 0 || !aligned16(x) ||
+        !aligned16(wq) || !aligned16(out) || (reinterpret_cast<uintptr_t>(scales) & 1u) != 0 || M * K * 2 >= (int64_t(1) << 32) ||
+        N * K >= (int64_t(1) << 32) || N * G * 2 >= (int64_t(1) << 32))
+        return AMCT_E_UNSUPPORTED;
+    if (smooth && !(workspace && workspace_bytes >= (size_t)(M * K * 2) && aligned16(workspace) && aligned16(smooth))) return AMCT_E_UNSUPPORTED;
+    const int64_t mt = (M + 127) / 128, nt64 = (N + 63) / 64, nt128 = (N + 127) / 128;
+    int shape = 0;
+    if (M <= 64 && nt64 <= cus) shape = 3;
+    else if (mt * nt64 <= cus) shape = 4;
+    else if (mt * nt128 <= cus) shape = 1;
+    if (!shape || mt > 65535) return AMCT_E_UNSUPPORTED;
+    W4A16Args a{(const uint16_t*)x, nullptr, wq, scales, offsets, bias, (uint16_t*)out, M, N, K, group, scale_dtype,
+                (uint32_t)(0x100000000ull / (uint64_t)group) + 1u};
+    if (smooth) {
+        const int64_t nvec = M * K / 8;
+        int64_t nb = (nvec + kBlock - 1) / kBlock;
+        if (nb > 16384) nb = 16384;
+        if (dtype == AMCT_F16) hipLaunchKernelGGL(smooth_rows_f16, dim3((unsigned)nb), dim3(kBlock), 0, st, a.x, (const uint16_t*)smooth, (uint16_t*)workspace, nvec, (int)(K / 8));
+        else hipLaunchKernelGGL(smooth_rows, dim3((unsigned)nb), dim3(kBlock), 0, st, a.x, (const uint16_t*)smooth, (uint16_t*)workspace, nvec, (int)(K / 8));
+        a.x = (const uint16_t*)workspace;
+    }
+#define AMCT_LAUNCH_SPEC8(SF, AF)                                                                                      \
+    {                                                                                                                  \
+        if (shape == 3) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3, 1, 1, 4, AF, 8>), dim3((unsigned)nt64, 1), dim3(kSpecThreads), 0, st, a); \
+        else if (shape == 4) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3, 2, 1, 4, AF, 8>), dim3((unsigned)nt64, (unsigned)mt), dim3(kSpecThreads), 0, st, a); \
+        else hipLaunchKernelGGL((w4a16_tile_spec<SF, 3, 2, 2, 4, AF, 8>), dim3((unsigned)nt128, (unsigned)mt), dim3(kSpecThreads), 0, st, a); \
+    }
+    if (dtype == AMCT_F16) {
+        if (scale_dtype == AMCT_F16) AMCT_LAUNCH_SPEC8(true, true) else AMCT_LAUNCH_SPEC8(false, true)
+    } else {
+        if (scale_dtype == AMCT_F16) AMCT_LAUNCH_SPEC8(true, false) else AMCT_LAUNCH_SPEC8(false, false)
+    }
+#undef AMCT_LAUNCH_SPEC8
+    return hip_status();
 }
 
 }  // namespace amct

@@ -508,12 +508,17 @@ static size_t w8a16_tiles_workspace(int64_t M, int64_t N, int64_t K, int group, 
 int w8a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
                           const uint8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group,
                           int dtype, hipStream_t st);      // gemm_w8a16_stream.hip
+int w8a16_spec_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
+                        const uint8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group, int dtype,
+                        void* workspace, size_t workspace_bytes, hipStream_t st);   // gemm_w4a16.hip
 }
 
 using namespace amct;
 
 extern "C" size_t amct_gemm_w8a16_workspace_bytes(int64_t M, int64_t N, int64_t K, int group, int has_smooth) {
-    return w8a16_tiles_workspace(M, N, K, group, has_smooth);
+    const size_t two = w8a16_tiles_workspace(M, N, K, group, has_smooth);   // many rows: the 16-bit weight as well
+    if (two) return two;
+    return has_smooth && M > 16 && N > 0 && K > 0 ? (size_t)M * (size_t)K * 2 : 0;   // tile kernels: x * smooth done once
 }
 
 extern "C" int amct_gemm_w8a16(const void* x, const void* smooth, const int8_t* wq, const void* scales, int scale_dtype,
@@ -538,6 +543,12 @@ extern "C" int amct_gemm_w8a16_ws(const void* x, const void* smooth, const int8_
     if (M <= 16) {                                   // K of 1024 / 2048 / 4096, groups of 128 .. K: the weight-streaming kernel
         const int rc = w8a16_stream_dispatch(x, smooth, reinterpret_cast<const uint8_t*>(wq), scales, scale_dtype,
                                              reinterpret_cast<const uint8_t*>(offsets), bias, out, M, N, K, group, dtype, st);
+        if (rc != AMCT_E_UNSUPPORTED) return rc;
+    }
+    if (M > 16) {                                    // while the blocks fit the CUs in one round: the kernels with specialised waves
+        const int rc = w8a16_spec_dispatch(x, smooth, reinterpret_cast<const uint8_t*>(wq), scales, scale_dtype,
+                                           reinterpret_cast<const uint8_t*>(offsets), bias, out, M, N, K, group, dtype, workspace,
+                                           workspace_bytes, st);
         if (rc != AMCT_E_UNSUPPORTED) return rc;
     }
     // many rows and a lent workspace: dequantise once, then the plain 16-bit GEMM on the large tiles

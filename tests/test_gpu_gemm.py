@@ -282,6 +282,40 @@ def test_w8a16_many_rows_through_the_workspace(dev, dtype, M, N, K, group):
     assert_bits_equal(out.cpu()[rows], want.to(dtype), "integer special case")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K,group", [(17, 14336, 4096, 128), (40, 520, 1024, 128), (64, 14336, 4096, 4096), (65, 200, 512, 64),
+                                         (128, 8200, 256, 64), (200, 1000, 768, 256), (256, 14336, 4096, 128), (100, 264, 320, 64),
+                                         (33, 20000, 256, 128)])
+def test_w8a16_medium_rows_specialised_waves(dev, dtype, M, N, K, group):
+    """Int8 weight-only Linear from 17 rows on, while the blocks fit the CUs in one round: the tile kernels with
+    specialised waves (K a multiple of 256; 64x64, 128x64 and 128x128 blocks), ragged M and N, per-channel and grouped
+    factors, symmetric and with offsets, with smoothing (through the workspace ops.gemm_w8a16 lends) and bias; one shape
+    the shared kernel keeps (K = 320).  dt((q - offset) * scale) and fp32 accumulation: within 1e-3 of the row's largest
+    output (plus half an ulp) of the fp64 anchor; small integers give an integer matmul bit for bit."""
+    from amct_amd import _lib
+    assert _lib.load().amct_gemm_w8a16_workspace_bytes(M, N, K, group, 1) >= M * K * 2
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    for sdt, sym in ((torch.float16, False), (torch.bfloat16, True)):
+        x, codes, scales, offsets, smooth, bias = w8a16_case(M, N, K, group, 190 + M % 97, dtype, sdt, sym)
+        for sm, b in ((None, None), (smooth, bias)):
+            out = ops.gemm_w8a16(x.to(dev), codes.to(dev), scales.to(dev), None if offsets is None else offsets.to(dev), group,
+                                 None if sm is None else sm.to(dev), None if b is None else b.to(dev)).cpu()
+            assert out.dtype == dtype
+            want = od.w4a16_forward_f64(x, codes.to(torch.int32), scales, None if offsets is None else -offsets.float(), group,
+                                        b, None if sm is None else sm.reshape(1, -1), round_weight=True)
+            err = (out.double() - want).abs()
+            tol = 1e-3 * want.abs().amax(dim=1, keepdim=True) + want.abs() * ulp
+            assert (err <= tol).all(), (float((err / tol).max()), sdt, sym, sm is not None)
+    g = torch.Generator().manual_seed(191)
+    xi = torch.randint(-4, 5, (M, K), generator=g).to(dtype)
+    wi = torch.randint(-7, 8, (N, K), generator=g, dtype=torch.int16).to(torch.int8)
+    zi = torch.randint(-3, 4, (N, K // group), generator=g, dtype=torch.int16).to(torch.int8)
+    ones = torch.ones(N, K // group, dtype=torch.float16)
+    out = ops.gemm_w8a16(xi.to(dev), wi.to(dev), ones.to(dev), zi.to(dev), group)
+    want = torch.matmul(xi.double(), (wi.double() - zi.double().repeat_interleave(group, dim=1)).t())
+    assert_bits_equal(out, want.to(dtype), "integer special case")
+
+
 def test_w4a16_reduces_to_plain_matmul(dev):
     """zero = 8 (code 0 in signed terms), scale = 1: the kernel is a bf16 GEMM against integer
     weights, checked against torch.matmul."""
