@@ -1889,9 +1889,10 @@ static int two_pass(const void* x, const void* smooth, const uint8_t* wq, const 
     return gemm16_tiles(xa, wdq, bias, out, M, N, K, dtype, st);
 }
 
-// The int8 weight-only Linear (gemm_wq16.hip) on the kernels with specialised waves: 17 rows and more, while the blocks
-// of the launch fit the CUs in one round (up to 256 rows on W[14336, 4096]); K a multiple of 256, groups a multiple of 64,
-// at most kSpecMaxG of them.  With `smooth` the activations go through the pre-pass into `workspace` (M * K * 2 bytes)
+// The int8 weight-only Linear (gemm_wq16.hip) on the kernels with specialised waves: 17 rows and more, while the 128x128
+// blocks of the launch fit the CUs in two rounds (up to 512 rows on W[14336, 4096]: 74 / 81 us at 384 / 512 rows against
+// 98 us for the dequantise-once form, which wins from there on: 640 rows 115 against 111 us); K a multiple of 256, groups
+// a multiple of 64, at most kSpecMaxG of them.  With `smooth` the activations go through the pre-pass into `workspace` (M * K * 2 bytes)
 // first.  AMCT_E_UNSUPPORTED when the shape or the workspace does not allow it (nothing has been launched then).
 int w8a16_spec_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
                         const uint8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group, int dtype,
@@ -1906,7 +1907,7 @@ int w8a16_spec_dispatch(const void* x, const void* smooth, const uint8_t* wq, co
     int shape = 0;
     if (M <= 64 && nt64 <= cus) shape = 3;
     else if (mt * nt64 <= cus) shape = 4;
-    else if (mt * nt128 <= cus) shape = 1;
+    else if (mt * nt128 <= 2 * cus) shape = 1;            // two rounds still beat dequantising the weight into a workspace first
     if (!shape || mt > 65535) return AMCT_E_UNSUPPORTED;
     W4A16Args a{(const uint16_t*)x, nullptr, wq, scales, offsets, bias, (uint16_t*)out, M, N, K, group, scale_dtype,
                 (uint32_t)(0x100000000ull / (uint64_t)group) + 1u};

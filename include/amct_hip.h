@@ -289,7 +289,7 @@ int amct_gemm_w8a16(const void* x, const void* smooth, const int8_t* wq, const v
  * GEMM on the 256x256 tiles of the W8A8 kernel: the same arithmetic as the tile kernel without workspace (the
  * dequantised weight rounded to dtype, fp32 accumulation), about three times as fast.  For fewer rows (M > 16) with smooth
  * the query asks for M * K * 2 bytes: the multiply is then done once up front and the fast tile kernels apply (while
- * their blocks fit the CUs in one round, K a multiple of 256, groups a multiple of 64; they take precedence up to 256
+ * their blocks fit the CUs in two rounds, K a multiple of 256, groups a multiple of 64; they take precedence up to 512
  * rows on W[14336, 4096]).  0 bytes are asked for otherwise; a null or smaller workspace is never an error. */
 size_t amct_gemm_w8a16_workspace_bytes(int64_t M, int64_t N, int64_t K, int group, int has_smooth);
 int amct_gemm_w8a16_ws(const void* x, const void* smooth, const int8_t* wq, const void* scales, int scale_dtype,
