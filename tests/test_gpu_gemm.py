@@ -250,7 +250,7 @@ def test_w8a16_weight_streaming_kernel(dev, dtype, M, N, K, group):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,N,K,group", [(2048, 14336, 4096, 128), (256, 264, 64, 64), (300, 1000, 320, 32), (513, 2056, 1024, 1024),
-                                         (1000, 4104, 192, 64)])
+                                         (1000, 4104, 192, 64), (300, 16, 65536, 256)])
 def test_w8a16_many_rows_through_the_workspace(dev, dtype, M, N, K, group):
     """Int8 weight-only Linear from 256 rows on: with the workspace the library asks for, the weight is dequantised once
     and the product is the plain 16-bit GEMM on the large tiles (uniform and mixed tile launches, ragged M and N, K of
@@ -407,7 +407,7 @@ def test_w4a16_fp16_at_the_benchmark_size(dev, M, N, K):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,N,K,group", [(1025, 1000, 320, 32), (3584, 1000, 320, 32), (4100, 264, 64, 64)])
+@pytest.mark.parametrize("M,N,K,group", [(1025, 1000, 320, 32), (3584, 1000, 320, 32), (4100, 264, 64, 64), (1100, 16, 65536, 128)])
 def test_w4a16_very_many_rows_dequantise_once(dev, dtype, M, N, K, group):
     """From 1025 rows on, with the workspace the library asks for (the 16-bit weight and the smoothed activations), the
     int4 weight is dequantised once and the product is the plain 16-bit GEMM on the large tiles; with the smaller
