@@ -316,6 +316,31 @@ def test_w8a16_medium_rows_specialised_waves(dev, dtype, M, N, K, group):
     assert_bits_equal(out, want.to(dtype), "integer special case")
 
 
+@pytest.mark.parametrize("M", [40, 300])
+def test_w8a16_smoothing_with_and_without_workspace(dev, M):
+    """With a smoothing vector the fast int8 weight-only tile kernels need the lent workspace (M * K * 2 bytes); without
+    it, or with one that is too small, the call is still served (shared kernel, smoothing inside the tile) and both
+    answers are within the tolerance of the fp64 anchor.  Through the C ABI."""
+    from amct_amd import _lib
+    lib = _lib.load()
+    N, K, group = 520, 1024, 128
+    x, codes, scales, offsets, smooth, bias = w8a16_case(M, N, K, group, 777, torch.bfloat16, torch.float16, False)
+    want = od.w4a16_forward_f64(x, codes.to(torch.int32), scales, -offsets.float(), group, bias, smooth.reshape(1, -1), round_weight=True)
+    tol = 1e-3 * want.abs().amax(dim=1, keepdim=True) + want.abs() * 2.0 ** -8
+    xd, cd, sd, zd, smd, bd = (t.to(dev) for t in (x, codes, scales, offsets, smooth, bias))
+    st = torch.cuda.current_stream(dev).cuda_stream
+    need = lib.amct_gemm_w8a16_workspace_bytes(M, N, K, group, 1)
+    assert need >= M * K * 2
+    for nbytes in (need, 0, M * K * 2 - 16):
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dev)
+        out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+        _lib.check(lib.amct_gemm_w8a16_ws(xd.data_ptr(), smd.data_ptr(), cd.data_ptr(), sd.data_ptr(), _lib.F16, zd.data_ptr(),
+                                          bd.data_ptr(), out.data_ptr(), M, N, K, group, _lib.BF16,
+                                          ws.data_ptr() if nbytes else None, nbytes, st))
+        err = (out.cpu().double() - want).abs()
+        assert (err <= tol).all(), (nbytes, float((err / tol).max()))
+
+
 def test_w4a16_reduces_to_plain_matmul(dev):
     """zero = 8 (code 0 in signed terms), scale = 1: the kernel is a bf16 GEMM against integer
     weights, checked against torch.matmul."""
