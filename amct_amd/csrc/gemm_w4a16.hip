@@ -35,6 +35,7 @@ struct W4A16Args {
     int group;
     int scale_dtype;
     uint32_t group_magic;                            // floor(2^32 / group) + 1: k / group == mulhi(k, magic) for k, group < 2^16
+    float* part;                                     // split-K launches (gridDim.z > 1): fp32 partial sums [gridDim.z, M, N]
 };
 
 AMCT_DEV float load_scale(const W4A16Args& a, int64_t i) {
@@ -1066,7 +1067,13 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int64_t m0 = (int64_t)blockIdx.y * kLM, n0 = (int64_t)blockIdx.x * kLN;
-    const int nsteps = (int)(a.K / kWK);
+    // Split K (gridDim.z > 1): block z takes the units of 256 elements [units z / S, units (z + 1) / S) of every row and
+    // leaves fp32 partial sums in a.part[z]; a second kernel adds them in order.  Rows keep their stride a.K.
+    const uint32_t units = (uint32_t)(a.K >> 8);
+    const uint32_t k0 = (units * blockIdx.z / gridDim.z) << 8;
+    const uint32_t klen = ((units * (blockIdx.z + 1) / gridDim.z) << 8) - k0;
+    const uint32_t gfirst = __umulhi(k0, a.group_magic);           // first group of the slice
+    const int nsteps = (int)(klen / kWK);
     const int last = nsteps - 1;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
     auto swz = [](int r) { return (r >> 1) & 7; };
@@ -1075,6 +1082,7 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
         // Per-step loads of a 2-byte scale and a 1-byte zero-point per thread touch 48 cache lines per wave
         // instruction; all of the tile's factors are fetched once instead, by all 512 threads.
         const uint32_t G = (uint32_t)(a.K / a.group);
+        const uint32_t Gs = __umulhi(k0 + klen - 1, a.group_magic) - gfirst + 1;   // groups the slice touches (<= kSpecMaxG: host)
         // kTPR threads share a row; all loads are issued before the first use (unconditional, clamped): a loop that
         // loads and stores entry by entry pays one memory latency per trip before the kernel's first MFMA
         constexpr int kTPR = kThreads / kLN, kIt = (kSpecMaxG + kTPR - 1) / kTPR;
@@ -1083,14 +1091,14 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
         uint32_t sb[kIt], zb[kIt];
 #pragma unroll
         for (int j = 0; j < kIt; ++j) {
-            const uint32_t g = g0 + j * kTPR < G ? g0 + j * kTPR : G - 1;
+            const uint32_t g = gfirst + (g0 + j * kTPR < Gs ? g0 + j * kTPR : Gs - 1);
             sb[j] = reinterpret_cast<const uint16_t*>(a.scales)[wr * G + g];
             if constexpr (WBITS == 4) zb[j] = a.zeros[wr * G + g];
             else zb[j] = a.zeros ? (uint32_t)((int)reinterpret_cast<const int8_t*>(a.zeros)[wr * G + g] + 128) : 128u;
         }
 #pragma unroll
         for (int j = 0; j < kIt; ++j)
-            if (g0 + j * kTPR < G) tab[row * (kSpecMaxG + 1) + g0 + j * kTPR] = sb[j] | (zb[j] << 16);
+            if (g0 + j * kTPR < Gs) tab[row * (kSpecMaxG + 1) + g0 + j * kTPR] = sb[j] | (zb[j] << 16);
         __syncthreads();
     }
 
@@ -1112,7 +1120,7 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
             const int st = step < last ? step : last;
 #pragma unroll
             for (int j = 0; j < kNA; ++j)
-                dma16s(lds0 + stg * kStageBytes + (pw * kNA + j) * 1024, a.x + (int64_t)st * kWK, goff[j]);
+                dma16s(lds0 + stg * kStageBytes + (pw * kNA + j) * 1024, a.x + k0 + (int64_t)st * kWK, goff[j]);
         };
         // weight row ptid/kPPR of the tile, 8*kBC weights (4*kBC bytes) per step, which part from ptid%kPPR
         const int brow = ptid / kPPR, bq = ptid % kPPR;
@@ -1129,7 +1137,7 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
         typename std::conditional<kWB * kBC == 16, wq4, typename std::conditional<kWB * kBC == 8, uint64_t, uint32_t>::type>::type wreg[kD];
         auto issue_b = [&](int slot, int step) {
             const int st = step < last ? step : last;
-            const uint8_t* src = a.wq + (uint32_t)st * (kWK * kWB / 8);
+            const uint8_t* src = a.wq + (k0 + (uint32_t)st * kWK) * kWB / 8;
             if constexpr (kWB * kBC == 16)
                 asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(wreg[slot]) : "v"(woff), "s"(src) : "memory");
             else if constexpr (kWB * kBC == 8)
@@ -1141,7 +1149,7 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
         // would otherwise head the chain table read -> arithmetic -> LDS write -> barrier that bounds a step
         auto factor_word = [&](int step) {
             const int st = step < last ? step : last;
-            return trow[__umulhi((uint32_t)st * kWK, a.group_magic)];          // k / group (k, group < 2^16); group % 64 == 0
+            return trow[__umulhi(k0 + (uint32_t)st * kWK, a.group_magic) - gfirst];   // k / group (k, group < 2^16); group % 64 == 0
         };
         uint32_t enext = factor_word(0);
         auto dequant_into = [&](int slot, int step, int stg) {      // the weights of K-step `step` (in `slot`) -> stage stg
@@ -1343,6 +1351,22 @@ __global__ __launch_bounds__(kSpecThreads) __attribute__((amdgpu_waves_per_eu(3,
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 
+    if (gridDim.z > 1) {
+        // split K: the raw fp32 sums of this slice, row 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32 of each 32x32 tile
+        float* const part = a.part + (int64_t)blockIdx.z * a.M * a.N;
+#pragma unroll
+        for (int i = 0; i < TI; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int64_t m = m0 + wm * 32 * TI + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+#pragma unroll
+                for (int j = 0; j < TJ; ++j) {
+                    const int64_t n = n0 + wn * 32 * TJ + j * 32 + (lane & 31);
+                    if (m < a.M && n < a.N) part[m * a.N + n] = acc[i][j][r];
+                }
+            }
+        return;
+    }
     // epilogue (matrix waves only): + bias (or + (-0.0f)), narrow to the activation type, transpose through a per-wave LDS patch
     constexpr int kPW = 32 * TJ, kPatchRow = kPW * 2 + 16, CPR = kPW * 2 / 16;
     uint8_t* patch = smem + wave * 16384;
@@ -1411,6 +1435,29 @@ __global__ __launch_bounds__(kBlock) void smooth_rows_f16(const uint16_t* x, con
 // time (4 bytes of nibbles in, 16 bytes out), the threads of a block walk along a row: a wave reads 256 and writes 1024
 // contiguous bytes per step.  group % 8 == 0, so the 8 weights share a group.
 constexpr int kDqRows = 4;      // rows of the weight per block, their loads in flight together (1 / 2 / 4 / 8: 209 / 206 / 205.6 / 206.8 us at M = 2048)
+// out = dt(part[0] + part[1] + ... + part[S - 1] + bias), the slices added in that order; 8 columns per thread (N % 8 == 0)
+template <bool AF16>
+__global__ __launch_bounds__(kBlock) void splitk_reduce16(const float* part, const float* bias, uint16_t* out, int64_t M, int64_t N, int S) {
+    const int64_t nvec = M * N / 8, stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += stride) {
+        const int64_t e = v * 8;
+        float4 lo = *reinterpret_cast<const float4*>(part + e), hi = *reinterpret_cast<const float4*>(part + e + 4);
+        for (int z = 1; z < S; ++z) {
+            const float4 a0 = *reinterpret_cast<const float4*>(part + (int64_t)z * M * N + e);
+            const float4 a1 = *reinterpret_cast<const float4*>(part + (int64_t)z * M * N + e + 4);
+            lo.x += a0.x, lo.y += a0.y, lo.z += a0.z, lo.w += a0.w;
+            hi.x += a1.x, hi.y += a1.y, hi.z += a1.z, hi.w += a1.w;
+        }
+        if (bias) {
+            const int64_t n = e % N;
+            const float4 b0 = *reinterpret_cast<const float4*>(bias + n), b1 = *reinterpret_cast<const float4*>(bias + n + 4);
+            lo.x += b0.x, lo.y += b0.y, lo.z += b0.z, lo.w += b0.w;
+            hi.x += b1.x, hi.y += b1.y, hi.z += b1.z, hi.w += b1.w;
+        }
+        stg16_nt(out + e, make_uint4(pack_act2<AF16>(lo.x, lo.y), pack_act2<AF16>(lo.z, lo.w), pack_act2<AF16>(hi.x, hi.y), pack_act2<AF16>(hi.z, hi.w)));
+    }
+}
+
 // The first `wblocks` blocks of the launch dequantise (kDqRows rows each); the others, if any, smooth the activations
 // into `xs` (two independent passes in one launch: the short one runs beside the long one).
 template <bool AF16>
@@ -1886,28 +1933,68 @@ static int two_pass(const void* x, const void* smooth, const uint8_t* wq, const 
     return gemm16_tiles(xa, wdq, bias, out, M, N, K, dtype, st);
 }
 
-// The int8 weight-only Linear (gemm_wq16.hip) on the kernels with specialised waves: 17 rows and more, while the 128x128
-// blocks of the launch fit the CUs in two rounds (up to 512 rows on W[14336, 4096]: 74 / 81 us at 384 / 512 rows against
-// 98 us for the dequantise-once form, which wins from there on: 640 rows 115 against 111 us); K a multiple of 256, groups
-// a multiple of 64, at most kSpecMaxG of them.  With `smooth` the activations go through the pre-pass into `workspace` (M * K * 2 bytes)
-// first.  AMCT_E_UNSUPPORTED when the shape or the workspace does not allow it (nothing has been launched then).
-int w8a16_spec_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
-                        const uint8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group, int dtype,
-                        void* workspace, size_t workspace_bytes, hipStream_t st) {
-    const int64_t G = K / group, cus = current_cu_count();
-    if (M <= 16 || cus <= 0 || K % 256 != 0 || K >= 65536 || G > kSpecMaxG || group % 64 != 0 || N % 8 != 0 || !aligned16(x) ||
-        !aligned16(wq) || !aligned16(out) || (reinterpret_cast<uintptr_t>(scales) & 1u) != 0 || M * K * 2 >= (int64_t(1) << 32) ||
-        N * K >= (int64_t(1) << 32) || N * G * 2 >= (int64_t(1) << 32))
-        return AMCT_E_UNSUPPORTED;
-    if (smooth && !(workspace && workspace_bytes >= (size_t)(M * K * 2) && aligned16(workspace) && aligned16(smooth))) return AMCT_E_UNSUPPORTED;
+// Block shape of the kernels with specialised waves (3: 64x64, 4: 128x64, 1: 128x128; 0: they do not apply) and the number
+// of K slices of the launch.  K is split over blocks when the tiles alone would leave CUs idle (few output columns, long
+// rows: the down projection of an MLP) or when a row has more groups than the kernel's factor table holds; a slice is
+// at least 2048 elements.  max_rounds: how many rounds of 128x128 blocks are still accepted.
+struct SpecPlan {
+    int shape;
+    int splits;
+};
+static SpecPlan spec_plan(int64_t M, int64_t N, int64_t K, int group, int64_t cus, int max_rounds) {
+    SpecPlan p{0, 1};
+    if (M <= 0 || cus <= 0 || K % 256 != 0 || K >= 65536 || group % 64 != 0 || group <= 0 || K % group != 0) return p;
     const int64_t mt = (M + 127) / 128, nt64 = (N + 63) / 64, nt128 = (N + 127) / 128;
-    int shape = 0;
-    if (M <= 64 && nt64 <= cus) shape = 3;
-    else if (mt * nt64 <= cus) shape = 4;
-    else if (mt * nt128 <= 2 * cus) shape = 1;            // two rounds still beat dequantising the weight into a workspace first
-    if (!shape || mt > 65535) return AMCT_E_UNSUPPORTED;
-    W4A16Args a{(const uint16_t*)x, nullptr, wq, scales, offsets, bias, (uint16_t*)out, M, N, K, group, scale_dtype,
-                (uint32_t)(0x100000000ull / (uint64_t)group) + 1u};
+    int64_t blocks;
+    if (M <= 64 && nt64 <= cus) p.shape = 3, blocks = nt64;
+    else if (mt * nt64 <= cus) p.shape = 4, blocks = mt * nt64;
+    else if (mt * nt128 <= max_rounds * cus) p.shape = 1, blocks = mt * nt128;
+    else return p;
+    const int64_t units = K / 256;
+    auto fits = [&](int64_t S) {                                    // the groups of every slice fit the factor table
+        for (int64_t z = 0; z < S; ++z) {
+            const int64_t k0 = units * z / S * 256, k1 = units * (z + 1) / S * 256;
+            if (k1 <= k0 || (k1 - 1) / group - k0 / group + 1 > kSpecMaxG) return false;
+        }
+        return true;
+    };
+    int64_t S = cus / blocks;
+    if (S > 8) S = 8;
+    while (S > 1 && K / S < 2048) --S;
+    if (S < 1) S = 1;
+    while (S <= 16 && S <= units && !fits(S)) ++S;
+    if (S > 16 || S > units || mt > 65535) return SpecPlan{0, 1};
+    p.splits = (int)S;
+    return p;
+}
+static size_t spec_part_bytes(const SpecPlan& p, int64_t M, int64_t N) {
+    return p.shape && p.splits > 1 ? (size_t)p.splits * (size_t)M * (size_t)N * 4 : 0;
+}
+
+// The kernels with specialised waves for int4 (WB = 4) or int8 (WB = 8) weights, with the plan above.  `smooth`: the
+// activations go through the pre-pass into the workspace first (M * K * 2 bytes; the partial sums of a split launch
+// follow).  only_split: serve only shapes whose plan splits K (the caller has its own kernels otherwise).
+// AMCT_E_UNSUPPORTED when the shape, the operands or the workspace do not allow it (nothing has been launched then).
+template <int WB>
+static int spec_launch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype, const uint8_t* zeros,
+                       const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group, int dtype, void* workspace,
+                       size_t workspace_bytes, hipStream_t st, int max_rounds, bool only_split) {
+    const int64_t G = group > 0 ? K / group : 0, cus = current_cu_count();
+    SpecPlan p = spec_plan(M, N, K, group, cus, max_rounds);
+    if (!p.shape || N % 8 != 0 || !aligned16(x) || !aligned16(wq) || !aligned16(out) || (reinterpret_cast<uintptr_t>(scales) & 1u) != 0 ||
+        M * K * 2 >= (int64_t(1) << 32) || N * K * WB / 8 >= (int64_t(1) << 32) || N * G * 2 >= (int64_t(1) << 32))
+        return AMCT_E_UNSUPPORTED;
+    const size_t xs_bytes = smooth ? (size_t)(M * K * 2) : 0;
+    const bool ws_ok = workspace && aligned16(workspace);
+    if (smooth && !(ws_ok && workspace_bytes >= xs_bytes && aligned16(smooth))) return AMCT_E_UNSUPPORTED;
+    if (p.splits > 1 && !(ws_ok && workspace_bytes >= xs_bytes + spec_part_bytes(p, M, N) && (!bias || aligned16(bias)))) {
+        // no room for the partial sums: the unsplit launch, if the factor table allows it
+        if (G > kSpecMaxG) return AMCT_E_UNSUPPORTED;
+        p.splits = 1;
+    }
+    if (only_split && p.splits == 1) return AMCT_E_UNSUPPORTED;
+    W4A16Args a{(const uint16_t*)x, nullptr, wq, scales, zeros, bias, (uint16_t*)out, M, N, K, group, scale_dtype,
+                (uint32_t)(0x100000000ull / (uint64_t)group) + 1u, nullptr};
     if (smooth) {
         const int64_t nvec = M * K / 8;
         int64_t nb = (nvec + kBlock - 1) / kBlock;
@@ -1916,19 +2003,40 @@ int w8a16_spec_dispatch(const void* x, const void* smooth, const uint8_t* wq, co
         else hipLaunchKernelGGL(smooth_rows, dim3((unsigned)nb), dim3(kBlock), 0, st, a.x, (const uint16_t*)smooth, (uint16_t*)workspace, nvec, (int)(K / 8));
         a.x = (const uint16_t*)workspace;
     }
-#define AMCT_LAUNCH_SPEC8(SF, AF)                                                                                      \
+    if (p.splits > 1) a.part = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + xs_bytes);
+    const unsigned mt = (unsigned)((M + 127) / 128), nt64 = (unsigned)((N + 63) / 64), nt128 = (unsigned)((N + 127) / 128), S = (unsigned)p.splits;
+#define AMCT_LAUNCH_SPEC(SF, AF)                                                                                       \
     {                                                                                                                  \
-        if (shape == 3) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3, 1, 1, 4, AF, 8>), dim3((unsigned)nt64, 1), dim3(kSpecThreads), 0, st, a); \
-        else if (shape == 4) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3, 2, 1, 4, AF, 8>), dim3((unsigned)nt64, (unsigned)mt), dim3(kSpecThreads), 0, st, a); \
-        else hipLaunchKernelGGL((w4a16_tile_spec<SF, 3, 2, 2, 4, AF, 8>), dim3((unsigned)nt128, (unsigned)mt), dim3(kSpecThreads), 0, st, a); \
+        if (p.shape == 3) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3, 1, 1, 4, AF, WB>), dim3(nt64, 1, S), dim3(kSpecThreads), 0, st, a); \
+        else if (p.shape == 4) hipLaunchKernelGGL((w4a16_tile_spec<SF, 3, 2, 1, 4, AF, WB>), dim3(nt64, mt, S), dim3(kSpecThreads), 0, st, a); \
+        else hipLaunchKernelGGL((w4a16_tile_spec<SF, 3, 2, 2, 4, AF, WB>), dim3(nt128, mt, S), dim3(kSpecThreads), 0, st, a); \
     }
     if (dtype == AMCT_F16) {
-        if (scale_dtype == AMCT_F16) AMCT_LAUNCH_SPEC8(true, true) else AMCT_LAUNCH_SPEC8(false, true)
+        if (scale_dtype == AMCT_F16) AMCT_LAUNCH_SPEC(true, true) else AMCT_LAUNCH_SPEC(false, true)
     } else {
-        if (scale_dtype == AMCT_F16) AMCT_LAUNCH_SPEC8(true, false) else AMCT_LAUNCH_SPEC8(false, false)
+        if (scale_dtype == AMCT_F16) AMCT_LAUNCH_SPEC(true, false) else AMCT_LAUNCH_SPEC(false, false)
     }
-#undef AMCT_LAUNCH_SPEC8
+#undef AMCT_LAUNCH_SPEC
+    if (p.splits > 1) {
+        int64_t nb = (M * N / 8 + kBlock - 1) / kBlock;
+        if (nb > 8192) nb = 8192;
+        if (dtype == AMCT_F16) hipLaunchKernelGGL((splitk_reduce16<true>), dim3((unsigned)nb), dim3(kBlock), 0, st, a.part, bias, (uint16_t*)out, M, N, p.splits);
+        else hipLaunchKernelGGL((splitk_reduce16<false>), dim3((unsigned)nb), dim3(kBlock), 0, st, a.part, bias, (uint16_t*)out, M, N, p.splits);
+    }
     return hip_status();
+}
+
+// The int8 weight-only Linear (gemm_wq16.hip) on the kernels with specialised waves: while the 128x128 blocks of the
+// launch fit the CUs in two rounds (up to 512 rows on W[14336, 4096]: 74 / 81 us at 384 / 512 rows against 98 us for the
+// dequantise-once form, which wins from there on: 640 rows 115 against 111 us); any number of rows when K is split.
+int w8a16_spec_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
+                        const uint8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group, int dtype,
+                        void* workspace, size_t workspace_bytes, hipStream_t st) {
+    return spec_launch<8>(x, smooth, wq, scales, scale_dtype, offsets, bias, out, M, N, K, group, dtype, workspace, workspace_bytes, st, 2, false);
+}
+// what that path wants lent beyond the smoothed activations: the partial sums of a split launch
+size_t w8a16_spec_part_bytes(int64_t M, int64_t N, int64_t K, int group) {
+    return spec_part_bytes(spec_plan(M, N, K, group, current_cu_count(), 2), M, N);
 }
 
 }  // namespace amct
@@ -1939,7 +2047,9 @@ extern "C" size_t amct_gemm_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t 
     if (M <= 0 || N <= 0 || K <= 0 || group <= 0) return 0;
     const size_t two = two_pass_workspace(M, N, K, group, has_smooth);    // many rows: the dequantised weight as well
     if (two) return two;
-    return has_smooth && M > 16 ? (size_t)M * (size_t)K * 2 : 0;          // tile kernels: x * smooth done once
+    // tile kernels: x * smooth done once; long rows on few column blocks: the partial sums of the K slices behind it
+    const size_t part = spec_part_bytes(spec_plan(M, N, K, group, current_cu_count(), 1), M, N);
+    return (has_smooth && (M > 16 || part) ? (size_t)M * (size_t)K * 2 : 0) + part;
 }
 
 extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t* wq, const void* scales,
@@ -1952,14 +2062,19 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
     if (dtype != AMCT_BF16 && dtype != AMCT_F16) return AMCT_E_UNSUPPORTED;
     if (K % group != 0 || K % 2 != 0) return AMCT_E_ALIGN;
     if (M == 0) return AMCT_OK;
-    // fp16 activations: a few rows take the weight-streaming kernel like bf16 ones; otherwise the kernels shared with
-    // the int8-weight path (gemm_wq16.hip), which smooth in the tile
+    if (M <= 16) {                                                 // K of 1024 / 2048 / 4096, group 128: the weight-streaming kernel
+        const int rc = w4a16_stream_dispatch(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, dtype,
+                                             (hipStream_t)stream);
+        if (rc != AMCT_E_UNSUPPORTED) return rc;
+    }
+    if (M < kTwoPassFrom) {                                        // long rows on few column blocks: specialised waves, K split over blocks
+        const int rc = spec_launch<4>(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, dtype, workspace,
+                                      workspace_bytes, (hipStream_t)stream, 1, true);
+        if (rc != AMCT_E_UNSUPPORTED) return rc;
+    }
+    // fp16 activations: otherwise the tile kernels below or the kernels shared with the int8-weight path (gemm_wq16.hip),
+    // which smooth in the tile
     if (dtype == AMCT_F16) {
-        if (M <= 16) {
-            const int rc = w4a16_stream_dispatch(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, dtype,
-                                                 (hipStream_t)stream);
-            if (rc != AMCT_E_UNSUPPORTED) return rc;
-        }
         if (M >= kTwoPassFrom) {
             const int rc = two_pass(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, dtype, workspace,
                                     workspace_bytes, (hipStream_t)stream);
@@ -2019,10 +2134,6 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
     W4A16Args a{(const uint16_t*)x, (const uint16_t*)smooth, wq, scales, zeros, bias, (uint16_t*)out, M, N, K, group, scale_dtype,
                 (uint32_t)(0x100000000ull / (uint64_t)group) + 1u};
     hipStream_t st = (hipStream_t)stream;
-    if (M <= 16) {                                                 // bf16, K % 1024 == 0, group 128: the weight-streaming kernel
-        const int rc = w4a16_stream_dispatch(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, dtype, st);
-        if (rc != AMCT_E_UNSUPPORTED) return rc;
-    }
     if (M >= kTwoPassFrom) {                                       // many rows and a workspace for the dequantised weight
         const int rc = two_pass(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, dtype, workspace,
                                 workspace_bytes, st);

@@ -511,14 +511,18 @@ int w8a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, 
 int w8a16_spec_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
                         const uint8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group, int dtype,
                         void* workspace, size_t workspace_bytes, hipStream_t st);   // gemm_w4a16.hip
+size_t w8a16_spec_part_bytes(int64_t M, int64_t N, int64_t K, int group);         // gemm_w4a16.hip
 }
 
 using namespace amct;
 
 extern "C" size_t amct_gemm_w8a16_workspace_bytes(int64_t M, int64_t N, int64_t K, int group, int has_smooth) {
+    if (M <= 0 || N <= 0 || K <= 0 || group <= 0) return 0;
+    // tile kernels: x * smooth done once; long rows on few column blocks: the partial sums of the K slices behind it
+    const size_t part = w8a16_spec_part_bytes(M, N, K, group);
+    const size_t spec = (has_smooth && (M > 16 || part) ? (size_t)M * (size_t)K * 2 : 0) + part;
     const size_t two = w8a16_tiles_workspace(M, N, K, group, has_smooth);   // many rows: the 16-bit weight as well
-    if (two) return two;
-    return has_smooth && M > 16 && N > 0 && K > 0 ? (size_t)M * (size_t)K * 2 : 0;   // tile kernels: x * smooth done once
+    return two > spec ? two : spec;
 }
 
 extern "C" int amct_gemm_w8a16(const void* x, const void* smooth, const int8_t* wq, const void* scales, int scale_dtype,
@@ -545,7 +549,7 @@ extern "C" int amct_gemm_w8a16_ws(const void* x, const void* smooth, const int8_
                                              reinterpret_cast<const uint8_t*>(offsets), bias, out, M, N, K, group, dtype, st);
         if (rc != AMCT_E_UNSUPPORTED) return rc;
     }
-    if (M > 16) {                                    // while the blocks fit the CUs in one round: the kernels with specialised waves
+    if (M > 16 || w8a16_spec_part_bytes(M, N, K, group)) {   // the tile kernels with specialised waves (a few rows: only with K split)
         const int rc = w8a16_spec_dispatch(x, smooth, reinterpret_cast<const uint8_t*>(wq), scales, scale_dtype,
                                            reinterpret_cast<const uint8_t*>(offsets), bias, out, M, N, K, group, dtype, workspace,
                                            workspace_bytes, st);
