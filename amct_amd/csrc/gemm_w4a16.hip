@@ -1936,7 +1936,7 @@ static int two_pass(const void* x, const void* smooth, const uint8_t* wq, const 
 // Block shape of the kernels with specialised waves (3: 64x64, 4: 128x64, 1: 128x128; 0: they do not apply) and the number
 // of K slices of the launch.  K is split over blocks when the tiles alone would leave CUs idle (few output columns, long
 // rows: the down projection of an MLP) or when a row has more groups than the kernel's factor table holds; a slice is
-// at least 2048 elements.  max_rounds: how many rounds of 128x128 blocks are still accepted.
+// at least 2048 elements.  max_rounds: how many rounds of 128x128 blocks are still accepted up to 512 rows.
 struct SpecPlan {
     int shape;
     int splits;
@@ -1948,7 +1948,7 @@ static SpecPlan spec_plan(int64_t M, int64_t N, int64_t K, int group, int64_t cu
     int64_t blocks;
     if (M <= 64 && nt64 <= cus) p.shape = 3, blocks = nt64;
     else if (mt * nt64 <= cus) p.shape = 4, blocks = mt * nt64;
-    else if (mt * nt128 <= max_rounds * cus) p.shape = 1, blocks = mt * nt128;
+    else if (mt * nt128 <= cus || (M <= 512 && mt * nt128 <= max_rounds * cus)) p.shape = 1, blocks = mt * nt128;
     else return p;
     const int64_t units = K / 256;
     auto fits = [&](int64_t S) {                                    // the groups of every slice fit the factor table
@@ -2067,7 +2067,10 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
                                              (hipStream_t)stream);
         if (rc != AMCT_E_UNSUPPORTED) return rc;
     }
-    if (M < kTwoPassFrom) {                                        // long rows on few column blocks: specialised waves, K split over blocks
+    // long rows on few column blocks: specialised waves, K split over blocks.  Measured on W[4096, 14336] / W[4096, 8192]
+    // (us, the older kernels for a few rows / this path): M = 2: 17.3 / 20.5 and 12.2 / 14.1; M = 4: 29.3 / 20.9 and
+    // 12.7 / 14.4; M = 8: 52.6 / 20.8 and 21.4 / 14.5; M = 32: 78.7 / 21.3 and 46.1 / 15.3.
+    if (M < kTwoPassFrom && (M >= 8 || (M >= 4 && K >= 12288))) {
         const int rc = spec_launch<4>(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, dtype, workspace,
                                       workspace_bytes, (hipStream_t)stream, 1, true);
         if (rc != AMCT_E_UNSUPPORTED) return rc;

@@ -41,6 +41,7 @@ struct W8A8Args {
     int64_t M, N, K;
     int bias_kind;
     int out_dtype;
+    int32_t* part;                                   // split-K launches (gridDim.z > 1): int32 partial sums [gridDim.z, M, N]
 };
 
 AMCT_DEV void w8a8_epilogue(const W8A8Args& a, int64_t m, int64_t n, int32_t acc) {
@@ -232,8 +233,14 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
-    const int nsteps = (int)(a.K / LK);
+    // Split K (gridDim.z > 1): block z takes the steps [steps z / S, steps (z + 1) / S) of every row and leaves its int32
+    // sums in a.part[z]; w8a8_splitk_reduce adds them (exactly) and applies the epilogue.  Rows keep their stride a.K.
+    const uint32_t steps_all = (uint32_t)(a.K / LK);
+    const uint32_t step0 = steps_all * blockIdx.z / gridDim.z;
+    const int nsteps = (int)(steps_all * (blockIdx.z + 1) / gridDim.z - step0);
     const int last = nsteps - 1;
+    const int8_t* const xk = a.xq + (int64_t)step0 * LK;
+    const int8_t* const wk = a.wq + (int64_t)step0 * LK;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t*)smem;
     // Rows are LK bytes, unpadded (a direct-to-LDS load writes the 64 lanes' 16-byte pieces to 1024 contiguous
     // bytes); 16-byte chunk c of row r lives at chunk position c ^ swz(r), which spreads the 16 rows that one
@@ -267,10 +274,10 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
     }
     auto dma_one = [&](int stg, int step, int j) {
         if (j < kNA) {
-            dma16s(lds0 + stg * kLStageBytes + (lw * kNA + j) * 1024, a.xq + (int64_t)step * LK, goff[j]);
+            dma16s(lds0 + stg * kLStageBytes + (lw * kNA + j) * 1024, xk + (int64_t)step * LK, goff[j]);
         } else {
             const int pb = lw * kNB + (j - kNA) < kLN / kRP ? lw * kNB + (j - kNA) : kLN / kRP - 1;
-            dma16s(lds0 + stg * kLStageBytes + kLM * LK + pb * 1024, a.wq + (int64_t)step * LK, goff[j]);
+            dma16s(lds0 + stg * kLStageBytes + kLM * LK + pb * 1024, wk + (int64_t)step * LK, goff[j]);
         }
     };
     auto dma_stage = [&](int stage, int step) {
@@ -315,7 +322,7 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
         const int64_t m = m0 + (tid - kLN) < a.M ? m0 + (tid - kLN) : a.M - 1;
         if (a.s_tok) fac0 = a.s_tok[m];
     }
-    if (a.bias_kind == 1) {
+    if (a.bias_kind == 1 && gridDim.z == 1) {
 #pragma unroll
         for (int j = 0; j < TJ; ++j) {
             const int64_t n = n0 + wn * 32 * TJ + j * 32 + (lane & 31);
@@ -431,7 +438,8 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
         sc[j] = ftab[wn * kPW + j * 32 + (lane & 31)];
         fb2[j] = ftab[256 + wn * kPW + j * 32 + (lane & 31)];
     }
-    if (a.acc_out) {                                                // accumulators on request (tests): plain stores
+    int32_t* const raw = gridDim.z > 1 ? a.part + (int64_t)blockIdx.z * a.M * a.N : a.acc_out;
+    if (raw) {                                                      // a slice's partial sums, or the accumulators on request (tests): plain stores
 #pragma unroll
         for (int i = 0; i < TI; ++i)
 #pragma unroll
@@ -440,8 +448,9 @@ AMCT_DEV void w8a8_dma_body(const W8A8Args& a, int8_t* smem, const int64_t m0, c
                 for (int j = 0; j < TJ; ++j) {
                     const int64_t m = m0 + wm * 32 * TI + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                     const int64_t n = n0 + wn * kPW + j * 32 + (lane & 31);
-                    if (m < a.M && n < a.N) a.acc_out[m * a.N + n] = acc[i][j][r];
+                    if (m < a.M && n < a.N) raw[m * a.N + n] = acc[i][j][r];
                 }
+        if (gridDim.z > 1) return;
     }
     const int h4 = 4 * (lane >> 5);
     int8_t* wbase = patch + h4 * kPatchRow + (lane & 31) * ES;      // this lane's element of patch row h4
@@ -1107,6 +1116,52 @@ __global__ __launch_bounds__(kBlock) void w8a8_general(W8A8Args a) {
     w8a8_epilogue(a, m, n, acc);
 }
 
+// out = dt(fp32(part[0] + ... + part[S - 1] + ibias) * s_ch * s_tok + fbias): the tile kernels' epilogue, operation for
+// operation, on the exact sum of the K slices; four columns per thread (N % 8 == 0)
+template <int ODT>
+__global__ __launch_bounds__(kBlock) void w8a8_splitk_reduce(W8A8Args a, int S) {
+    const int64_t nvec = a.M * a.N / 4, stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += stride) {
+        const int64_t e = v * 4, m = e / a.N, n = e - m * a.N;
+        int4 sum = *reinterpret_cast<const int4*>(a.part + e);
+        for (int z = 1; z < S; ++z) {
+            const int4 p = *reinterpret_cast<const int4*>(a.part + (int64_t)z * a.M * a.N + e);
+            sum.x += p.x, sum.y += p.y, sum.z += p.z, sum.w += p.w;
+        }
+        int32_t acc[4] = {sum.x, sum.y, sum.z, sum.w};
+        const float tk = a.s_tok ? a.s_tok[m] : 1.0f;
+        float f[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            if (a.bias_kind == 1) acc[c] += reinterpret_cast<const int32_t*>(a.bias)[n + c];
+            f[c] = (float)acc[c] * (a.s_ch ? a.s_ch[n + c] : 1.0f);
+            f[c] = f[c] * tk;
+            f[c] = f[c] + (a.bias_kind == 2 ? reinterpret_cast<const float*>(a.bias)[n + c] : -0.0f);
+        }
+        if (a.acc_out) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) a.acc_out[e + c] = acc[c];
+        }
+        if constexpr (ODT == AMCT_F32) {
+            *reinterpret_cast<float4*>(reinterpret_cast<float*>(a.out) + e) = make_float4(f[0], f[1], f[2], f[3]);
+        } else {
+            uint32_t h[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) h[c] = ODT == AMCT_BF16 ? f32_to_bf16_bits(f[c]) : f32_to_f16_bits(f[c]);
+            *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(a.out) + e) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+        }
+    }
+}
+
+// K slices of a launch of `blocks` tile blocks: as many as fill the CUs, at most 8, a slice of at least 2048 bytes of K
+static int w8a8_splits(int64_t blocks, int64_t K, int64_t cus) {
+    if (blocks <= 0 || cus <= 0) return 1;
+    int64_t S = cus / blocks;
+    if (S > 8) S = 8;
+    while (S > 1 && K / S < 2048) --S;
+    return S < 1 ? 1 : (int)S;
+}
+
 int w8a8_stream_dispatch(const int8_t* xq, const int8_t* wq, const float* s_tok, const float* s_ch, const void* bias,
                          int bias_kind, void* out, int32_t* acc_out, int64_t M, int64_t N, int64_t K, int out_dtype,
                          hipStream_t st);
@@ -1142,9 +1197,37 @@ int gemm16_tiles(const void* x, const void* w, const float* bias, void* out, int
 
 using namespace amct;
 
+// block shape of the small and medium tile launches (1: 64x64, 2: 128x64, 3: 128x128, 4: 128x256; 0: none of them) and
+// the number of blocks it takes
+static int w8a8_mid_shape(int64_t M, int64_t N, int64_t cus, int64_t* blocks) {
+    const int64_t mt = (M + 127) / 128, nt64 = (N + 63) / 64, nt128 = (N + 127) / 128, nt256 = (N + 255) / 256;
+    int shape = 0;
+    if (cus > 0 && M <= 64 && nt64 <= cus) shape = 1, *blocks = nt64;
+    else if (cus > 0 && mt * nt64 <= cus) shape = 2, *blocks = mt * nt64;
+    else if (cus > 0 && mt * nt128 <= cus) shape = 3, *blocks = mt * nt128;
+    else if (cus > 0 && (mt * nt256 <= cus || M < 256)) shape = 4, *blocks = mt * nt256;
+    return shape;
+}
+
+extern "C" size_t amct_gemm_w8a8_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 2 || N <= 0 || K <= 0 || K % 128 != 0 || N % 8 != 0) return 0;
+    if (M <= 16 && (K == 1024 || K == 2048 || K == 4096)) return 0;      // the weight-streaming kernel
+    int64_t blocks = 0;
+    const int64_t cus = current_cu_count();
+    if (!w8a8_mid_shape(M, N, cus, &blocks)) return 0;
+    const int S = w8a8_splits(blocks, K, cus);
+    return S > 1 ? (size_t)S * (size_t)M * (size_t)N * 4 : 0;
+}
+
 extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s_tok, const float* s_ch,
                               const void* bias, int bias_kind, void* out, int32_t* acc_out, int64_t M, int64_t N,
                               int64_t K, int out_dtype, amct_stream_t stream) {
+    return amct_gemm_w8a8_ws(xq, wq, s_tok, s_ch, bias, bias_kind, out, acc_out, M, N, K, out_dtype, nullptr, 0, stream);
+}
+
+extern "C" int amct_gemm_w8a8_ws(const int8_t* xq, const int8_t* wq, const float* s_tok, const float* s_ch,
+                                 const void* bias, int bias_kind, void* out, int32_t* acc_out, int64_t M, int64_t N,
+                                 int64_t K, int out_dtype, void* workspace, size_t workspace_bytes, amct_stream_t stream) {
     if (M < 0 || N <= 0 || K <= 0 || bias_kind < 0 || bias_kind > 2) return AMCT_E_BADARG;
     if (M != 0 && (!xq || !wq || !s_ch || !out || (bias_kind != 0 && !bias))) return AMCT_E_BADARG;   // M == 0 reads nothing
     if (out_dtype != AMCT_F32 && out_dtype != AMCT_F16 && out_dtype != AMCT_BF16) return AMCT_E_BADARG;
@@ -1184,18 +1267,26 @@ extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s
     if (tile_ok) {
         const int64_t cus = current_cu_count();
         const int64_t mt = (M + 127) / 128, nt64 = (N + 63) / 64, nt128 = (N + 127) / 128, nt256 = (N + 255) / 256;
-        int shape = 0;
-        if (cus > 0 && M <= 64 && nt64 <= cus) shape = 1;
-        else if (cus > 0 && mt * nt64 <= cus) shape = 2;
-        else if (cus > 0 && mt * nt128 <= cus) shape = 3;
-        else if (cus > 0 && (mt * nt256 <= cus || M < 256)) shape = 4;
+        int64_t blocks = 0;
+        const int shape = w8a8_mid_shape(M, N, cus, &blocks);
         if (shape && mt <= 65535) {
+            // Few blocks and long rows (the down projection of an MLP): K is split over S blocks per tile, which leave
+            // int32 partial sums in the lent workspace; a second kernel adds them - exactly - and applies the epilogue,
+            // so the result is that of the unsplit launch bit for bit.
+            unsigned S = (unsigned)w8a8_splits(blocks, K, cus);
+            if (S > 1 && !(workspace && aligned16(workspace) && workspace_bytes >= (size_t)S * (size_t)M * (size_t)N * 4)) S = 1;
+            if (S > 1) a.part = reinterpret_cast<int32_t*>(workspace);
 #define AMCT_LAUNCH_MID(ODT)                                                                                          \
     {                                                                                                                 \
-        if (shape == 1) hipLaunchKernelGGL((w8a8_tile_shape<ODT, 2, 2, 1, 1, 4, 128>), dim3((unsigned)nt64, 1), dim3(256), 0, st, a);             \
-        else if (shape == 2) hipLaunchKernelGGL((w8a8_tile_shape<ODT, 2, 2, 2, 1, 4, 128>), dim3((unsigned)nt64, (unsigned)mt), dim3(256), 0, st, a);  \
-        else if (shape == 3) hipLaunchKernelGGL((w8a8_tile_shape<ODT, 2, 2, 2, 2, 3, 128>), dim3((unsigned)nt128, (unsigned)mt), dim3(256), 0, st, a); \
-        else hipLaunchKernelGGL((w8a8_tile_shape<ODT, 2, 4, 2, 2, 3, 128>), dim3((unsigned)nt256, (unsigned)mt), dim3(512), 0, st, a);            \
+        if (shape == 1) hipLaunchKernelGGL((w8a8_tile_shape<ODT, 2, 2, 1, 1, 4, 128>), dim3((unsigned)nt64, 1, S), dim3(256), 0, st, a);             \
+        else if (shape == 2) hipLaunchKernelGGL((w8a8_tile_shape<ODT, 2, 2, 2, 1, 4, 128>), dim3((unsigned)nt64, (unsigned)mt, S), dim3(256), 0, st, a);  \
+        else if (shape == 3) hipLaunchKernelGGL((w8a8_tile_shape<ODT, 2, 2, 2, 2, 3, 128>), dim3((unsigned)nt128, (unsigned)mt, S), dim3(256), 0, st, a); \
+        else hipLaunchKernelGGL((w8a8_tile_shape<ODT, 2, 4, 2, 2, 3, 128>), dim3((unsigned)nt256, (unsigned)mt, S), dim3(512), 0, st, a);            \
+        if (S > 1) {                                                                                                  \
+            int64_t nb = (M * N / 4 + kBlock - 1) / kBlock;                                                           \
+            if (nb > 8192) nb = 8192;                                                                                 \
+            hipLaunchKernelGGL((w8a8_splitk_reduce<ODT>), dim3((unsigned)nb), dim3(kBlock), 0, st, a, (int)S);        \
+        }                                                                                                             \
     }
             if (out_dtype == AMCT_BF16) AMCT_LAUNCH_MID(AMCT_BF16)
             else if (out_dtype == AMCT_F16) AMCT_LAUNCH_MID(AMCT_F16)

@@ -459,9 +459,15 @@ def gemm_w8a8(xq, wq_nk, s_ch, s_tok=None, bias=None, out_dtype=torch.bfloat16, 
             bias = _c(bias.to(torch.float32))
     out = torch.empty(M, N, dtype=out_dtype, device=dev)
     acc = torch.empty(M, N, dtype=torch.int32, device=dev) if want_acc else None
+    # the workspace the library asks for (partial sums, when it splits long rows over several blocks per tile)
+    ws = None
+    nbytes = _lib.load().amct_gemm_w8a8_workspace_bytes(M, N, K)
+    if nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
-        _lib.check(_lib.load().amct_gemm_w8a8(_p(xq), _p(wq_nk), _p(s_tok), _p(s_ch), _p(bias), kind, _p(out), _p(acc),
-                                              M, N, K, dtype_code(out_dtype), _stream(dev)))
+        _lib.check(_lib.load().amct_gemm_w8a8_ws(_p(xq), _p(wq_nk), _p(s_tok), _p(s_ch), _p(bias), kind, _p(out), _p(acc),
+                                                 M, N, K, dtype_code(out_dtype), _p(ws), 0 if ws is None else ws.numel(),
+                                                 _stream(dev)))
     return (out, acc) if want_acc else out
 
 

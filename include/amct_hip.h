@@ -243,6 +243,17 @@ int amct_hif8_decode(const uint8_t* x, void* y, int64_t n, int dtype, amct_strea
 int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s_tok, const float* s_ch,
                    const void* bias, int bias_kind, void* out, int32_t* acc_out,
                    int64_t M, int64_t N, int64_t K, int out_dtype, amct_stream_t stream);
+/* The same with a workspace (may be null): amct_gemm_w8a8_workspace_bytes(M, N, K) bytes the caller lends, 16-byte
+ * aligned, contents irrelevant before and after the call.  The query asks for memory when the tiles of the launch would
+ * leave CUs idle and the rows are long (few output columns against the number of CUs, K >= 4096: the down projection of
+ * an MLP at 3 .. a few hundred rows): K is then split over several blocks per tile, which leave int32 partial sums in the
+ * workspace, and a second kernel adds them and applies the epilogue.  Integer sums are exact, so the result is that of
+ * amct_gemm_w8a8 bit for bit; 0 bytes otherwise; a null or smaller workspace is never an error. */
+size_t amct_gemm_w8a8_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int amct_gemm_w8a8_ws(const int8_t* xq, const int8_t* wq, const float* s_tok, const float* s_ch,
+                      const void* bias, int bias_kind, void* out, int32_t* acc_out,
+                      int64_t M, int64_t N, int64_t K, int out_dtype, void* workspace, size_t workspace_bytes,
+                      amct_stream_t stream);
 
 /* ---- K7: W4A16 Linear -------------------------------------------------------------------------------------
  * Replaces torch_npu.npu_weight_quant_batchmatmul as called at
@@ -256,8 +267,10 @@ int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s_tok, const
  * once up front instead of inside every column tile (same results; the fast bf16 tile kernels need it, without it such
  * calls take slower kernels that smooth in place).  From M = 1025 on the query also asks for N * K * 2 bytes: the weight
  * is then dequantised once into the workspace and the product runs as a plain 16-bit GEMM, which beats dequantising inside
- * every row tile from there on (same arithmetic; a smaller workspace keeps the fused kernels).  0 bytes are asked for
- * otherwise; a null or smaller workspace is never an error.
+ * every row tile from there on (same arithmetic; a smaller workspace keeps the fused kernels).  For long rows on few
+ * column blocks (the down projection of an MLP at up to a few hundred rows) the query also asks for S * M * N * 4 bytes:
+ * K is then split over S blocks per tile, whose fp32 partial sums a second kernel adds in a fixed order.  0 bytes are
+ * asked for otherwise; a null or smaller workspace is never an error.
  * Arithmetic of the dequantisation: the tile kernels (M > 16) feed dtype((u - zero) * scale) to the matrix pipe; the
  * weight-streaming kernel for M <= 16 (bf16 or fp16, K of 1024 / 2048 / 4096, group = 128) keeps the weight as the exact integer and applies
  * scale and zero per group in fp32, i.e. the dequantised weight is not rounded to bf16 there (the fp32 weight * scale of
@@ -290,7 +303,9 @@ int amct_gemm_w8a16(const void* x, const void* smooth, const int8_t* wq, const v
  * dequantised weight rounded to dtype, fp32 accumulation), about three times as fast.  For fewer rows (M > 16) with smooth
  * the query asks for M * K * 2 bytes: the multiply is then done once up front and the fast tile kernels apply (while
  * their blocks fit the CUs in two rounds, K a multiple of 256, groups a multiple of 64; they take precedence up to 512
- * rows on W[14336, 4096]).  0 bytes are asked for otherwise; a null or smaller workspace is never an error. */
+ * rows on W[14336, 4096]; for long rows on few column blocks with K split over blocks, whose fp32 partial sums follow the
+ * activations in the workspace: S * M * N * 4 bytes more).  0 bytes are asked for otherwise; a null or smaller workspace
+ * is never an error. */
 size_t amct_gemm_w8a16_workspace_bytes(int64_t M, int64_t N, int64_t K, int group, int has_smooth);
 int amct_gemm_w8a16_ws(const void* x, const void* smooth, const int8_t* wq, const void* scales, int scale_dtype,
                        const int8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group,

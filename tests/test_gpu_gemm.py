@@ -70,10 +70,13 @@ def test_w8a8_vs_oracle(dev, M, N, K, per_token, bias):
 @pytest.mark.parametrize("M,N,K", [(300, 1000, 320), (256, 448, 128), (512, 832, 256), (2048, 14336, 192), (1100, 9000, 64),
                                    (2000, 14328, 128), (100, 1000, 256), (200, 520, 384), (384, 14336, 128), (17, 72, 128),
                                    (640, 14336, 128), (33, 40000, 128), (5, 64, 128), (3, 14336, 384), (64, 200, 384),
-                                   (33, 14336, 256), (100, 14336, 128), (128, 8200, 256), (16, 40000, 128), (1, 16392, 128)])
+                                   (33, 14336, 256), (100, 14336, 128), (128, 8200, 256), (16, 40000, 128), (1, 16392, 128),
+                                   (16, 520, 14336), (40, 1000, 8192), (130, 2056, 8192), (300, 1000, 4224), (5, 64, 6144)])
 def test_w8a8_large_shapes_mixed_blocks(dev, M, N, K):
     """Block shapes of the tile kernels: 64x64 and 128x64 blocks for small M, 128x128 and 128x256 for medium M, 256x256 for large M, where a launch
-    may mix in 256x192 blocks so that the blocks fill the CUs evenly; ragged edges in M and N, accumulators bit for bit."""
+    may mix in 256x192 blocks so that the blocks fill the CUs evenly; ragged edges in M and N, accumulators bit for bit.
+    The last shapes (few column blocks, long rows) split K over several blocks per tile (ops.gemm_w8a8 lends the
+    workspace for the int32 partial sums): the same bits."""
     xq, wq, s_ch, s_tok, b = w8a8_case(M, N, K, 131, True, 'float')
     want_acc = od.int8_matmul_exact(xq, wq.t())
     for odt in (torch.bfloat16, torch.float32):
@@ -132,10 +135,12 @@ def w4a16_oracle(x, codes, scales, zeros, group, smooth, bias, rows=None):
                                          (130, 40000, 128, 64), (640, 14336, 256, 128), (100, 1000, 512, 128), (256, 136, 1024, 64),
                                          (65, 14336, 256, 256), (25, 200, 128, 64), (40, 14336, 256, 128), (48, 40000, 128, 64),
                                          (100, 14336, 128, 128), (128, 8200, 256, 64), (64, 14336, 128, 128), (300, 14336, 128, 128),
-                                         (512, 14328, 256, 64), (257, 1000, 384, 128), (33, 200, 512, 64), (100, 520, 768, 128), (64, 14336, 256, 128)])
+                                         (512, 14328, 256, 64), (257, 1000, 384, 128), (33, 200, 512, 64), (100, 520, 768, 128), (64, 14336, 256, 128),
+                                         (40, 520, 8192, 128), (8, 1000, 14336, 128), (100, 4096, 4096, 128), (200, 264, 11008, 64)])
 def test_w4a16_large_shapes_ragged(dev, M, N, K, group):
     """The wide tile kernels (M > 24, group % 64 == 0) in their block shapes (64x64, 128x64, 128x128 with and without specialised
-    waves, 128x256, 256x256; two or three LDS stages) on ragged edges in M and N, both scale dtypes."""
+    waves, 128x256, 256x256; two or three LDS stages) on ragged edges in M and N, both scale dtypes; the last shapes (few
+    column blocks, long rows) with K split over several blocks per tile and the partial sums added by a second kernel."""
     for sdt in (torch.float16, torch.bfloat16):
         x, codes, scales, zeros, smooth, bias = w4a16_case(M, N, K, group, 137, sdt)
         packed = workloads.pack_nibbles(codes)
@@ -285,12 +290,14 @@ def test_w8a16_many_rows_through_the_workspace(dev, dtype, M, N, K, group):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,N,K,group", [(17, 14336, 4096, 128), (40, 520, 1024, 128), (64, 14336, 4096, 4096), (65, 200, 512, 64),
                                          (128, 8200, 256, 64), (200, 1000, 768, 256), (256, 14336, 4096, 128), (100, 264, 320, 64),
-                                         (33, 20000, 256, 128), (512, 14336, 1024, 128)])
+                                         (33, 20000, 256, 128), (512, 14336, 1024, 128), (8, 520, 8192, 128), (100, 2048, 8192, 256),
+                                         (1, 1000, 14336, 128)])
 def test_w8a16_medium_rows_specialised_waves(dev, dtype, M, N, K, group):
     """Int8 weight-only Linear from 17 rows on, while the blocks fit the CUs in two rounds: the tile kernels with
     specialised waves (K a multiple of 256; 64x64, 128x64 and 128x128 blocks), ragged M and N, per-channel and grouped
     factors, symmetric and with offsets, with smoothing (through the workspace ops.gemm_w8a16 lends) and bias; one shape
-    the shared kernel keeps (K = 320).  dt((q - offset) * scale) and fp32 accumulation: within 1e-3 of the row's largest
+    the shared kernel keeps (K = 320); the last shapes (few column blocks, long rows, any number of rows) with K split
+    over several blocks per tile.  dt((q - offset) * scale) and fp32 accumulation: within 1e-3 of the row's largest
     output (plus half an ulp) of the fp64 anchor; small integers give an integer matmul bit for bit."""
     from amct_amd import _lib
     assert _lib.load().amct_gemm_w8a16_workspace_bytes(M, N, K, group, 1) >= M * K * 2
@@ -407,7 +414,8 @@ def test_gemms_at_the_benchmark_size(dev, M):
 
 @pytest.mark.parametrize("M,N,K", [(2048, 14336, 4096), (520, 14336, 4096), (300, 14336, 4096), (130, 14336, 4096),
                                    (70, 14336, 4096), (200, 20000, 1024), (65, 72, 128), (17, 14336, 4096), (40, 14336, 4096),
-                                   (64, 520, 1024), (33, 200, 512), (100, 1000, 768), (128, 20000, 256), (24, 72, 128)])
+                                   (64, 520, 1024), (33, 200, 512), (100, 1000, 768), (128, 20000, 256), (24, 72, 128),
+                                   (32, 1000, 8192), (9, 520, 14336)])
 def test_w4a16_fp16_at_the_benchmark_size(dev, M, N, K):
     """fp16 activations, more than 16 rows: the tile kernels with fp16 operands, every block shape the dispatch knows
     (256x256, 256x128, 128x256, 128x128, 128x64, 64x64; with specialised waves when K is a multiple of 256, the only
