@@ -1891,7 +1891,8 @@ int w4a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, 
                           int dtype, hipStream_t st);              // gemm_w4a16_stream.hip
 
 int gemm16_tiles(const void* x, const void* w, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int dtype,
-                 hipStream_t st);                                  // gemm_w8a8.hip
+                 void* workspace, size_t workspace_bytes, hipStream_t st);   // gemm_w8a8.hip
+size_t gemm16_part_bytes(int64_t M, int64_t N, int64_t K);         // gemm_w8a8.hip: partial sums it wants lent for few tiles
 
 // From this many rows on, dequantising the weight once into a lent workspace and running the plain 16-bit GEMM beats
 // dequantising inside every row tile.  Measured on W[14336,4096] with smoothing, fused kernel / two passes: M = 1024
@@ -1904,15 +1905,16 @@ static size_t two_pass_workspace(int64_t M, int64_t N, int64_t K, int group, int
     if (M < kTwoPassFrom || K % 64 != 0 || N % 8 != 0 || group % 32 != 0 || K % group != 0 || N * K * 2 >= (int64_t(1) << 32) ||
         M * K * 2 >= (int64_t(1) << 32))
         return 0;
-    return (size_t)N * (size_t)K * 2 + (has_smooth ? (size_t)M * (size_t)K * 2 : 0);
+    return (size_t)N * (size_t)K * 2 + (has_smooth ? (size_t)M * (size_t)K * 2 : 0) + gemm16_part_bytes(M, N, K);
 }
 
 // dequantise, smooth, multiply; AMCT_E_UNSUPPORTED when the shape or the workspace does not allow it
 static int two_pass(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype, const uint8_t* zeros,
                     const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group, int dtype, void* workspace,
                     size_t workspace_bytes, hipStream_t st) {
-    const size_t need = two_pass_workspace(M, N, K, group, smooth != nullptr);
-    if (!need || !workspace || workspace_bytes < need || !aligned16(workspace) || !aligned16(x) || !aligned16(wq) || !aligned16(out) ||
+    const size_t part = gemm16_part_bytes(M, N, K);
+    const size_t need = two_pass_workspace(M, N, K, group, smooth != nullptr) - part;   // the partial sums are optional
+    if (!two_pass_workspace(M, N, K, group, smooth != nullptr) || !workspace || workspace_bytes < need || !aligned16(workspace) || !aligned16(x) || !aligned16(wq) || !aligned16(out) ||
         (smooth && !aligned16(smooth)))
         return AMCT_E_UNSUPPORTED;
     W4A16Args a{(const uint16_t*)x, (const uint16_t*)smooth, wq, scales, zeros, bias, (uint16_t*)out, M, N, K, group, scale_dtype,
@@ -1930,7 +1932,8 @@ static int two_pass(const void* x, const void* smooth, const uint8_t* wq, const 
     if (dtype == AMCT_F16) hipLaunchKernelGGL((w4_dequant_rows<true>), grid, dim3(kBlock), 0, st, a, wdq, xs, (unsigned)wblocks);
     else hipLaunchKernelGGL((w4_dequant_rows<false>), grid, dim3(kBlock), 0, st, a, wdq, xs, (unsigned)wblocks);
     const void* xa = smooth ? (const void*)xs : x;
-    return gemm16_tiles(xa, wdq, bias, out, M, N, K, dtype, st);
+    char* const rest = reinterpret_cast<char*>(workspace) + need;
+    return gemm16_tiles(xa, wdq, bias, out, M, N, K, dtype, rest, workspace_bytes - need, st);
 }
 
 // Block shape of the kernels with specialised waves (3: 64x64, 4: 128x64, 1: 128x128; 0: they do not apply) and the number

@@ -519,8 +519,14 @@ AMCT_DEV void w8a8_dma_body16(const W8A8Args& a, int8_t* smem, const int64_t m0,
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
-    const int nsteps = (int)(a.K / LK);
+    // Split K (gridDim.z > 1): block z takes the steps [steps z / S, steps (z + 1) / S) of every row and leaves its sums
+    // (int32, or fp32 in the 16-bit modes) in a.part[z]; a second kernel adds them and applies the epilogue.
+    const uint32_t steps_all = (uint32_t)(a.K / LK);
+    const uint32_t step0 = steps_all * blockIdx.z / gridDim.z;
+    const int nsteps = (int)(steps_all * (blockIdx.z + 1) / gridDim.z - step0);
     const int last = nsteps - 1;
+    const int8_t* const xk = a.xq + (int64_t)step0 * LK;
+    const int8_t* const wk = a.wq + (int64_t)step0 * LK;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t*)smem;
     // Rows are LK bytes, unpadded (a direct-to-LDS load writes the 64 lanes' 16-byte pieces to 1024 contiguous
     // bytes); 16-byte chunk c of row r lives at chunk position c ^ swz(r), which spreads the 16 rows that one
@@ -554,10 +560,10 @@ AMCT_DEV void w8a8_dma_body16(const W8A8Args& a, int8_t* smem, const int64_t m0,
     }
     auto dma_one = [&](int stg, int step, int j) {
         if (j < kNA) {
-            dma16s(lds0 + stg * kLStageBytes + (lw * kNA + j) * 1024, a.xq + (int64_t)step * LK, goff[j]);
+            dma16s(lds0 + stg * kLStageBytes + (lw * kNA + j) * 1024, xk + (int64_t)step * LK, goff[j]);
         } else {
             const int pb = lw * kNB + (j - kNA) < kLN / kRP ? lw * kNB + (j - kNA) : kLN / kRP - 1;
-            dma16s(lds0 + stg * kLStageBytes + kLM * LK + pb * 1024, a.wq + (int64_t)step * LK, goff[j]);
+            dma16s(lds0 + stg * kLStageBytes + kLM * LK + pb * 1024, wk + (int64_t)step * LK, goff[j]);
         }
     };
     auto dma_stage = [&](int stage, int step) {
@@ -614,7 +620,7 @@ AMCT_DEV void w8a8_dma_body16(const W8A8Args& a, int8_t* smem, const int64_t m0,
     // and moves them with one LDS write.  An integer bias is where the accumulators start (its loads wait together with
     // the first stage's), so the epilogue never sees it.
     if constexpr (MODE == 0) {
-        if (a.bias_kind == 1) {
+        if (a.bias_kind == 1 && gridDim.z == 1) {
 #pragma unroll
             for (int j = 0; j < TB; ++j)
 #pragma unroll
@@ -709,6 +715,19 @@ AMCT_DEV void w8a8_dma_body16(const W8A8Args& a, int8_t* smem, const int64_t m0,
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 
+    if (gridDim.z > 1) {
+        // the raw sums of this slice: a lane's four adjacent columns of row 16 t + lane % 16 as one 16-byte store
+        int32_t* const part = a.part + (int64_t)blockIdx.z * a.M * a.N;
+#pragma unroll
+        for (int t = 0; t < 2 * TI; ++t)
+#pragma unroll
+            for (int j = 0; j < TB; ++j) {
+                const int64_t m = m0 + wm * 32 * TI + t * 16 + (lane & 15);
+                const int64_t n = n0 + wn * 32 * TJ + j * 16 + 4 * (lane >> 4);
+                if (m < a.M && n < a.N) *reinterpret_cast<acc_t*>(part + m * a.N + n) = acc[t][j];
+            }
+        return;
+    }
     // epilogue: fp32(acc, integer bias included) * s_ch * s_tok + fbias, narrowed, through a per-wave LDS patch of 32 rows x
     // 32*TJ columns, stored as 16-byte pieces of full rows.  Branch-free per element: absent factors are replaced by
     // their neutral elements (x * 1.0f and x + (-0.0f) return x bit for bit).  A lane holds the factors of its 4 TB
@@ -1153,6 +1172,28 @@ __global__ __launch_bounds__(kBlock) void w8a8_splitk_reduce(W8A8Args a, int S) 
     }
 }
 
+// the same for the 16-bit GEMM: out = dt(part[0] + ... + part[S - 1] + bias), fp32 partial sums added in that order
+template <int ODT>
+__global__ __launch_bounds__(kBlock) void gemm16_splitk_reduce(W8A8Args a, int S) {
+    const int64_t nvec = a.M * a.N / 4, stride = (int64_t)gridDim.x * kBlock;
+    const float* part = reinterpret_cast<const float*>(a.part);
+    for (int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += stride) {
+        const int64_t e = v * 4, n = e % a.N;
+        float4 sum = *reinterpret_cast<const float4*>(part + e);
+        for (int z = 1; z < S; ++z) {
+            const float4 p = *reinterpret_cast<const float4*>(part + (int64_t)z * a.M * a.N + e);
+            sum.x += p.x, sum.y += p.y, sum.z += p.z, sum.w += p.w;
+        }
+        float f[4] = {sum.x, sum.y, sum.z, sum.w};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) f[c] = f[c] + (a.bias_kind == 2 ? reinterpret_cast<const float*>(a.bias)[n + c] : -0.0f);
+        uint32_t h[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) h[c] = ODT == AMCT_BF16 ? f32_to_bf16_bits(f[c]) : f32_to_f16_bits(f[c]);
+        *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(a.out) + e) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+    }
+}
+
 // K slices of a launch of `blocks` tile blocks: as many as fill the CUs, at most 8, a slice of at least 2048 bytes of K
 static int w8a8_splits(int64_t blocks, int64_t K, int64_t cus) {
     if (blocks <= 0 || cus <= 0) return 1;
@@ -1170,8 +1211,17 @@ int w8a8_stream_dispatch(const int8_t* xq, const int8_t* wq, const float* s_tok,
 // fp16), K contiguous: the 256x256 / 256x192 tiles of the W8A8 kernel on the 16-bit MFMAs.  Returns AMCT_E_UNSUPPORTED
 // for shapes the tiles do not take (fewer than 256 rows, K not a multiple of 64, N not a multiple of 8, unaligned or
 // 4 GiB operands).  Used by the int8 weight-only Linear, which dequantises its weight into a workspace first.
+// K slices of the uniform 256x256 launch of the 16-bit GEMM (1: not split), and the bytes of their fp32 partial sums
+static int gemm16_splits(int64_t M, int64_t N, int64_t Kb, int cus) {
+    return w8a8_splits(((M + 255) / 256) * ((N + 255) / 256), Kb, cus);
+}
+size_t gemm16_part_bytes(int64_t M, int64_t N, int64_t K) {
+    const int S = M >= 256 ? gemm16_splits(M, N, K * 2, current_cu_count()) : 1;
+    return S > 1 ? (size_t)S * (size_t)M * (size_t)N * 4 : 0;
+}
+
 int gemm16_tiles(const void* x, const void* w, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int dtype,
-                 hipStream_t st) {
+                 void* workspace, size_t workspace_bytes, hipStream_t st) {
     const int64_t Kb = K * 2;                                       // bytes of a row
     if (dtype != AMCT_BF16 && dtype != AMCT_F16) return AMCT_E_UNSUPPORTED;
     if (M < 256 || Kb % 128 != 0 || N % 8 != 0 || !aligned16(x) || !aligned16(w) || !aligned16(out) ||
@@ -1181,14 +1231,27 @@ int gemm16_tiles(const void* x, const void* w, const float* bias, void* out, int
     if (grid.y > 65535) return AMCT_E_UNSUPPORTED;
     W8A8Args a{reinterpret_cast<const int8_t*>(x), reinterpret_cast<const int8_t*>(w), nullptr, nullptr, bias, out, nullptr,
                M, N, Kb, bias ? 2 : 0, dtype};
-    const MixPlan plan = plan_mix(M, N, current_cu_count());
-    if (plan.nbig >= 0) {
+    const int cus = current_cu_count();
+    // few tiles (half the CUs or fewer: few output columns): K split over S blocks per uniform tile, fp32 partial sums in
+    // the lent workspace; otherwise the plan that mixes in narrower tiles where that fills the CUs better
+    unsigned S = (unsigned)gemm16_splits(M, N, Kb, cus);
+    if (S > 1 && !(workspace && aligned16(workspace) && workspace_bytes >= (size_t)S * (size_t)M * (size_t)N * 4)) S = 1;
+    const MixPlan plan = plan_mix(M, N, cus);
+    if (S == 1 && plan.nbig >= 0) {
         const dim3 g1((unsigned)(plan.big + plan.mtiles * plan.nsmall));
         if (dtype == AMCT_BF16) hipLaunchKernelGGL((w8a8_tile_mix16<AMCT_BF16, 1>), g1, dim3(512), 0, st, a, plan);
         else hipLaunchKernelGGL((w8a8_tile_mix16<AMCT_F16, 2>), g1, dim3(512), 0, st, a, plan);
     } else {
-        if (dtype == AMCT_BF16) hipLaunchKernelGGL((w8a8_tile_dma16<AMCT_BF16, 1>), grid, dim3(512), 0, st, a);
-        else hipLaunchKernelGGL((w8a8_tile_dma16<AMCT_F16, 2>), grid, dim3(512), 0, st, a);
+        if (S > 1) a.part = reinterpret_cast<int32_t*>(workspace);
+        const dim3 g(grid.x, grid.y, S);
+        if (dtype == AMCT_BF16) hipLaunchKernelGGL((w8a8_tile_dma16<AMCT_BF16, 1>), g, dim3(512), 0, st, a);
+        else hipLaunchKernelGGL((w8a8_tile_dma16<AMCT_F16, 2>), g, dim3(512), 0, st, a);
+        if (S > 1) {
+            int64_t nb = (M * N / 4 + kBlock - 1) / kBlock;
+            if (nb > 8192) nb = 8192;
+            if (dtype == AMCT_BF16) hipLaunchKernelGGL((gemm16_splitk_reduce<AMCT_BF16>), dim3((unsigned)nb), dim3(kBlock), 0, st, a, (int)S);
+            else hipLaunchKernelGGL((gemm16_splitk_reduce<AMCT_F16>), dim3((unsigned)nb), dim3(kBlock), 0, st, a, (int)S);
+        }
     }
     return hip_status();
 }
@@ -1214,7 +1277,10 @@ extern "C" size_t amct_gemm_w8a8_workspace_bytes(int64_t M, int64_t N, int64_t K
     if (M <= 16 && (K == 1024 || K == 2048 || K == 4096)) return 0;      // the weight-streaming kernel
     int64_t blocks = 0;
     const int64_t cus = current_cu_count();
-    if (!w8a8_mid_shape(M, N, cus, &blocks)) return 0;
+    if (!w8a8_mid_shape(M, N, cus, &blocks)) {                      // the large tiles, when their launch is uniform
+        if (M < 256 || plan_mix(M, N, (int)cus).nbig >= 0) return 0;
+        blocks = ((M + 255) / 256) * ((N + 255) / 256);
+    }
     const int S = w8a8_splits(blocks, K, cus);
     return S > 1 ? (size_t)S * (size_t)M * (size_t)N * 4 : 0;
 }
@@ -1318,6 +1384,13 @@ extern "C" int amct_gemm_w8a8_ws(const int8_t* xq, const int8_t* wq, const float
         // operands (register-only loops: 3.74 against 3.24 POP/s; with the large tile's fragment reads interleaved 3.8
         // against 3.4), at equal LDS traffic per wave tile: 98 against 105 us on M = 2048, N = 14336, K = 4096.
         constexpr bool mi16 = true;
+        // few tiles (few output columns): K split over S blocks per tile, int32 partial sums in the lent workspace
+        unsigned S = 1;
+        if (wide && mi16 && plan.nbig < 0) {
+            S = (unsigned)w8a8_splits((int64_t)grid.x * grid.y, K, cus);
+            if (S > 1 && !(workspace && aligned16(workspace) && workspace_bytes >= (size_t)S * (size_t)M * (size_t)N * 4)) S = 1;
+            if (S > 1) a.part = reinterpret_cast<int32_t*>(workspace);
+        }
 #define AMCT_LAUNCH_DMA(ODT)                                                                                        \
     {                                                                                                               \
         if (plan.nbig >= 0) {                                                                                       \
@@ -1326,9 +1399,14 @@ extern "C" int amct_gemm_w8a8_ws(const int8_t* xq, const int8_t* wq, const float
             else if (wide) hipLaunchKernelGGL((w8a8_tile_mix<ODT, 2, 128>), g1, dim3(512), 0, st, a, plan);         \
             else hipLaunchKernelGGL((w8a8_tile_mix<ODT, 4, 64>), g1, dim3(512), 0, st, a, plan);                    \
         } else {                                                                                                    \
-            if (wide && mi16) hipLaunchKernelGGL((w8a8_tile_dma16<ODT>), grid, dim3(512), 0, st, a);                \
+            if (wide && mi16) hipLaunchKernelGGL((w8a8_tile_dma16<ODT>), dim3(grid.x, grid.y, S), dim3(512), 0, st, a); \
             else if (wide) hipLaunchKernelGGL((w8a8_tile_dma<ODT, 2, 4, 2, 128>), grid, dim3(512), 0, st, a);       \
             else hipLaunchKernelGGL((w8a8_tile_dma<ODT, 2, 4, 4, 64>), grid, dim3(512), 0, st, a);                  \
+            if (S > 1) {                                                                                            \
+                int64_t nb = (M * N / 4 + kBlock - 1) / kBlock;                                                     \
+                if (nb > 8192) nb = 8192;                                                                           \
+                hipLaunchKernelGGL((w8a8_splitk_reduce<ODT>), dim3((unsigned)nb), dim3(kBlock), 0, st, a, (int)S);  \
+            }                                                                                                       \
         }                                                                                                           \
     }
         if (out_dtype == AMCT_BF16) AMCT_LAUNCH_DMA(AMCT_BF16)

@@ -496,13 +496,14 @@ __global__ __launch_bounds__(kBlock) void w8_dequant_rows(WqArgs a, uint16_t* wd
 }
 
 int gemm16_tiles(const void* x, const void* w, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int dtype,
-                 hipStream_t st);                           // gemm_w8a8.hip
+                 void* workspace, size_t workspace_bytes, hipStream_t st);   // gemm_w8a8.hip
+size_t gemm16_part_bytes(int64_t M, int64_t N, int64_t K);  // gemm_w8a8.hip: partial sums it wants lent for few tiles
 
 static size_t w8a16_tiles_workspace(int64_t M, int64_t N, int64_t K, int group, int has_smooth) {
     if (M < 256 || N <= 0 || K <= 0 || group <= 0 || K % 64 != 0 || K % 16 != 0 || group % 16 != 0 || K % group != 0 || N % 8 != 0 ||
         N * K * 2 >= (int64_t(1) << 32) || M * K * 2 >= (int64_t(1) << 32))
         return 0;
-    return (size_t)N * (size_t)K * 2 + (has_smooth ? (size_t)M * (size_t)K * 2 : 0);
+    return (size_t)N * (size_t)K * 2 + (has_smooth ? (size_t)M * (size_t)K * 2 : 0) + gemm16_part_bytes(M, N, K);
 }
 
 int w8a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
@@ -556,7 +557,8 @@ extern "C" int amct_gemm_w8a16_ws(const void* x, const void* smooth, const int8_
         if (rc != AMCT_E_UNSUPPORTED) return rc;
     }
     // many rows and a lent workspace: dequantise once, then the plain 16-bit GEMM on the large tiles
-    const size_t need = w8a16_tiles_workspace(M, N, K, group, smooth != nullptr);
+    const size_t full = w8a16_tiles_workspace(M, N, K, group, smooth != nullptr);
+    const size_t need = full ? full - gemm16_part_bytes(M, N, K) : 0;      // the partial sums are optional
     if (need && workspace && workspace_bytes >= need && aligned16(workspace) && aligned16(x) && aligned16(wq) && aligned16(out) &&
         (!smooth || aligned16(smooth)) && (reinterpret_cast<uintptr_t>(scales) & 1u) == 0) {
         uint16_t* wdq = reinterpret_cast<uint16_t*>(workspace);
@@ -571,7 +573,7 @@ extern "C" int amct_gemm_w8a16_ws(const void* x, const void* smooth, const int8_
         if (dtype == AMCT_BF16) hipLaunchKernelGGL((w8_dequant_rows<AMCT_BF16>), grid, dim3(kBlock), 0, st, a, wdq, xs, (unsigned)wblocks);
         else hipLaunchKernelGGL((w8_dequant_rows<AMCT_F16>), grid, dim3(kBlock), 0, st, a, wdq, xs, (unsigned)wblocks);
         const void* xa = smooth ? (const void*)xs : x;
-        const int rc = gemm16_tiles(xa, wdq, bias, out, M, N, K, dtype, st);
+        const int rc = gemm16_tiles(xa, wdq, bias, out, M, N, K, dtype, reinterpret_cast<char*>(workspace) + need, workspace_bytes - need, st);
         if (rc != AMCT_E_UNSUPPORTED) return rc;
         // (the two preparatory kernels above only wrote the workspace: the call below starts from the caller's operands)
     }

@@ -71,7 +71,8 @@ def test_w8a8_vs_oracle(dev, M, N, K, per_token, bias):
                                    (2000, 14328, 128), (100, 1000, 256), (200, 520, 384), (384, 14336, 128), (17, 72, 128),
                                    (640, 14336, 128), (33, 40000, 128), (5, 64, 128), (3, 14336, 384), (64, 200, 384),
                                    (33, 14336, 256), (100, 14336, 128), (128, 8200, 256), (16, 40000, 128), (1, 16392, 128),
-                                   (16, 520, 14336), (40, 1000, 8192), (130, 2056, 8192), (300, 1000, 4224), (5, 64, 6144)])
+                                   (16, 520, 14336), (40, 1000, 8192), (130, 2056, 8192), (300, 1000, 4224), (5, 64, 6144),
+                                   (1000, 1032, 4096), (520, 4096, 2304)])
 def test_w8a8_large_shapes_mixed_blocks(dev, M, N, K):
     """Block shapes of the tile kernels: 64x64 and 128x64 blocks for small M, 128x128 and 128x256 for medium M, 256x256 for large M, where a launch
     may mix in 256x192 blocks so that the blocks fill the CUs evenly; ragged edges in M and N, accumulators bit for bit.
@@ -255,7 +256,7 @@ def test_w8a16_weight_streaming_kernel(dev, dtype, M, N, K, group):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,N,K,group", [(2048, 14336, 4096, 128), (256, 264, 64, 64), (300, 1000, 320, 32), (513, 2056, 1024, 1024),
-                                         (1000, 4104, 192, 64), (300, 16, 65536, 256)])
+                                         (1000, 4104, 192, 64), (300, 16, 65536, 256), (700, 1032, 4096, 128)])
 def test_w8a16_many_rows_through_the_workspace(dev, dtype, M, N, K, group):
     """Int8 weight-only Linear from 256 rows on: with the workspace the library asks for, the weight is dequantised once
     and the product is the plain 16-bit GEMM on the large tiles (uniform and mixed tile launches, ragged M and N, K of
@@ -266,7 +267,7 @@ def test_w8a16_many_rows_through_the_workspace(dev, dtype, M, N, K, group):
     lib = _lib.load()
     ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
     rows = [r for r in FULL_ROWS if r < M]
-    assert lib.amct_gemm_w8a16_workspace_bytes(M, N, K, group, 1) == N * K * 2 + M * K * 2
+    assert lib.amct_gemm_w8a16_workspace_bytes(M, N, K, group, 1) >= N * K * 2 + M * K * 2
     for sdt, sym in ((torch.float16, False), (torch.bfloat16, True)):
         x, codes, scales, offsets, smooth, bias = w8a16_case(M, N, K, group, 170 + M % 97, dtype, sdt, sym)
         for sm, b in ((None, None), (smooth, bias)):
@@ -440,7 +441,8 @@ def test_w4a16_fp16_at_the_benchmark_size(dev, M, N, K):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,N,K,group", [(1025, 1000, 320, 32), (3584, 1000, 320, 32), (4100, 264, 64, 64), (1100, 16, 65536, 128)])
+@pytest.mark.parametrize("M,N,K,group", [(1025, 1000, 320, 32), (3584, 1000, 320, 32), (4100, 264, 64, 64), (1100, 16, 65536, 128),
+                                         (1300, 1000, 4096, 128)])
 def test_w4a16_very_many_rows_dequantise_once(dev, dtype, M, N, K, group):
     """From 1025 rows on, with the workspace the library asks for (the 16-bit weight and the smoothed activations), the
     int4 weight is dequantised once and the product is the plain 16-bit GEMM on the large tiles; with the smaller
@@ -448,8 +450,9 @@ def test_w4a16_very_many_rows_dequantise_once(dev, dtype, M, N, K, group):
     sampled rows of both within the tolerance of the fp64 anchor; small integers bit for bit."""
     from amct_amd import _lib
     lib = _lib.load()
-    assert lib.amct_gemm_w4a16_workspace_bytes(M, N, K, group, 1) == N * K * 2 + M * K * 2
-    assert lib.amct_gemm_w4a16_workspace_bytes(M, N, K, group, 0) == N * K * 2
+    # the 16-bit weight and the smoothed activations, plus the partial sums of a K-split GEMM when its tiles are few
+    assert lib.amct_gemm_w4a16_workspace_bytes(M, N, K, group, 1) >= N * K * 2 + M * K * 2
+    assert lib.amct_gemm_w4a16_workspace_bytes(M, N, K, group, 0) >= N * K * 2
     ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
     rows = sorted({r for r in FULL_ROWS + [M - 1, M - 2, 1023] if r < M})
     x, codes, scales, zeros, smooth, bias = w4a16_case(M, N, K, group, 333, torch.float16)
@@ -458,7 +461,7 @@ def test_w4a16_very_many_rows_dequantise_once(dev, dtype, M, N, K, group):
     want = w4a16_oracle(x[rows], codes, scales, zeros, group, smooth, bias, rows=M)
     tol = 1e-3 * want.abs().amax(dim=1, keepdim=True) + want.abs() * ulp
     st = torch.cuda.current_stream(dev).cuda_stream
-    for nbytes in (N * K * 2 + M * K * 2, M * K * 2):
+    for nbytes in (lib.amct_gemm_w4a16_workspace_bytes(M, N, K, group, 1), N * K * 2 + M * K * 2, M * K * 2):
         ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
         out = torch.empty(M, N, dtype=dtype, device=dev)
         _lib.check(lib.amct_gemm_w4a16(xd.data_ptr(), smd.data_ptr(), packed.data_ptr(), sd.data_ptr(), _lib.F16, zd.data_ptr(),
