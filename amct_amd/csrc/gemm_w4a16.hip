@@ -1951,7 +1951,8 @@ static SpecPlan spec_plan(int64_t M, int64_t N, int64_t K, int group, int64_t cu
     int64_t blocks;
     if (M <= 64 && nt64 <= cus) p.shape = 3, blocks = nt64;
     else if (mt * nt64 <= cus) p.shape = 4, blocks = mt * nt64;
-    else if (mt * nt128 <= cus || (M <= 512 && mt * nt128 <= max_rounds * cus)) p.shape = 1, blocks = mt * nt128;
+    else if (mt * nt128 <= cus || (M <= 512 && mt * nt128 <= max_rounds * cus) || (max_rounds > 1 && M <= 128))
+        p.shape = 1, blocks = mt * nt128;                          // (up to 128 rows any number of rounds: the weight streams once)
     else return p;
     const int64_t units = K / 256;
     auto fits = [&](int64_t S) {                                    // the groups of every slice fit the factor table
@@ -2073,9 +2074,13 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
     // long rows on few column blocks: specialised waves, K split over blocks.  Measured on W[4096, 14336] / W[4096, 8192]
     // (us, the older kernels for a few rows / this path): M = 2: 17.3 / 20.5 and 12.2 / 14.1; M = 4: 29.3 / 20.9 and
     // 12.7 / 14.4; M = 8: 52.6 / 20.8 and 21.4 / 14.5; M = 32: 78.7 / 21.3 and 46.1 / 15.3.
-    if (M < kTwoPassFrom && (M >= 8 || (M >= 4 && K >= 12288))) {
+    // Rows whose 256-element units do not split evenly over four waves leave the older kernels one wave per block
+    // (W[4096, 11008], M = 1: 43 us), so they come here for any M; many rows come here too while the 128x128 blocks fit
+    // the CUs in one round (W[1024, 4096], M = 2048: 27 us against 51 us for the dequantise-once form).
+    if (M >= 8 || (M >= 4 && K >= 12288) || (K / 256) % 4 != 0) {
+        // (below kTwoPassFrom rows only launches that split K: the dispatch further down takes the unsplit ones)
         const int rc = spec_launch<4>(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, dtype, workspace,
-                                      workspace_bytes, (hipStream_t)stream, 1, true);
+                                      workspace_bytes, (hipStream_t)stream, 1, M < kTwoPassFrom);
         if (rc != AMCT_E_UNSUPPORTED) return rc;
     }
     // fp16 activations: otherwise the tile kernels below or the kernels shared with the int8-weight path (gemm_wq16.hip),
