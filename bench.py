@@ -394,6 +394,58 @@ def build_cases(dev, only):
         cases.append(Case("w8a16_m16", "hbm", N9 * K9 + 16 * K9 * 2 + 16 * N9 * 2 + N9 * 2, "B", launch, 6, "bf16",
                           "int8 weight-only Linear M=16 N=14336 K=4096, per-channel scales, bf16 activations (decode): weight streaming"))
 
+    # ---- the three Linears on a down-projection shape, W[4096,14336] at M = 16: few column blocks and long rows, so the
+    # tile kernels split K over blocks (partial sums in the lent workspace, a second kernel adds them)
+    if want("w8a8_down_m16") or want("w4a16_down_m16") or want("w8a16_down_m16"):
+        Nd, Kd, Md, gd = 4096, 14336, 16, 128
+        gen = torch.Generator().manual_seed(2031)
+        nwd = 8                                          # 8 x 58.7 MB (int8) / 29.4 MB (int4) of weights rotate
+        xd16 = (torch.randn(Md, Kd, generator=gen) * 0.5).to(torch.bfloat16).to(dev)
+        wd8 = dev_copies(torch.randint(-128, 128, (Nd, Kd), generator=gen, dtype=torch.int16).to(torch.int8), nwd)
+        if want("w8a8_down_m16"):
+            xqd = torch.randint(-128, 128, (Md, Kd), generator=gen, dtype=torch.int16).to(torch.int8).to(dev)
+            stk = (0.01 + torch.rand(Md, generator=gen)).to(dev)
+            sch = (1e-3 + 9e-3 * torch.rand(Nd, generator=gen)).to(dev)
+            outs_d = [torch.empty(Md, Nd, dtype=torch.bfloat16, device=dev) for _ in range(nwd)]
+            wsd = torch.empty(max(16, lib.amct_gemm_w8a8_workspace_bytes(Md, Nd, Kd)), dtype=torch.uint8, device=dev)
+
+            def launch(i, xqd=xqd, wd8=wd8, stk=stk, sch=sch, outs_d=outs_d, wsd=wsd):
+                j = i % len(wd8)
+                rc = lib.amct_gemm_w8a8_ws(xqd.data_ptr(), wd8[j].data_ptr(), stk.data_ptr(), sch.data_ptr(), None, 0,
+                                           outs_d[j].data_ptr(), None, Md, Nd, Kd, _lib.BF16, wsd.data_ptr(), wsd.numel(), st)
+                assert rc == 0, rc
+            cases.append(Case("w8a8_down_m16", "hbm", Nd * Kd + Md * Kd + Md * Nd * 2 + Nd * 4 + Md * 4, "B", launch, nwd, "int8",
+                              "W8A8 Linear M=16 N=4096 K=14336 (down projection, decode): 64x64 tiles, K split over 4 blocks per tile, "
+                              "int32 partial sums + reduce kernel"))
+        if want("w4a16_down_m16"):
+            pkd = dev_copies(torch.randint(0, 256, (Nd, Kd // 2), generator=gen, dtype=torch.int16).to(torch.uint8), nwd)
+            scd4 = (1e-3 + 9e-3 * torch.rand(Nd, Kd // gd, generator=gen)).to(torch.float16).to(dev)
+            zd4 = torch.randint(0, 16, (Nd, Kd // gd), generator=gen, dtype=torch.int16).to(torch.uint8).to(dev)
+            outs_d4 = [torch.empty(Md, Nd, dtype=torch.bfloat16, device=dev) for _ in range(nwd)]
+            wsd4 = torch.empty(max(16, lib.amct_gemm_w4a16_workspace_bytes(Md, Nd, Kd, gd, 0)), dtype=torch.uint8, device=dev)
+
+            def launch(i, pkd=pkd, scd4=scd4, zd4=zd4, outs_d4=outs_d4, wsd4=wsd4, xd16=xd16):
+                j = i % len(pkd)
+                rc = lib.amct_gemm_w4a16(xd16.data_ptr(), None, pkd[j].data_ptr(), scd4.data_ptr(), _lib.F16, zd4.data_ptr(), None,
+                                         outs_d4[j].data_ptr(), Md, Nd, Kd, gd, _lib.BF16, wsd4.data_ptr(), wsd4.numel(), st)
+                assert rc == 0, rc
+            cases.append(Case("w4a16_down_m16", "hbm", Nd * Kd // 2 + Nd * (Kd // gd) * 3 + Md * Kd * 2 + Md * Nd * 2, "B", launch, nwd, "bf16",
+                              "W4A16 Linear M=16 N=4096 K=14336 (down projection, decode): specialised-wave 64x64 tiles, K split over "
+                              "4 blocks per tile, fp32 partial sums + reduce kernel"))
+        if want("w8a16_down_m16"):
+            scd8 = (1e-3 + 9e-3 * torch.rand(Nd, Kd // gd, generator=gen)).to(torch.bfloat16).to(dev)
+            outs_d8 = [torch.empty(Md, Nd, dtype=torch.bfloat16, device=dev) for _ in range(nwd)]
+            wsd8 = torch.empty(max(16, lib.amct_gemm_w8a16_workspace_bytes(Md, Nd, Kd, gd, 0)), dtype=torch.uint8, device=dev)
+
+            def launch(i, wd8=wd8, scd8=scd8, outs_d8=outs_d8, wsd8=wsd8, xd16=xd16):
+                j = i % len(wd8)
+                rc = lib.amct_gemm_w8a16_ws(xd16.data_ptr(), None, wd8[j].data_ptr(), scd8.data_ptr(), _lib.BF16, None, None,
+                                            outs_d8[j].data_ptr(), Md, Nd, Kd, gd, _lib.BF16, wsd8.data_ptr(), wsd8.numel(), st)
+                assert rc == 0, rc
+            cases.append(Case("w8a16_down_m16", "hbm", Nd * Kd + Nd * (Kd // gd) * 2 + Md * Kd * 2 + Md * Nd * 2, "B", launch, nwd, "bf16",
+                              "int8 weight-only Linear M=16 N=4096 K=14336 group 128 (down projection, decode): specialised-wave 64x64 "
+                              "tiles, K split over 4 blocks per tile"))
+
     # ---- the same operator at M = 2048: dequantise the weight once into the lent workspace, then the 16-bit GEMM on the
     # large tiles (three launches with smoothing)
     if want("w8a16_m2048"):
