@@ -229,6 +229,7 @@ static int run_token(const void* x, const void* smooth, int8_t* q, float* scale,
     else if (vec_ok && S <= 2 * kBlock) hipLaunchKernelGGL((act_quant_token<DT, 2>), grid, block, 0, st, x, smooth, q, scale, K, mode);
     else if (vec_ok && S <= 4 * kBlock) hipLaunchKernelGGL((act_quant_token<DT, 4>), grid, block, 0, st, x, smooth, q, scale, K, mode);
     else if (vec_ok && S <= 8 * kBlock) hipLaunchKernelGGL((act_quant_token<DT, 8>), grid, block, 0, st, x, smooth, q, scale, K, mode);
+    else if (vec_ok && S <= 16 * kBlock) hipLaunchKernelGGL((act_quant_token<DT, 16>), grid, block, 0, st, x, smooth, q, scale, K, mode);   // rows of up to 32768 16-bit elements
     else hipLaunchKernelGGL((act_quant_token_general<DT>), grid, block, 0, st, x, smooth, q, scale, K, mode);
     return hip_status();
 }

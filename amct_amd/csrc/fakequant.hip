@@ -520,7 +520,7 @@ static bool dispatch_fused(const FqArgs& a, hipStream_t st) {
     else if (S <= 512) launch_fused<DT, 64, 8, 1>(a, st);
     else if (S <= 1024) launch_fused<DT, 256, 4, 1>(a, st);
     else if (S <= 2048) launch_fused<DT, 256, 8, 1>(a, st);
-    else if (VEC == 4 && S <= 4096) launch_fused<DT, 256, VEC == 4 ? 16 : 8, 1>(a, st);   // fp32 rows up to 16384 elements (64 values per lane)
+    else if (S <= 4096) launch_fused<DT, 256, 16, 1>(a, st);        // rows up to 16384 fp32 / 32768 16-bit elements (64 / 128 values per lane)
     else return false;
     return true;
 }

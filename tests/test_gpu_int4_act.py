@@ -87,7 +87,7 @@ def test_int4_word_layouts(dev, k, n):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
-@pytest.mark.parametrize("shape", [(12, 128), (33, 4096), (5, 100), (2, 16384), (3, 20000), (1, 8)])
+@pytest.mark.parametrize("shape", [(12, 128), (33, 4096), (5, 100), (2, 16384), (3, 20000), (1, 8), (3, 28672), (2, 40000)])
 def test_dynamic_per_token(dev, dtype, shape):
     g = torch.Generator().manual_seed(71)
     x = torch.randn(*shape, generator=g).to(dtype)

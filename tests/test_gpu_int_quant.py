@@ -94,7 +94,7 @@ def test_scale_offset_bad_count(dev):
 FUSED_CASES = [((16, 96), 0), ((16, 96), 32), ((64, 64), 0), ((7, 80), 32), ((5, 37), 0), ((12, 128), 128),
                ((8, 4096), 0), ((8, 4096), 128), ((4, 8192), 0), ((3, 16384), 0), ((2, 20000), 0),
                ((6, 1024), 256), ((6, 4096), 2048), ((2, 16384), 8192), ((1, 8), 0), ((130, 256), 64),
-               ((5, 11008), 0), ((4, 14336), 0)]
+               ((5, 11008), 0), ((4, 14336), 0), ((2, 28672), 0), ((2, 40000), 0)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
