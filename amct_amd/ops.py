@@ -2,6 +2,8 @@
 device pointers and the current HIP stream, raise on error codes.  All
 arithmetic happens in the HIP kernels; torch is used for memory only.
 """
+import contextlib
+
 import torch
 
 from . import _lib
@@ -53,8 +55,22 @@ def _segments(rows, cols, group):
     return rows if group == 0 else 1
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_SAME_DEVICE = contextlib.nullcontext()
+
+
 def _stream(dev):
+    """Handle of torch's current stream on dev (the raw getter skips building a Stream object per call)."""
+    if _raw_stream is not None and dev.index is not None:
+        return _raw_stream(dev.index)
     return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _on(dev):
+    """Device guard for a launch: nothing to switch (the common case) when dev is already current."""
+    if dev.index is None or dev.index == torch.cuda.current_device():
+        return _SAME_DEVICE
+    return torch.cuda.device(dev)
 
 
 def _c(t):
@@ -72,7 +88,7 @@ def minmax(w, group=0):
     n = rows if group == 0 else rows * ((cols + group - 1) // group)
     mn = torch.empty(n, dtype=torch.float32, device=dev)
     mx = torch.empty(n, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(_lib.load().amct_minmax(_p(w), _p(mn), _p(mx), rows, cols, group, dtype_code(w.dtype), _stream(dev)))
     if group:
         return mn.reshape(rows, -1), mx.reshape(rows, -1)
@@ -102,7 +118,7 @@ def col_minmax(x, col_max=None, col_min=None, absolute=False):
     lib = _lib.load()
     nbytes = lib.amct_col_minmax_workspace_bytes(rows, cols)
     ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(lib.amct_col_minmax(_p(x), _p(col_max), None if absolute else _p(col_min), rows, cols, int(absolute),
                                        int(accumulate), dtype_code(x.dtype), _p(ws), nbytes, _stream(dev)))
     return col_max if absolute else (col_max, col_min)
@@ -119,7 +135,7 @@ def awq_loss(y, yhat):
     nbytes = lib.amct_awq_loss_workspace_bytes()
     ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     loss = torch.empty((), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(lib.amct_awq_loss(_p(y), _p(yhat), y.numel(), dtype_code(y.dtype), _p(loss), _p(ws), nbytes, _stream(dev)))
     return loss
 
@@ -137,7 +153,7 @@ def hessian_update(hessian, x, beta, alpha):
     tokens, cols = x.shape
     nbytes = lib.amct_hessian_update_workspace_bytes(tokens, cols)
     ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(lib.amct_hessian_update(_p(hessian), _p(x), tokens, cols, float(beta), float(alpha), dtype_code(x.dtype),
                                            _p(ws), ws.numel(), _stream(dev)))
     return hessian
@@ -151,7 +167,7 @@ def scale_offset(vmax, vmin, bits, symmetric, scope_rule=SCOPE_AMCT, bad=None):
     vmax, vmin = _c(vmax), _c(vmin)
     scale = torch.empty(vmax.shape, dtype=torch.float32, device=dev)
     offset = None if symmetric else torch.empty(vmax.shape, dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(_lib.load().amct_scale_offset(_p(vmax), _p(vmin), _p(scale), _p(offset), _p(bad), vmax.numel(), bits,
                                                  int(symmetric), scope_rule, dtype_code(vmax.dtype), _stream(dev)))
     return scale, offset
@@ -185,7 +201,7 @@ def quant_with_params(w, scale, offset, group, qmin, qmax, want_dq=True, codes_k
         codes = torch.empty(w.shape, dtype=torch.int32, device=dev)
     if col_scale is not None:
         col_scale = _c(col_scale.to(w.dtype))
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(_lib.load().amct_quant_with_params(
             _p(w), _p(scale), _p(offset), _p(dq), _p(codes), codes_kind, _p(col_scale), col_mode, rows, cols, group,
             qmin, qmax, int(via_src), stage, dtype_code(w.dtype), _stream(dev)))
@@ -230,7 +246,7 @@ def fakequant_int(w, bits, symmetric, group=0, want_dq=True, codes_kind=CODES_NO
         codes = torch.empty(w.shape, dtype=torch.int32, device=dev)
     if col_scale is not None:
         col_scale = _c(col_scale.to(w.dtype))
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(_lib.load().amct_fakequant_int(
             _p(w), _p(dq), _p(codes), codes_kind, _p(scale), _p(offset), _p(bad), _p(col_scale), col_mode, rows, cols,
             group, bits, int(symmetric), scope_rule, qmin, qmax, int(via_src), dtype_code(w.dtype), _stream(dev)))
@@ -261,7 +277,7 @@ def quant_int4_group_pack(w, group, symmetric=False, scale_dtype=torch.float16, 
     zeros = torch.empty(rows, g, dtype=torch.uint8, device=dev)
     if col_scale is not None:
         col_scale = _c(col_scale.to(w.dtype))
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(_lib.load().amct_quant_int4_group_pack(
             _p(w), _p(packed), _p(s16), dtype_code(scale_dtype), _p(s32), _p(zeros), _p(bad), _p(col_scale), col_mode,
             rows, cols, group, int(symmetric), dtype_code(w.dtype), _stream(dev)))
@@ -278,7 +294,7 @@ def pack_int4_words(codes_i32):
     if n % 8:
         raise RuntimeError("int4 packing needs the last dim to be a multiple of 8")
     words = torch.empty(k, n // 8, dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(_lib.load().amct_pack_int4_words(_p(codes_i32), _p(words), k, n, _stream(dev)))
     return words
 
@@ -288,7 +304,7 @@ def words_to_nibbles_nk(words, k, n):
     dev = _dev(words)
     words = _c(words)
     packed = torch.empty(n, k // 2, dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(_lib.load().amct_words_to_nibbles_nk(_p(words), _p(packed), k, n, _stream(dev)))
     return packed
 
@@ -301,7 +317,7 @@ def pack_nibbles_nk(codes_i8):
         raise RuntimeError("nibble packing expects int8 codes with an even number of columns")
     n, k = codes_i8.shape
     packed = torch.empty(n, k // 2, dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(_lib.load().amct_pack_nibbles_nk(_p(codes_i8), _p(packed), n, k, _stream(dev)))
     return packed
 
@@ -312,7 +328,7 @@ def unpack_nibbles_to_i32_kn(packed):
     packed = _c(packed)
     n, k = packed.shape[0], packed.shape[1] * 2
     codes = torch.empty(k, n, dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(_lib.load().amct_nibbles_nk_to_codes_kn(_p(packed), _p(codes), k, n, _stream(dev)))
     return codes
 
@@ -340,7 +356,7 @@ def act_quant_per_token_int8(x, smooth=None, mode=0):
         smooth = _c(smooth.reshape(-1).to(x.dtype))
         if smooth.numel() != K:
             raise RuntimeError("smooth factor must have K elements")
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(_lib.load().amct_act_quant_per_token_int8(_p(x), _p(smooth), _p(q), _p(s), M, K, mode,
                                                              dtype_code(x.dtype), _stream(dev)))
     return q, s
@@ -369,7 +385,7 @@ def quantize_static(x, scales, zero_points, per_token, smooth=None):
             zero_points = zero_points.repeat(reps) if zero_points is not None else None
             n_scales = rows
     q = torch.empty(x.shape, dtype=torch.int8, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(_lib.load().amct_quantize(_p(x), _p(smooth), _p(scales), _p(zero_points), _p(q), rows, K, n_scales,
                                              int(per_token), dtype_code(x.dtype), _stream(dev)))
     return q
@@ -387,7 +403,7 @@ def mx_quant(x, fmt, scale_mode=MX_FLOOR):
         raise ValueError("MX quantisation needs the last dim to be a multiple of 32")
     el = torch.empty(*x.shape[:-1], cols if fmt == MX_E4M3 else cols // 2, dtype=torch.uint8, device=dev)
     e8 = torch.empty(*x.shape[:-1], cols // 32, dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(_lib.load().amct_mx_quant(_p(x), _p(el), _p(e8), rows, cols, fmt, scale_mode, dtype_code(x.dtype),
                                              _stream(dev)))
     return el, e8
@@ -403,7 +419,7 @@ def mx_dequant(el, e8, fmt, dtype=torch.bfloat16):
     dev = _dev(el, e8)
     el, e8 = _c(el), _c(e8)
     y = torch.empty(*e8.shape[:-1], cols, dtype=dtype, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(_lib.load().amct_mx_dequant(_p(el), _p(e8), _p(y), rows, cols, fmt, dtype_code(dtype), _stream(dev)))
     return y
 
@@ -412,7 +428,7 @@ def hif8_encode(x, saturate=False):
     dev = _dev(x)
     x = _c(x)
     y = torch.empty(x.shape, dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(_lib.load().amct_hif8_encode(_p(x), _p(y), x.numel(), dtype_code(x.dtype), int(saturate), _stream(dev)))
     return y
 
@@ -421,7 +437,7 @@ def hif8_decode(c, dtype=torch.bfloat16):
     dev = _dev(c)
     c = _c(c)
     y = torch.empty(c.shape, dtype=dtype, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(_lib.load().amct_hif8_decode(_p(c), _p(y), c.numel(), dtype_code(dtype), _stream(dev)))
     return y
 
@@ -464,7 +480,7 @@ def gemm_w8a8(xq, wq_nk, s_ch, s_tok=None, bias=None, out_dtype=torch.bfloat16, 
     nbytes = _lib.load().amct_gemm_w8a8_workspace_bytes(M, N, K)
     if nbytes:
         ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(_lib.load().amct_gemm_w8a8_ws(_p(xq), _p(wq_nk), _p(s_tok), _p(s_ch), _p(bias), kind, _p(out), _p(acc),
                                                  M, N, K, dtype_code(out_dtype), _p(ws), 0 if ws is None else ws.numel(),
                                                  _stream(dev)))
@@ -510,7 +526,7 @@ def gemm_w4a16(x, wq_packed, scales, zeros, group, smooth=None, bias=None):
     nbytes = _lib.load().amct_gemm_w4a16_workspace_bytes(M, N, K, group, int(smooth is not None))
     if nbytes:
         ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(_lib.load().amct_gemm_w4a16(_p(x), _p(smooth), _p(wq_packed), _p(scales), dtype_code(scales.dtype),
                                                _p(zeros), _p(bias), _p(out), M, N, K, group, dtype_code(x.dtype),
                                                _p(ws), 0 if ws is None else ws.numel(), _stream(dev)))
@@ -536,7 +552,7 @@ def gemm_w8a16(x, wq_nk, scales, offsets, group, smooth=None, bias=None):
     nbytes = _lib.load().amct_gemm_w8a16_workspace_bytes(M, N, K, group, int(smooth is not None))
     if nbytes:
         ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(_lib.load().amct_gemm_w8a16_ws(_p(x), _p(smooth), _p(wq_nk), _p(scales), dtype_code(scales.dtype),
                                                   _p(offsets), _p(bias), _p(out), M, N, K, group, dtype_code(x.dtype),
                                                   _p(ws), 0 if ws is None else ws.numel(), _stream(dev)))
