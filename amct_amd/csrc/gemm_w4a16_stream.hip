@@ -17,6 +17,7 @@
 // The partial sums of the KS waves are added in wave order, so the result does not depend on the launch shape
 // beyond KS.
 #include "amct_common.h"
+#include "gemm_plan.h"
 
 namespace amct {
 
@@ -32,6 +33,7 @@ struct StreamArgs {
     const uint16_t* scales;
     const uint8_t* zeros;
     const float* bias;
+    const float* bias_src;                           // bias, or any readable N floats when there is none
     uint16_t* out;
     int M, N, K, G;                                  // G = K / group
     int group;
@@ -98,9 +100,133 @@ AMCT_DEV uint4 st_smooth8(const uint4& x, const uint4& c) {
     return make_uint4(o[0], o[1], o[2], o[3]);
 }
 
-// XJ: 16-byte activation vectors a thread stages (clamped duplicates beyond the tensor)
+// What a wave holds of one tile of CG x 16 columns: its whole weight stream and the factors of its lane's column.
+template <int NL>
+struct StTile {
+    u4v wv[NL];
+    uint32_t fsw[NL / 2], fzw[(NL + 3) / 4];
+    float bias;
+};
 
-template <int DT, int KS, int CG, int NL, int XJ, bool SMOOTH>
+// Issues every load of one tile (factors first, then the NL weight registers) and waits for none of them.
+template <int KS, int CG, int NL>
+AMCT_DEV void st_load_tile(const StreamArgs& a, StTile<NL>& t, int n0, int cg, int ks, int lane) {
+    const uint32_t K = (uint32_t)a.K, G = (uint32_t)a.G;
+    const int r16 = lane & 15;
+    // the scales and zero-points of this lane's column for the NL groups of this wave: 2 NL and NL contiguous bytes.
+    // They come from HBM like the weights and are only needed when the first group is folded, so they are loaded into
+    // registers by every lane itself (a block-wide table in LDS would hold up the barrier below for as long as an
+    // HBM access takes under the load of the whole launch's weight requests).
+    const int fcol = n0 + cg * 16 + r16;
+    const size_t fidx = (size_t)(fcol < a.N ? fcol : a.N - 1) * G + ks * NL;
+    // the bias too: a load issued in the epilogue would queue behind the next tile's weights
+    // (unconditional, from `bias_src`, which is always readable: a branch here makes the wait counts of the two paths differ
+    // and the compiler then waits for everything in flight)
+    t.bias = a.bias_src[fcol < a.N ? fcol : a.N - 1];
+#pragma unroll
+    for (int q = 0; q < NL / 2; ++q) t.fsw[q] = *reinterpret_cast<const uint32_t*>(a.scales + fidx + 2 * q);
+    if constexpr (NL >= 4) {
+#pragma unroll
+        for (int q = 0; q < NL / 4; ++q) t.fzw[q] = *reinterpret_cast<const uint32_t*>(a.zeros + fidx + 4 * q);
+    } else {
+        t.fzw[0] = *reinterpret_cast<const uint16_t*>(a.zeros + fidx);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // A load instruction fetches 8 weight rows x one whole 128-byte line (256 elements of K): lane l reads row l % 8
+    // (the second instruction of a pair rows 8 .. 15) and the 16-byte chunk chunk_of(l / 8) of the line.  Whole lines per
+    // instruction stream 1.3 us faster over W[14336,4096] than 16 rows x 64 bytes.  The MFMA wants 16 different rows in
+    // lanes 0 .. 15 of a lane group, so the two registers of a pair swap halves afterwards (two DPP moves per word):
+    // the first then holds chunks 0 .. 3 (one group of 128, chunk g in lane group g) for rows 0 .. 15, the second chunks
+    // 4 .. 7 (the next group).
+    const uint32_t kw = K / KS;                      // elements of K of this wave: NL steps of 128
+    const uint32_t oct = lane >> 3;
+    const uint32_t chunk = (oct & 1) ? 4 + (oct >> 1) : (oct >> 1);
+    const int rlo = n0 + cg * 16 + (lane & 7), rhi = rlo + 8;
+    const uint8_t* wlo = a.wq + (size_t)(rlo < a.N ? rlo : a.N - 1) * (K / 2) + (ks * kw) / 2 + chunk * 16;
+    const uint8_t* whi = a.wq + (size_t)(rhi < a.N ? rhi : a.N - 1) * (K / 2) + (ks * kw) / 2 + chunk * 16;
+#pragma unroll
+    for (int i = 0; i < NL; i += 2) {
+        t.wv[i] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wlo + (i / 2) * 128));
+        t.wv[i + 1] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(whi + (i / 2) * 128));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// Follows the weights of one tile as they land, adds the KS partial sums of a column group in wave order through
+// `red` ((KS - 1) * CG * 64 * 16 bytes of LDS that nobody else touches until the next barrier but one), writes.
+// FIRST_SYNC: `red` overlays the activations, so every wave has to be done reading them first.
+template <int DT, int KS, int CG, int NL, bool FIRST_SYNC>
+AMCT_DEV void st_compute_tile(const StreamArgs& a, StTile<NL>& t, int n0, int cg, int ks, int lane, const uint8_t* xlane,
+                              const float* xsum, float* red) {
+    const uint32_t kw = (uint32_t)a.K / KS;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int M = a.M;
+    s4f acc = {0.f, 0.f, 0.f, 0.f}, P = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+        // the loads retire in order: step i waits for wv[i] only, the younger ones stay in flight
+        uint4 fa[4];
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4) fa[s4] = *reinterpret_cast<const uint4*>(xlane + i * 256 + s4 * 16);
+        if ((i & 1) == 0) {                          // both registers of the pair have landed: swap halves
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const uint32_t lo = t.wv[i][d], hi = t.wv[i + 1][d];
+                // row_ror:8 inside each row of 16 lanes; bank_mask picks the lanes that take the rotated value
+                t.wv[i][d] = (uint32_t)__builtin_amdgcn_update_dpp((int)lo, (int)hi, 0x128, 0xF, 0xC, false);
+                t.wv[i + 1][d] = (uint32_t)__builtin_amdgcn_update_dpp((int)hi, (int)lo, 0x128, 0xF, 0x3, false);
+            }
+        }
+        const uint32_t ws[4] = {t.wv[i].x, t.wv[i].y, t.wv[i].z, t.wv[i].w};
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4)
+            P = StAct<DT>::mfma(fa[s4], StAct<DT>::int8x(ws[s4]), P);
+        {                                             // a step is one group of 128: fold it into the result
+            const uint32_t gi = (ks * kw) / 128 + i;
+            const uint32_t sbits = (t.fsw[i / 2] >> (16 * (i & 1))) & 0xFFFFu;
+            const uint32_t zu = (t.fzw[i / 4] >> (8 * (i & 3))) & 0xFFu;
+            const float s_h = f16_bits_to_f32(sbits), s_b = bf16_bits_to_f32(sbits);
+            const float sc = a.scale_f16 ? s_h : s_b;
+            const float c = -(sc * (float)(16u + zu));                        // exact: 5 bits x 11 bits
+            const s4f X = *reinterpret_cast<const s4f*>(xsum + gi * 16 + 4 * g);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[r] = __builtin_fmaf(sc, P[r], __builtin_fmaf(c, X[r], acc[r]));
+            P = s4f{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    s4f y = acc;
+    if constexpr (KS > 1) {
+        if constexpr (FIRST_SYNC) __syncthreads();
+        if (ks > 0) *reinterpret_cast<s4f*>(red + (((ks - 1) * CG + cg) * 64 + lane) * 4) = y;
+        __syncthreads();
+        if (ks == 0) {
+#pragma unroll
+            for (int w = 0; w < KS - 1; ++w) {
+                const s4f o = *reinterpret_cast<const s4f*>(red + ((w * CG + cg) * 64 + lane) * 4);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) y[r] = y[r] + o[r];
+            }
+        }
+    }
+    const int ncol = n0 + cg * 16 + r16;
+    if (ks == 0 && ncol < a.N) {
+        int m0 = 4 * g;
+        asm volatile("" : "+v"(m0));                  // the output addresses are computed here, per tile, not kept in registers
+        uint16_t* o = a.out + (size_t)m0 * a.N + ncol;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float v = y[r];
+            if (a.bias) v = v + t.bias;
+            if (m0 + r < M) o[(size_t)r * a.N] = (uint16_t)StAct<DT>::out_bits(v);
+        }
+    }
+}
+
+// XJ: 16-byte activation vectors a thread stages (clamped duplicates beyond the tensor).
+// LOOP: a block walks the tiles blockIdx.x, blockIdx.x + gridDim.x, ... on one staged copy of the activations, the
+// next tile's loads issued before the current tile is consumed (two register sets); for weights with more tiles than
+// the device runs blocks at once, where staging the activations per tile costs as much traffic as the tile's weights.
+template <int DT, int KS, int CG, int NL, int XJ, bool SMOOTH, bool LOOP>
 __global__ __launch_bounds__(KS * CG * 64) void w4a16_stream(StreamArgs a) {
     static_assert(NL % 2 == 0, "the weight loads come in pairs");
     extern __shared__ __align__(16) uint8_t lds[];
@@ -110,15 +236,14 @@ __global__ __launch_bounds__(KS * CG * 64) void w4a16_stream(StreamArgs a) {
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int cg = wave / KS, ks = wave % KS;
     const int r16 = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * COLS;
     const uint32_t K = (uint32_t)a.K, M = (uint32_t)a.M, G = (uint32_t)a.G;
     const uint32_t xstride = K * 2 + 16;             // 16 bytes of padding: the 16 rows of a fragment read hit different banks
     const uint32_t xbytes = M * xstride;
-    const uint32_t red_bytes = (KS - 1) * CG * 64 * 16;
+    constexpr uint32_t kRedBytes = (KS - 1) * CG * 64 * 16;
     uint8_t* xs = lds;
     float* xsum = reinterpret_cast<float*>(lds + xbytes);   // [G][16]: sum of x' per group and row
 
-    // ---- staging loads (activations, smoothing factors, this block's scales and zero-points) ----------------
+    // ---- staging loads (activations, smoothing factors) --------------------------------------------------------
     const uint32_t KV = K / 8, n_xv = M * KV;
     uint4 xv[XJ], cv[XJ];
     uint32_t xrow[XJ], xkv[XJ];
@@ -131,43 +256,10 @@ __global__ __launch_bounds__(KS * CG * 64) void w4a16_stream(StreamArgs a) {
         xv[j] = ldg16(a.x + (size_t)xrow[j] * K + xkv[j] * 8);
         if constexpr (SMOOTH) cv[j] = ldg16(a.smooth + xkv[j] * 8);
     }
-    // the scales and zero-points of this lane's column for the NL groups of this wave: 2 NL and NL contiguous bytes.
-    // They come from HBM like the weights and are only needed when the first group is folded, so they are loaded into
-    // registers by every lane itself (a block-wide table in LDS would hold up the barrier below for as long as an
-    // HBM access takes under the load of the whole launch's weight requests).
-    const int fcol = n0 + cg * 16 + r16;
-    const size_t fidx = (size_t)(fcol < a.N ? fcol : a.N - 1) * G + ks * NL;
-    uint32_t fsw[NL / 2], fzw[(NL + 3) / 4];
-#pragma unroll
-    for (int q = 0; q < NL / 2; ++q) fsw[q] = *reinterpret_cast<const uint32_t*>(a.scales + fidx + 2 * q);
-    if constexpr (NL >= 4) {
-#pragma unroll
-        for (int q = 0; q < NL / 4; ++q) fzw[q] = *reinterpret_cast<const uint32_t*>(a.zeros + fidx + 4 * q);
-    } else {
-        fzw[0] = *reinterpret_cast<const uint16_t*>(a.zeros + fidx);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    // ---- the whole weight stream of this wave ---------------------------------------------------------------------
-    // A load instruction fetches 8 weight rows x one whole 128-byte line (256 elements of K): lane l reads row l % 8
-    // (the second instruction of a pair rows 8 .. 15) and the 16-byte chunk chunk_of(l / 8) of the line.  Whole lines per
-    // instruction stream 1.3 us faster over W[14336,4096] than 16 rows x 64 bytes.  The MFMA wants 16 different rows in
-    // lanes 0 .. 15 of a lane group, so the two registers of a pair swap halves afterwards (two DPP moves per word):
-    // the first then holds chunks 0 .. 3 (one group of 128, chunk g in lane group g) for rows 0 .. 15, the second chunks
-    // 4 .. 7 (the next group).
-    const uint32_t kw = K / KS;                      // elements of K of this wave: NL steps of 128
-    const int ncol = n0 + cg * 16 + r16;
-    const uint32_t oct = lane >> 3;
-    const uint32_t chunk = (oct & 1) ? 4 + (oct >> 1) : (oct >> 1);
-    const int rlo = n0 + cg * 16 + (lane & 7), rhi = rlo + 8;
-    const uint8_t* wlo = a.wq + (size_t)(rlo < a.N ? rlo : a.N - 1) * (K / 2) + (ks * kw) / 2 + chunk * 16;
-    const uint8_t* whi = a.wq + (size_t)(rhi < a.N ? rhi : a.N - 1) * (K / 2) + (ks * kw) / 2 + chunk * 16;
-    u4v wv[NL];
-#pragma unroll
-    for (int i = 0; i < NL; i += 2) {
-        wv[i] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wlo + (i / 2) * 128));
-        wv[i + 1] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(whi + (i / 2) * 128));
-    }
-    __builtin_amdgcn_sched_barrier(0);
+    // ---- the whole weight stream of this wave for its first tile -------------------------------------------------
+    int tile = blockIdx.x;
+    StTile<NL> ta;
+    st_load_tile<KS, CG, NL>(a, ta, tile * COLS, cg, ks, lane);
 
     // ---- stage the activations: smoothed, interleaved to the operand order of st_int8x, summed per group ----------
 #pragma unroll
@@ -190,79 +282,47 @@ __global__ __launch_bounds__(KS * CG * 64) void w4a16_stream(StreamArgs a) {
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
 
-    // ---- follow the weights as they land ---------------------------------------------------------------------------
-    s4f acc = {0.f, 0.f, 0.f, 0.f}, P = {0.f, 0.f, 0.f, 0.f};
+    const uint32_t kw = K / KS;
     const uint8_t* xlane = xs + (r16 < (int)M ? r16 : (int)M - 1) * xstride + (ks * kw + g * 32) * 2;
-#pragma unroll
-    for (int i = 0; i < NL; ++i) {
-        // the loads retire in order: step i waits for wv[i] only, the NL - 1 - i younger ones stay in flight
-        uint4 fa[4];
-#pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4) fa[s4] = *reinterpret_cast<const uint4*>(xlane + i * 256 + s4 * 16);
-        if ((i & 1) == 0) {                          // both registers of the pair have landed: swap halves
-#pragma unroll
-            for (int d = 0; d < 4; ++d) {
-                const uint32_t lo = wv[i][d], hi = wv[i + 1][d];
-                // row_ror:8 inside each row of 16 lanes; bank_mask picks the lanes that take the rotated value
-                wv[i][d] = (uint32_t)__builtin_amdgcn_update_dpp((int)lo, (int)hi, 0x128, 0xF, 0xC, false);
-                wv[i + 1][d] = (uint32_t)__builtin_amdgcn_update_dpp((int)hi, (int)lo, 0x128, 0xF, 0x3, false);
+    if constexpr (!LOOP) {
+        st_compute_tile<DT, KS, CG, NL, true>(a, ta, tile * COLS, cg, ks, lane, xlane, xsum, reinterpret_cast<float*>(lds));
+    } else {
+        // two reduction buffers behind the activation image, used in turn: a tile's partial sums are read before the
+        // reading wave reaches the next tile's barrier, and written again only after that barrier
+        float* red0 = reinterpret_cast<float*>(lds + xbytes + G * 64);
+        float* red1 = red0 + kRedBytes / 4;
+        const int tiles = (a.N + COLS - 1) / COLS, stride = gridDim.x;
+        StTile<NL> tb;
+        for (;;) {
+            int next = tile + stride;
+            if (next >= tiles) {
+                st_compute_tile<DT, KS, CG, NL, false>(a, ta, tile * COLS, cg, ks, lane, xlane, xsum, red0);
+                break;
             }
-        }
-        const uint32_t ws[4] = {wv[i].x, wv[i].y, wv[i].z, wv[i].w};
-#pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4)
-            P = StAct<DT>::mfma(fa[s4], StAct<DT>::int8x(ws[s4]), P);
-        {                                             // a step is one group of 128: fold it into the result
-            const uint32_t gi = (ks * kw) / 128 + i;
-            const uint32_t sbits = (fsw[i / 2] >> (16 * (i & 1))) & 0xFFFFu;
-            const uint32_t zu = (fzw[i / 4] >> (8 * (i & 3))) & 0xFFu;
-            const float s_h = f16_bits_to_f32(sbits), s_b = bf16_bits_to_f32(sbits);
-            const float sc = a.scale_f16 ? s_h : s_b;
-            const float c = -(sc * (float)(16u + zu));                        // exact: 5 bits x 11 bits
-            const s4f X = *reinterpret_cast<const s4f*>(xsum + gi * 16 + 4 * g);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) acc[r] = __builtin_fmaf(sc, P[r], __builtin_fmaf(c, X[r], acc[r]));
-            P = s4f{0.f, 0.f, 0.f, 0.f};
-        }
-    }
-    s4f y = acc;
-
-    // ---- add the KS partial sums of a column group in wave order, write ------------------------------------
-    if constexpr (KS > 1) {
-        __syncthreads();                              // every wave is done reading activations: their rows are reused
-        float* red = reinterpret_cast<float*>(lds);
-        if (ks > 0) *reinterpret_cast<s4f*>(red + (((ks - 1) * CG + cg) * 64 + lane) * 4) = y;
-        __syncthreads();
-        if (ks == 0) {
-#pragma unroll
-            for (int w = 0; w < KS - 1; ++w) {
-                const s4f o = *reinterpret_cast<const s4f*>(red + ((w * CG + cg) * 64 + lane) * 4);
-#pragma unroll
-                for (int r = 0; r < 4; ++r) y[r] = y[r] + o[r];
+            st_load_tile<KS, CG, NL>(a, tb, next * COLS, cg, ks, lane);
+            st_compute_tile<DT, KS, CG, NL, false>(a, ta, tile * COLS, cg, ks, lane, xlane, xsum, red0);
+            tile = next;
+            next = tile + stride;
+            if (next >= tiles) {
+                st_compute_tile<DT, KS, CG, NL, false>(a, tb, tile * COLS, cg, ks, lane, xlane, xsum, red1);
+                break;
             }
-        }
-    }
-    if (ks == 0 && ncol < a.N) {
-        const float b = a.bias ? a.bias[ncol] : 0.f;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int m = 4 * g + r;
-            float v = y[r];
-            if (a.bias) v = v + b;
-            if (m < (int)M) a.out[(size_t)m * a.N + ncol] = (uint16_t)StAct<DT>::out_bits(v);
+            st_load_tile<KS, CG, NL>(a, ta, next * COLS, cg, ks, lane);
+            st_compute_tile<DT, KS, CG, NL, false>(a, tb, tile * COLS, cg, ks, lane, xlane, xsum, red1);
+            tile = next;
         }
     }
 }
 
-template <int DT, int KS, int CG, int NL, bool SMOOTH>
-static int stream_launch_x(const StreamArgs& a, size_t lds_bytes, hipStream_t st) {
+template <int DT, int KS, int CG, int NL, bool SMOOTH, bool LOOP>
+static int stream_launch_x(const StreamArgs& a, size_t lds_bytes, unsigned blocks, hipStream_t st) {
     constexpr int NT = KS * CG * 64;
     const int n_xv = a.M * (a.K / 8);
     const int xj = (n_xv + NT - 1) / NT;
-    const dim3 grid((unsigned)((a.N + CG * 16 - 1) / (CG * 16)));
+    const dim3 grid(blocks);
 #define AMCT_STREAM_GO(XJ)                                                                                          \
     {                                                                                                               \
-        auto kern = &w4a16_stream<DT, KS, CG, NL, XJ, SMOOTH>;                                                          \
+        auto kern = &w4a16_stream<DT, KS, CG, NL, XJ, SMOOTH, LOOP>;                                                \
         if (lds_bytes > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                       \
                                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess) { \
             (void)hipGetLastError();                                                                                \
@@ -286,8 +346,9 @@ int w4a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, 
     if (M < 1 || M > 16 || (K != 1024 && K != 2048 && K != 4096) || group != 128 || N > (int64_t(1) << 30)) return AMCT_E_UNSUPPORTED;
     if (!aligned16(x) || !aligned16(wq) || (smooth && !aligned16(smooth)) || ((uintptr_t)scales & 3) || ((uintptr_t)zeros & 3))
         return AMCT_E_UNSUPPORTED;
-    StreamArgs a{(const uint16_t*)x, (const uint16_t*)smooth, wq, (const uint16_t*)scales, zeros, bias, (uint16_t*)out,
-                 (int)M, (int)N, (int)K, (int)(K / group), group, scale_dtype == AMCT_F16 ? 1 : 0,
+    StreamArgs a{(const uint16_t*)x, (const uint16_t*)smooth, wq, (const uint16_t*)scales, zeros, bias,
+                 bias ? bias : reinterpret_cast<const float*>(scales),   // N * K / group * 2 >= N * 4 bytes (K >= 1024)
+                 (uint16_t*)out, (int)M, (int)N, (int)K, (int)(K / group), group, scale_dtype == AMCT_F16 ? 1 : 0,
                  (uint32_t)(0x100000000ull / (uint64_t)(K / 8)) + 1u};
     // A wave streams K / 4 elements of 16 columns in NL = K / 512 steps, all of them in flight from the start.  Large
     // activation blocks are staged by few, wide blocks (16 waves share one copy in LDS); small ones by many narrow
@@ -298,16 +359,32 @@ int w4a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, 
     const int cg = xbytes > 40 * 1024 ? 4 : xbytes > 12 * 1024 ? 2 : 1;
     const int64_t nl = K / 512;
     const size_t red = (size_t)3 * cg * 64 * 16, img = xbytes + (size_t)(K / group) * 64;
-    const size_t lds_bytes = img > red ? img : red;
+    // More tiles than CUs under a wide block (one per CU: its activation image fills most of the LDS): one block per CU
+    // walks its share of the tiles on one staged copy of the activations.  W[128256,4096] at M = 8 / 16: 82 / 96 ->
+    // 62 / 63 us; W[28672,4096]: 22.6 / 25.4 -> 19.1 / 20.0 us.  The narrower blocks for smaller activation images (several
+    // per CU, which overlap one block's staging with another's stream) were 5 - 15 % slower in this form.
+    const int64_t tiles = (N + cg * 16 - 1) / (cg * 16), cus = current_cu_count();
+    const size_t loop_bytes = img + 2 * red;
+    const bool loop = cg == 4 && cus > 0 && tiles > cus && loop_bytes <= 160 * 1024;
+    const size_t lds_bytes = loop ? loop_bytes : img > red ? img : red;
+    const unsigned blocks = (unsigned)(loop ? cus : tiles);
     if (lds_bytes > 160 * 1024) return AMCT_E_UNSUPPORTED;
+#define AMCT_STREAM_DT(DT_, CG_, NL_, LOOP_)                                                              \
+    return smooth ? stream_launch_x<DT_, 4, CG_, NL_, true, LOOP_>(a, lds_bytes, blocks, st)              \
+                  : stream_launch_x<DT_, 4, CG_, NL_, false, LOOP_>(a, lds_bytes, blocks, st);
 #define AMCT_STREAM_SHAPE(CG_, NL_)                                                                       \
     if (cg == CG_ && nl == NL_) {                                                                         \
-        if (dtype == AMCT_F16)                                                                            \
-            return smooth ? stream_launch_x<AMCT_F16, 4, CG_, NL_, true>(a, lds_bytes, st)                \
-                          : stream_launch_x<AMCT_F16, 4, CG_, NL_, false>(a, lds_bytes, st);              \
-        return smooth ? stream_launch_x<AMCT_BF16, 4, CG_, NL_, true>(a, lds_bytes, st)                   \
-                      : stream_launch_x<AMCT_BF16, 4, CG_, NL_, false>(a, lds_bytes, st);                 \
+        if (dtype == AMCT_F16) { AMCT_STREAM_DT(AMCT_F16, CG_, NL_, false) }                              \
+        AMCT_STREAM_DT(AMCT_BF16, CG_, NL_, false)                                                        \
     }
+#define AMCT_STREAM_SHAPE_LOOP(NL_)                                                                       \
+    if (cg == 4 && nl == NL_ && loop) {                                                                   \
+        if (dtype == AMCT_F16) { AMCT_STREAM_DT(AMCT_F16, 4, NL_, true) }                                 \
+        AMCT_STREAM_DT(AMCT_BF16, 4, NL_, true)                                                           \
+    }
+    AMCT_STREAM_SHAPE_LOOP(8)
+    AMCT_STREAM_SHAPE_LOOP(4)
+    AMCT_STREAM_SHAPE_LOOP(2)
     AMCT_STREAM_SHAPE(4, 8)
     AMCT_STREAM_SHAPE(2, 8)
     AMCT_STREAM_SHAPE(1, 8)
@@ -317,7 +394,9 @@ int w4a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, 
     AMCT_STREAM_SHAPE(4, 2)
     AMCT_STREAM_SHAPE(2, 2)
     AMCT_STREAM_SHAPE(1, 2)
+#undef AMCT_STREAM_SHAPE_LOOP
 #undef AMCT_STREAM_SHAPE
+#undef AMCT_STREAM_DT
     return AMCT_E_UNSUPPORTED;                        // K / 512 steps per wave beyond 8: the other kernels
 }
 

@@ -178,11 +178,14 @@ def test_w4a16_vs_oracle(dev, M, N, K, group, sdt):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 64, 1024), (16, 200, 2048), (9, 72, 1024), (5, 33, 2048), (16, 1000, 1024),
-                                   (13, 14336, 4096), (1, 14336, 2048), (3, 16, 4096), (16, 15, 1024)])
+                                   (13, 14336, 4096), (1, 14336, 2048), (3, 16, 4096), (16, 15, 1024),
+                                   (16, 40000, 1024), (16, 20008, 4096), (1, 70000, 1024), (4, 33000, 2048), (2, 16392, 4096)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_w4a16_weight_streaming_kernel(dev, M, N, K, dtype):
     """The kernel for a few rows (M <= 16, K of 1024/2048/4096, groups of 128): every block width, ragged N, both factor
-    dtypes, with and without smoothing, against the fp64 anchor whose dequantised weight is not rounded; then the
+    dtypes, with and without smoothing, against the fp64 anchor whose dequantised weight is not rounded (the last
+    shapes: more column tiles than the device runs blocks at once, so that a block walks several tiles -- one, two, three
+    or more, with a ragged last one -- on one staged copy of the activations); then the
     integer special case (scale 1, small integer activations), where both readings of the dequantisation give the same
     bits as an integer matmul."""
     assert od.w4a16_streams(M, K, 128, dtype)
