@@ -1939,7 +1939,7 @@ static int two_pass(const void* x, const void* smooth, const uint8_t* wq, const 
 // Block shape of the kernels with specialised waves (3: 64x64, 4: 128x64, 1: 128x128; 0: they do not apply) and the number
 // of K slices of the launch.  K is split over blocks when the tiles alone would leave CUs idle (few output columns, long
 // rows: the down projection of an MLP) or when a row has more groups than the kernel's factor table holds; a slice is
-// at least 2048 elements.  max_rounds: how many rounds of 128x128 blocks are still accepted up to 512 rows.
+// at least 2048 elements.  max_rounds: 1 = only launches whose 128x128 blocks run at once; 2 = the rule for int8 weights below.
 struct SpecPlan {
     int shape;
     int splits;
@@ -1951,8 +1951,11 @@ static SpecPlan spec_plan(int64_t M, int64_t N, int64_t K, int group, int64_t cu
     int64_t blocks;
     if (M <= 64 && nt64 <= cus) p.shape = 3, blocks = nt64;
     else if (mt * nt64 <= cus) p.shape = 4, blocks = mt * nt64;
-    else if (mt * nt128 <= cus || (M <= 512 && mt * nt128 <= max_rounds * cus) || (max_rounds > 1 && M <= 128))
-        p.shape = 1, blocks = mt * nt128;                          // (up to 128 rows any number of rounds: the weight streams once)
+    else if (mt * nt128 <= cus ||
+             (max_rounds > 1 && (M <= 384 || (M <= 512 && (mt * nt128 <= max_rounds * cus || mt * nt128 > 4 * cus)))))
+        // (int8 weights: any number of rounds up to 384 rows -- dequantising the weight once costs more than the rounds --
+        // and up to 512 rows unless the last round of three or four would run half empty)
+        p.shape = 1, blocks = mt * nt128;
     else return p;
     const int64_t units = K / 256;
     auto fits = [&](int64_t S) {                                    // the groups of every slice fit the factor table
@@ -2030,9 +2033,10 @@ static int spec_launch(const void* x, const void* smooth, const uint8_t* wq, con
     return hip_status();
 }
 
-// The int8 weight-only Linear (gemm_wq16.hip) on the kernels with specialised waves: while the 128x128 blocks of the
-// launch fit the CUs in two rounds (up to 512 rows on W[14336, 4096]: 74 / 81 us at 384 / 512 rows against 98 us for the
-// dequantise-once form, which wins from there on: 640 rows 115 against 111 us); any number of rows when K is split.
+// The int8 weight-only Linear (gemm_wq16.hip) on the kernels with specialised waves: up to 384 rows, and up to 512 rows
+// unless the last of three or four rounds of 128x128 blocks would run half empty (W[14336, 4096]: 74 / 81 us at 384 / 512 rows
+// against 98 us for the dequantise-once form, which wins from there on: 640 rows 115 against 111 us; W[57344, 4096] at
+// 256 / 384 / 512 rows: 167 / 245 / 313 us against 285 / 347 / 357 us); any number of rows when K is split.
 int w8a16_spec_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
                         const uint8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group, int dtype,
                         void* workspace, size_t workspace_bytes, hipStream_t st) {

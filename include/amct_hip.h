@@ -301,9 +301,9 @@ int amct_gemm_w8a16(const void* x, const void* smooth, const int8_t* wq, const v
  * dequantised once into it (N * K * 2 bytes; the smoothed activations follow), and the product runs as a plain 16-bit
  * GEMM on the 256x256 tiles of the W8A8 kernel: the same arithmetic as the tile kernel without workspace (the
  * dequantised weight rounded to dtype, fp32 accumulation), about three times as fast.  For fewer rows (M > 16) with smooth
- * the query asks for M * K * 2 bytes: the multiply is then done once up front and the fast tile kernels apply (while
- * their blocks fit the CUs in two rounds, K a multiple of 256, groups a multiple of 64; they take precedence up to 512
- * rows on W[14336, 4096]; for long rows on few column blocks with K split over blocks, whose fp32 partial sums follow the
+ * the query asks for M * K * 2 bytes: the multiply is then done once up front and the fast tile kernels apply (K a
+ * multiple of 256, groups a multiple of 64; they take precedence up to 384 rows, and up to 512 rows unless a last round
+ * of 128x128 blocks would run half empty; for long rows on few column blocks with K split over blocks, whose fp32 partial sums follow the
  * activations in the workspace: S * M * N * 4 bytes more).  0 bytes are asked for otherwise; a null or smaller workspace
  * is never an error. */
 size_t amct_gemm_w8a16_workspace_bytes(int64_t M, int64_t N, int64_t K, int group, int has_smooth);

@@ -295,10 +295,11 @@ def test_w8a16_many_rows_through_the_workspace(dev, dtype, M, N, K, group):
 @pytest.mark.parametrize("M,N,K,group", [(17, 14336, 4096, 128), (40, 520, 1024, 128), (64, 14336, 4096, 4096), (65, 200, 512, 64),
                                          (128, 8200, 256, 64), (200, 1000, 768, 256), (256, 14336, 4096, 128), (100, 264, 320, 64),
                                          (33, 20000, 256, 128), (512, 14336, 1024, 128), (8, 520, 8192, 128), (100, 2048, 8192, 256),
-                                         (1, 1000, 14336, 128)])
+                                         (1, 1000, 14336, 128), (300, 40000, 256, 128), (500, 70000, 256, 256)])
 def test_w8a16_medium_rows_specialised_waves(dev, dtype, M, N, K, group):
-    """Int8 weight-only Linear from 17 rows on, while the blocks fit the CUs in two rounds: the tile kernels with
-    specialised waves (K a multiple of 256; 64x64, 128x64 and 128x128 blocks), ragged M and N, per-channel and grouped
+    """Int8 weight-only Linear from 17 rows on, up to 384 rows (512 unless a last round of blocks would run half empty):
+    the tile kernels with specialised waves (K a multiple of 256; 64x64, 128x64 and 128x128 blocks, the latter in as
+    many rounds as it takes: the two widest shapes), ragged M and N, per-channel and grouped
     factors, symmetric and with offsets, with smoothing (through the workspace ops.gemm_w8a16 lends) and bias; one shape
     the shared kernel keeps (K = 320); the last shapes (few column blocks, long rows, any number of rows) with K split
     over several blocks per tile.  dt((q - offset) * scale) and fp32 accumulation: within 1e-3 of the row's largest
