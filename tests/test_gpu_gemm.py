@@ -137,7 +137,8 @@ def w4a16_oracle(x, codes, scales, zeros, group, smooth, bias, rows=None):
                                          (65, 14336, 256, 256), (25, 200, 128, 64), (40, 14336, 256, 128), (48, 40000, 128, 64),
                                          (100, 14336, 128, 128), (128, 8200, 256, 64), (64, 14336, 128, 128), (300, 14336, 128, 128),
                                          (512, 14328, 256, 64), (257, 1000, 384, 128), (33, 200, 512, 64), (100, 520, 768, 128), (64, 14336, 256, 128),
-                                         (40, 520, 8192, 128), (8, 1000, 14336, 128), (100, 4096, 4096, 128), (200, 264, 11008, 64)])
+                                         (40, 520, 8192, 128), (8, 1000, 14336, 128), (100, 4096, 4096, 128), (200, 264, 11008, 64),
+                                         (17, 14336, 4096, 128), (64, 1000, 2048, 64), (33, 4104, 4096, 256), (50, 8200, 3072, 128)])
 def test_w4a16_large_shapes_ragged(dev, M, N, K, group):
     """The wide tile kernels (M > 24, group % 64 == 0) in their block shapes (64x64, 128x64, 128x128 with and without specialised
     waves, 128x256, 256x256; two or three LDS stages) on ragged edges in M and N, both scale dtypes; the last shapes (few
