@@ -1888,7 +1888,8 @@ int wq16_int4_f16(const void* x, const void* smooth, const uint8_t* wq, const vo
                   hipStream_t st);                                 // gemm_wq16.hip
 int w4a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
                           const uint8_t* zeros, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group,
-                          int dtype, hipStream_t st);              // gemm_w4a16_stream.hip
+                          int dtype, void* workspace, size_t workspace_bytes, hipStream_t st);
+size_t w4a16_stream_part_bytes(int64_t M, int64_t N, int64_t K, int group);   // partial sums of its launches over slices of K              // gemm_w4a16_stream.hip
 
 int gemm16_tiles(const void* x, const void* w, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int dtype,
                  void* workspace, size_t workspace_bytes, hipStream_t st);   // gemm_w8a8.hip
@@ -2033,6 +2034,16 @@ static int spec_launch(const void* x, const void* smooth, const uint8_t* wq, con
     return hip_status();
 }
 
+// out = dt(part[0] + ... + part[splits - 1] + bias) for the other files' split launches (N % 8 == 0; part, bias and out
+// 16-byte aligned)
+int splitk_reduce16_launch(const float* part, const float* bias, void* out, int64_t M, int64_t N, int splits, int dtype, hipStream_t st) {
+    int64_t nb = (M * N / 8 + kBlock - 1) / kBlock;
+    if (nb > 8192) nb = 8192;
+    if (dtype == AMCT_F16) hipLaunchKernelGGL((splitk_reduce16<true>), dim3((unsigned)nb), dim3(kBlock), 0, st, part, bias, (uint16_t*)out, M, N, splits);
+    else hipLaunchKernelGGL((splitk_reduce16<false>), dim3((unsigned)nb), dim3(kBlock), 0, st, part, bias, (uint16_t*)out, M, N, splits);
+    return hip_status();
+}
+
 // The int8 weight-only Linear (gemm_wq16.hip) on the kernels with specialised waves: up to 384 rows, and up to 512 rows
 // unless the last of three or four rounds of 128x128 blocks would run half empty (W[14336, 4096]: 74 / 81 us at 384 / 512 rows
 // against 98 us for the dequantise-once form, which wins from there on: 640 rows 115 against 111 us; W[57344, 4096] at
@@ -2057,7 +2068,9 @@ extern "C" size_t amct_gemm_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t 
     if (two) return two;
     // tile kernels: x * smooth done once; long rows on few column blocks: the partial sums of the K slices behind it
     const size_t part = spec_part_bytes(spec_plan(M, N, K, group, current_cu_count(), 1), M, N);
-    return (has_smooth && (M > 16 || part) ? (size_t)M * (size_t)K * 2 : 0) + part;
+    const size_t tiles = (has_smooth && (M > 16 || part) ? (size_t)M * (size_t)K * 2 : 0) + part;
+    const size_t stream = w4a16_stream_part_bytes(M, N, K, group);     // a few rows, K in slices: its partial sums only
+    return tiles > stream ? tiles : stream;
 }
 
 extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t* wq, const void* scales,
@@ -2072,7 +2085,7 @@ extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t*
     if (M == 0) return AMCT_OK;
     if (M <= 16) {                                                 // K of 1024 / 2048 / 4096, group 128: the weight-streaming kernel
         const int rc = w4a16_stream_dispatch(x, smooth, wq, scales, scale_dtype, zeros, bias, out, M, N, K, group, dtype,
-                                             (hipStream_t)stream);
+                                             workspace, workspace_bytes, (hipStream_t)stream);
         if (rc != AMCT_E_UNSUPPORTED) return rc;
     }
     // long rows on few column blocks: specialised waves, K split over blocks.  Measured on W[4096, 14336] / W[4096, 8192]

@@ -35,10 +35,14 @@ struct StreamArgs {
     const float* bias;
     const float* bias_src;                           // bias, or any readable N floats when there is none
     uint16_t* out;
-    int M, N, K, G;                                  // G = K / group
+    int M, N, K, G;                                  // K: elements of a row one block walks (a slice); G = K / group
     int group;
     int scale_f16;
     uint32_t kv_magic;                               // floor(2^32 / (K / 8)) + 1: v / (K / 8) == mulhi(v, magic)
+    // Rows longer than a slice: blockIdx.y picks the slice; rows keep their full length as stride; every slice leaves
+    // fp32 partial sums part[slice][M][N] that a second kernel adds in slice order (plus bias, rounding to the output type)
+    int row_k;                                       // elements of a full row of x and of the weight
+    float* part;                                     // null: one slice, the result goes to `out`
 };
 
 typedef _Float16 s8h __attribute__((ext_vector_type(8)));
@@ -118,7 +122,8 @@ AMCT_DEV void st_load_tile(const StreamArgs& a, StTile<NL>& t, int n0, int cg, i
     // registers by every lane itself (a block-wide table in LDS would hold up the barrier below for as long as an
     // HBM access takes under the load of the whole launch's weight requests).
     const int fcol = n0 + cg * 16 + r16;
-    const size_t fidx = (size_t)(fcol < a.N ? fcol : a.N - 1) * G + ks * NL;
+    const uint32_t slice = blockIdx.y;
+    const size_t fidx = (size_t)(fcol < a.N ? fcol : a.N - 1) * (size_t)(a.row_k / a.group) + slice * G + ks * NL;
     // the bias too: a load issued in the epilogue would queue behind the next tile's weights
     // (unconditional, from `bias_src`, which is always readable: a branch here makes the wait counts of the two paths differ
     // and the compiler then waits for everything in flight)
@@ -142,8 +147,9 @@ AMCT_DEV void st_load_tile(const StreamArgs& a, StTile<NL>& t, int n0, int cg, i
     const uint32_t oct = lane >> 3;
     const uint32_t chunk = (oct & 1) ? 4 + (oct >> 1) : (oct >> 1);
     const int rlo = n0 + cg * 16 + (lane & 7), rhi = rlo + 8;
-    const uint8_t* wlo = a.wq + (size_t)(rlo < a.N ? rlo : a.N - 1) * (K / 2) + (ks * kw) / 2 + chunk * 16;
-    const uint8_t* whi = a.wq + (size_t)(rhi < a.N ? rhi : a.N - 1) * (K / 2) + (ks * kw) / 2 + chunk * 16;
+    const size_t wrow = (size_t)(a.row_k / 2), woff = (size_t)slice * (K / 2) + (ks * kw) / 2 + chunk * 16;
+    const uint8_t* wlo = a.wq + (size_t)(rlo < a.N ? rlo : a.N - 1) * wrow + woff;
+    const uint8_t* whi = a.wq + (size_t)(rhi < a.N ? rhi : a.N - 1) * wrow + woff;
 #pragma unroll
     for (int i = 0; i < NL; i += 2) {
         t.wv[i] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wlo + (i / 2) * 128));
@@ -212,12 +218,19 @@ AMCT_DEV void st_compute_tile(const StreamArgs& a, StTile<NL>& t, int n0, int cg
     if (ks == 0 && ncol < a.N) {
         int m0 = 4 * g;
         asm volatile("" : "+v"(m0));                  // the output addresses are computed here, per tile, not kept in registers
-        uint16_t* o = a.out + (size_t)m0 * a.N + ncol;
+        if (a.part) {
+            float* o = a.part + ((size_t)blockIdx.y * M + m0) * a.N + ncol;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            float v = y[r];
-            if (a.bias) v = v + t.bias;
-            if (m0 + r < M) o[(size_t)r * a.N] = (uint16_t)StAct<DT>::out_bits(v);
+            for (int r = 0; r < 4; ++r)
+                if (m0 + r < M) o[(size_t)r * a.N] = y[r];
+        } else {
+            uint16_t* o = a.out + (size_t)m0 * a.N + ncol;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float v = y[r];
+                if (a.bias) v = v + t.bias;
+                if (m0 + r < M) o[(size_t)r * a.N] = (uint16_t)StAct<DT>::out_bits(v);
+            }
         }
     }
 }
@@ -253,8 +266,8 @@ __global__ __launch_bounds__(KS * CG * 64) void w4a16_stream(StreamArgs a) {
         const uint32_t vc = v < n_xv ? v : n_xv - 1;
         xrow[j] = __umulhi(vc, a.kv_magic);           // vc / KV
         xkv[j] = vc - xrow[j] * KV;
-        xv[j] = ldg16(a.x + (size_t)xrow[j] * K + xkv[j] * 8);
-        if constexpr (SMOOTH) cv[j] = ldg16(a.smooth + xkv[j] * 8);
+        xv[j] = ldg16(a.x + (size_t)xrow[j] * a.row_k + blockIdx.y * K + xkv[j] * 8);
+        if constexpr (SMOOTH) cv[j] = ldg16(a.smooth + blockIdx.y * K + xkv[j] * 8);
     }
     // ---- the whole weight stream of this wave for its first tile -------------------------------------------------
     int tile = blockIdx.x;
@@ -314,12 +327,15 @@ __global__ __launch_bounds__(KS * CG * 64) void w4a16_stream(StreamArgs a) {
     }
 }
 
+int splitk_reduce16_launch(const float* part, const float* bias, void* out, int64_t M, int64_t N, int splits, int dtype,
+                           hipStream_t st);                          // gemm_w4a16.hip
+
 template <int DT, int KS, int CG, int NL, bool SMOOTH, bool LOOP>
-static int stream_launch_x(const StreamArgs& a, size_t lds_bytes, unsigned blocks, hipStream_t st) {
+static int stream_launch_x(const StreamArgs& a, size_t lds_bytes, dim3 blocks, hipStream_t st) {
     constexpr int NT = KS * CG * 64;
     const int n_xv = a.M * (a.K / 8);
     const int xj = (n_xv + NT - 1) / NT;
-    const dim3 grid(blocks);
+    const dim3 grid = blocks;
 #define AMCT_STREAM_GO(XJ)                                                                                          \
     {                                                                                                               \
         auto kern = &w4a16_stream<DT, KS, CG, NL, XJ, SMOOTH, LOOP>;                                                \
@@ -329,6 +345,7 @@ static int stream_launch_x(const StreamArgs& a, size_t lds_bytes, unsigned block
             return AMCT_E_HIP;                                                                                      \
         }                                                                                                           \
         hipLaunchKernelGGL(kern, grid, dim3(NT), lds_bytes, st, a);                                                 \
+        if (a.part) return splitk_reduce16_launch(a.part, a.bias, a.out, a.M, a.N, (int)grid.y, DT, st);            \
         return hip_status();                                                                                        \
     }
     if (xj <= 2) AMCT_STREAM_GO(2)
@@ -338,18 +355,48 @@ static int stream_launch_x(const StreamArgs& a, size_t lds_bytes, unsigned block
     return AMCT_E_UNSUPPORTED;
 }
 
+// The slice of K one block walks: K itself when it is 1024, 2048 or 4096, else the largest of those that divides K into at
+// most 16 slices (8192 = 2 x 4096, 14336 = 7 x 2048, 5120 = 5 x 1024, 28672 = 7 x 4096); 0: none (odd multiples of 512).
+static int64_t stream_slice(int64_t K) {
+    if (K == 1024 || K == 2048 || K == 4096) return K;
+#ifdef AMCT_ST_SLICE
+    if (K % AMCT_ST_SLICE == 0 && K / AMCT_ST_SLICE <= 16) return AMCT_ST_SLICE;
+#endif
+    for (int64_t ks = 4096; ks >= 1024; ks /= 2)
+        if (K % ks == 0 && K / ks <= 16) return ks;
+    return 0;
+}
+// Sliced rows pay a second launch: taken from 5 rows on, or for rows of 12288 elements and more (measured against the
+// older kernels for a few rows, us: W[8192,8192] M = 1 / 4 / 16: 13.2 / 14.0 / 22.3 against 16.1 / 16.0 / 16.3 sliced;
+// W[28672,8192]: 30.6 / 38.6 / 86.9 against 34.7 / 35.5 / 37.2; W[8192,28672]: 105 / 80 / 79 against 31 / 34 / 41).
+static bool stream_slices_pay(int64_t M, int64_t K) { return M >= 5 || K >= 12288; }
+size_t w4a16_stream_part_bytes(int64_t M, int64_t N, int64_t K, int group) {
+    const int64_t ks = stream_slice(K);
+    if (M < 1 || M > 16 || group != 128 || !ks || ks == K || N % 8 != 0 || !stream_slices_pay(M, K)) return 0;
+    return (size_t)(K / ks) * (size_t)M * (size_t)N * 4;
+}
+
 // Returns AMCT_E_UNSUPPORTED when the shape is not one this kernel takes (the caller then uses its other kernels).
 int w4a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
-                          const uint8_t* zeros, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group,
-                          int dtype, hipStream_t st) {
+                          const uint8_t* zeros, const float* bias, void* out, int64_t M, int64_t N, int64_t K_row, int group,
+                          int dtype, void* workspace, size_t workspace_bytes, hipStream_t st) {
     // one group per step of 128 elements of K (the per-group partial sums of a step cannot be separated otherwise)
-    if (M < 1 || M > 16 || (K != 1024 && K != 2048 && K != 4096) || group != 128 || N > (int64_t(1) << 30)) return AMCT_E_UNSUPPORTED;
+    const int64_t K = stream_slice(K_row), S = K ? K_row / K : 0;
+    if (M < 1 || M > 16 || !K || group != 128 || N > (int64_t(1) << 30)) return AMCT_E_UNSUPPORTED;
     if (!aligned16(x) || !aligned16(wq) || (smooth && !aligned16(smooth)) || ((uintptr_t)scales & 3) || ((uintptr_t)zeros & 3))
         return AMCT_E_UNSUPPORTED;
+    float* part = nullptr;
+    if (S > 1) {
+        // rows of several slices: the partial sums go through the lent workspace
+        const size_t need = w4a16_stream_part_bytes(M, N, K_row, group);
+        if (!need || !workspace || !aligned16(workspace) || workspace_bytes < need || !aligned16(out) || (bias && !aligned16(bias)))
+            return AMCT_E_UNSUPPORTED;
+        part = reinterpret_cast<float*>(workspace);
+    }
     StreamArgs a{(const uint16_t*)x, (const uint16_t*)smooth, wq, (const uint16_t*)scales, zeros, bias,
                  bias ? bias : reinterpret_cast<const float*>(scales),   // N * K / group * 2 >= N * 4 bytes (K >= 1024)
                  (uint16_t*)out, (int)M, (int)N, (int)K, (int)(K / group), group, scale_dtype == AMCT_F16 ? 1 : 0,
-                 (uint32_t)(0x100000000ull / (uint64_t)(K / 8)) + 1u};
+                 (uint32_t)(0x100000000ull / (uint64_t)(K / 8)) + 1u, (int)K_row, part};
     // A wave streams K / 4 elements of 16 columns in NL = K / 512 steps, all of them in flight from the start.  Large
     // activation blocks are staged by few, wide blocks (16 waves share one copy in LDS); small ones by many narrow
     // blocks, several per CU.  Measured on W[14336,4096]: 8.8 us at M = 1 (11.0 us for the kernel this one replaced),
@@ -365,9 +412,10 @@ int w4a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, 
     // per CU, which overlap one block's staging with another's stream) were 5 - 15 % slower in this form.
     const int64_t tiles = (N + cg * 16 - 1) / (cg * 16), cus = current_cu_count();
     const size_t loop_bytes = img + 2 * red;
-    const bool loop = cg == 4 && cus > 0 && tiles > cus && loop_bytes <= 160 * 1024;
+    const bool loop = cg == 4 && cus > 0 && tiles * S > cus && tiles > 1 && loop_bytes <= 160 * 1024;
     const size_t lds_bytes = loop ? loop_bytes : img > red ? img : red;
-    const unsigned blocks = (unsigned)(loop ? cus : tiles);
+    const int64_t per_slice = cus / S > 0 ? cus / S : 1;            // blocks per slice when they walk tiles
+    const dim3 blocks((unsigned)(loop ? (tiles < per_slice ? tiles : per_slice) : tiles), (unsigned)S);
     if (lds_bytes > 160 * 1024) return AMCT_E_UNSUPPORTED;
 #define AMCT_STREAM_DT(DT_, CG_, NL_, LOOP_)                                                              \
     return smooth ? stream_launch_x<DT_, 4, CG_, NL_, true, LOOP_>(a, lds_bytes, blocks, st)              \

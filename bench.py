@@ -430,8 +430,8 @@ def build_cases(dev, only):
                                          outs_d4[j].data_ptr(), Md, Nd, Kd, gd, _lib.BF16, wsd4.data_ptr(), wsd4.numel(), st)
                 assert rc == 0, rc
             cases.append(Case("w4a16_down_m16", "hbm", Nd * Kd // 2 + Nd * (Kd // gd) * 3 + Md * Kd * 2 + Md * Nd * 2, "B", launch, nwd, "bf16",
-                              "W4A16 Linear M=16 N=4096 K=14336 (down projection, decode): specialised-wave 64x64 tiles, K split over "
-                              "4 blocks per tile, fp32 partial sums + reduce kernel"))
+                              "W4A16 Linear M=16 N=4096 K=14336 (down projection, decode): weight-streaming kernel on 7 slices of 2048 "
+                              "elements of K, fp32 partial sums + reduce kernel"))
         if want("w8a16_down_m16"):
             scd8 = (1e-3 + 9e-3 * torch.rand(Nd, Kd // gd, generator=gen)).to(torch.bfloat16).to(dev)
             outs_d8 = [torch.empty(Md, Nd, dtype=torch.bfloat16, device=dev) for _ in range(nwd)]

@@ -269,10 +269,12 @@ int amct_gemm_w8a8_ws(const int8_t* xq, const int8_t* wq, const float* s_tok, co
  * is then dequantised once into the workspace and the product runs as a plain 16-bit GEMM, which beats dequantising inside
  * every row tile from there on (same arithmetic; a smaller workspace keeps the fused kernels).  For long rows on few
  * column blocks (the down projection of an MLP at up to a few hundred rows) the query also asks for S * M * N * 4 bytes:
- * K is then split over S blocks per tile, whose fp32 partial sums a second kernel adds in a fixed order.  0 bytes are
+ * K is then split over S blocks per tile, whose fp32 partial sums a second kernel adds in a fixed order; likewise for
+ * M <= 16 (from 5 rows on, or K >= 12288) when K is 2 ... 16 slices of 4096, 2048 or 1024 elements, which the
+ * weight-streaming kernel then walks one per block.  0 bytes are
  * asked for otherwise; a null or smaller workspace is never an error.
  * Arithmetic of the dequantisation: the tile kernels (M > 16) feed dtype((u - zero) * scale) to the matrix pipe; the
- * weight-streaming kernel for M <= 16 (bf16 or fp16, K of 1024 / 2048 / 4096, group = 128) keeps the weight as the exact integer and applies
+ * weight-streaming kernel for M <= 16 (bf16 or fp16, K of 1024 / 2048 / 4096 or slices of those, group = 128) keeps the weight as the exact integer and applies
  * scale and zero per group in fp32, i.e. the dequantised weight is not rounded to bf16 there (the fp32 weight * scale of
  * tests/amct_pytorch/mock_torch_npu.py:33-55).  Both stay within 1e-3 of the exact result. */
 size_t amct_gemm_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K, int group, int has_smooth);

@@ -274,10 +274,16 @@ def w4a16_forward_f64(x, codes_nk, scale_ng, antioffset_ng, group_size, bias=Non
     return weight_quant_matmul_f64(x2, wdq, bias).reshape(*shp[:-1], -1)
 
 
-def w4a16_streams(M, K, group_size, dtype=torch.bfloat16):
+def w4a16_streams(M, K, group_size, dtype=torch.bfloat16, N=None):
     """Whether the int4 GEMM takes its weight-streaming kernel for this shape (a few rows of bf16 or fp16 activations, K
-    of 1024, 2048 or 4096, groups of 128): that kernel does not round the dequantised weight."""
-    return dtype in (torch.bfloat16, torch.float16) and 1 <= M <= 16 and K in (1024, 2048, 4096) and group_size == 128
+    of 1024, 2048 or 4096, or -- from 5 rows on or for K >= 12288, N a multiple of 8 -- at most 16 slices of one of those;
+    groups of 128): that kernel does not round the dequantised weight."""
+    if dtype not in (torch.bfloat16, torch.float16) or not 1 <= M <= 16 or group_size != 128:
+        return False
+    if K in (1024, 2048, 4096):
+        return True
+    sliced = any(K % ks == 0 and K // ks <= 16 for ks in (4096, 2048, 1024)) and (M >= 5 or K >= 12288)
+    return sliced and (N is None or N % 8 == 0)
 
 
 # --------------------------------------------------------------------------

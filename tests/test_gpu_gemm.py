@@ -128,7 +128,7 @@ def w4a16_oracle(x, codes, scales, zeros, group, smooth, bias, rows=None):
     anti = -(zeros.to(torch.float32) - 8)
     m = x.shape[0] if rows is None else rows
     return od.w4a16_forward_f64(x, signed, scales, anti, group, bias, None if smooth is None else smooth.reshape(1, -1),
-                                round_weight=not od.w4a16_streams(m, x.shape[1], group, x.dtype))
+                                round_weight=not od.w4a16_streams(m, x.shape[1], group, x.dtype, N=codes.shape[0]))
 
 
 @pytest.mark.parametrize("M,N,K,group", [(300, 1000, 256, 64), (256, 448, 128, 128), (2048, 14336, 256, 128), (2000, 14328, 128, 64),
@@ -180,13 +180,16 @@ def test_w4a16_vs_oracle(dev, M, N, K, group, sdt):
 
 @pytest.mark.parametrize("M,N,K", [(1, 64, 1024), (16, 200, 2048), (9, 72, 1024), (5, 33, 2048), (16, 1000, 1024),
                                    (13, 14336, 4096), (1, 14336, 2048), (3, 16, 4096), (16, 15, 1024),
-                                   (16, 40000, 1024), (16, 20008, 4096), (1, 70000, 1024), (4, 33000, 2048), (2, 16392, 4096)])
+                                   (16, 40000, 1024), (16, 20008, 4096), (1, 70000, 1024), (4, 33000, 2048), (2, 16392, 4096),
+                                   (16, 1000, 8192), (8, 520, 14336), (6, 264, 5120), (16, 20008, 8192), (12, 200, 28672),
+                                   (1, 72, 12288)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_w4a16_weight_streaming_kernel(dev, M, N, K, dtype):
     """The kernel for a few rows (M <= 16, K of 1024/2048/4096, groups of 128): every block width, ragged N, both factor
     dtypes, with and without smoothing, against the fp64 anchor whose dequantised weight is not rounded (the last
     shapes: more column tiles than the device runs blocks at once, so that a block walks several tiles -- one, two, three
-    or more, with a ragged last one -- on one staged copy of the activations); then the
+    or more, with a ragged last one -- on one staged copy of the activations; rows of 2 ... 14 slices of 1024, 2048 or 4096
+    elements, whose partial sums a second kernel adds in slice order); then the
     integer special case (scale 1, small integer activations), where both readings of the dequantisation give the same
     bits as an integer matmul."""
     assert od.w4a16_streams(M, K, 128, dtype)
