@@ -13,6 +13,7 @@
 // matrix pipe; both are within the 1e-3 tolerance of the fp64 result.  Groups of 128, 256, ... up to the whole of K
 // (per-channel and per-tensor factors) are spans of whole steps.
 #include "amct_common.h"
+#include "gemm_plan.h"
 
 namespace amct {
 
@@ -59,6 +60,11 @@ struct Stream16Args {
     int spans;                                       // such spans per wave
     int scale_f16;
     uint32_t kv_magic;                               // floor(2^32 / (K / 8)) + 1: v / (K / 8) == mulhi(v, magic)
+    // Rows longer than a slice (K above is the slice one block walks): blockIdx.y picks the slice; rows keep their full
+    // length as stride; every slice leaves fp32 partial sums part[slice][M][N] that a second kernel adds in slice order
+    int row_k;                                       // elements of a full row of x and of the weight
+    int row_g;                                       // groups of a full row
+    float* part;                                     // null: one slice, the result goes to `out`
 };
 
 // 8 bytes (two words) -> 8 values of dt, in byte order
@@ -106,7 +112,7 @@ __global__ __launch_bounds__(4 * CG * 64) void w8a16_stream(Stream16Args a) {
     const int cg = wave / KS, ks = wave % KS;
     const int r16 = lane & 15, g = lane >> 4;
     const int n0 = blockIdx.x * COLS;
-    const uint32_t K = (uint32_t)a.K, M = (uint32_t)a.M, G = (uint32_t)a.G;
+    const uint32_t K = (uint32_t)a.K, M = (uint32_t)a.M;
     const uint32_t xstride = K * 2 + 16;             // 16 bytes of padding: the 16 rows of a fragment read hit different banks
     const uint32_t xbytes = M * xstride;
     uint8_t* xs = lds;
@@ -122,9 +128,9 @@ __global__ __launch_bounds__(4 * CG * 64) void w8a16_stream(Stream16Args a) {
         const uint32_t vc = v < n_xv ? v : n_xv - 1;
         xrow[j] = __umulhi(vc, a.kv_magic);           // vc / KV
         xkv[j] = vc - xrow[j] * KV;
-        xv[j] = ldg16(a.x + (size_t)xrow[j] * K + xkv[j] * 8);
+        xv[j] = ldg16(a.x + (size_t)xrow[j] * a.row_k + blockIdx.y * K + xkv[j] * 8);
         if constexpr (SMOOTH) {
-            if (j < CVN) cv[j] = ldg16(a.smooth + xkv[j] * 8);
+            if (j < CVN) cv[j] = ldg16(a.smooth + blockIdx.y * K + xkv[j] * 8);
         }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -134,8 +140,9 @@ __global__ __launch_bounds__(4 * CG * 64) void w8a16_stream(Stream16Args a) {
     const uint32_t oct = lane >> 3;
     const uint32_t chunk = (oct & 1) ? 4 + (oct >> 1) : (oct >> 1);
     const int rlo = n0 + cg * 16 + (lane & 7), rhi = rlo + 8;
-    const uint8_t* wlo = a.wq + (size_t)(rlo < a.N ? rlo : a.N - 1) * K + ks * kw + chunk * 16;
-    const uint8_t* whi = a.wq + (size_t)(rhi < a.N ? rhi : a.N - 1) * K + ks * kw + chunk * 16;
+    const size_t woff = (size_t)blockIdx.y * K + ks * kw + chunk * 16;
+    const uint8_t* wlo = a.wq + (size_t)(rlo < a.N ? rlo : a.N - 1) * (size_t)a.row_k + woff;
+    const uint8_t* whi = a.wq + (size_t)(rhi < a.N ? rhi : a.N - 1) * (size_t)a.row_k + woff;
     // Blocks of 16 waves have 128 registers per lane: the activation vectors in flight (32) and all of the weights
     // (64) do not fit beside each other, so such a block requests the second half of its lines when the activations have
     // gone to LDS (the first half is still arriving then; narrower blocks request everything at once).
@@ -149,14 +156,15 @@ __global__ __launch_bounds__(4 * CG * 64) void w8a16_stream(Stream16Args a) {
     __builtin_amdgcn_sched_barrier(0);
     // the factors of this lane's column for the spans of this wave (at most NLN), needed when the first span ends
     const int nc = ncol < a.N ? ncol : a.N - 1;
-    const uint32_t g_first = ((uint32_t)ks * NLN) / (uint32_t)a.per_group;     // the group of the wave's first span
+    const uint32_t g_first = (blockIdx.y * (K / 128) + (uint32_t)ks * NLN) / (uint32_t)a.per_group;   // the group of the wave's first span
+    const uint32_t RG = (uint32_t)a.row_g;
     float fs[NLN], fc[NLN];
 #pragma unroll
     for (int q = 0; q < NLN; ++q) {
         const uint32_t gi = q < a.spans ? g_first + q : g_first;
-        const uint32_t gidx = gi < G ? gi : G - 1;
-        const uint32_t sbits = a.scales[(size_t)nc * G + gidx];
-        const int zq = a.offsets ? (int)reinterpret_cast<const int8_t*>(a.offsets)[(size_t)nc * G + gidx] : 0;
+        const uint32_t gidx = gi < RG ? gi : RG - 1;
+        const uint32_t sbits = a.scales[(size_t)nc * RG + gidx];
+        const int zq = a.offsets ? (int)reinterpret_cast<const int8_t*>(a.offsets)[(size_t)nc * RG + gidx] : 0;
         fs[q] = a.scale_f16 ? f16_bits_to_f32(sbits) : bf16_bits_to_f32(sbits);
         fc[q] = -(fs[q] * (float)(zq + 128));                                  // exact: 8 bits x 11 bits
     }
@@ -244,7 +252,13 @@ __global__ __launch_bounds__(4 * CG * 64) void w8a16_stream(Stream16Args a) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) y[r] = y[r] + o[r];
         }
-        if (ncol < a.N) {
+        if (ncol < a.N && a.part) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = 4 * g + r;
+                if (m < (int)M) a.part[((size_t)blockIdx.y * M + m) * a.N + ncol] = y[r];
+            }
+        } else if (ncol < a.N) {
             const float b = a.bias ? a.bias[ncol] : 0.f;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
@@ -257,12 +271,15 @@ __global__ __launch_bounds__(4 * CG * 64) void w8a16_stream(Stream16Args a) {
     }
 }
 
+int splitk_reduce16_launch(const float* part, const float* bias, void* out, int64_t M, int64_t N, int splits, int dtype,
+                           hipStream_t st);                          // gemm_w4a16.hip
+
 template <int DT, int CG, int NLN, bool SMOOTH>
 static int stream16_launch_x(const Stream16Args& a, size_t lds_bytes, hipStream_t st) {
     constexpr int NT = 4 * CG * 64;
     const int n_xv = a.M * (a.K / 8);
     const int xj = (n_xv + NT - 1) / NT;
-    const dim3 grid((unsigned)((a.N + CG * 16 - 1) / (CG * 16)));
+    const dim3 grid((unsigned)((a.N + CG * 16 - 1) / (CG * 16)), (unsigned)(a.row_k / a.K));
 #define AMCT_STREAM16_GO(XJ, CVN_)                                                                                    \
     {                                                                                                               \
         auto kern = &w8a16_stream<DT, CG, NLN, XJ, CVN_, SMOOTH>;                                                         \
@@ -272,6 +289,7 @@ static int stream16_launch_x(const Stream16Args& a, size_t lds_bytes, hipStream_
             return AMCT_E_HIP;                                                                                      \
         }                                                                                                           \
         hipLaunchKernelGGL(kern, grid, dim3(NT), lds_bytes, st, a);                                                 \
+        if (a.part) return splitk_reduce16_launch(a.part, a.bias, a.out, a.M, a.N, (int)grid.y, DT, st);            \
         return hip_status();                                                                                        \
     }
     const int kv = a.K / 8;
@@ -306,19 +324,58 @@ static int stream16_dispatch_dt(const Stream16Args& a, bool smooth, int cg, int 
     return AMCT_E_UNSUPPORTED;
 }
 
+// The slice of K one block walks: K itself when it is 1024, 2048 or 4096, else the largest of those that divides K into at
+// most 16 slices; 0: none.
+static int64_t stream16_slice(int64_t K) {
+    if (K == 1024 || K == 2048 || K == 4096) return K;
+    for (int64_t ks = 4096; ks >= 1024; ks /= 2)
+        if (K % ks == 0 && K / ks <= 16) return ks;
+    return 0;
+}
+// groups the kernel takes for slices of `ks`: 128, 256, ... up to the slice, or whole slices (per-channel factors: the row)
+static bool stream16_group_ok(int64_t K_row, int64_t ks, int group) {
+    if (group < 128 || K_row % group != 0) return false;
+    if (group <= ks) return (group & (group - 1)) == 0;
+    return group % ks == 0;
+}
+// Sliced rows pay a second launch and stage the activations once per block: taken for long rows (K >= 12288), for four
+// and more slices (slices of 1024), or while blocks of 64 columns per slice run in one round.  Measured against the
+// kernels that served these shapes before (specialised waves with K split, shared kernel), us at M = 1 / 4 / 16,
+// per-channel factors: W[8192,28672] 87 / 87 / 87 -> 58 / 65 / 77; W[8192,8192] 30 / 30 / 29 -> 21 / 29 / 23;
+// W[13824,5120] 24 / 26 / 28 -> 19 / 20 / 25; not taken: W[28672,8192] 53 / 56 / 65 (sliced: 56 / 83 / 73),
+// W[10240,8192] 27 / 29 / 33 (sliced: 25 / 35 / 38).
+static bool stream16_slices_pay(int64_t N, int64_t K, int64_t ks) {
+    const int64_t S = K / ks, cus = current_cu_count();
+    return K >= 12288 || S >= 4 || ((N + 63) / 64) * S <= cus;
+}
+size_t w8a16_stream_part_bytes(int64_t M, int64_t N, int64_t K, int group) {
+    const int64_t ks = stream16_slice(K);
+    if (M < 1 || M > 16 || !ks || ks == K || N % 8 != 0 || !stream16_group_ok(K, ks, group) || !stream16_slices_pay(N, K, ks)) return 0;
+    return (size_t)(K / ks) * (size_t)M * (size_t)N * 4;
+}
+
 // Returns AMCT_E_UNSUPPORTED when the shape is not one this kernel takes (the caller then uses its other kernels).
 int w8a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
-                          const uint8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group,
-                          int dtype, hipStream_t st) {
-    if (M < 1 || M > 16 || (K != 1024 && K != 2048 && K != 4096) || N > (int64_t(1) << 30)) return AMCT_E_UNSUPPORTED;
-    if (group < 128 || (group & (group - 1)) != 0 || group > K) return AMCT_E_UNSUPPORTED;     // 128, 256, ..., K
+                          const uint8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K_row, int group,
+                          int dtype, void* workspace, size_t workspace_bytes, hipStream_t st) {
+    const int64_t K = stream16_slice(K_row), S = K ? K_row / K : 0;
+    if (M < 1 || M > 16 || !K || N > (int64_t(1) << 30)) return AMCT_E_UNSUPPORTED;
+    if (!stream16_group_ok(K_row, K, group)) return AMCT_E_UNSUPPORTED;
     if (!aligned16(x) || !aligned16(wq) || (smooth && !aligned16(smooth)) || ((uintptr_t)scales & 1)) return AMCT_E_UNSUPPORTED;
-    const int nln = (int)(K / 512);                  // lines of 128 per wave (a quarter of K)
+    float* part = nullptr;
+    if (S > 1) {
+        // rows of several slices: the partial sums go through the lent workspace
+        const size_t need = w8a16_stream_part_bytes(M, N, K_row, group);
+        if (!need || !workspace || !aligned16(workspace) || workspace_bytes < need || !aligned16(out) || (bias && !aligned16(bias)))
+            return AMCT_E_UNSUPPORTED;
+        part = reinterpret_cast<float*>(workspace);
+    }
+    const int nln = (int)(K / 512);                  // lines of 128 per wave (a quarter of the slice)
     const int per_group = group / 128;               // steps that share a scale
     const int span = per_group < nln ? per_group : nln;
     Stream16Args a{(const uint16_t*)x, (const uint16_t*)smooth, wq, (const uint16_t*)scales, offsets, bias, (uint16_t*)out,
-                   (int)M, (int)N, (int)K, (int)(K / group), per_group, span, nln / span, scale_dtype == AMCT_F16 ? 1 : 0,
-                   (uint32_t)(0x100000000ull / (uint64_t)(K / 8)) + 1u};
+                   (int)M, (int)N, (int)K, (int)(K_row / group), per_group, span, nln / span, scale_dtype == AMCT_F16 ? 1 : 0,
+                   (uint32_t)(0x100000000ull / (uint64_t)(K / 8)) + 1u, (int)K_row, (int)(K_row / group), part};
     const size_t xbytes = (size_t)M * ((size_t)K * 2 + 16);
     const int cg = xbytes > 40 * 1024 ? 4 : xbytes > 12 * 1024 ? 2 : 1;
     const size_t red = (size_t)3 * cg * 64 * 16, img = xbytes + (size_t)(K / 128) * 64;

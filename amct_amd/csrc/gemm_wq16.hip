@@ -508,7 +508,8 @@ static size_t w8a16_tiles_workspace(int64_t M, int64_t N, int64_t K, int group, 
 
 int w8a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
                           const uint8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group,
-                          int dtype, hipStream_t st);      // gemm_w8a16_stream.hip
+                          int dtype, void* workspace, size_t workspace_bytes, hipStream_t st);      // gemm_w8a16_stream.hip
+size_t w8a16_stream_part_bytes(int64_t M, int64_t N, int64_t K, int group);   // partial sums of its launches over slices of K
 int w8a16_spec_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
                         const uint8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group, int dtype,
                         void* workspace, size_t workspace_bytes, hipStream_t st);   // gemm_w4a16.hip
@@ -523,7 +524,9 @@ extern "C" size_t amct_gemm_w8a16_workspace_bytes(int64_t M, int64_t N, int64_t 
     const size_t part = w8a16_spec_part_bytes(M, N, K, group);
     const size_t spec = (has_smooth && (M > 16 || part) ? (size_t)M * (size_t)K * 2 : 0) + part;
     const size_t two = w8a16_tiles_workspace(M, N, K, group, has_smooth);   // many rows: the 16-bit weight as well
-    return two > spec ? two : spec;
+    const size_t stream = w8a16_stream_part_bytes(M, N, K, group);          // a few rows, K in slices: its partial sums
+    const size_t most = two > spec ? two : spec;
+    return most > stream ? most : stream;
 }
 
 extern "C" int amct_gemm_w8a16(const void* x, const void* smooth, const int8_t* wq, const void* scales, int scale_dtype,
@@ -547,7 +550,8 @@ extern "C" int amct_gemm_w8a16_ws(const void* x, const void* smooth, const int8_
     hipStream_t st = (hipStream_t)stream;
     if (M <= 16) {                                   // K of 1024 / 2048 / 4096, groups of 128 .. K: the weight-streaming kernel
         const int rc = w8a16_stream_dispatch(x, smooth, reinterpret_cast<const uint8_t*>(wq), scales, scale_dtype,
-                                             reinterpret_cast<const uint8_t*>(offsets), bias, out, M, N, K, group, dtype, st);
+                                             reinterpret_cast<const uint8_t*>(offsets), bias, out, M, N, K, group, dtype, workspace,
+                                             workspace_bytes, st);
         if (rc != AMCT_E_UNSUPPORTED) return rc;
     }
     if (M > 16 || w8a16_spec_part_bytes(M, N, K, group)) {   // the tile kernels with specialised waves (a few rows: only with K split)

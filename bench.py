@@ -443,8 +443,8 @@ def build_cases(dev, only):
                                             outs_d8[j].data_ptr(), Md, Nd, Kd, gd, _lib.BF16, wsd8.data_ptr(), wsd8.numel(), st)
                 assert rc == 0, rc
             cases.append(Case("w8a16_down_m16", "hbm", Nd * Kd + Nd * (Kd // gd) * 2 + Md * Kd * 2 + Md * Nd * 2, "B", launch, nwd, "bf16",
-                              "int8 weight-only Linear M=16 N=4096 K=14336 group 128 (down projection, decode): specialised-wave 64x64 "
-                              "tiles, K split over 4 blocks per tile"))
+                              "int8 weight-only Linear M=16 N=4096 K=14336 group 128 (down projection, decode): weight-streaming kernel on "
+                              "7 slices of 2048 elements of K, fp32 partial sums + reduce kernel"))
 
     # ---- the same operator at M = 2048: dequantise the weight once into the lent workspace, then the 16-bit GEMM on the
     # large tiles (three launches with smoothing)

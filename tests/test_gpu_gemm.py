@@ -230,9 +230,12 @@ def w8a16_case(M, N, K, group, seed, dtype, sdt, sym):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,N,K,group", [(1, 64, 1024, 128), (16, 200, 2048, 256), (9, 72, 1024, 1024), (5, 33, 2048, 128),
                                          (16, 1000, 4096, 4096), (13, 14336, 4096, 128), (1, 14336, 4096, 4096),
-                                         (3, 16, 4096, 512), (16, 15, 1024, 512), (2, 300, 4096, 2048), (16, 520, 4096, 1024)])
+                                         (3, 16, 4096, 512), (16, 15, 1024, 512), (2, 300, 4096, 2048), (16, 520, 4096, 1024),
+                                         (16, 1000, 8192, 128), (8, 520, 14336, 14336), (6, 264, 5120, 256), (12, 200, 28672, 4096),
+                                         (1, 72, 12288, 12288), (16, 136, 8192, 8192)])
 def test_w8a16_weight_streaming_kernel(dev, dtype, M, N, K, group):
-    """The int8 weight-only kernel for a few rows (M <= 16, K of 1024/2048/4096, groups of 128, 256, ... up to K, i.e.
+    """The int8 weight-only kernel for a few rows (M <= 16, K of 1024/2048/4096 or 2 ... 14 slices of those, whose partial
+    sums a second kernel adds in slice order; groups of 128, 256, ... up to K, i.e.
     per-channel factors too): every block width, ragged N, both activation and factor dtypes, symmetric and with
     offsets, with and without smoothing and bias, against the fp64 anchor whose dequantised weight is not rounded; then
     the integer special case (scale 1, small integer activations), where the result is an integer matmul bit for bit."""
@@ -318,7 +321,8 @@ def test_w8a16_medium_rows_specialised_waves(dev, dtype, M, N, K, group):
                                  None if sm is None else sm.to(dev), None if b is None else b.to(dev)).cpu()
             assert out.dtype == dtype
             want = od.w4a16_forward_f64(x, codes.to(torch.int32), scales, None if offsets is None else -offsets.float(), group,
-                                        b, None if sm is None else sm.reshape(1, -1), round_weight=True)
+                                        b, None if sm is None else sm.reshape(1, -1),
+                                        round_weight=not od.w8a16_streams(M, K, group, dtype, N=N))
             err = (out.double() - want).abs()
             tol = 1e-3 * want.abs().amax(dim=1, keepdim=True) + want.abs() * ulp
             assert (err <= tol).all(), (float((err / tol).max()), sdt, sym, sm is not None)
