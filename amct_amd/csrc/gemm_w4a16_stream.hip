@@ -123,7 +123,11 @@ AMCT_DEV void st_load_tile(const StreamArgs& a, StTile<NL>& t, int n0, int cg, i
     // HBM access takes under the load of the whole launch's weight requests).
     const int fcol = n0 + cg * 16 + r16;
     const uint32_t slice = blockIdx.y;
-    const size_t fidx = (size_t)(fcol < a.N ? fcol : a.N - 1) * (size_t)(a.row_k / a.group) + slice * G + ks * NL;
+    // (a wave whose part of a last, shorter slice lies beyond the row reads the row's last factors and its first weights:
+    // its activations are zeros)
+    const uint32_t row_g = (uint32_t)(a.row_k / a.group);
+    const uint32_t gwave = slice * G + ks * NL;
+    const size_t fidx = (size_t)(fcol < a.N ? fcol : a.N - 1) * (size_t)row_g + (gwave + NL <= row_g ? gwave : row_g - NL);
     // the bias too: a load issued in the epilogue would queue behind the next tile's weights
     // (unconditional, from `bias_src`, which is always readable: a branch here makes the wait counts of the two paths differ
     // and the compiler then waits for everything in flight)
@@ -147,7 +151,8 @@ AMCT_DEV void st_load_tile(const StreamArgs& a, StTile<NL>& t, int n0, int cg, i
     const uint32_t oct = lane >> 3;
     const uint32_t chunk = (oct & 1) ? 4 + (oct >> 1) : (oct >> 1);
     const int rlo = n0 + cg * 16 + (lane & 7), rhi = rlo + 8;
-    const size_t wrow = (size_t)(a.row_k / 2), woff = (size_t)slice * (K / 2) + (ks * kw) / 2 + chunk * 16;
+    const uint32_t kwave = slice * K + ks * kw;      // first element of K of this wave
+    const size_t wrow = (size_t)(a.row_k / 2), woff = (size_t)(kwave < (uint32_t)a.row_k ? kwave / 2 : 0u) + chunk * 16;
     const uint8_t* wlo = a.wq + (size_t)(rlo < a.N ? rlo : a.N - 1) * wrow + woff;
     const uint8_t* whi = a.wq + (size_t)(rhi < a.N ? rhi : a.N - 1) * wrow + woff;
 #pragma unroll
@@ -266,8 +271,12 @@ __global__ __launch_bounds__(KS * CG * 64) void w4a16_stream(StreamArgs a) {
         const uint32_t vc = v < n_xv ? v : n_xv - 1;
         xrow[j] = __umulhi(vc, a.kv_magic);           // vc / KV
         xkv[j] = vc - xrow[j] * KV;
-        xv[j] = ldg16(a.x + (size_t)xrow[j] * a.row_k + blockIdx.y * K + xkv[j] * 8);
-        if constexpr (SMOOTH) cv[j] = ldg16(a.smooth + blockIdx.y * K + xkv[j] * 8);
+        // (a last slice may reach beyond the row: those elements are staged as zeros, read from the row's start)
+        const uint32_t xk = blockIdx.y * K + xkv[j] * 8;
+        const bool inside = xk < (uint32_t)a.row_k;
+        xv[j] = ldg16(a.x + (size_t)xrow[j] * a.row_k + (inside ? xk : 0u));
+        if (!inside) xv[j] = make_uint4(0u, 0u, 0u, 0u);
+        if constexpr (SMOOTH) cv[j] = ldg16(a.smooth + (inside ? xk : 0u));
     }
     // ---- the whole weight stream of this wave for its first tile -------------------------------------------------
     int tile = blockIdx.x;
@@ -356,7 +365,7 @@ static int stream_launch_x(const StreamArgs& a, size_t lds_bytes, dim3 blocks, h
 }
 
 // The slice of K one block walks: K itself when it is 1024, 2048 or 4096, else the largest of those that divides K into at
-// most 16 slices (8192 = 2 x 4096, 14336 = 7 x 2048, 5120 = 5 x 1024, 28672 = 7 x 4096); 0: none (odd multiples of 512).
+// most 16 slices (8192 = 2 x 4096, 14336 = 7 x 2048, 5120 = 5 x 1024, 28672 = 7 x 4096); 0: none.
 static int64_t stream_slice(int64_t K) {
     if (K == 1024 || K == 2048 || K == 4096) return K;
 #ifdef AMCT_ST_SLICE
@@ -364,16 +373,22 @@ static int64_t stream_slice(int64_t K) {
 #endif
     for (int64_t ks = 4096; ks >= 1024; ks /= 2)
         if (K % ks == 0 && K / ks <= 16) return ks;
+    // other multiples of 256 (11008, 13824): slices of 1024 whose last one is shorter -- a wave walks 256 elements, so it
+    // lies inside the row or beyond it as a whole
+    if (K % 256 == 0 && K > 1024 && (K + 1023) / 1024 <= 16) return 1024;
     return 0;
 }
 // Sliced rows pay a second launch: taken from 5 rows on, or for rows of 12288 elements and more (measured against the
 // older kernels for a few rows, us: W[8192,8192] M = 1 / 4 / 16: 13.2 / 14.0 / 22.3 against 16.1 / 16.0 / 16.3 sliced;
 // W[28672,8192]: 30.6 / 38.6 / 86.9 against 34.7 / 35.5 / 37.2; W[8192,28672]: 105 / 80 / 79 against 31 / 34 / 41).
-static bool stream_slices_pay(int64_t M, int64_t K) { return M >= 5 || K >= 12288; }
+// Rows whose 256-element units do not split evenly over the four waves of those older kernels (11008, 13824) come here for any M
+// (W[4096,11008], us at M = 1 / 5 / 8 / 16: 18.6 / 18.1 / 18.1 / 18.2 on the split tile kernels against 16 / 16.1 / 15.0 / 17.7;
+// W[5120,13824]: 34.5 against 18 - 24).
+static bool stream_slices_pay(int64_t M, int64_t K) { return M >= 5 || K >= 12288 || (K / 256) % 4 != 0; }
 size_t w4a16_stream_part_bytes(int64_t M, int64_t N, int64_t K, int group) {
     const int64_t ks = stream_slice(K);
     if (M < 1 || M > 16 || group != 128 || !ks || ks == K || N % 8 != 0 || !stream_slices_pay(M, K)) return 0;
-    return (size_t)(K / ks) * (size_t)M * (size_t)N * 4;
+    return (size_t)((K + ks - 1) / ks) * (size_t)M * (size_t)N * 4;
 }
 
 // Returns AMCT_E_UNSUPPORTED when the shape is not one this kernel takes (the caller then uses its other kernels).
@@ -381,7 +396,7 @@ int w4a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, 
                           const uint8_t* zeros, const float* bias, void* out, int64_t M, int64_t N, int64_t K_row, int group,
                           int dtype, void* workspace, size_t workspace_bytes, hipStream_t st) {
     // one group per step of 128 elements of K (the per-group partial sums of a step cannot be separated otherwise)
-    const int64_t K = stream_slice(K_row), S = K ? K_row / K : 0;
+    const int64_t K = stream_slice(K_row), S = K ? (K_row + K - 1) / K : 0;
     if (M < 1 || M > 16 || !K || group != 128 || N > (int64_t(1) << 30)) return AMCT_E_UNSUPPORTED;
     if (!aligned16(x) || !aligned16(wq) || (smooth && !aligned16(smooth)) || ((uintptr_t)scales & 3) || ((uintptr_t)zeros & 3))
         return AMCT_E_UNSUPPORTED;

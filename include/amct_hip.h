@@ -270,8 +270,9 @@ int amct_gemm_w8a8_ws(const int8_t* xq, const int8_t* wq, const float* s_tok, co
  * every row tile from there on (same arithmetic; a smaller workspace keeps the fused kernels).  For long rows on few
  * column blocks (the down projection of an MLP at up to a few hundred rows) the query also asks for S * M * N * 4 bytes:
  * K is then split over S blocks per tile, whose fp32 partial sums a second kernel adds in a fixed order; likewise for
- * M <= 16 (from 5 rows on, or K >= 12288) when K is 2 ... 16 slices of 4096, 2048 or 1024 elements, which the
- * weight-streaming kernel then walks one per block.  0 bytes are
+ * M <= 16 (from 5 rows on, for K >= 12288, or when K / 256 is not a multiple of 4) when K is 2 ... 16 slices of 4096, 2048
+ * or 1024 elements (the last one shorter for other multiples of 256, e.g. 11008), which the weight-streaming kernel then
+ * walks one per block.  0 bytes are
  * asked for otherwise; a null or smaller workspace is never an error.
  * Arithmetic of the dequantisation: the tile kernels (M > 16) feed dtype((u - zero) * scale) to the matrix pipe; the
  * weight-streaming kernel for M <= 16 (bf16 or fp16, K of 1024 / 2048 / 4096 or slices of those, group = 128) keeps the weight as the exact integer and applies

@@ -276,13 +276,15 @@ def w4a16_forward_f64(x, codes_nk, scale_ng, antioffset_ng, group_size, bias=Non
 
 def w4a16_streams(M, K, group_size, dtype=torch.bfloat16, N=None):
     """Whether the int4 GEMM takes its weight-streaming kernel for this shape (a few rows of bf16 or fp16 activations, K
-    of 1024, 2048 or 4096, or -- from 5 rows on or for K >= 12288, N a multiple of 8 -- at most 16 slices of one of those;
+    of 1024, 2048 or 4096, or -- from 5 rows on, for K >= 12288 or when K / 256 is not a multiple of 4; N a multiple of 8 -- at most 16 slices of one of those
+    (the last one shorter for other multiples of 256);
     groups of 128): that kernel does not round the dequantised weight."""
     if dtype not in (torch.bfloat16, torch.float16) or not 1 <= M <= 16 or group_size != 128:
         return False
     if K in (1024, 2048, 4096):
         return True
-    sliced = any(K % ks == 0 and K // ks <= 16 for ks in (4096, 2048, 1024)) and (M >= 5 or K >= 12288)
+    sliced = any(K % ks == 0 and K // ks <= 16 for ks in (4096, 2048, 1024)) or (K % 256 == 0 and 1024 < K <= 16384)
+    sliced = sliced and (M >= 5 or K >= 12288 or (K // 256) % 4 != 0)
     return sliced and (N is None or N % 8 == 0)
 
 

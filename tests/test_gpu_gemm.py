@@ -182,14 +182,14 @@ def test_w4a16_vs_oracle(dev, M, N, K, group, sdt):
                                    (13, 14336, 4096), (1, 14336, 2048), (3, 16, 4096), (16, 15, 1024),
                                    (16, 40000, 1024), (16, 20008, 4096), (1, 70000, 1024), (4, 33000, 2048), (2, 16392, 4096),
                                    (16, 1000, 8192), (8, 520, 14336), (6, 264, 5120), (16, 20008, 8192), (12, 200, 28672),
-                                   (1, 72, 12288)])
+                                   (1, 72, 12288), (16, 520, 11008), (8, 264, 13824), (5, 200, 2816), (1, 72, 13824), (2, 136, 11008)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_w4a16_weight_streaming_kernel(dev, M, N, K, dtype):
     """The kernel for a few rows (M <= 16, K of 1024/2048/4096, groups of 128): every block width, ragged N, both factor
     dtypes, with and without smoothing, against the fp64 anchor whose dequantised weight is not rounded (the last
     shapes: more column tiles than the device runs blocks at once, so that a block walks several tiles -- one, two, three
     or more, with a ragged last one -- on one staged copy of the activations; rows of 2 ... 14 slices of 1024, 2048 or 4096
-    elements, whose partial sums a second kernel adds in slice order); then the
+    elements, whose partial sums a second kernel adds in slice order, the last slice shorter for K = 11008, 13824, 2816); then the
     integer special case (scale 1, small integer activations), where both readings of the dequantisation give the same
     bits as an integer matmul."""
     assert od.w4a16_streams(M, K, 128, dtype)
