@@ -57,6 +57,8 @@ SIGNATURES = {
     "amct_gemm_w8a8": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _L, _L, _L, _I, _P]),
     "amct_gemm_w8a8_workspace_bytes": (ctypes.c_size_t, [_L, _L, _L]),
     "amct_gemm_w8a8_ws": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _L, _L, _L, _I, _P, ctypes.c_size_t, _P]),
+    "amct_linear_w8a8_workspace_bytes": (ctypes.c_size_t, [_L, _L, _L]),
+    "amct_linear_w8a8": (_I, [_P, _I, _P, _P, _P, _L, _I, _P, _P, _P, _P, _I, _P, _L, _L, _L, _I, _P, ctypes.c_size_t, _P]),
     "amct_gemm_w8a16": (_I, [_P, _P, _P, _P, _I, _P, _P, _P, _L, _L, _L, _I, _I, _P]),
     "amct_gemm_w8a16_workspace_bytes": (ctypes.c_size_t, [_L, _L, _L, _I, _I]),
     "amct_gemm_w8a16_ws": (_I, [_P, _P, _P, _P, _I, _P, _P, _P, _L, _L, _L, _I, _I, _P, ctypes.c_size_t, _P]),

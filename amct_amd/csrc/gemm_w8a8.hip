@@ -1285,6 +1285,42 @@ extern "C" size_t amct_gemm_w8a8_workspace_bytes(int64_t M, int64_t N, int64_t K
     return S > 1 ? (size_t)S * (size_t)M * (size_t)N * 4 : 0;
 }
 
+namespace amct {
+int w8a8_stream_quant_dispatch(const void* x, int x_dtype, const void* smooth, const void* act_scale, const void* act_zp,
+                               int per_token, const int8_t* wq, const float* s_tok, const float* s_ch, const void* bias,
+                               int bias_kind, void* out, int64_t M, int64_t N, int64_t K, int out_dtype, hipStream_t st);   // gemm_w8a8_stream.hip
+}
+
+// the int8 activations of the two-kernel form (rounded up to 16 bytes), then what the GEMM asks for
+extern "C" size_t amct_linear_w8a8_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    return (((size_t)M * (size_t)K + 15) & ~(size_t)15) + amct_gemm_w8a8_workspace_bytes(M, N, K);
+}
+
+extern "C" int amct_linear_w8a8(const void* x, int x_dtype, const void* smooth, const void* act_scale, const void* act_offset,
+                                int64_t n_scales, int per_token, const int8_t* wq, const float* s_tok, const float* s_ch,
+                                const void* bias, int bias_kind, void* out, int64_t M, int64_t N, int64_t K, int out_dtype,
+                                void* workspace, size_t workspace_bytes, amct_stream_t stream) {
+    if (M < 0 || N <= 0 || K <= 0 || bias_kind < 0 || bias_kind > 2) return AMCT_E_BADARG;
+    if (x_dtype != AMCT_F32 && x_dtype != AMCT_F16 && x_dtype != AMCT_BF16) return AMCT_E_BADARG;
+    if (out_dtype != AMCT_F32 && out_dtype != AMCT_F16 && out_dtype != AMCT_BF16) return AMCT_E_BADARG;
+    if (per_token ? (n_scales != M) : (n_scales != 1 && n_scales != K)) return AMCT_E_BADARG;
+    if (M == 0) return AMCT_OK;
+    if (!x || !act_scale || !wq || !s_ch || !out || (bias_kind != 0 && !bias)) return AMCT_E_BADARG;
+    if (per_token || n_scales == 1) {
+        const int rc = w8a8_stream_quant_dispatch(x, x_dtype, smooth, act_scale, act_offset, per_token, wq, s_tok, s_ch, bias,
+                                                  bias_kind, out, M, N, K, out_dtype, (hipStream_t)stream);
+        if (rc != AMCT_E_UNSUPPORTED) return rc;
+    }
+    const size_t xq_bytes = ((size_t)M * (size_t)K + 15) & ~(size_t)15;
+    if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 15u) != 0 || workspace_bytes < xq_bytes) return AMCT_E_BADARG;
+    int8_t* xq = reinterpret_cast<int8_t*>(workspace);
+    const int rc = amct_quantize(x, smooth, act_scale, act_offset, xq, M, K, n_scales, per_token, x_dtype, stream);
+    if (rc != AMCT_OK) return rc;
+    return amct_gemm_w8a8_ws(xq, wq, s_tok, s_ch, bias, bias_kind, out, nullptr, M, N, K, out_dtype,
+                             reinterpret_cast<char*>(workspace) + xq_bytes, workspace_bytes - xq_bytes, stream);
+}
+
 extern "C" int amct_gemm_w8a8(const int8_t* xq, const int8_t* wq, const float* s_tok, const float* s_ch,
                               const void* bias, int bias_kind, void* out, int32_t* acc_out, int64_t M, int64_t N,
                               int64_t K, int out_dtype, amct_stream_t stream) {

@@ -83,16 +83,24 @@ class HipQuantizationLinear(torch.nn.Module):
             out = ops.gemm_w8a8(xq.reshape(-1, x.shape[-1]), self.quantized_weight.t(), s_ch, s_tok,
                                 self._float_bias(), self.output_dtype)
             return out.reshape(*lead, -1)
-        xq = ops.quantize_static(x, self.act_scale, self.act_offset, self.act_granularity == 'PER_TOKEN', smooth)
-        s_tok = self.pertoken_scale
-        m = xq.numel() // xq.shape[-1]
+        per_token = self.act_granularity == 'PER_TOKEN'
+        x2 = x.reshape(-1, x.shape[-1])
+        m = x2.shape[0]
+        act_scale, act_offset, s_tok = self.act_scale, self.act_offset, self.pertoken_scale
+        if per_token and act_scale.numel() != m:
+            # one scale per token of the last-but-one dim, shared by every leading batch index
+            if act_scale.numel() != x.shape[-2]:
+                raise RuntimeError("per-token quantize needs one scale per token ({} vs {})".format(
+                    act_scale.numel(), x.shape[-2]))
+            act_scale, act_offset = act_scale.repeat(m // act_scale.numel()), act_offset.repeat(m // act_offset.numel())
         if s_tok is not None and s_tok.numel() != m:
             if s_tok.numel() != x.shape[-2]:
                 raise RuntimeError("per-token scales were calibrated for {} tokens, the input has {}".format(
                     s_tok.numel(), x.shape[-2]))
             s_tok = s_tok.repeat(m // s_tok.numel())
-        out = ops.gemm_w8a8(xq.reshape(-1, x.shape[-1]), self.quantized_weight.t(), self.deq_scale, s_tok,
-                            self.bias, self.output_dtype)
+        # npu_quantize and npu_quant_matmul (npu_quantization_linear.py:98-102) in one library call
+        out = ops.linear_w8a8(x2, act_scale, act_offset, per_token, self.quantized_weight.t(), self.deq_scale, s_tok,
+                              self.bias, self.output_dtype, smooth)
         return out.reshape(*lead, -1)
 
     def _scale_w(self):

@@ -487,6 +487,56 @@ def gemm_w8a8(xq, wq_nk, s_ch, s_tok=None, bias=None, out_dtype=torch.bfloat16, 
     return (out, acc) if want_acc else out
 
 
+def linear_w8a8(x, act_scale, act_offset, per_token, wq_nk, s_ch, s_tok=None, bias=None, out_dtype=torch.bfloat16,
+                smooth=None):
+    """quantize_static followed by gemm_w8a8 in one library call (the forward of the W8A8 deploy module): x [M,K]
+    fp32|fp16|bf16; act_scale / act_offset one per tensor or (per_token) one per row, in x's dtype; the other operands as
+    for gemm_w8a8.  Up to 16 rows the activations are quantised inside the weight-streaming kernel."""
+    _need(x.dim() == 2 and wq_nk.dim() == 2 and wq_nk.dtype == torch.int8, "W8A8 Linear expects x [M,K] and an int8 weight [N,K]")
+    M, K = x.shape
+    N = wq_nk.shape[0]
+    _need(wq_nk.shape[1] == K, "W8A8 Linear: K mismatch ({} vs {})", K, wq_nk.shape[1])
+    _need(s_ch.numel() in (1, N), "W8A8 Linear: {} channel scales for {} output channels", s_ch.numel(), N)
+    _need(s_tok is None or s_tok.numel() == M, "W8A8 Linear: {} token scales for {} rows",
+          0 if s_tok is None else s_tok.numel(), M)
+    _need(bias is None or bias.numel() == N, "W8A8 Linear: bias has {} entries, {} output channels",
+          0 if bias is None else bias.numel(), N)
+    n_scales = act_scale.numel()
+    _need(n_scales == M if per_token else n_scales in (1, K), "W8A8 Linear: {} activation scales for x of shape {}",
+          n_scales, tuple(x.shape))
+    _need(act_offset is None or act_offset.numel() == n_scales, "W8A8 Linear: activation offsets do not match the scales")
+    _need(smooth is None or smooth.numel() == K, "W8A8 Linear: smooth factor must have K elements")
+    dev = _dev(x, act_scale, act_offset, wq_nk, s_ch, s_tok, bias, smooth)
+    x, wq_nk = _c(x), _c(wq_nk)
+    act_scale = _c(act_scale.reshape(-1).to(x.dtype))
+    if act_offset is not None:
+        act_offset = _c(act_offset.reshape(-1).to(x.dtype))
+    if smooth is not None:
+        smooth = _c(smooth.reshape(-1).to(x.dtype))
+    s_ch = _c(s_ch.reshape(-1).to(torch.float32))
+    if s_ch.numel() == 1:
+        s_ch = s_ch.expand(N).contiguous()
+    if s_tok is not None:
+        s_tok = _c(s_tok.reshape(-1).to(torch.float32))
+    kind = 0
+    if bias is not None:
+        if bias.dtype == torch.int32:
+            kind, bias = 1, _c(bias)
+        else:
+            kind, bias = 2, _c(bias.to(torch.float32))
+    out = torch.empty(M, N, dtype=out_dtype, device=dev)
+    lib = _lib.load()
+    fused = M <= 16 and K in (1024, 2048, 4096) and x.dtype != torch.float32 and (per_token or n_scales == 1)
+    ws = None
+    if not fused:                                    # the int8 activations (and the GEMM's partial sums) go through a workspace
+        ws = torch.empty(max(16, lib.amct_linear_w8a8_workspace_bytes(M, N, K)), dtype=torch.uint8, device=dev)
+    with _on(dev):
+        _lib.check(lib.amct_linear_w8a8(_p(x), dtype_code(x.dtype), _p(smooth), _p(act_scale), _p(act_offset), n_scales,
+                                        int(bool(per_token)), _p(wq_nk), _p(s_tok), _p(s_ch), _p(bias), kind, _p(out), M, N, K,
+                                        dtype_code(out_dtype), _p(ws), 0 if ws is None else ws.numel(), _stream(dev)))
+    return out
+
+
 def _check_weight_only(x, N, K, scales, zeros, group, smooth, bias, zeros_dtype, what):
     _need(x.dim() == 2 and x.shape[1] == K, "{}: activations must be [M, {}], got {}", what, K, tuple(x.shape))
     _need(x.dtype in (torch.bfloat16, torch.float16), "Not support tensor dtype {}, support dtypes {}.", x.dtype,

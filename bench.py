@@ -41,10 +41,10 @@ MEASURED_TRAFFIC = {
     "act_quant_per_token": ("act_quant_token<2, 2>", 25292715),
     "col_minmax": ("col_partial_k<2, false> + col_final_k", 69345307),
     "w8a8_m2048": ("w8a8_tile_mix16<2, 0>", 255069388),
-    "w8a8_m16": ("w8a8_stream<2, 4, 4, 16, 4>", 59796000),
+    "w8a8_m16": ("w8a8_stream<2, 4, 4, 16, 4, 0>", 59796000),
     "w4a16_m2048": ("w4_dequant_rows<false> + smooth_rows + w8a8_tile_mix16<2, 1>", 632207001),
-    "w4a16_m16": ("w4a16_stream<2, 4, 4, 8, 8, true>", 32474218),
-    "w4a16_m1": ("w4a16_stream<2, 4, 1, 8, 2, true>", 31011237),
+    "w4a16_m16": ("w4a16_stream<2, 4, 4, 8, 8, true, false>", 32474218),
+    "w4a16_m1": ("w4a16_stream<2, 4, 1, 8, 2, true, false>", 31011237),
 }
 
 
@@ -298,7 +298,7 @@ def build_cases(dev, only):
 
     # ---- K6: W8A8 Linear, W[14336,4096] int8 ----------------------------------------------------------
     chain = {"w8a8_dynamic_m2048": 2048, "w8a8_dynamic_m16": 16}
-    if want("w8a8_m2048") or want("w8a8_m16") or any(want(n) for n in chain):
+    if want("w8a8_m2048") or want("w8a8_m16") or want("w8a8_linear_m16") or any(want(n) for n in chain):
         x6, wq6, sw6 = workloads.c4_w8a8()
         N6, K6 = wq6.shape
         nw = 6                                           # 6 x 58.7 MB of weights rotate through HBM
@@ -321,6 +321,24 @@ def build_cases(dev, only):
             else:
                 cases.append(Case(name, "hbm", N6 * K6 + M6 * K6 + M6 * N6 * 2 + N6 * 4 + M6 * 4, "B", launch, nw, "int8",
                                   "W8A8 Linear M=%d (decode): weight streaming (config 4)" % M6))
+
+        # the deploy module's forward for 16 rows in one call: the static per-tensor quantisation of the bf16 activations
+        # (npu_quantize) done inside the weight-streaming kernel while it stages them, then the Linear
+        if want("w8a8_linear_m16"):
+            ML = 16
+            xl = x6[:ML].to(dev)
+            asc = torch.full((1,), 24.0, dtype=torch.bfloat16, device=dev)
+            azp = torch.zeros(1, dtype=torch.bfloat16, device=dev)
+            outs_l = [torch.empty(ML, N6, dtype=torch.bfloat16, device=dev) for _ in range(nw)]
+
+            def launch(i, xl=xl, asc=asc, azp=azp, outs_l=outs_l, ML=ML, wqs=wqs, swd=swd, N6=N6, K6=K6):
+                j = i % len(wqs)
+                rc = lib.amct_linear_w8a8(xl.data_ptr(), _lib.BF16, None, asc.data_ptr(), azp.data_ptr(), 1, 0, wqs[j].data_ptr(), None,
+                                          swd.data_ptr(), None, 0, outs_l[j].data_ptr(), ML, N6, K6, _lib.BF16, None, 0, st)
+                assert rc == 0, rc
+            cases.append(Case("w8a8_linear_m16", "hbm", N6 * K6 + ML * K6 * 2 + ML * N6 * 2 + N6 * 4, "B", launch, nw, "int8",
+                              "static activation quantisation + W8A8 Linear M=16 in one launch (decode, config 4): bf16 x "
+                              "quantised while the weight-streaming kernel stages it"))
 
         # config 4 as the deployed module runs it with dynamic activation quantisation: K3 (per-token scales and codes
         # of the bf16 activations) and K6 back to back on one stream, two launches per step.  (Quantising inside the

@@ -255,6 +255,21 @@ int amct_gemm_w8a8_ws(const int8_t* xq, const int8_t* wq, const float* s_tok, co
                       int64_t M, int64_t N, int64_t K, int out_dtype, void* workspace, size_t workspace_bytes,
                       amct_stream_t stream);
 
+/* The deploy module's forward in one call: the static quantisation of the activations followed by the W8A8 Linear
+ * (amct_pytorch/deploy_op/npu_quantization_linear.py:96-102: x * scale_factor, torch_npu.npu_quantize,
+ * torch_npu.npu_quant_matmul).  x [M, K] of x_dtype; smooth, act_scale, act_offset as for amct_quantize (n_scales,
+ * per_token likewise); the other operands as for amct_gemm_w8a8.  The result is that of amct_quantize followed by
+ * amct_gemm_w8a8 bit for bit.  For M <= 16, K of 1024 / 2048 / 4096, bf16 or fp16 x and one scale per tensor or per
+ * row, the activations are quantised inside the weight-streaming kernel while it stages them (one launch, no int8
+ * copy of x in memory); otherwise the two kernels run one after the other and the int8 activations go through the
+ * workspace: amct_linear_w8a8_workspace_bytes(M, N, K) bytes, 16-byte aligned, contents irrelevant before and after
+ * (AMCT_E_BADARG when such a call comes without it). */
+size_t amct_linear_w8a8_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int amct_linear_w8a8(const void* x, int x_dtype, const void* smooth, const void* act_scale, const void* act_offset,
+                     int64_t n_scales, int per_token, const int8_t* wq, const float* s_tok, const float* s_ch,
+                     const void* bias, int bias_kind, void* out, int64_t M, int64_t N, int64_t K, int out_dtype,
+                     void* workspace, size_t workspace_bytes, amct_stream_t stream);
+
 /* ---- K7: W4A16 Linear -------------------------------------------------------------------------------------
  * Replaces torch_npu.npu_weight_quant_batchmatmul as called at
  * amct_pytorch/deploy_op/weight_npu_quant_module.py:116-117 (with the x * scale_factor of :113-114

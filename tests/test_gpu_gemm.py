@@ -110,6 +110,37 @@ def test_w8a8_weight_streaming_kernel(dev, M, N, K):
             assert_bits_equal(out, od.quant_matmul(xq, wq.t(), s_ch, s_tok, b, odt), "out %s" % odt)
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 64, 1024), (16, 200, 2048), (9, 72, 4096), (16, 14336, 4096), (5, 33, 2048), (3, 4104, 4096),
+                                   (16, 1000, 1024), (40, 200, 1024), (7, 136, 8192), (300, 520, 4096)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_linear_w8a8_one_call(dev, M, N, K, dtype):
+    """Static activation quantisation + W8A8 Linear in one library call (the deploy module's forward): up to 16 rows and K
+    of 1024/2048/4096 the activations are quantised inside the weight-streaming kernel, otherwise the two kernels run through
+    the workspace (the last shapes).  Per-tensor and per-token scales, with and without offsets and smoothing, both bias
+    kinds, every output dtype: the bits of npu_quantize followed by npu_quant_matmul (the oracle), and of the two separate
+    library calls."""
+    from oracle import int_quant as iq
+    g = torch.Generator().manual_seed(300 + M)
+    x = (torch.randn(M, K, generator=g) * 3).to(dtype)
+    smooth = (0.5 + torch.rand(K, generator=g)).to(dtype)
+    for per_token, zp, sm, bias_kind, odt in ((False, False, False, 'int', torch.bfloat16), (True, True, True, 'float', torch.float16),
+                                              (True, False, False, None, torch.float32), (False, True, True, 'float', torch.bfloat16)):
+        _, wq, s_ch, s_tok, b = w8a8_case(M, N, K, 310 + M, per_token, bias_kind)
+        ns = M if per_token else 1
+        act_scale = (20 + 20 * torch.rand(ns, generator=g)).to(dtype)
+        act_off = torch.randint(-20, 21, (ns,), generator=g).to(dtype) if zp else None
+        dv = lambda t: None if t is None else t.to(dev)
+        out = ops.linear_w8a8(x.to(dev), act_scale.to(dev), dv(act_off), per_token, wq.to(dev), s_ch.to(dev), dv(s_tok), dv(b), odt,
+                              smooth.to(dev) if sm else None)
+        xq = ops.quantize_static(x.to(dev), act_scale.to(dev), dv(act_off), per_token, smooth.to(dev) if sm else None)
+        two = ops.gemm_w8a8(xq, wq.to(dev), s_ch.to(dev), dv(s_tok), dv(b), odt)
+        assert_bits_equal(out, two.cpu(), "one call against two")
+        xs = (x * smooth).to(dtype) if sm else x
+        xq_o = iq.static_quantize(xs, act_scale, act_off if zp else torch.zeros(ns, dtype=dtype), axis=-2 if per_token else -1)
+        assert torch.equal(xq.cpu(), xq_o), "codes"
+        assert_bits_equal(out, od.quant_matmul(xq_o, wq.t(), s_ch, s_tok, b, odt), "against the oracle")
+
+
 def w4a16_case(M, N, K, group, seed, sdt=torch.float16):
     g = torch.Generator().manual_seed(seed)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)
