@@ -41,10 +41,13 @@ MEASURED_TRAFFIC = {
     "act_quant_per_token": ("act_quant_token<2, 2>", 25292715),
     "col_minmax": ("col_partial_k<2, false> + col_final_k", 69345307),
     "w8a8_m2048": ("w8a8_tile_mix16<2, 0>", 255069388),
-    "w8a8_m16": ("w8a8_stream<2, 4, 4, 16, 4, 0>", 59796000),
+    "w8a8_m16": ("w8a8_stream<2, 4, 4, 16, 4, 0>", 59805700),
+    "w8a8_linear_m16": ("w8a8_stream<2, 4, 4, 16, 8, 2>", 60417600),
     "w4a16_m2048": ("w4_dequant_rows<false> + smooth_rows + w8a8_tile_mix16<2, 1>", 632207001),
-    "w4a16_m16": ("w4a16_stream<2, 4, 4, 8, 8, true, false>", 32474218),
-    "w4a16_m1": ("w4a16_stream<2, 4, 1, 8, 2, true, false>", 31011237),
+    "w4a16_m16": ("w4a16_stream<2, 4, 4, 8, 8, true, false>", 32535100),
+    "w4a16_m1": ("w4a16_stream<2, 4, 1, 8, 2, true, false>", 31110041),
+    "w4a16_down_m16": ("w4a16_stream<2, 4, 4, 4, 4, false, true> + splitk_reduce16<false>", 39848448),
+    "w8a16_down_m16": ("w8a16_stream<2, 4, 4, 4, 1, false> + splitk_reduce16<false>", 67237581),
 }
 
 
