@@ -213,7 +213,7 @@ def test_w4a16_vs_oracle(dev, M, N, K, group, sdt):
                                    (13, 14336, 4096), (1, 14336, 2048), (3, 16, 4096), (16, 15, 1024),
                                    (16, 40000, 1024), (16, 20008, 4096), (1, 70000, 1024), (4, 33000, 2048), (2, 16392, 4096),
                                    (16, 1000, 8192), (8, 520, 14336), (6, 264, 5120), (16, 20008, 8192), (12, 200, 28672),
-                                   (1, 72, 12288), (16, 520, 11008), (8, 264, 13824), (5, 200, 2816), (1, 72, 13824), (2, 136, 11008)])
+                                   (1, 72, 12288), (16, 520, 11008), (8, 264, 13824), (5, 200, 2816), (1, 72, 13824), (2, 136, 11008), (16, 4104, 11008)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_w4a16_weight_streaming_kernel(dev, M, N, K, dtype):
     """The kernel for a few rows (M <= 16, K of 1024/2048/4096, groups of 128): every block width, ragged N, both factor
