@@ -128,9 +128,13 @@ __global__ __launch_bounds__(4 * CG * 64) void w8a16_stream(Stream16Args a) {
         const uint32_t vc = v < n_xv ? v : n_xv - 1;
         xrow[j] = __umulhi(vc, a.kv_magic);           // vc / KV
         xkv[j] = vc - xrow[j] * KV;
-        xv[j] = ldg16(a.x + (size_t)xrow[j] * a.row_k + blockIdx.y * K + xkv[j] * 8);
+        // (a last slice may reach beyond the row: those elements are staged as zeros, read from the row's start)
+        const uint32_t xk = blockIdx.y * K + xkv[j] * 8;
+        const bool inside = xk < (uint32_t)a.row_k;
+        xv[j] = ldg16(a.x + (size_t)xrow[j] * a.row_k + (inside ? xk : 0u));
+        if (!inside) xv[j] = make_uint4(0u, 0u, 0u, 0u);
         if constexpr (SMOOTH) {
-            if (j < CVN) cv[j] = ldg16(a.smooth + blockIdx.y * K + xkv[j] * 8);
+            if (j < CVN) cv[j] = ldg16(a.smooth + (inside ? xk : 0u));
         }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -140,7 +144,9 @@ __global__ __launch_bounds__(4 * CG * 64) void w8a16_stream(Stream16Args a) {
     const uint32_t oct = lane >> 3;
     const uint32_t chunk = (oct & 1) ? 4 + (oct >> 1) : (oct >> 1);
     const int rlo = n0 + cg * 16 + (lane & 7), rhi = rlo + 8;
-    const size_t woff = (size_t)blockIdx.y * K + ks * kw + chunk * 16;
+    // (a wave whose part of a last, shorter slice lies beyond the row reads the row's first weights: its activations are zeros)
+    const uint32_t kwave = blockIdx.y * K + ks * kw;
+    const size_t woff = (size_t)(kwave < (uint32_t)a.row_k ? kwave : 0u) + chunk * 16;
     const uint8_t* wlo = a.wq + (size_t)(rlo < a.N ? rlo : a.N - 1) * (size_t)a.row_k + woff;
     const uint8_t* whi = a.wq + (size_t)(rhi < a.N ? rhi : a.N - 1) * (size_t)a.row_k + woff;
     // Blocks of 16 waves have 128 registers per lane: the activation vectors in flight (32) and all of the weights
@@ -279,7 +285,7 @@ static int stream16_launch_x(const Stream16Args& a, size_t lds_bytes, hipStream_
     constexpr int NT = 4 * CG * 64;
     const int n_xv = a.M * (a.K / 8);
     const int xj = (n_xv + NT - 1) / NT;
-    const dim3 grid((unsigned)((a.N + CG * 16 - 1) / (CG * 16)), (unsigned)(a.row_k / a.K));
+    const dim3 grid((unsigned)((a.N + CG * 16 - 1) / (CG * 16)), (unsigned)((a.row_k + a.K - 1) / a.K));
 #define AMCT_STREAM16_GO(XJ, CVN_)                                                                                    \
     {                                                                                                               \
         auto kern = &w8a16_stream<DT, CG, NLN, XJ, CVN_, SMOOTH>;                                                         \
@@ -330,13 +336,16 @@ static int64_t stream16_slice(int64_t K) {
     if (K == 1024 || K == 2048 || K == 4096) return K;
     for (int64_t ks = 4096; ks >= 1024; ks /= 2)
         if (K % ks == 0 && K / ks <= 16) return ks;
+    // other multiples of 256 (11008, 13824): slices of 1024 whose last one is shorter -- a wave walks 256 elements, so it
+    // lies inside the row or beyond it as a whole
+    if (K % 256 == 0 && K > 1024 && (K + 1023) / 1024 <= 16) return 1024;
     return 0;
 }
-// groups the kernel takes for slices of `ks`: 128, 256, ... up to the slice, or whole slices (per-channel factors: the row)
+// groups the kernel takes for slices of `ks`: 128, 256, ... up to the slice, whole slices, or the whole row (per-channel factors)
 static bool stream16_group_ok(int64_t K_row, int64_t ks, int group) {
     if (group < 128 || K_row % group != 0) return false;
     if (group <= ks) return (group & (group - 1)) == 0;
-    return group % ks == 0;
+    return group % ks == 0 || group == K_row;
 }
 // Sliced rows pay a second launch and stage the activations once per block: taken for long rows (K >= 12288), for four
 // and more slices (slices of 1024), or while blocks of 64 columns per slice run in one round.  Measured against the
@@ -345,20 +354,20 @@ static bool stream16_group_ok(int64_t K_row, int64_t ks, int group) {
 // W[13824,5120] 24 / 26 / 28 -> 19 / 20 / 25; not taken: W[28672,8192] 53 / 56 / 65 (sliced: 56 / 83 / 73),
 // W[10240,8192] 27 / 29 / 33 (sliced: 25 / 35 / 38).
 static bool stream16_slices_pay(int64_t N, int64_t K, int64_t ks) {
-    const int64_t S = K / ks, cus = current_cu_count();
+    const int64_t S = (K + ks - 1) / ks, cus = current_cu_count();
     return K >= 12288 || S >= 4 || ((N + 63) / 64) * S <= cus;
 }
 size_t w8a16_stream_part_bytes(int64_t M, int64_t N, int64_t K, int group) {
     const int64_t ks = stream16_slice(K);
     if (M < 1 || M > 16 || !ks || ks == K || N % 8 != 0 || !stream16_group_ok(K, ks, group) || !stream16_slices_pay(N, K, ks)) return 0;
-    return (size_t)(K / ks) * (size_t)M * (size_t)N * 4;
+    return (size_t)((K + ks - 1) / ks) * (size_t)M * (size_t)N * 4;
 }
 
 // Returns AMCT_E_UNSUPPORTED when the shape is not one this kernel takes (the caller then uses its other kernels).
 int w8a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
                           const uint8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K_row, int group,
                           int dtype, void* workspace, size_t workspace_bytes, hipStream_t st) {
-    const int64_t K = stream16_slice(K_row), S = K ? K_row / K : 0;
+    const int64_t K = stream16_slice(K_row), S = K ? (K_row + K - 1) / K : 0;
     if (M < 1 || M > 16 || !K || N > (int64_t(1) << 30)) return AMCT_E_UNSUPPORTED;
     if (!stream16_group_ok(K_row, K, group)) return AMCT_E_UNSUPPORTED;
     if (!aligned16(x) || !aligned16(wq) || (smooth && !aligned16(smooth)) || ((uintptr_t)scales & 1)) return AMCT_E_UNSUPPORTED;

@@ -309,8 +309,8 @@ int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t* wq, const 
  * out [M, N] of dtype = x' @ dtype((q - offset) * scale)^T + bias, fp32 accumulate.
  * As for the int4 weight there are two readings of the dequantisation: the tile kernels feed dtype((q - offset) * scale)
  * to the matrix pipe; the weight-streaming kernel for M <= 16 (K of 1024 / 2048 / 4096, group a power of two from 128 to K; through
- * amct_gemm_w8a16_ws and its workspace also rows of 2 ... 16 such slices -- K = 8192, 14336, 28672, 5120 ... --, groups up to a
- * slice or whole slices, where that beats the other kernels) keeps the weight as the exact integer and applies scale and offset per group in fp32, i.e. the dequantised weight is
+ * amct_gemm_w8a16_ws and its workspace also rows of 2 ... 16 such slices, the last one shorter if need be -- K = 8192, 11008, 14336, 28672, 5120 ... --,
+ * groups up to a slice, whole slices or the whole row, where that beats the other kernels) keeps the weight as the exact integer and applies scale and offset per group in fp32, i.e. the dequantised weight is
  * not rounded to 16 bits there.  Both stay within 1e-3 of the exact result. */
 int amct_gemm_w8a16(const void* x, const void* smooth, const int8_t* wq, const void* scales, int scale_dtype,
                     const int8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K,

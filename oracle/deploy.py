@@ -296,14 +296,17 @@ def w8a16_streams(M, K, group_size, dtype=torch.bfloat16, N=None, cus=256):
     if dtype not in (torch.bfloat16, torch.float16) or not 1 <= M <= 16 or group_size < 128 or K % group_size:
         return False
     ks = K if K in (1024, 2048, 4096) else next((c for c in (4096, 2048, 1024) if K % c == 0 and K // c <= 16), 0)
+    if not ks and K % 256 == 0 and 1024 < K <= 16384:
+        ks = 1024                                   # the last slice shorter (11008, 13824)
     if not ks:
         return False
     if ks != K:
+        slices = -(-K // ks)
         if N is None or N % 8:
             return False
-        if not (K >= 12288 or K // ks >= 4 or -(-N // 64) * (K // ks) <= cus):
+        if not (K >= 12288 or slices >= 4 or -(-N // 64) * slices <= cus):
             return False
-    return group_size & (group_size - 1) == 0 if group_size <= ks else group_size % ks == 0
+    return group_size & (group_size - 1) == 0 if group_size <= ks else (group_size % ks == 0 or group_size == K)
 
 
 # --------------------------------------------------------------------------

@@ -263,7 +263,8 @@ def w8a16_case(M, N, K, group, seed, dtype, sdt, sym):
                                          (16, 1000, 4096, 4096), (13, 14336, 4096, 128), (1, 14336, 4096, 4096),
                                          (3, 16, 4096, 512), (16, 15, 1024, 512), (2, 300, 4096, 2048), (16, 520, 4096, 1024),
                                          (16, 1000, 8192, 128), (8, 520, 14336, 14336), (6, 264, 5120, 256), (12, 200, 28672, 4096),
-                                         (1, 72, 12288, 12288), (16, 136, 8192, 8192)])
+                                         (1, 72, 12288, 12288), (16, 136, 8192, 8192), (16, 520, 11008, 11008), (3, 264, 13824, 128),
+                                         (9, 200, 2816, 256)])
 def test_w8a16_weight_streaming_kernel(dev, dtype, M, N, K, group):
     """The int8 weight-only kernel for a few rows (M <= 16, K of 1024/2048/4096 or 2 ... 14 slices of those, whose partial
     sums a second kernel adds in slice order; groups of 128, 256, ... up to K, i.e.
