@@ -4,8 +4,9 @@ npu_convert_weight_to_int4pack -- call sites amct_pytorch/deploy_op/npu_quantiza
 and amct_pytorch/deploy_op/weight_npu_quant_module.py:54-57,116-117).  Same keyword names and operand
 layouts as those calls; each runs HIP kernels only.
 
-The weight operands arrive here in the reference's [K, N] layouts and are re-laid out for the kernels
-on every call; the deploy modules in amct_amd.deploy_op do that once at construction instead.
+The weight operands arrive here in the reference's [K, N] layouts; their kernel layouts are computed on the
+first call and cached per tensor and version (the deploy modules in amct_amd.deploy_op convert once at
+construction instead).
 """
 import torch
 
