@@ -138,9 +138,25 @@ __global__ __launch_bounds__(4 * CG * 64) void w8a16_stream(Stream16Args a) {
         }
     }
     __builtin_amdgcn_sched_barrier(0);
+    // the factors of this lane's column for the spans of this wave (at most NLN), needed when the first span ends:
+    // requested BEFORE the weights (a load issued behind the weight stream returns behind it) and kept as raw bits until
+    // the fold that uses them, so that nothing waits for them here
+    const int ncol = n0 + cg * 16 + r16;
+    const int nc = ncol < a.N ? ncol : a.N - 1;
+    const uint32_t g_first = (blockIdx.y * (K / 128) + (uint32_t)ks * NLN) / (uint32_t)a.per_group;   // the group of the wave's first span
+    const uint32_t RG = (uint32_t)a.row_g;
+    uint32_t fs_raw[NLN];
+    int fz_raw[NLN];
+#pragma unroll
+    for (int q = 0; q < NLN; ++q) {
+        const uint32_t gi = q < a.spans ? g_first + q : g_first;
+        const uint32_t gidx = gi < RG ? gi : RG - 1;
+        fs_raw[q] = a.scales[(size_t)nc * RG + gidx];
+        fz_raw[q] = a.offsets ? (int)reinterpret_cast<const int8_t*>(a.offsets)[(size_t)nc * RG + gidx] : 0;
+    }
+    __builtin_amdgcn_sched_barrier(0);
     // ---- the whole weight stream of this wave: NLN lines of 16 rows, two load instructions (rows 0 .. 7, 8 .. 15) each
     constexpr uint32_t kw = NLN * 128;               // elements (= bytes) of K of this wave
-    const int ncol = n0 + cg * 16 + r16;
     const uint32_t oct = lane >> 3;
     const uint32_t chunk = (oct & 1) ? 4 + (oct >> 1) : (oct >> 1);
     const int rlo = n0 + cg * 16 + (lane & 7), rhi = rlo + 8;
@@ -160,22 +176,6 @@ __global__ __launch_bounds__(4 * CG * 64) void w8a16_stream(Stream16Args a) {
         wv[2 * i + 1] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(whi + i * 128));
     }
     __builtin_amdgcn_sched_barrier(0);
-    // the factors of this lane's column for the spans of this wave (at most NLN), needed when the first span ends
-    const int nc = ncol < a.N ? ncol : a.N - 1;
-    const uint32_t g_first = (blockIdx.y * (K / 128) + (uint32_t)ks * NLN) / (uint32_t)a.per_group;   // the group of the wave's first span
-    const uint32_t RG = (uint32_t)a.row_g;
-    float fs[NLN], fc[NLN];
-#pragma unroll
-    for (int q = 0; q < NLN; ++q) {
-        const uint32_t gi = q < a.spans ? g_first + q : g_first;
-        const uint32_t gidx = gi < RG ? gi : RG - 1;
-        const uint32_t sbits = a.scales[(size_t)nc * RG + gidx];
-        const int zq = a.offsets ? (int)reinterpret_cast<const int8_t*>(a.offsets)[(size_t)nc * RG + gidx] : 0;
-        fs[q] = a.scale_f16 ? f16_bits_to_f32(sbits) : bf16_bits_to_f32(sbits);
-        fc[q] = -(fs[q] * (float)(zq + 128));                                  // exact: 8 bits x 11 bits
-    }
-    __builtin_amdgcn_sched_barrier(0);
-
     // ---- stage the activations: smoothed, summed per step of 128 --------------------------------------------------
 #pragma unroll
     for (int j = 0; j < XJ; ++j) {
@@ -232,10 +232,13 @@ __global__ __launch_bounds__(4 * CG * 64) void w8a16_stream(Stream16Args a) {
             for (int r = 0; r < 4; ++r) X[r] = X[r] + Xi[r];
         }
         if (++in_span == a.span) {                   // the span's scale ends here (the same for every wave of the launch)
-            float sc = fs[0], c = fc[0];
+            uint32_t sbits = fs_raw[0];
+            int zq = fz_raw[0];
 #pragma unroll
             for (int q = 1; q < NLN; ++q)
-                if (q == span_idx) { sc = fs[q]; c = fc[q]; }
+                if (q == span_idx) { sbits = fs_raw[q]; zq = fz_raw[q]; }
+            const float sc = a.scale_f16 ? f16_bits_to_f32(sbits) : bf16_bits_to_f32(sbits);
+            const float c = -(sc * (float)(zq + 128));                         // exact: 8 bits x 11 bits
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[r] = __builtin_fmaf(sc, P[r], __builtin_fmaf(c, X[r], acc[r]));
             P = w8f4{0.f, 0.f, 0.f, 0.f};
