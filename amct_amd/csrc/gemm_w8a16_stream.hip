@@ -356,13 +356,15 @@ static bool stream16_group_ok(int64_t K_row, int64_t ks, int group) {
 // per-channel factors: W[8192,28672] 87 / 87 / 87 -> 58 / 65 / 77; W[8192,8192] 30 / 30 / 29 -> 21 / 29 / 23;
 // W[13824,5120] 24 / 26 / 28 -> 19 / 20 / 25; not taken: W[28672,8192] 53 / 56 / 65 (sliced: 56 / 83 / 73),
 // W[10240,8192] 27 / 29 / 33 (sliced: 25 / 35 / 38).
-static bool stream16_slices_pay(int64_t N, int64_t K, int64_t ks) {
+// (And whenever the activation image of a slice is small enough for the narrow blocks, several per CU: W[28672,8192] /
+// W[57344,8192] at M = 1: 53 / 103 -> 40 / 73 us.)
+static bool stream16_slices_pay(int64_t M, int64_t N, int64_t K, int64_t ks) {
     const int64_t S = (K + ks - 1) / ks, cus = current_cu_count();
-    return K >= 12288 || S >= 4 || ((N + 63) / 64) * S <= cus;
+    return K >= 12288 || S >= 4 || ((N + 63) / 64) * S <= cus || M * (ks * 2 + 16) <= 12 * 1024;
 }
 size_t w8a16_stream_part_bytes(int64_t M, int64_t N, int64_t K, int group) {
     const int64_t ks = stream16_slice(K);
-    if (M < 1 || M > 16 || !ks || ks == K || N % 8 != 0 || !stream16_group_ok(K, ks, group) || !stream16_slices_pay(N, K, ks)) return 0;
+    if (M < 1 || M > 16 || !ks || ks == K || N % 8 != 0 || !stream16_group_ok(K, ks, group) || !stream16_slices_pay(M, N, K, ks)) return 0;
     return (size_t)((K + ks - 1) / ks) * (size_t)M * (size_t)N * 4;
 }
 

@@ -290,8 +290,8 @@ def w4a16_streams(M, K, group_size, dtype=torch.bfloat16, N=None):
 
 def w8a16_streams(M, K, group_size, dtype=torch.bfloat16, N=None, cus=256):
     """The same question for the int8 weight-only GEMM: a few rows, K of 1024, 2048 or 4096 or (N a multiple of 8) at most
-    16 slices of one of those -- for K >= 12288, four and more slices, or few enough columns that 64-column blocks per
-    slice run at once on `cus` compute units; groups of 128, 256, ... up to the slice, or whole slices (per-channel
+    16 slices of one of those -- for K >= 12288, four and more slices, few enough columns that 64-column blocks per
+    slice run at once on `cus` compute units, or a slice of the activations below 12 KB; groups of 128, 256, ... up to the slice, or whole slices (per-channel
     factors)."""
     if dtype not in (torch.bfloat16, torch.float16) or not 1 <= M <= 16 or group_size < 128 or K % group_size:
         return False
@@ -304,7 +304,7 @@ def w8a16_streams(M, K, group_size, dtype=torch.bfloat16, N=None, cus=256):
         slices = -(-K // ks)
         if N is None or N % 8:
             return False
-        if not (K >= 12288 or slices >= 4 or -(-N // 64) * slices <= cus):
+        if not (K >= 12288 or slices >= 4 or -(-N // 64) * slices <= cus or M * (ks * 2 + 16) <= 12 * 1024):
             return False
     return group_size & (group_size - 1) == 0 if group_size <= ks else (group_size % ks == 0 or group_size == K)
 
