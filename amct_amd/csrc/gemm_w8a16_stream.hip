@@ -145,6 +145,7 @@ __global__ __launch_bounds__(4 * CG * 64) void w8a16_stream(Stream16Args a) {
     const int nc = ncol < a.N ? ncol : a.N - 1;
     const uint32_t g_first = (blockIdx.y * (K / 128) + (uint32_t)ks * NLN) / (uint32_t)a.per_group;   // the group of the wave's first span
     const uint32_t RG = (uint32_t)a.row_g;
+    const float bias_v = (a.bias && ks == 0) ? a.bias[nc] : 0.f;    // with the factors: a load in the epilogue would cost a memory latency there
     uint32_t fs_raw[NLN];
     int fz_raw[NLN];
 #pragma unroll
@@ -268,12 +269,11 @@ __global__ __launch_bounds__(4 * CG * 64) void w8a16_stream(Stream16Args a) {
                 if (m < (int)M) a.part[((size_t)blockIdx.y * M + m) * a.N + ncol] = y[r];
             }
         } else if (ncol < a.N) {
-            const float b = a.bias ? a.bias[ncol] : 0.f;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int m = 4 * g + r;
                 float v = y[r];
-                if (a.bias) v = v + b;
+                if (a.bias) v = v + bias_v;
                 if (m < (int)M) a.out[(size_t)m * a.N + ncol] = (uint16_t)W8Act<DT>::out_bits(v);
             }
         }
