@@ -63,6 +63,8 @@ SIGNATURES = {
     "amct_gemm_w8a16_workspace_bytes": (ctypes.c_size_t, [_L, _L, _L, _I, _I]),
     "amct_gemm_w8a16_ws": (_I, [_P, _P, _P, _P, _I, _P, _P, _P, _L, _L, _L, _I, _I, _P, ctypes.c_size_t, _P]),
     "amct_gemm_w4a16_workspace_bytes": (ctypes.c_size_t, [_L, _L, _L, _I, _I]),
+    "amct_gemm_w4a16_weight_rounded": (_I, [_L, _L, _L, _I, _I, ctypes.c_size_t]),
+    "amct_gemm_w8a16_weight_rounded": (_I, [_L, _L, _L, _I, _I, ctypes.c_size_t]),
     "amct_gemm_w4a16": (_I, [_P, _P, _P, _P, _I, _P, _P, _P, _L, _L, _L, _I, _I, _P, ctypes.c_size_t, _P]),
 }
 

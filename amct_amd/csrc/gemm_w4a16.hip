@@ -1889,7 +1889,8 @@ int wq16_int4_f16(const void* x, const void* smooth, const uint8_t* wq, const vo
 int w4a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
                           const uint8_t* zeros, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group,
                           int dtype, void* workspace, size_t workspace_bytes, hipStream_t st);
-size_t w4a16_stream_part_bytes(int64_t M, int64_t N, int64_t K, int group);   // partial sums of its launches over slices of K              // gemm_w4a16_stream.hip
+size_t w4a16_stream_part_bytes(int64_t M, int64_t N, int64_t K, int group);   // partial sums of its launches over slices of K
+bool w4a16_stream_takes(int64_t M, int64_t N, int64_t K, int group, size_t workspace_bytes);   // gemm_w4a16_stream.hip
 
 int gemm16_tiles(const void* x, const void* w, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int dtype,
                  void* workspace, size_t workspace_bytes, hipStream_t st);   // gemm_w8a8.hip
@@ -2071,6 +2072,13 @@ extern "C" size_t amct_gemm_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t 
     const size_t tiles = (has_smooth && (M > 16 || part) ? (size_t)M * (size_t)K * 2 : 0) + part;
     const size_t stream = w4a16_stream_part_bytes(M, N, K, group);     // a few rows, K in slices: its partial sums only
     return tiles > stream ? tiles : stream;
+}
+
+extern "C" int amct_gemm_w4a16_weight_rounded(int64_t M, int64_t N, int64_t K, int group, int dtype, size_t workspace_bytes) {
+    if (M < 0 || N <= 0 || K <= 0 || group <= 0) return AMCT_E_BADARG;
+    if (dtype != AMCT_BF16 && dtype != AMCT_F16) return AMCT_E_UNSUPPORTED;
+    // the weight-streaming kernel is the only one that keeps the integer weight; amct_gemm_w4a16 tries it first
+    return M <= 16 && w4a16_stream_takes(M, N, K, group, workspace_bytes) ? 0 : 1;
 }
 
 extern "C" int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t* wq, const void* scales,

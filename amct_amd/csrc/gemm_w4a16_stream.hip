@@ -368,9 +368,6 @@ static int stream_launch_x(const StreamArgs& a, size_t lds_bytes, dim3 blocks, h
 // most 16 slices (8192 = 2 x 4096, 14336 = 7 x 2048, 5120 = 5 x 1024, 28672 = 7 x 4096); 0: none.
 static int64_t stream_slice(int64_t K) {
     if (K == 1024 || K == 2048 || K == 4096) return K;
-#ifdef AMCT_ST_SLICE
-    if (K % AMCT_ST_SLICE == 0 && K / AMCT_ST_SLICE <= 16) return AMCT_ST_SLICE;
-#endif
     for (int64_t ks = 4096; ks >= 1024; ks /= 2)
         if (K % ks == 0 && K / ks <= 16) return ks;
     // other multiples of 256 (11008, 13824): slices of 1024 whose last one is shorter -- a wave walks 256 elements, so it
@@ -391,21 +388,34 @@ size_t w4a16_stream_part_bytes(int64_t M, int64_t N, int64_t K, int group) {
     return (size_t)((K + ks - 1) / ks) * (size_t)M * (size_t)N * 4;
 }
 
+// Whether this kernel takes a call of this shape with a workspace of this size (operands suitably aligned): the one
+// rule behind the dispatch below and behind amct_gemm_w4a16_weight_rounded.
+bool w4a16_stream_takes(int64_t M, int64_t N, int64_t K_row, int group, size_t workspace_bytes) {
+    // one group per step of 128 elements of K (the per-group partial sums of a step cannot be separated otherwise)
+    const int64_t K = stream_slice(K_row), S = K ? (K_row + K - 1) / K : 0;
+    if (M < 1 || M > 16 || !K || group != 128 || N <= 0 || N > (int64_t(1) << 30)) return false;
+    if (S > 1) {
+        // rows of several slices: the partial sums go through the lent workspace
+        const size_t need = w4a16_stream_part_bytes(M, N, K_row, group);
+        if (!need || workspace_bytes < need) return false;
+    }
+    // what the launch shapes below hold: an activation image of at most 160 KB, at most 8 vectors staged per thread
+    const size_t xbytes = (size_t)M * ((size_t)K * 2 + 16), img = xbytes + (size_t)(K / group) * 64;
+    const int64_t cg = xbytes > 40 * 1024 ? 4 : xbytes > 12 * 1024 ? 2 : 1;
+    return img <= 160 * 1024 && (M * (K / 8) + 256 * cg - 1) / (256 * cg) <= 8;
+}
+
 // Returns AMCT_E_UNSUPPORTED when the shape is not one this kernel takes (the caller then uses its other kernels).
 int w4a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
                           const uint8_t* zeros, const float* bias, void* out, int64_t M, int64_t N, int64_t K_row, int group,
                           int dtype, void* workspace, size_t workspace_bytes, hipStream_t st) {
-    // one group per step of 128 elements of K (the per-group partial sums of a step cannot be separated otherwise)
-    const int64_t K = stream_slice(K_row), S = K ? (K_row + K - 1) / K : 0;
-    if (M < 1 || M > 16 || !K || group != 128 || N > (int64_t(1) << 30)) return AMCT_E_UNSUPPORTED;
+    if (!w4a16_stream_takes(M, N, K_row, group, workspace ? workspace_bytes : 0)) return AMCT_E_UNSUPPORTED;
+    const int64_t K = stream_slice(K_row), S = (K_row + K - 1) / K;
     if (!aligned16(x) || !aligned16(wq) || (smooth && !aligned16(smooth)) || ((uintptr_t)scales & 3) || ((uintptr_t)zeros & 3))
         return AMCT_E_UNSUPPORTED;
     float* part = nullptr;
     if (S > 1) {
-        // rows of several slices: the partial sums go through the lent workspace
-        const size_t need = w4a16_stream_part_bytes(M, N, K_row, group);
-        if (!need || !workspace || !aligned16(workspace) || workspace_bytes < need || !aligned16(out) || (bias && !aligned16(bias)))
-            return AMCT_E_UNSUPPORTED;
+        if (!aligned16(workspace) || !aligned16(out) || (bias && !aligned16(bias))) return AMCT_E_UNSUPPORTED;
         part = reinterpret_cast<float*>(workspace);
     }
     StreamArgs a{(const uint16_t*)x, (const uint16_t*)smooth, wq, (const uint16_t*)scales, zeros, bias,

@@ -368,20 +368,36 @@ size_t w8a16_stream_part_bytes(int64_t M, int64_t N, int64_t K, int group) {
     return (size_t)((K + ks - 1) / ks) * (size_t)M * (size_t)N * 4;
 }
 
+// Whether this kernel takes a call of this shape with a workspace of this size (operands suitably aligned): the one
+// rule behind the dispatch below and behind amct_gemm_w8a16_weight_rounded.
+bool w8a16_stream_takes(int64_t M, int64_t N, int64_t K_row, int group, size_t workspace_bytes) {
+    const int64_t K = stream16_slice(K_row), S = K ? (K_row + K - 1) / K : 0;
+    if (M < 1 || M > 16 || !K || N <= 0 || N > (int64_t(1) << 30)) return false;
+    if (!stream16_group_ok(K_row, K, group)) return false;
+    if (S > 1) {
+        // rows of several slices: the partial sums go through the lent workspace
+        const size_t need = w8a16_stream_part_bytes(M, N, K_row, group);
+        if (!need || workspace_bytes < need) return false;
+    }
+    // the launch shapes below: threads whose staged vectors share a column (or M = 1 on K = 4096), at most 8 of them
+    const size_t xbytes = (size_t)M * ((size_t)K * 2 + 16);
+    const int64_t cg = xbytes > 40 * 1024 ? 4 : xbytes > 12 * 1024 ? 2 : 1, nt = 256 * cg, kv = K / 8;
+    const int64_t xj = (M * kv + nt - 1) / nt;
+    if (xbytes + (size_t)(K / 128) * 64 > 160 * 1024) return false;
+    if (nt % kv == 0) return xj <= 8;
+    return kv == 2 * nt && cg == 1 && K / 512 == 8 && xj <= 2;
+}
+
 // Returns AMCT_E_UNSUPPORTED when the shape is not one this kernel takes (the caller then uses its other kernels).
 int w8a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
                           const uint8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K_row, int group,
                           int dtype, void* workspace, size_t workspace_bytes, hipStream_t st) {
-    const int64_t K = stream16_slice(K_row), S = K ? (K_row + K - 1) / K : 0;
-    if (M < 1 || M > 16 || !K || N > (int64_t(1) << 30)) return AMCT_E_UNSUPPORTED;
-    if (!stream16_group_ok(K_row, K, group)) return AMCT_E_UNSUPPORTED;
+    if (!w8a16_stream_takes(M, N, K_row, group, workspace ? workspace_bytes : 0)) return AMCT_E_UNSUPPORTED;
+    const int64_t K = stream16_slice(K_row), S = (K_row + K - 1) / K;
     if (!aligned16(x) || !aligned16(wq) || (smooth && !aligned16(smooth)) || ((uintptr_t)scales & 1)) return AMCT_E_UNSUPPORTED;
     float* part = nullptr;
     if (S > 1) {
-        // rows of several slices: the partial sums go through the lent workspace
-        const size_t need = w8a16_stream_part_bytes(M, N, K_row, group);
-        if (!need || !workspace || !aligned16(workspace) || workspace_bytes < need || !aligned16(out) || (bias && !aligned16(bias)))
-            return AMCT_E_UNSUPPORTED;
+        if (!aligned16(workspace) || !aligned16(out) || (bias && !aligned16(bias))) return AMCT_E_UNSUPPORTED;
         part = reinterpret_cast<float*>(workspace);
     }
     const int nln = (int)(K / 512);                  // lines of 128 per wave (a quarter of the slice)

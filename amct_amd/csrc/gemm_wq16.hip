@@ -510,6 +510,7 @@ int w8a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, 
                           const uint8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group,
                           int dtype, void* workspace, size_t workspace_bytes, hipStream_t st);      // gemm_w8a16_stream.hip
 size_t w8a16_stream_part_bytes(int64_t M, int64_t N, int64_t K, int group);   // partial sums of its launches over slices of K
+bool w8a16_stream_takes(int64_t M, int64_t N, int64_t K, int group, size_t workspace_bytes);
 int w8a16_spec_dispatch(const void* x, const void* smooth, const uint8_t* wq, const void* scales, int scale_dtype,
                         const uint8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K, int group, int dtype,
                         void* workspace, size_t workspace_bytes, hipStream_t st);   // gemm_w4a16.hip
@@ -527,6 +528,13 @@ extern "C" size_t amct_gemm_w8a16_workspace_bytes(int64_t M, int64_t N, int64_t 
     const size_t stream = w8a16_stream_part_bytes(M, N, K, group);          // a few rows, K in slices: its partial sums
     const size_t most = two > spec ? two : spec;
     return most > stream ? most : stream;
+}
+
+extern "C" int amct_gemm_w8a16_weight_rounded(int64_t M, int64_t N, int64_t K, int group, int dtype, size_t workspace_bytes) {
+    if (M < 0 || N <= 0 || K <= 0 || group <= 0) return AMCT_E_BADARG;
+    if (dtype != AMCT_BF16 && dtype != AMCT_F16) return AMCT_E_UNSUPPORTED;
+    // the weight-streaming kernel is the only one that keeps the integer weight; amct_gemm_w8a16_ws tries it first
+    return M <= 16 && w8a16_stream_takes(M, N, K, group, workspace_bytes) ? 0 : 1;
 }
 
 extern "C" int amct_gemm_w8a16(const void* x, const void* smooth, const int8_t* wq, const void* scales, int scale_dtype,

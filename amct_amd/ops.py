@@ -77,6 +77,37 @@ def _c(t):
     return t if t.is_contiguous() else t.contiguous()
 
 
+# Scratch memory the GEMM wrappers lend to the library (it never allocates): ONE grow-only byte tensor per device and
+# stream, shared by every call on that stream.  Calls on one stream run in order, so they can share it; a fresh
+# torch.empty per forward would pass a dequantise-once call (the weight as 16 bits: N * K * 2 bytes) through the
+# allocator every time.  `workspace_limit_bytes` caps what is lent: a call that asks for more gets the capped size and
+# the library then takes the kernels that need less (documented per entry point: never an error), which bounds the
+# memory a deployment pays for the faster many-row kernels.  None: no cap.
+workspace_limit_bytes = None
+_WORKSPACES = {}
+
+
+def lent_workspace(dev, nbytes):
+    """A uint8 tensor of at least min(nbytes, workspace_limit_bytes) bytes on dev for the current stream, or None."""
+    if workspace_limit_bytes is not None:
+        nbytes = min(nbytes, int(workspace_limit_bytes))
+    if nbytes <= 0:
+        return None
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), _stream(dev))
+    ws = _WORKSPACES.get(key)
+    if ws is None or ws.numel() < nbytes:
+        _WORKSPACES.pop(key, None)                   # let the smaller one go before the larger one is allocated
+        ws = None
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        _WORKSPACES[key] = ws
+    return ws
+
+
+def release_workspaces():
+    """Drops the lent scratch tensors (they come back on the next call that needs one)."""
+    _WORKSPACES.clear()
+
+
 # ---------------------------------------------------------------------------
 # A1 / A2
 # ---------------------------------------------------------------------------
@@ -476,10 +507,7 @@ def gemm_w8a8(xq, wq_nk, s_ch, s_tok=None, bias=None, out_dtype=torch.bfloat16, 
     out = torch.empty(M, N, dtype=out_dtype, device=dev)
     acc = torch.empty(M, N, dtype=torch.int32, device=dev) if want_acc else None
     # the workspace the library asks for (partial sums, when it splits long rows over several blocks per tile)
-    ws = None
-    nbytes = _lib.load().amct_gemm_w8a8_workspace_bytes(M, N, K)
-    if nbytes:
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    ws = lent_workspace(dev, _lib.load().amct_gemm_w8a8_workspace_bytes(M, N, K))
     with _on(dev):
         _lib.check(_lib.load().amct_gemm_w8a8_ws(_p(xq), _p(wq_nk), _p(s_tok), _p(s_ch), _p(bias), kind, _p(out), _p(acc),
                                                  M, N, K, dtype_code(out_dtype), _p(ws), 0 if ws is None else ws.numel(),
@@ -526,10 +554,9 @@ def linear_w8a8(x, act_scale, act_offset, per_token, wq_nk, s_ch, s_tok=None, bi
             kind, bias = 2, _c(bias.to(torch.float32))
     out = torch.empty(M, N, dtype=out_dtype, device=dev)
     lib = _lib.load()
-    fused = M <= 16 and K in (1024, 2048, 4096) and x.dtype != torch.float32 and (per_token or n_scales == 1)
-    ws = None
-    if not fused:                                    # the int8 activations (and the GEMM's partial sums) go through a workspace
-        ws = torch.empty(max(16, lib.amct_linear_w8a8_workspace_bytes(M, N, K)), dtype=torch.uint8, device=dev)
+    # whatever the library asks for (the int8 activations of the two-kernel form, the GEMM's partial sums): which calls
+    # quantise inside the weight-streaming kernel and need none of it is the library's rule, not restated here
+    ws = lent_workspace(dev, lib.amct_linear_w8a8_workspace_bytes(M, N, K))
     with _on(dev):
         _lib.check(lib.amct_linear_w8a8(_p(x), dtype_code(x.dtype), _p(smooth), _p(act_scale), _p(act_offset), n_scales,
                                         int(bool(per_token)), _p(wq_nk), _p(s_tok), _p(s_ch), _p(bias), kind, _p(out), M, N, K,
@@ -554,6 +581,33 @@ def _check_weight_only(x, N, K, scales, zeros, group, smooth, bias, zeros_dtype,
           0 if bias is None else bias.numel(), N)
 
 
+def gemm_w4a16_weight_rounded(M, N, K, group, dtype, workspace_bytes=None):
+    """Whether amct_gemm_w4a16 rounds the dequantised weight to `dtype` for a call of this shape (True) or keeps it
+    exact (False); workspace_bytes None: the workspace gemm_w4a16 lends."""
+    lib = _lib.load()
+    if workspace_bytes is None:
+        workspace_bytes = lib.amct_gemm_w4a16_workspace_bytes(M, N, K, group, 0)
+        if workspace_limit_bytes is not None:
+            workspace_bytes = min(workspace_bytes, int(workspace_limit_bytes))
+    r = lib.amct_gemm_w4a16_weight_rounded(M, N, K, group, dtype_code(dtype), workspace_bytes)
+    if r < 0:
+        _lib.check(r)
+    return bool(r)
+
+
+def gemm_w8a16_weight_rounded(M, N, K, group, dtype, workspace_bytes=None):
+    """The same question for amct_gemm_w8a16_ws."""
+    lib = _lib.load()
+    if workspace_bytes is None:
+        workspace_bytes = lib.amct_gemm_w8a16_workspace_bytes(M, N, K, group, 0)
+        if workspace_limit_bytes is not None:
+            workspace_bytes = min(workspace_bytes, int(workspace_limit_bytes))
+    r = lib.amct_gemm_w8a16_weight_rounded(M, N, K, group, dtype_code(dtype), workspace_bytes)
+    if r < 0:
+        _lib.check(r)
+    return bool(r)
+
+
 def gemm_w4a16(x, wq_packed, scales, zeros, group, smooth=None, bias=None):
     """x [M,K] bf16|f16; wq_packed uint8 [N,K/2]; scales [N,K/g] f16|bf16; zeros uint8 [N,K/g]."""
     _need(wq_packed.dim() == 2 and wq_packed.dtype == torch.uint8, "int4 GEMM: the weight must be uint8 [N, K/2]")
@@ -572,10 +626,7 @@ def gemm_w4a16(x, wq_packed, scales, zeros, group, smooth=None, bias=None):
     out = torch.empty(M, N, dtype=x.dtype, device=dev)
     # the workspace the library asks for: the smoothed activations for the tile kernels, or the activation image the
     # weight-streaming kernel for a few rows fetches
-    ws = None
-    nbytes = _lib.load().amct_gemm_w4a16_workspace_bytes(M, N, K, group, int(smooth is not None))
-    if nbytes:
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    ws = lent_workspace(dev, _lib.load().amct_gemm_w4a16_workspace_bytes(M, N, K, group, int(smooth is not None)))
     with _on(dev):
         _lib.check(_lib.load().amct_gemm_w4a16(_p(x), _p(smooth), _p(wq_packed), _p(scales), dtype_code(scales.dtype),
                                                _p(zeros), _p(bias), _p(out), M, N, K, group, dtype_code(x.dtype),
@@ -598,10 +649,7 @@ def gemm_w8a16(x, wq_nk, scales, offsets, group, smooth=None, bias=None):
         bias = _c(bias.reshape(-1).to(torch.float32))
     out = torch.empty(M, N, dtype=x.dtype, device=dev)
     # the workspace the library asks for: from 256 rows on, the dequantised weight (and the smoothed activations)
-    ws = None
-    nbytes = _lib.load().amct_gemm_w8a16_workspace_bytes(M, N, K, group, int(smooth is not None))
-    if nbytes:
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    ws = lent_workspace(dev, _lib.load().amct_gemm_w8a16_workspace_bytes(M, N, K, group, int(smooth is not None)))
     with _on(dev):
         _lib.check(_lib.load().amct_gemm_w8a16_ws(_p(x), _p(smooth), _p(wq_nk), _p(scales), dtype_code(scales.dtype),
                                                   _p(offsets), _p(bias), _p(out), M, N, K, group, dtype_code(x.dtype),

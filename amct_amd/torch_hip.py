@@ -5,8 +5,8 @@ and amct_pytorch/deploy_op/weight_npu_quant_module.py:54-57,116-117).  Same keyw
 layouts as those calls; each runs HIP kernels only.
 
 The weight operands arrive here in the reference's [K, N] layouts; their kernel layouts are computed on the
-first call and cached per tensor and version (the deploy modules in amct_amd.deploy_op convert once at
-construction instead).
+first call and cached per tensor and version for as long as the tensor lives (the deploy modules in
+amct_amd.deploy_op convert once at construction instead).
 """
 import torch
 
@@ -78,17 +78,32 @@ def npu_convert_weight_to_int4pack(weight, inner_k_tiles=0):
 class _LayoutCache:
     """Converted operands of npu_weight_quant_batchmatmul, keyed on the identity and version of the tensors the
     caller passed.  A deploy module calls the operator with the same registered buffers on every forward; their
-    kernel layout ([N, K] weights, [N, K/g] factors) is computed on the first call only.  Entries hold weak
-    references to their sources, so a buffer that is freed, replaced or written in place is converted again."""
+    kernel layout ([N, K] weights, [N, K/g] factors) is computed on the first call only.
 
-    def __init__(self, capacity=256):
-        self.capacity = capacity
-        self.entries = {}
+    Lifetime: an entry holds weak references to its source tensors and is dropped the moment one of them is freed
+    (weakref.finalize), so the cache never outlives the model: at most one converted copy per live weight.  There
+    is no entry count limit (a model of any number of layers hits on every forward after the first); `max_bytes`
+    (None: unbounded) caps the converted bytes kept, evicting the least recently used entry first.
+    Contract: a write that bumps the tensor's version counter (copy_, add_, ...) is seen and converts again; a
+    write that does not (through `.data`, `set_()` onto the same storage, a kernel outside torch) is NOT seen --
+    call clear_layout_cache() after such a write."""
+
+    def __init__(self, max_bytes=None):
+        import collections
+        self.max_bytes = max_bytes
+        self.entries = collections.OrderedDict()      # key -> (weakrefs, value, nbytes), least recently used first
+        self.bytes = 0
+        self.conversions = 0
 
     @staticmethod
     def _key(tensors, extra):
-        return tuple((t.data_ptr(), t._version, tuple(t.shape), t.dtype) if t is not None else None
+        return tuple((id(t), t.data_ptr(), t._version, tuple(t.shape), t.dtype) if t is not None else None
                      for t in tensors) + (extra,)
+
+    def _drop(self, key):
+        hit = self.entries.pop(key, None)
+        if hit is not None:
+            self.bytes -= hit[2]
 
     def get(self, tensors, extra, make):
         import weakref
@@ -96,18 +111,46 @@ class _LayoutCache:
         hit = self.entries.get(key)
         if hit is not None and all((r is None and t is None) or (r is not None and r() is t)
                                    for r, t in zip(hit[0], tensors)):
+            self.entries.move_to_end(key)
             return hit[1]
+        self._drop(key)
+        # an older version of the same source tensors is of no further use
+        ids = tuple(None if t is None else id(t) for t in tensors)
+        for k in [k for k in self.entries if tuple(None if e is None else e[0] for e in k[:-1]) == ids and k[-1] == extra]:
+            self._drop(k)
         value = make()
-        if len(self.entries) >= self.capacity:
-            self.entries.pop(next(iter(self.entries)))
-        self.entries[key] = ([None if t is None else weakref.ref(t) for t in tensors], value)
+        self.conversions += 1
+        nbytes = sum(v.numel() * v.element_size() for v in value if isinstance(v, torch.Tensor))
+        refs = []
+        for t in tensors:
+            if t is None:
+                refs.append(None)
+                continue
+            refs.append(weakref.ref(t))
+            weakref.finalize(t, self._drop, key)        # the source is gone: so is the converted copy
+        self.entries[key] = (refs, value, nbytes)
+        self.bytes += nbytes
+        while self.max_bytes is not None and self.bytes > self.max_bytes and len(self.entries) > 1:
+            self._drop(next(iter(self.entries)))
         return value
 
     def clear(self):
         self.entries.clear()
+        self.bytes = 0
 
 
 _layout_cache = _LayoutCache()
+
+
+def clear_layout_cache():
+    """Forgets every converted operand (needed after a write to a weight or factor tensor that torch's version
+    counter does not see)."""
+    _layout_cache.clear()
+
+
+def set_layout_cache_limit(max_bytes):
+    """Caps the converted bytes the operator keeps (None: no cap; entries always die with their source tensors)."""
+    _layout_cache.max_bytes = max_bytes
 
 
 def npu_weight_quant_batchmatmul(x, weight, antiquant_scale, antiquant_offset=None, quant_scale=None,

@@ -104,9 +104,12 @@ int amct_col_minmax(const void* x, float* col_max, float* col_min, int64_t rows,
  * hipMalloc).  Same arguments, kernels and results as amct_col_minmax; the per-chunk partials go to a fixed array
  * inside the library's device image instead (64 chunks x 2 x AMCT_COL_MINMAX_NOALLOC_MAX_COLS floats = 4 MiB, held
  * by every GPU the library runs on until the process ends).  cols > AMCT_COL_MINMAX_NOALLOC_MAX_COLS returns
- * AMCT_E_TOO_LARGE and enqueues nothing.  The call allocates and frees nothing.  All calls on one GPU share that
- * array: calls that overlap on one GPU (different streams or threads) race; calls on one stream do not.  Nothing
- * has to be cleared between calls (the first pass overwrites every partial the second pass reads). */
+ * AMCT_E_TOO_LARGE and enqueues nothing.  The call allocates and frees nothing.  The FIRST call on a device asks the
+ * runtime for the array's address on that device (hipGetDevice, hipGetSymbolAddress: the runtime may load the
+ * library's code object then), so make one ordinary call per device before capturing the entry point in a graph.
+ * All calls on one GPU share that array, whatever their stream: calls that overlap on one GPU (different streams or
+ * threads) race; calls on one stream do not.  Nothing has to be cleared between calls (the first pass overwrites
+ * every partial the second pass reads). */
 #define AMCT_COL_MINMAX_NOALLOC_MAX_COLS 8192
 int amct_col_minmax_noalloc(const void* x, float* col_max, float* col_min, int64_t rows, int64_t cols, int absolute,
                             int accumulate, int dtype, amct_stream_t stream);
@@ -289,10 +292,23 @@ int amct_linear_w8a8(const void* x, int x_dtype, const void* smooth, const void*
  * or 1024 elements (the last one shorter for other multiples of 256, e.g. 11008), which the weight-streaming kernel then
  * walks one per block.  0 bytes are
  * asked for otherwise; a null or smaller workspace is never an error.
- * Arithmetic of the dequantisation: the tile kernels (M > 16) feed dtype((u - zero) * scale) to the matrix pipe; the
- * weight-streaming kernel for M <= 16 (bf16 or fp16, K of 1024 / 2048 / 4096 or slices of those, group = 128) keeps the weight as the exact integer and applies
- * scale and zero per group in fp32, i.e. the dequantised weight is not rounded to bf16 there (the fp32 weight * scale of
- * tests/amct_pytorch/mock_torch_npu.py:33-55).  Both stay within 1e-3 of the exact result. */
+ * Arithmetic of the dequantisation (the operator's own lives inside the un-vendored torch_npu, so the library fixes
+ * two readings and says which one a call takes):
+ *   exact    the weight-streaming kernel for M <= 16 (bf16 or fp16, K of 1024 / 2048 / 4096 or slices of those,
+ *            group = 128) keeps the weight as the exact integer and applies scale and zero per group in fp32: the
+ *            dequantised weight is not rounded (the fp32 weight * scale of tests/amct_pytorch/mock_torch_npu.py:33-55).
+ *            Within 1e-5 of the row's largest output (+ the rounding of the output) of the exact result.
+ *   rounded  every other kernel feeds dtype((u - zero) * scale) to the matrix pipe, whose operands are 16 bits wide.
+ *            Each weight then carries a relative error of up to u = 2^-8 (bf16; 2^-11 for fp16), so an output differs
+ *            from the exact result by at most u * sum_k |x'_k * w_k|, and for errors of independent sign by about
+ *            u / sqrt(3) * sqrt(sum_k (x'_k * w_k)^2).  On W[14336, 4096] with N(0, 1) activations that is up to
+ *            2.5e-3 of the row's largest output for bf16 (3e-4 for fp16): bf16 calls of more than 16 rows are NOT
+ *            within 1e-3 of the exact result at K = 4096, and a token's output differs by that much between a call
+ *            of up to 16 rows and a larger one.
+ * amct_gemm_w4a16_weight_rounded answers 0 (exact) or 1 (rounded) for a call of that shape, dtype and workspace size
+ * with 16-byte aligned operands (unaligned operands always take a rounding kernel); a negative error code for
+ * arguments amct_gemm_w4a16 rejects. */
+int amct_gemm_w4a16_weight_rounded(int64_t M, int64_t N, int64_t K, int group, int dtype, size_t workspace_bytes);
 size_t amct_gemm_w4a16_workspace_bytes(int64_t M, int64_t N, int64_t K, int group, int has_smooth);
 int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t* wq, const void* scales,
                     int scale_dtype, const uint8_t* zeros, const float* bias, void* out,
@@ -307,11 +323,16 @@ int amct_gemm_w4a16(const void* x, const void* smooth, const uint8_t* wq, const 
  * channel, the reference's antiquant_group_size = 0); offsets int8 [N, K/group] = the quantiser's offset_w, null
  * when symmetric (the module registers its negation as antiquant_offset, :62-64); bias fp32 [N] or null.
  * out [M, N] of dtype = x' @ dtype((q - offset) * scale)^T + bias, fp32 accumulate.
- * As for the int4 weight there are two readings of the dequantisation: the tile kernels feed dtype((q - offset) * scale)
- * to the matrix pipe; the weight-streaming kernel for M <= 16 (K of 1024 / 2048 / 4096, group a power of two from 128 to K; through
- * amct_gemm_w8a16_ws and its workspace also rows of 2 ... 16 such slices, the last one shorter if need be -- K = 8192, 11008, 14336, 28672, 5120 ... --,
- * groups up to a slice, whole slices or the whole row, where that beats the other kernels) keeps the weight as the exact integer and applies scale and offset per group in fp32, i.e. the dequantised weight is
- * not rounded to 16 bits there.  Both stay within 1e-3 of the exact result. */
+ * As for the int4 weight there are two readings of the dequantisation: the weight-streaming kernel for M <= 16 (K of
+ * 1024 / 2048 / 4096, group a power of two from 128 to K; through amct_gemm_w8a16_ws and its workspace also rows of
+ * 2 ... 16 such slices, the last one shorter if need be -- K = 8192, 11008, 14336, 28672, 5120 ... --, groups up to a
+ * slice, whole slices or the whole row, where that beats the other kernels) keeps the weight as the exact integer and
+ * applies scale and offset per group in fp32 (within 2e-5 of the row's largest output of the exact result); every other
+ * kernel feeds dtype((q - offset) * scale) to the matrix pipe, with the error bound stated for amct_gemm_w4a16 (up to
+ * 2.5e-3 of the row's largest output for bf16 at K = 4096).  amct_gemm_w8a16_weight_rounded answers 0 (exact) or
+ * 1 (rounded) for a call of that shape, dtype and workspace size (0 for amct_gemm_w8a16, which has none) with 16-byte
+ * aligned operands. */
+int amct_gemm_w8a16_weight_rounded(int64_t M, int64_t N, int64_t K, int group, int dtype, size_t workspace_bytes);
 int amct_gemm_w8a16(const void* x, const void* smooth, const int8_t* wq, const void* scales, int scale_dtype,
                     const int8_t* offsets, const float* bias, void* out, int64_t M, int64_t N, int64_t K,
                     int group, int dtype, amct_stream_t stream);

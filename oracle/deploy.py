@@ -30,10 +30,15 @@ documented arithmetic.  Pin status:
                         the output dtype.
   w4a16 dequant         PARITY UNPINNED against torch_npu (precision of the
                         dequantised weight); this repo fixes: (q - z) * s
-                        exact in fp32, rounded once to x's dtype (tile
-                        kernels) or not rounded at all (the weight-streaming
-                        kernel for M <= 16, as the reference's CPU stand-in
+                        exact in fp32, rounded once to x's dtype (every
+                        kernel that feeds the matrix pipe a 16-bit weight)
+                        or not rounded at all (the weight-streaming kernels
+                        for M <= 16, as the reference's CPU stand-in
                         mock_torch_npu.py:33-55 does), fp32 accumulate.
+                        The library says which reading a call takes
+                        (amct_gemm_w4a16_weight_rounded); the tests compare
+                        EVERY call with the exact anchor, the rounding ones
+                        within weight_only_error_bounds().
                         Special case z=8 (unsigned), s=1 reduces to a plain
                         matmul -- tested against torch.matmul.
   int4 word packing     PARITY UNPINNED against torch_npu (nibble order);
@@ -274,39 +279,30 @@ def w4a16_forward_f64(x, codes_nk, scale_ng, antioffset_ng, group_size, bias=Non
     return weight_quant_matmul_f64(x2, wdq, bias).reshape(*shp[:-1], -1)
 
 
-def w4a16_streams(M, K, group_size, dtype=torch.bfloat16, N=None):
-    """Whether the int4 GEMM takes its weight-streaming kernel for this shape (a few rows of bf16 or fp16 activations, K
-    of 1024, 2048 or 4096, or -- from 5 rows on, for K >= 12288 or when K / 256 is not a multiple of 4; N a multiple of 8 -- at most 16 slices of one of those
-    (the last one shorter for other multiples of 256);
-    groups of 128): that kernel does not round the dequantised weight."""
-    if dtype not in (torch.bfloat16, torch.float16) or not 1 <= M <= 16 or group_size != 128:
-        return False
-    if K in (1024, 2048, 4096):
-        return True
-    sliced = any(K % ks == 0 and K // ks <= 16 for ks in (4096, 2048, 1024)) or (K % 256 == 0 and 1024 < K <= 16384)
-    sliced = sliced and (M >= 5 or K >= 12288 or (K // 256) % 4 != 0)
-    return sliced and (N is None or N % 8 == 0)
+def smoothed_rows(x, scale_factor=None):
+    """x' of the forward (weight_npu_quant_module.py:112-114): rows flattened, times scale_factor, rounded to x's dtype."""
+    x2 = x.reshape(-1, x.shape[-1])
+    if scale_factor is not None:
+        x2 = torch.mul(x2, scale_factor.to(x2.dtype))
+    return x2
 
 
-def w8a16_streams(M, K, group_size, dtype=torch.bfloat16, N=None, cus=256):
-    """The same question for the int8 weight-only GEMM: a few rows, K of 1024, 2048 or 4096 or (N a multiple of 8) at most
-    16 slices of one of those -- for K >= 12288, four and more slices, few enough columns that 64-column blocks per
-    slice run at once on `cus` compute units, or a slice of the activations below 12 KB; groups of 128, 256, ... up to the slice, or whole slices (per-channel
-    factors)."""
-    if dtype not in (torch.bfloat16, torch.float16) or not 1 <= M <= 16 or group_size < 128 or K % group_size:
-        return False
-    ks = K if K in (1024, 2048, 4096) else next((c for c in (4096, 2048, 1024) if K % c == 0 and K // c <= 16), 0)
-    if not ks and K % 256 == 0 and 1024 < K <= 16384:
-        ks = 1024                                   # the last slice shorter (11008, 13824)
-    if not ks:
-        return False
-    if ks != K:
-        slices = -(-K // ks)
-        if N is None or N % 8:
-            return False
-        if not (K >= 12288 or slices >= 4 or -(-N // 64) * slices <= cus or M * (ks * 2 + 16) <= 12 * 1024):
-            return False
-    return group_size & (group_size - 1) == 0 if group_size <= ks else (group_size % ks == 0 or group_size == K)
+def weight_only_error_bounds(x2d, w_exact_nk):
+    """How far a kernel that rounds the dequantised weight to x's dtype may be from the exact result
+    (w4a16_forward_f64 with round_weight=False), per output, derived from the arithmetic alone.  x2d: the smoothed
+    activations [M, K] (smoothed_rows), w_exact_nk: dequant_weight(..., dtype=None).
+
+    Rounding w to nearest in a format with p significand bits (hidden bit included) gives w(1 + d) with
+    |d| <= u = 2^-p (bf16: p = 8, u = 2^-8; fp16: p = 11, u = 2^-11), so the output moves by sum_k x'_k w_k d_k:
+      hard   u * sum_k |x'_k w_k|                       (every d_k at its limit with the worst sign)
+      likely 7 u * sqrt(sum_k (x'_k w_k)^2)             (Hoeffding for independent bounded errors: exceeded with
+                                                         probability < 2 exp(-24.5) = 5e-11 per output)
+    Returns (hard, likely) as fp64 [M, N]."""
+    u = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[x2d.dtype]
+    xa, wa = x2d.double().abs(), w_exact_nk.double().abs()
+    hard = u * (xa @ wa.t())
+    likely = 7.0 * u * torch.sqrt((xa * xa) @ (wa * wa).t())
+    return hard, likely
 
 
 # --------------------------------------------------------------------------

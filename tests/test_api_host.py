@@ -118,3 +118,46 @@ def test_operand_sizes_are_checked_before_any_launch():
         ops.mx_dequant(torch.zeros(4, 60, dtype=torch.uint8), torch.zeros(4, 2, dtype=torch.uint8), ops.MX_E4M3)
     with pytest.raises(RuntimeError, match="col_max must be"):
         ops.col_minmax(torch.zeros(4, 64), col_max=torch.zeros(63))
+
+
+def test_layout_cache_hits_for_any_number_of_layers_and_dies_with_its_sources():
+    """The operand cache of npu_weight_quant_batchmatmul (host logic only: CPU tensors, a counting converter): a model of
+    more layers than any fixed capacity, walked in the same order twice, converts every layer once; a version bump
+    converts again and replaces the old entry; freeing a source drops its entry at once; a byte cap evicts the least
+    recently used entry."""
+    import gc
+    import torch
+    from amct_amd.torch_hip import _LayoutCache
+    cache = _LayoutCache()
+    layers = [(torch.zeros(4, 8, dtype=torch.int8), torch.ones(1, 8), None) for _ in range(600)]
+    made = []
+
+    def walk():
+        for i, t in enumerate(layers):
+            cache.get(t, (0, torch.bfloat16), lambda i=i: (made.append(i), torch.zeros(8, 4))[1:])
+    walk()
+    walk()
+    assert len(made) == 600 and cache.conversions == 600 and len(cache.entries) == 600
+    # an in-place write that torch sees: converted again, the stale entry is gone
+    layers[5][0].add_(1)
+    walk()
+    assert len(made) == 601 and made[-1] == 5 and len(cache.entries) == 600
+    # the source is freed: no converted copy stays behind
+    before = cache.bytes
+    del layers[10:]
+    gc.collect()
+    assert len(cache.entries) == 10 and cache.bytes == before * 10 // 600
+    # byte cap: the least recently used entry goes first
+    small = _LayoutCache(max_bytes=3 * 8 * 4 * 4)
+    keep = [(torch.zeros(2, 2), None, None) for _ in range(5)]
+    for t in keep:
+        small.get(t, 0, lambda: (torch.zeros(8, 4),))
+    assert len(small.entries) == 3 and small.bytes == 3 * 128
+    small.get(keep[2], 0, lambda: (torch.zeros(8, 4),))            # a hit: now the most recent
+    small.get(keep[0], 0, lambda: (torch.zeros(8, 4),))            # evicts keep[3], the oldest
+    assert small.conversions == 6
+    n = small.conversions
+    small.get(keep[2], 0, lambda: (torch.zeros(8, 4),))
+    assert small.conversions == n
+    small.get(keep[3], 0, lambda: (torch.zeros(8, 4),))
+    assert small.conversions == n + 1

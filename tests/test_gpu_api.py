@@ -12,7 +12,7 @@ from amct_amd.quantize_op import utils as qutils
 from amct_amd.utils import data_utils, quant_util
 from oracle import deploy as od
 from oracle import int_quant as iq
-from util import assert_bits_equal
+from util import assert_bits_equal, check_weight_only
 
 pytestmark = pytest.mark.gpu
 
@@ -115,6 +115,16 @@ def test_awq_process_weights(dev, strategy, group, sym):
         want_q = iq.ungroup(t, w.shape).to(w.dtype)
         got = awq.do_quant(w.to(dev), s.to(dev), None if z is None else z.to(dev), strategy, group)
         assert_bits_equal(got, want_q, "do_quant")
+
+
+def module_forward_check(got, x, buf, N, K, g, scale_factor, kind):
+    """A weight-only module's forward (any leading dims) against the exact anchor, with the bound of the reading the
+    library reports for the flattened call."""
+    rows = x.numel() // K
+    query = ops.gemm_w4a16_weight_rounded if kind == 'int4' else ops.gemm_w8a16_weight_rounded
+    check_weight_only(got.reshape(rows, N), x.reshape(rows, K), buf['codes_nk'].reshape(N, K), buf['scale_w'].t(),
+                      None if buf['offset_w'] is None else buf['offset_w'].t().float(), g, buf['bias'], scale_factor,
+                      query(rows, N, K, g, x.dtype), what=kind, exact_rel=2e-5)
 
 
 def quant_module(weight, bias, **kw):
@@ -231,13 +241,8 @@ def test_w4a16_module(dev, group, sym, with_awq):
     assert mod.bias.dtype == torch.float32
     got = mod(x.to(dev))
     g = group or K
-    want = od.w4a16_forward_f64(x, buf['codes_nk'].reshape(N, K), buf['scale_w'].t(),
-                                None if buf['offset_w'] is None else buf['offset_w'].t().float(), g, buf['bias'],
-                                awq_scale)
     assert got.shape == (3, M, N)
-    err = (got.cpu().double() - want).abs()
-    tol = 1e-3 * want.abs().amax(dim=-1, keepdim=True) + want.abs() * 2.0 ** -8
-    assert (err <= tol).all()
+    module_forward_check(got, x, buf, N, K, g, awq_scale, 'int4')
     # operator-level drop-in with the reference's operand layouts gives the same result
     xs = x.to(dev) if awq_scale is None else torch.mul(x.to(dev), awq_scale.to(dev))
     out2 = torch_hip.npu_weight_quant_batchmatmul(xs.reshape(-1, K), words, sw, antiquant_offset=ow if not sym else None,
@@ -280,13 +285,7 @@ def test_weight_only_module_matrix(dev, kind, dtype, strategy, group, sym, with_
     got = mod(x.to(dev))
     assert got.shape == (2, M, N) and got.dtype == dtype
     g = group or K
-    want = od.w4a16_forward_f64(x, buf['codes_nk'].reshape(N, K), buf['scale_w'].t(),
-                                None if buf['offset_w'] is None else buf['offset_w'].t().float(), g,
-                                buf['bias'], awq_scale)
-    err = (got.cpu().double() - want).abs()
-    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
-    tol = 1e-3 * want.abs().amax(dim=-1, keepdim=True) + want.abs() * ulp
-    assert (err <= tol).all(), float((err / tol).max())
+    module_forward_check(got, x, buf, N, K, g, awq_scale, kind)
     # operator-level drop-in with the reference's operand layouts: same bits as the module
     xs = x.to(dev) if awq_scale is None else torch.mul(x.to(dev), awq_scale.to(dev))
     for _ in range(2):                                               # the second call takes the cached layouts

@@ -30,13 +30,32 @@ def _with_workspace(x, absolute, running=None):
     return cmax, cmin
 
 
+_WARM = set()
+
+
+def _warm_up(dev):
+    """The first call on a device asks the runtime for the scratch array's address (which may load the library's code
+    object): done once per device, before any call whose memory use is measured or that is captured in a graph."""
+    if dev in _WARM:
+        return
+    x = torch.zeros(4, 8, dtype=torch.float32, device=dev)
+    o = torch.empty(8, dtype=torch.float32, device=dev)
+    _lib.check(_lib.load().amct_col_minmax_noalloc(x.data_ptr(), o.data_ptr(), o.data_ptr(), 4, 8, 0, 0, _lib.F32, _stream(dev)))
+    torch.cuda.synchronize(dev)
+    _WARM.add(dev)
+
+
 def _no_alloc(x, cmax, cmin, absolute, accumulate):
-    """Outputs are allocated by the caller beforehand: the call itself must not allocate."""
+    """Outputs are allocated by the caller beforehand: the call itself must not allocate -- neither through torch's
+    caching allocator nor behind its back (the device's free memory as the runtime reports it, hipMemGetInfo)."""
     lib = _lib.load()
     rows, cols = x.shape
+    _warm_up(x.device)
     before = torch.cuda.memory_stats(x.device)["allocation.all.allocated"]
+    free_before = torch.cuda.mem_get_info(x.device)[0]
     _lib.check(lib.amct_col_minmax_noalloc(x.data_ptr(), cmax.data_ptr(), None if absolute else cmin.data_ptr(), rows,
                                            cols, int(absolute), int(accumulate), _DT[x.dtype], _stream(x.device)))
+    assert torch.cuda.mem_get_info(x.device)[0] == free_before
     assert torch.cuda.memory_stats(x.device)["allocation.all.allocated"] == before
 
 
@@ -99,3 +118,30 @@ def test_too_wide_is_rejected(dev):
     want = _with_workspace(x, False)
     assert_bits_equal(cmax, want[0], "widest max")
     assert_bits_equal(cmin, want[1], "widest min")
+
+
+def test_captured_in_a_graph_after_a_warm_up(dev):
+    """What the entry point is for: after one eager call per device (the address look-up), the call is captured in a HIP
+    graph; every replay -- with eager work and synchronisations between them, on new input values in the same buffers
+    -- gives the bits of the workspace form."""
+    _warm_up(dev)
+    g = torch.Generator().manual_seed(13)
+    x = torch.randn(1000, 2048, generator=g).to(torch.bfloat16).to(dev)
+    cmax = torch.empty(2048, dtype=torch.float32, device=dev)
+    cmin = torch.empty(2048, dtype=torch.float32, device=dev)
+    lib = _lib.load()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _lib.check(lib.amct_col_minmax_noalloc(x.data_ptr(), cmax.data_ptr(), cmin.data_ptr(), 1000, 2048, 0, 0, _lib.BF16,
+                                               _stream(dev)))
+    for i in range(4):
+        x.copy_(torch.randn(1000, 2048, generator=g).to(torch.bfloat16))         # eager work between the replays
+        cmax.fill_(-1.0)
+        cmin.fill_(-1.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = _with_workspace(x, False)
+        assert_bits_equal(cmax, want[0], "replay %d max" % i)
+        assert_bits_equal(cmin, want[1], "replay %d min" % i)

@@ -77,3 +77,37 @@ def load_int_quant_kat16():
                     "codes": torch.tensor(c["codes"], dtype=torch.int32).reshape(1, -1),
                     "dq": dec(c["dq"], fmt).reshape(1, -1), "awq_dq": dec(c["awq_dq"], fmt).reshape(1, -1)})
     return out
+
+
+def check_weight_only(out, x, codes_signed, scales, antioffset, group, bias, smooth, rounded, what="", exact_rel=1e-5):
+    """A weight-only Linear result against the EXACT anchor (dequantised weight not rounded, fp64 contraction), with the
+    bound that follows from the reading the library says it took (`rounded`: ops.gemm_w*a16_weight_rounded):
+
+      exact reading    |err| <= exact_rel * max|row| + ulp * |y|         (fp32 accumulation, one rounding of the output)
+      rounded reading  |err| <= min(hard, likely) + the same              (oracle.deploy.weight_only_error_bounds)
+                       and, against the anchor with the SAME rounding of the weight, the exact reading's bound
+
+    x may be a sample of the call's rows (then `out` holds those rows).  Returns the largest |err| / max|row| against
+    the exact anchor, for the tests that record it."""
+    import torch
+    from oracle import deploy as od
+    ulp = 2.0 ** -8 if x.dtype == torch.bfloat16 else 2.0 ** -11
+    x2 = od.smoothed_rows(x, None if smooth is None else smooth.reshape(1, -1))
+    w = od.dequant_weight(codes_signed, scales, antioffset, group, None)             # exact, fp64
+    want = od.weight_quant_matmul_f64(x2, w, bias)
+    rowmax = want.abs().amax(dim=1, keepdim=True)
+    got = out.detach().cpu().double().reshape(want.shape)
+    err = (got - want).abs()
+    base = exact_rel * rowmax + want.abs() * ulp
+    if not rounded:
+        assert (err <= base).all(), (what, "exact reading", float((err / base).max()))
+    else:
+        hard, likely = od.weight_only_error_bounds(x2, w)
+        tol = torch.minimum(hard, likely) + base
+        assert (err <= tol).all(), (what, "rounded reading against the exact anchor", float((err / tol).max()))
+        # (q - z) * s is exact in fp32 (at most 9 x 11 bits), so one rounding of the fp64 value is the kernel's rounding
+        own = od.weight_quant_matmul_f64(x2, w.to(x.dtype), bias)
+        err_own = (got - own).abs()
+        base_own = exact_rel * own.abs().amax(dim=1, keepdim=True) + own.abs() * ulp
+        assert (err_own <= base_own).all(), (what, "rounded reading against its own anchor", float((err_own / base_own).max()))
+    return float((err / rowmax.clamp_min(1e-300)).max())
