@@ -28,19 +28,41 @@ FLAGS = [
 # iteration): a register spill would add scratch loads and stores to that count and make them read registers before
 # their data has landed.  The build refuses such a kernel instead of shipping it.
 NO_SPILL = ("w8a8_tile_", "w4a16_tile_")
+# Kernels that are built around "every load of a wave in flight at once" at a fixed register budget (16 waves per
+# block: 128 registers).  A spill there costs speed, not correctness: reported, the build goes on.
+REPORT_SPILL = ("_stream<",)
+_TAG = "[-Rpass-analysis=kernel-resource-usage]"
 
 
-def _spilling_kernels(remarks):
-    """Names of NO_SPILL kernels for which the compiler reports spilled vector registers or scratch memory."""
+def _spilling_kernels(remarks, families=NO_SPILL):
+    """Names of kernels of `families` for which the compiler reports spilled vector registers or scratch memory."""
     bad, name = [], None
     for line in remarks.splitlines():
         if "Function Name:" in line:
             name = line.split("Function Name:")[1].split("[")[0].strip()
-        elif name and any(k in name for k in NO_SPILL):
+        elif name and any(k in name for k in families):
             for key in ("VGPRs Spill:", "ScratchSize [bytes/lane]:"):
                 if key in line and int(line.split(key)[1].split("[")[0].strip()) != 0:
                     bad.append("{} ({} {})".format(name, key, line.split(key)[1].split("[")[0].strip()))
     return sorted(set(bad))
+
+
+def _without_resource_remarks(text):
+    """Compiler output minus the resource-usage remarks and their source-context lines; warnings and errors keep
+    theirs."""
+    keep, skipping = [], False
+    for line in text.splitlines():
+        if _TAG in line:
+            skipping = True
+            continue
+        if "warning:" in line or "error:" in line or "note:" in line:
+            skipping = False
+        elif skipping and (line.strip().startswith(("|", "^")) or " | " in line or "__launch_bounds__" in line or not line.strip()):
+            continue
+        else:
+            skipping = False
+        keep.append(line)
+    return "\n".join(keep)
 
 
 def _compile(src):
@@ -53,7 +75,10 @@ def _compile(src):
         bad = _spilling_kernels(out)
         if bad:
             return src, obj, 1, "kernels with hand-counted waits must not spill:\n  " + "\n  ".join(bad)
-        out = "\n".join(l for l in out.splitlines() if "remark:" not in l and "__launch_bounds__" not in l and not l.strip().startswith(("|", "^")))
+        slow = _spilling_kernels(out, REPORT_SPILL)
+        out = _without_resource_remarks(out)
+        if slow:
+            out += "\nwarning: weight-streaming kernels that spill (slower, still correct):\n  " + "\n  ".join(slow)
     return src, obj, p.returncode, out
 
 

@@ -12,7 +12,11 @@ from .utils import calculate_scale_offset, get_weight_min_max_by_granularity
 
 @torch.no_grad()
 def update_hessian(hessian, nsamples, input_data, columns):
-    """:161-186.  Returns (hessian, nsamples); the matrix stays on the device instead of moving to the host."""
+    """:161-186.  Returns (hessian, nsamples); the matrix stays on the device instead of moving to the host.
+    For bf16 / fp16 activations on the device the update runs in place: the returned tensor IS the `hessian` passed in
+    (the reference and the fp32 branch below build a new tensor per call) -- pass a clone to keep the earlier value.
+    That branch applies 2 / n to the fp32 sum of exact products instead of scaling every element by sqrt(2 / n) first,
+    so it matches the reference to fp32 rounding, not bit for bit."""
     if len(input_data.shape) == 2:
         input_data = input_data.unsqueeze(0)
     batch_size = input_data.shape[0]

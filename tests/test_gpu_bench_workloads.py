@@ -41,12 +41,13 @@ def test_config4_dynamic_quant_then_w8a8_at_bench_size(dev, c4, M):
     assert_bits_equal(out.cpu()[rows], od.quant_matmul(want_q[rows], wq.t(), sw, want_s[rows], None, torch.bfloat16), "w8a8 out")
 
 
-# Largest deviation from the exact anchor, as a fraction of the row's largest output, that the tests below allow
-# on config 5 (K = 4096, N(0, 1) activations, fp16 scales in [1e-3, 1e-2]) beyond the per-output bound of
-# tests.util.check_weight_only:
-#   exact reading (M <= 16)   fp32 accumulation and the output's rounding only: measured 1e-6 .. 4e-6, allowed 1e-5
-#   rounded reading (M > 16)  bf16 weight, u = 2^-8: about u / sqrt(3) * sqrt(K) * rms(x'w) against a row maximum of
-#                             about 4.5 * sqrt(K) * rms(x'(w - mean)), measured 2.0e-3 .. 2.3e-3, allowed 3e-3.
+# Largest deviation from the exact anchor, as a fraction of the row's largest output and not counting the rounding of
+# the bf16 output itself, that the tests below allow on config 5 (K = 4096, N(0, 1) activations, fp16 scales in
+# [1e-3, 1e-2]) on top of the per-output bound of tests.util.check_weight_only:
+#   exact reading (M <= 16)   fp32 accumulation only: allowed 1e-5
+#   rounded reading (M > 16)  bf16 weight, u = 2^-8: each weight moves by up to u, about u / sqrt(3) on average, and
+#                             the 4096 moves add up like a random walk; on these tensors the two anchors differ by up
+#                             to 2.6e-3 of the row's largest output (mean over rows of the largest: 1.8e-3), allowed 3e-3.
 #                             This is NOT within the 1e-3 the operator is asked for: a deviation that is stated, not hidden.
 C5_ROWMAX_FRACTION = {False: 1e-5, True: 3e-3}
 
@@ -93,8 +94,8 @@ def test_config5_same_tokens_through_a_decode_and_a_prefill_call(dev, c5):
     """One module serves a token through the weight-streaming kernel in a call of up to 16 rows (exact weights) and
     through a tile kernel in a larger call (weights rounded to bf16).  The first 16 rows of config 5 through both:
     each within its own bound of the exact anchor (the tests above), and the two within the SUM of those bounds of each
-    other -- the difference a caller sees between decode and prefill for the same token, up to 3e-3 of the row's
-    largest output at K = 4096."""
+    other -- the difference a caller sees between decode and prefill for the same token: up to 3e-3 of the row's
+    largest output at K = 4096 from the weight rounding, plus the rounding of the two bf16 outputs."""
     from oracle import deploy as od
     x, codes, scales, zeros, smooth_recip = c5
     packed = workloads.pack_nibbles(codes).to(dev)
@@ -109,7 +110,9 @@ def test_config5_same_tokens_through_a_decode_and_a_prefill_call(dev, c5):
     tol = torch.minimum(hard, likely) + 2 * (1e-5 * rowmax + want.abs() * 2.0 ** -8)
     diff = (small - large).abs()
     assert (diff <= tol).all(), float((diff / tol).max())
-    assert float((diff / rowmax).max()) <= 3e-3
+    # not counting the two roundings of the bf16 outputs: the weight rounding alone, as a fraction of the row maximum
+    beyond = ((diff - 2 * want.abs() * 2.0 ** -8).clamp_min(0.0) / rowmax).max()
+    assert float(beyond) <= C5_ROWMAX_FRACTION[True], float(beyond)
     assert float((diff / rowmax).max()) > 1e-4, "the two calls are expected to differ: one of them does not round the weight"
 
 

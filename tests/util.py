@@ -87,8 +87,9 @@ def check_weight_only(out, x, codes_signed, scales, antioffset, group, bias, smo
       rounded reading  |err| <= min(hard, likely) + the same              (oracle.deploy.weight_only_error_bounds)
                        and, against the anchor with the SAME rounding of the weight, the exact reading's bound
 
-    x may be a sample of the call's rows (then `out` holds those rows).  Returns the largest |err| / max|row| against
-    the exact anchor, for the tests that record it."""
+    x may be a sample of the call's rows (then `out` holds those rows).  Returns, for the tests that state it, the
+    largest deviation from the exact anchor as a fraction of the row's largest output, not counting the rounding of
+    the output itself: max((|err| - ulp * |y|)+ / max|row|)."""
     import torch
     from oracle import deploy as od
     ulp = 2.0 ** -8 if x.dtype == torch.bfloat16 else 2.0 ** -11
@@ -110,4 +111,4 @@ def check_weight_only(out, x, codes_signed, scales, antioffset, group, bias, smo
         err_own = (got - own).abs()
         base_own = exact_rel * own.abs().amax(dim=1, keepdim=True) + own.abs() * ulp
         assert (err_own <= base_own).all(), (what, "rounded reading against its own anchor", float((err_own / base_own).max()))
-    return float((err / rowmax.clamp_min(1e-300)).max())
+    return float(((err - want.abs() * ulp).clamp_min(0.0) / rowmax.clamp_min(1e-300)).max())
