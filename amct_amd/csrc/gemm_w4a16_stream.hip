@@ -12,80 +12,19 @@
 // each group of `group` columns is accumulated on its own (P = sum x' * (16 + u), fp32) and folded into the result
 // as acc += s * P - s * (16 + z) * X with X = sum of the group's x' (computed once per block while staging).  That is
 // sum x' * (u - z) * s with the dequantised weight NOT rounded to bf16 -- the fp32 `weight * scale` of the reference's
-// CPU stand-in for this operator (tests/amct_pytorch/mock_torch_npu.py:33-55) -- whereas the tile kernels for larger M
-// feed bf16((u - z) * s) to the matrix pipe; both are within the 1e-3 tolerance of the fp64 result, this one closer.
+// CPU stand-in for this operator (tests/amct_pytorch/mock_torch_npu.py:33-55): within 1e-5 of the row's largest output
+// (plus the rounding of the output) of the exact result.  The tile kernels for larger M feed bf16((u - z) * s) to the
+// matrix pipe, which moves an output by up to 2^-8 * sum |x' w| (2.6e-3 of the row's largest output on W[14336,4096]
+// with N(0,1) activations): the two readings are NOT within 1e-3 of each other at K = 4096, and
+// amct_gemm_w4a16_weight_rounded says which one a call takes.
 // The partial sums of the KS waves are added in wave order, so the result does not depend on the launch shape
 // beyond KS.
 #include "amct_common.h"
 #include "gemm_plan.h"
+#include "w4a16_stream_act.h"
 
 namespace amct {
 
-typedef float s4f __attribute__((ext_vector_type(4)));
-typedef __bf16 s8bf __attribute__((ext_vector_type(8)));
-typedef __bf16 s2bf __attribute__((ext_vector_type(2)));
-typedef float s2f __attribute__((ext_vector_type(2)));
-
-struct StreamArgs {
-    const uint16_t* x;
-    const uint16_t* smooth;
-    const uint8_t* wq;
-    const uint16_t* scales;
-    const uint8_t* zeros;
-    const float* bias;
-    const float* bias_src;                           // bias, or any readable N floats when there is none
-    uint16_t* out;
-    int M, N, K, G;                                  // K: elements of a row one block walks (a slice); G = K / group
-    int group;
-    int scale_f16;
-    uint32_t kv_magic;                               // floor(2^32 / (K / 8)) + 1: v / (K / 8) == mulhi(v, magic)
-    // Rows longer than a slice: blockIdx.y picks the slice; rows keep their full length as stride; every slice leaves
-    // fp32 partial sums part[slice][M][N] that a second kernel adds in slice order (plus bias, rounding to the output type)
-    int row_k;                                       // elements of a full row of x and of the weight
-    float* part;                                     // null: one slice, the result goes to `out`
-};
-
-typedef _Float16 s8h __attribute__((ext_vector_type(8)));
-
-// what differs between the two activation types: the pack, the unpack, the bit pattern of the integer 16 + u, the MFMA
-template <int DT> struct StAct;
-template <> struct StAct<AMCT_BF16> {
-    static AMCT_DEV uint32_t pack2(float lo, float hi) {
-        const s2f f = {lo, hi};
-        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, s2bf));      // v_cvt_pk_bf16_f32, round-half-even
-    }
-    static AMCT_DEV float lo(uint32_t w) { return __uint_as_float(w << 16); }
-    static AMCT_DEV float hi(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
-    // 8 nibbles of w (nibble p = weight k0 + p) -> 4 words of two integers 16 + u each, word j = (weight j, weight j + 4)
-    static AMCT_DEV uint4 int8x(uint32_t w) {
-        constexpr uint32_t kMask = 0x00780078u, kBase = 0x41804180u;   // bf16(16 + u) = 0x4180 | u << 3
-        return make_uint4(((w << 3) & kMask) | kBase, ((w >> 1) & kMask) | kBase, ((w >> 5) & kMask) | kBase,
-                          ((w >> 9) & kMask) | kBase);
-    }
-    static AMCT_DEV s4f mfma(const uint4& a, const uint4& b, s4f c) {
-        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(s8bf, a), __builtin_bit_cast(s8bf, b), c, 0, 0, 0);
-    }
-    static AMCT_DEV uint32_t out_bits(float v) { return f32_to_bf16_bits(v); }
-};
-template <> struct StAct<AMCT_F16> {
-    static AMCT_DEV uint32_t pack2(float lo, float hi) { return f32_to_f16_bits(lo) | (f32_to_f16_bits(hi) << 16); }
-    static AMCT_DEV float lo(uint32_t w) { return f16_bits_to_f32(w & 0xFFFFu); }
-    static AMCT_DEV float hi(uint32_t w) { return f16_bits_to_f32(w >> 16); }
-    static AMCT_DEV uint4 int8x(uint32_t w) {
-        constexpr uint32_t kMask = 0x03C003C0u, kBase = 0x4C004C00u;   // f16(16 + u) = 0x4C00 | u << 6
-        return make_uint4(((w << 6) & kMask) | kBase, ((w << 2) & kMask) | kBase, ((w >> 2) & kMask) | kBase,
-                          ((w >> 6) & kMask) | kBase);
-    }
-    static AMCT_DEV s4f mfma(const uint4& a, const uint4& b, s4f c) {
-        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(s8h, a), __builtin_bit_cast(s8h, b), c, 0, 0, 0);
-    }
-    static AMCT_DEV uint32_t out_bits(float v) { return f32_to_f16_bits(v); }
-};
-// the matching order of 8 activations: (k0, k4), (k1, k5), (k2, k6), (k3, k7)
-AMCT_DEV uint4 st_interleave8(const uint4& x) {
-    return make_uint4(__builtin_amdgcn_perm(x.z, x.x, 0x05040100u), __builtin_amdgcn_perm(x.z, x.x, 0x07060302u),
-                      __builtin_amdgcn_perm(x.w, x.y, 0x05040100u), __builtin_amdgcn_perm(x.w, x.y, 0x07060302u));
-}
 template <int DT>
 AMCT_DEV float st_sum8(const uint4& x) {
     const uint32_t xs[4] = {x.x, x.y, x.z, x.w};
@@ -173,6 +112,8 @@ AMCT_DEV void st_compute_tile(const StreamArgs& a, StTile<NL>& t, int n0, int cg
     const int r16 = lane & 15, g = lane >> 4;
     const int M = a.M;
     s4f acc = {0.f, 0.f, 0.f, 0.f}, P = {0.f, 0.f, 0.f, 0.f};
+    uint32_t km = StAct<DT>::kMask, kb = StAct<DT>::kBase;
+    asm volatile("" : "+v"(km), "+v"(kb));           // in registers: (x & m) | b is then one instruction per word
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
         // the loads retire in order: step i waits for wv[i] only, the younger ones stay in flight
@@ -191,7 +132,7 @@ AMCT_DEV void st_compute_tile(const StreamArgs& a, StTile<NL>& t, int n0, int cg
         const uint32_t ws[4] = {t.wv[i].x, t.wv[i].y, t.wv[i].z, t.wv[i].w};
 #pragma unroll
         for (int s4 = 0; s4 < 4; ++s4)
-            P = StAct<DT>::mfma(fa[s4], StAct<DT>::int8x(ws[s4]), P);
+            P = StAct<DT>::mfma(fa[s4], StAct<DT>::int8x(ws[s4], km, kb), P);
         {                                             // a step is one group of 128: fold it into the result
             const uint32_t gi = (ks * kw) / 128 + i;
             const uint32_t sbits = (t.fsw[i / 2] >> (16 * (i & 1))) & 0xFFFFu;
@@ -338,6 +279,8 @@ __global__ __launch_bounds__(KS * CG * 64) void w4a16_stream(StreamArgs a) {
 
 int splitk_reduce16_launch(const float* part, const float* bias, void* out, int64_t M, int64_t N, int splits, int dtype,
                            hipStream_t st);                          // gemm_w4a16.hip
+bool w4a16_wave_fits(int64_t N, int64_t K_slice, int64_t slices);    // gemm_w4a16_wave.hip: the form with wave-private staging
+int w4a16_wave_launch(const StreamArgs& a, int slices, int dtype, hipStream_t st);
 
 template <int DT, int KS, int CG, int NL, bool SMOOTH, bool LOOP>
 static int stream_launch_x(const StreamArgs& a, size_t lds_bytes, dim3 blocks, hipStream_t st) {
@@ -422,6 +365,15 @@ int w4a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, 
                  bias ? bias : reinterpret_cast<const float*>(scales),   // N * K / group * 2 >= N * 4 bytes (K >= 1024)
                  (uint16_t*)out, (int)M, (int)N, (int)K, (int)(K / group), group, scale_dtype == AMCT_F16 ? 1 : 0,
                  (uint32_t)(0x100000000ull / (uint64_t)(K / 8)) + 1u, (int)K_row, part};
+    // launches whose blocks all run at once: every wave stages its own 256 elements of K (gemm_w4a16_wave.hip)
+    // Taken where it measured faster than the form below (us on W[14336,4096] / W[4096,4096] / W[8192,8192], this form
+    // against that one): with smoothing M = 5: 10.7 / 10.5 / 13.4 against 10.9 / 10.2 / 13.4, M = 8: 10.8 / 10.6 / 13.4
+    // against 11.2 / 10.4 / 13.9, M = 16: 11.4 / 10.9 / 14.1 against 13.2 / 12.5 / 16.0; without smoothing M = 12:
+    // 11.0 / 10.8 / 14.1 against 11.4 / 10.8 / 14.1, M = 16: 11.2 / 10.9 / 14.1 against 11.9 / 11.1 / 14.8.  Below that the
+    // narrow blocks of the form below win (M = 1: 8.5 against 10.2 us: a block of this form is a whole CU's work however
+    // few rows there are); slices shorter than 4096 (W[4096,14336]: 7 x 2048) stay below as well (M = 16: 15.2 against 15.9).
+    if ((smooth ? M >= 5 : M >= 12) && (S == 1 || K == 4096) && w4a16_wave_fits(N, K, S))
+        return w4a16_wave_launch(a, (int)S, dtype, st);
     // A wave streams K / 4 elements of 16 columns in NL = K / 512 steps, all of them in flight from the start.  Large
     // activation blocks are staged by few, wide blocks (16 waves share one copy in LDS); small ones by many narrow
     // blocks, several per CU.  Measured on W[14336,4096]: 8.8 us at M = 1 (11.0 us for the kernel this one replaced),
