@@ -30,16 +30,46 @@ npu = _Npu()
 
 
 def npu_quantize(input, scales, zero_points=None, dtype=torch.int8, axis=-1, div_mode=False):
-    """int8 = saturate(round_half_even(input * scales + zero_points)) (div_mode=False) or
-    input / scales (div_mode=True is not used by the reference's deploy path)."""
+    """int8 = saturate(round_half_even(input * scales + zero_points)) with div_mode=False -- the call of
+    amct_pytorch/deploy_op/npu_quantization_linear.py:98-99 -- or of input / scales + zero_points with div_mode=True
+    (the operator's default; signature in tests/amct_pytorch/mock_torch_npu.py:69-70).  One scale per tensor, or one per
+    index of `axis` (the last dim's neighbour, -2: per token).  The arithmetic inside torch_npu is not vendored:
+    this library multiplies / divides and adds in fp32 (the division is the exactly rounded one of the weight
+    quantiser, amct_quant_with_params) and rounds once.  Only dtype=torch.int8."""
     if dtype != torch.int8:
         raise RuntimeError("npu_quantize: only dtype=torch.int8 is supported")
-    if div_mode:
-        raise RuntimeError("npu_quantize: div_mode=True is not supported")
     if axis not in (-1, -2, input.dim() - 1, input.dim() - 2):
         raise RuntimeError("npu_quantize: axis must address one of the last two dims")
     per_token = axis in (-2, input.dim() - 2)
-    return ops.quantize_static(input, scales, zero_points, per_token)
+    if not div_mode:
+        return ops.quantize_static(input, scales, zero_points, per_token)
+    if input.dim() < 2:
+        raise RuntimeError("npu_quantize: the input must have at least two dims")
+    K = input.shape[-1]
+    x2 = input.reshape(-1, K)
+    n = scales.numel()
+    zp = None
+    if zero_points is not None:
+        zf = zero_points.reshape(-1).to(torch.float32)
+        zp = zf.round().to(torch.int32)
+        if not torch.equal(zp.to(torch.float32), zf):
+            raise RuntimeError("npu_quantize: div_mode=True takes integer zero_points")
+        if zp.numel() != n:
+            raise RuntimeError("npu_quantize: {} zero_points for {} scales".format(zp.numel(), n))
+    sc = scales.reshape(-1).to(torch.float32)
+    if n == 1:
+        group = -1                                   # one scale for the tensor
+    elif per_token and n == input.shape[-2]:
+        group = 0                                    # one per token, shared by every leading batch index
+        reps = x2.shape[0] // n
+        if reps > 1:
+            sc = sc.repeat(reps)
+            zp = None if zp is None else zp.repeat(reps)
+    else:
+        raise RuntimeError("npu_quantize: div_mode=True takes one scale per tensor or one per token, got {} scales "
+                           "for an input of shape {}".format(n, tuple(input.shape)))
+    _, codes = ops.quant_with_params(x2, sc, zp, group, -128, 127, want_dq=False, codes_kind=ops.CODES_I8)
+    return codes.reshape(input.shape)
 
 
 def _weight_nk(x2):

@@ -43,9 +43,13 @@ MEASURED_TRAFFIC = {
     "w8a8_m2048": ("w8a8_tile_mix16<2, 0>", 255069388),
     "w8a8_m16": ("w8a8_stream<2, 4, 4, 16, 4, 0>", 59805700),
     "w8a8_linear_m16": ("w8a8_stream<2, 4, 4, 16, 8, 2>", 60417600),
-    "w4a16_m2048": ("w4_dequant_rows<false> + smooth_rows + w8a8_tile_mix16<2, 1>", 632207001),
-    "w4a16_m16": ("w4a16_stream<2, 4, 4, 8, 8, true, false>", 32535100),
-    "w4a16_m1": ("w4a16_stream<2, 4, 1, 8, 2, true, false>", 31110041),
+    "w4a16_m2048": ("w4_dequant_rows<false> + w8a8_tile_mix16<2, 1>", 632207001),
+    "w4a16_m2048_fused": ("smooth_rows + w4a16_tile_wide16<true, 2, 4, 4, 2, 2, 2, false>", 303595344),
+    "w4a16_m16": ("w4a16_wave<2, true, true, 8>", 32471413),
+    "w4a16_m1": ("w4a16_stream<2, 4, 1, 8, 2, true, false>", 31100571),
+    "w8a16_m16": ("w8a16_stream<2, 4, 8, 8, 1, false>", 60426092),
+    "w8a16_m2048": ("w8_dequant_rows<2> + w8a8_tile_mix16<2, 1>", 659261016),
+    "w8a8_down_m16": ("w8a8_tile_shape<2, 2, 2, 1, 1, 4, 128> + w8a8_splitk_reduce<2>", 62957888),
     "w4a16_down_m16": ("w4a16_stream<2, 4, 4, 4, 4, false, true> + splitk_reduce16<false>", 39848448),
     "w8a16_down_m16": ("w8a16_stream<2, 4, 4, 4, 1, false> + splitk_reduce16<false>", 67237581),
 }
@@ -369,20 +373,23 @@ def build_cases(dev, only):
                                   "dynamic per-token quantise + W8A8 Linear, M=%d (decode), two launches" % M6))
 
     # ---- K7: W4A16 Linear, W[14336,4096] int4 g128 ------------------------------------------------------
-    if want("w4a16_m2048") or want("w4a16_m16") or want("w4a16_m1"):
+    if want("w4a16_m2048") or want("w4a16_m2048_fused") or want("w4a16_m16") or want("w4a16_m1"):
         x7, codes7, sc7, z7, smr7 = workloads.c5_w4a16(2048)
         N7, K7 = codes7.shape
         g7 = 128
         nw7 = 12                                         # 12 x 29.4 MB of packed weights rotate
         pk7 = dev_copies(workloads.pack_nibbles(codes7), nw7)
         scd, zd, smd = sc7.to(dev), z7.to(dev), smr7.to(dev)
-        for name, M7 in (("w4a16_m2048", 2048), ("w4a16_m16", 16), ("w4a16_m1", 1)):
+        for name, M7 in (("w4a16_m2048", 2048), ("w4a16_m2048_fused", 2048), ("w4a16_m16", 16), ("w4a16_m1", 1)):
             if not want(name):
                 continue
+            fused = name.endswith("_fused")
             xd = x7[:M7].contiguous().to(dev)
             outs7 = [torch.empty(M7, N7, dtype=torch.bfloat16, device=dev) for _ in range(nw7)]
             # the workspace the library asks for: the smoothed activations and, from 1025 rows on, the 16-bit weight
-            ws7 = torch.empty(max(16, lib.amct_gemm_w4a16_workspace_bytes(M7, N7, K7, g7, 1)), dtype=torch.uint8, device=dev)
+            # (the fused form: only the smoothed activations, M * K * 2 bytes -- the library then dequantises inside every tile)
+            ws7 = torch.empty(M7 * K7 * 2 if fused else max(16, lib.amct_gemm_w4a16_workspace_bytes(M7, N7, K7, g7, 1)),
+                              dtype=torch.uint8, device=dev)
 
             def launch(i, xd=xd, outs7=outs7, M7=M7, pk7=pk7, scd=scd, zd=zd, smd=smd, N7=N7, K7=K7, g7=g7, ws7=ws7):
                 j = i % len(pk7)
@@ -391,10 +398,16 @@ def build_cases(dev, only):
                                          ws7.data_ptr(), ws7.numel(), st)
                 assert rc == 0, rc
             wbytes = N7 * K7 // 2 + N7 * (K7 // g7) * 3
-            if M7 >= 256:
+            if fused:
                 cases.append(Case(name, "mfma_bf16", 2 * M7 * N7 * K7, "flop", launch, nw7, "bf16",
-                                  "W4A16 Linear M=%d N=14336 K=4096, group 128, with smoothing (config 5): the weight dequantised once into the "
-                                  "lent workspace + smoothing pre-pass + 16-bit GEMM on the 256x256 tiles" % M7))
+                                  "W4A16 Linear M=%d N=14336 K=4096, group 128, with smoothing (config 5), dequantisation FUSED into the "
+                                  "GEMM's main loop (the form a call without the 117 MB weight workspace takes): smoothing pre-pass "
+                                  "(smooth_rows) + w4a16_tile_wide16 on 256x256 tiles" % M7))
+            elif M7 >= 256:
+                cases.append(Case(name, "mfma_bf16", 2 * M7 * N7 * K7, "flop", launch, nw7, "bf16",
+                                  "W4A16 Linear M=%d N=14336 K=4096, group 128, with smoothing (config 5), as ops.gemm_w4a16 runs it: two "
+                                  "launches -- w4_dequant_rows (the weight dequantised once into the lent workspace, the activations "
+                                  "smoothed by the same launch) + the 16-bit GEMM w8a8_tile_mix16<bf16> on 256x256 / 256x192 tiles" % M7))
             else:
                 cases.append(Case(name, "hbm", wbytes + M7 * K7 * 2 + M7 * N7 * 2, "B", launch, nw7, "bf16",
                                   "W4A16 Linear M=%d (decode): weight streaming (config 5)" % M7))

@@ -161,3 +161,29 @@ def test_layout_cache_hits_for_any_number_of_layers_and_dies_with_its_sources():
     assert small.conversions == n
     small.get(keep[3], 0, lambda: (torch.zeros(8, 4),))
     assert small.conversions == n + 1
+
+
+def test_weight_rounding_queries_answer_without_a_gpu():
+    """amct_gemm_w4a16_weight_rounded / amct_gemm_w8a16_weight_rounded are host logic: which reading of the dequantised
+    weight a call takes follows from its shape, dtype and workspace size alone."""
+    from amct_amd import _lib
+    lib = _lib.load()
+    q4, q8 = lib.amct_gemm_w4a16_weight_rounded, lib.amct_gemm_w8a16_weight_rounded
+    for dt in (_lib.BF16, _lib.F16):
+        for M in (1, 2, 5, 16):
+            for K in (1024, 2048, 4096):
+                assert q4(M, 14336, K, 128, dt, 0) == 0                 # the weight-streaming kernels keep the integer weight
+                assert q8(M, 14336, K, 128, dt, 0) == 0
+                assert q8(M, 14336, K, K, dt, 0) == 0                   # per-channel factors
+        for M in (17, 64, 256, 1024, 2048):
+            assert q4(M, 14336, 4096, 128, dt, 1 << 30) == 1            # every tile kernel rounds it to the activation dtype
+            assert q8(M, 14336, 4096, 128, dt, 1 << 30) == 1
+        assert q4(16, 14336, 4096, 64, dt, 0) == 1                      # groups the streaming kernel does not take
+        assert q4(16, 14336, 4000, 100, dt, 0) == 1
+    # long rows walk slices whose partial sums need the lent workspace: without it another (rounding) kernel serves the call
+    need = lib.amct_gemm_w4a16_workspace_bytes(16, 4096, 14336, 128, 0)
+    assert need >= 7 * 16 * 4096 * 4
+    assert q4(16, 4096, 14336, 128, _lib.BF16, need) == 0 and q4(16, 4096, 14336, 128, _lib.BF16, 0) == 1
+    # what the GEMM entry points reject, the queries reject
+    assert q4(16, 0, 4096, 128, _lib.BF16, 0) < 0 and q4(16, 64, 4096, 0, _lib.BF16, 0) < 0
+    assert q4(16, 64, 4096, 128, _lib.F32, 0) < 0 and q8(16, 64, 4096, 128, _lib.F32, 0) < 0

@@ -356,6 +356,35 @@ def test_dispatcher_operators(dev):
         torch.ops.amct_hip.convert_weight_to_int4pack(codes)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_npu_quantize_div_mode(dev, dtype):
+    """npu_quantize(div_mode=True), the operator's default mode (tests/amct_pytorch/mock_torch_npu.py:69-76: input / scales
+    + zero_points): one scale per tensor or per token, with and without integer zero-points, leading batch dims; the
+    codes are those of the weight quantiser's division (oracle.int_quant.quant_codes: fp32 x / s + z, round half even,
+    saturate), bit for bit, and differ from the reciprocal-multiply mode only where that mode's rounded reciprocal moves
+    a value across a rounding boundary."""
+    g = torch.Generator().manual_seed(91)
+    x = (torch.randn(2, 9, 192, generator=g) * 40).to(dtype)
+    x[0, 0, :4] = torch.tensor([1e4, -1e4, 0.5 * 0.37, -0.0]).to(dtype)          # saturation both ways
+    s1 = torch.tensor([0.37], dtype=dtype)
+    st = (0.2 + torch.rand(9, generator=g)).to(dtype)
+    zt = torch.randint(-20, 21, (9,), generator=g).to(dtype)
+    for scales, zp, axis in ((s1, None, -1), (s1, torch.tensor([3.0]).to(dtype), -1), (st, None, -2), (st, zt, -2)):
+        got = torch_hip.npu_quantize(x.to(dev), scales.to(dev), None if zp is None else zp.to(dev), torch.int8, axis, True)
+        assert got.dtype == torch.int8 and got.shape == x.shape
+        sc = scales.float().reshape(-1)
+        z = None if zp is None else zp.float().round().to(torch.int32).reshape(-1)
+        if sc.numel() == 1:
+            want = iq.quant_codes(x.reshape(-1, 192), 'int8', sc.reshape(1, 1), None if z is None else z.reshape(1, 1))
+        else:
+            want = iq.quant_codes(x.reshape(-1, 192), 'int8', sc.repeat(2).reshape(-1, 1), None if z is None else z.repeat(2).reshape(-1, 1))
+        assert torch.equal(got.cpu().reshape(-1, 192), want.to(torch.int8)), (axis, zp is not None)
+    with pytest.raises(RuntimeError, match="integer zero_points"):
+        torch_hip.npu_quantize(x.to(dev), s1.to(dev), torch.tensor([0.5]).to(dev), torch.int8, -1, True)
+    with pytest.raises(RuntimeError, match="one scale per tensor or one per token"):
+        torch_hip.npu_quantize(x.to(dev), torch.ones(5, dtype=dtype).to(dev), None, torch.int8, -2, True)
+
+
 class _TwoLinears(torch.nn.Module):
     """Two linears on the same input, as the q/k/v projections of a block share theirs."""
 
