@@ -5,13 +5,15 @@
 // A block owns CG groups of 16 output columns; 4 waves per column group split K.
 // Arithmetic: x' = dt(x * smooth) as everywhere.  A weight enters the MFMA as the EXACT integer u = q + 128 in
 // 0 .. 255 (one v_cvt_f32_ubyte per weight and one pack per pair; 255 needs 8 significant bits, which both 16-bit
-// types have), every span of K that shares a scale is accumulated on its own (P = sum x' * u, fp32) and folded into
-// the result as acc += s * P - s * (offset + 128) * X with X = the sum of the span's x' (one sum per 128 elements of
-// K and row, computed once per block while staging).  That is sum x' * (q - offset) * s with the dequantised weight
-// NOT rounded to 16 bits -- the fp32 `weight * scale` of the reference's CPU stand-in for this operator
+// types have), and the offset leaves on the matrix pipe as well: behind every weight MFMA a second one multiplies the
+// same activations with the constant -(128 + offset) of the lane's column (0 .. 255 too, exact), so the accumulators
+// of a span of K that shares a scale hold P = sum x' * (q - offset) (fp32) and the fold is acc += s * P -- no sums of
+// activations are needed anywhere.  That is sum x' * (q - offset) * s with the dequantised weight NOT rounded to 16
+// bits -- the fp32 `weight * scale` of the reference's CPU stand-in for this operator
 // (tests/amct_pytorch/mock_torch_npu.py:33-55) -- whereas the tile kernels for larger M feed dt((q - offset) * s) to the
-// matrix pipe; both are within the 1e-3 tolerance of the fp64 result.  Groups of 128, 256, ... up to the whole of K
-// (per-channel and per-tensor factors) are spans of whole steps.
+// matrix pipe, which moves an output by up to 2^-8 (bf16; fp16: 2^-11) of sum |x' w|: amct_gemm_w8a16_weight_rounded tells
+// which of the two a call takes.  Groups of 128, 256, ... up to the whole of K (per-channel and per-tensor factors) are
+// spans of whole steps.
 #include "amct_common.h"
 #include "gemm_plan.h"
 
@@ -81,14 +83,6 @@ AMCT_DEV uint4 w8_expand(uint32_t w0, uint32_t w1) {
 }
 
 template <int DT>
-AMCT_DEV float w8_sum8(const uint4& x) {
-    const uint32_t xs[4] = {x.x, x.y, x.z, x.w};
-    float t = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) t = t + (W8Act<DT>::lo(xs[i]) + W8Act<DT>::hi(xs[i]));
-    return t;
-}
-template <int DT>
 AMCT_DEV uint4 w8_smooth8(const uint4& x, const uint4& c) {
     const uint32_t xs[4] = {x.x, x.y, x.z, x.w}, cs[4] = {c.x, c.y, c.z, c.w};
     uint32_t o[4];
@@ -114,9 +108,7 @@ __global__ __launch_bounds__(4 * CG * 64) void w8a16_stream(Stream16Args a) {
     const int n0 = blockIdx.x * COLS;
     const uint32_t K = (uint32_t)a.K, M = (uint32_t)a.M;
     const uint32_t xstride = K * 2 + 16;             // 16 bytes of padding: the 16 rows of a fragment read hit different banks
-    const uint32_t xbytes = M * xstride;
     uint8_t* xs = lds;
-    float* xsum = reinterpret_cast<float*>(lds + xbytes);   // [K / 128][16]: sum of x' per step and row
 
     // ---- staging loads (activations, smoothing factors) ------------------------------------------------------------
     const uint32_t KV = K / 8, n_xv = M * KV;
@@ -177,21 +169,12 @@ __global__ __launch_bounds__(4 * CG * 64) void w8a16_stream(Stream16Args a) {
         wv[2 * i + 1] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(whi + i * 128));
     }
     __builtin_amdgcn_sched_barrier(0);
-    // ---- stage the activations: smoothed, summed per step of 128 --------------------------------------------------
+    // ---- stage the activations, smoothed ----------------------------------------------------------------------------
 #pragma unroll
     for (int j = 0; j < XJ; ++j) {
         const uint32_t v = tid + NT * j;
         if constexpr (SMOOTH) xv[j] = w8_smooth8<DT>(xv[j], cv[j % CVN]);
-        // 16 consecutive lanes hold 128 consecutive elements of one row; whole groups of 16 lanes are valid or not
-        float t = w8_sum8<DT>(xv[j]);
-        t = t + __shfl_xor(t, 1);
-        t = t + __shfl_xor(t, 2);
-        t = t + __shfl_xor(t, 4);
-        t = t + __shfl_xor(t, 8);
-        if (v < n_xv) {
-            *reinterpret_cast<uint4*>(xs + xrow[j] * xstride + xkv[j] * 16) = xv[j];
-            if ((tid & 15) == 0) xsum[(xkv[j] >> 4) * 16 + xrow[j]] = t;
-        }
+        if (v < n_xv) *reinterpret_cast<uint4*>(xs + xrow[j] * xstride + xkv[j] * 16) = xv[j];
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -207,11 +190,22 @@ __global__ __launch_bounds__(4 * CG * 64) void w8a16_stream(Stream16Args a) {
     // line, register 2 i + 1 the same of the second 64.  A register feeds two MFMAs of 32 elements of K: lane group g
     // brings elements 16 g .. 16 g + 7 to the first and 16 g + 8 .. 16 g + 15 to the second; the activation fragments are
     // read from the same places.
-    w8f4 acc = {0.f, 0.f, 0.f, 0.f}, P = {0.f, 0.f, 0.f, 0.f}, X = {0.f, 0.f, 0.f, 0.f};
+    // (two accumulator chains, so that an MFMA does not wait for the one just issued)
+    w8f4 acc = {0.f, 0.f, 0.f, 0.f}, P0 = {0.f, 0.f, 0.f, 0.f}, P1 = {0.f, 0.f, 0.f, 0.f};
     const uint8_t* xlane = xs + (r16 < (int)M ? r16 : (int)M - 1) * xstride + (ks * kw + g * 16) * 2;
     int in_span = 0, span_idx = 0;
+    uint4 nz = make_uint4(0u, 0u, 0u, 0u);           // -(128 + offset) of the lane's column in the current span, 8 times
 #pragma unroll
     for (int i = 0; i < NLN; ++i) {
+        if (in_span == 0) {                          // a span starts (the same for every wave of the launch)
+            int zq = fz_raw[0];
+#pragma unroll
+            for (int q = 1; q < NLN; ++q)
+                if (q == span_idx) zq = fz_raw[q];
+            const float nf = -(float)(zq + 128);
+            const uint32_t nb = W8Act<DT>::pack2(nf, nf);
+            nz = make_uint4(nb, nb, nb, nb);
+        }
         uint4 fa[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) fa[q] = *reinterpret_cast<const uint4*>(xlane + i * 256 + (q >> 1) * 128 + (q & 1) * 16);
@@ -223,27 +217,24 @@ __global__ __launch_bounds__(4 * CG * 64) void w8a16_stream(Stream16Args a) {
             b0[d] = (uint32_t)__builtin_amdgcn_update_dpp((int)lo, (int)hi, 0x128, 0xF, 0xC, false);
             b1[d] = (uint32_t)__builtin_amdgcn_update_dpp((int)hi, (int)lo, 0x128, 0xF, 0x3, false);
         }
-        P = W8Act<DT>::mfma(fa[0], w8_expand<DT>(b0.x, b0.y), P);
-        P = W8Act<DT>::mfma(fa[1], w8_expand<DT>(b0.z, b0.w), P);
-        P = W8Act<DT>::mfma(fa[2], w8_expand<DT>(b1.x, b1.y), P);
-        P = W8Act<DT>::mfma(fa[3], w8_expand<DT>(b1.z, b1.w), P);
-        {
-            const w8f4 Xi = *reinterpret_cast<const w8f4*>(xsum + (ks * NLN + i) * 16 + 4 * g);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) X[r] = X[r] + Xi[r];
-        }
-        if (++in_span == a.span) {                   // the span's scale ends here (the same for every wave of the launch)
+        P0 = W8Act<DT>::mfma(fa[0], w8_expand<DT>(b0.x, b0.y), P0);
+        P1 = W8Act<DT>::mfma(fa[1], w8_expand<DT>(b0.z, b0.w), P1);
+        P0 = W8Act<DT>::mfma(fa[2], w8_expand<DT>(b1.x, b1.y), P0);
+        P1 = W8Act<DT>::mfma(fa[3], w8_expand<DT>(b1.z, b1.w), P1);
+        P0 = W8Act<DT>::mfma(fa[0], nz, P0);
+        P1 = W8Act<DT>::mfma(fa[1], nz, P1);
+        P0 = W8Act<DT>::mfma(fa[2], nz, P0);
+        P1 = W8Act<DT>::mfma(fa[3], nz, P1);
+        if (++in_span == a.span) {                   // the span's scale ends here
             uint32_t sbits = fs_raw[0];
-            int zq = fz_raw[0];
 #pragma unroll
             for (int q = 1; q < NLN; ++q)
-                if (q == span_idx) { sbits = fs_raw[q]; zq = fz_raw[q]; }
+                if (q == span_idx) sbits = fs_raw[q];
             const float sc = a.scale_f16 ? f16_bits_to_f32(sbits) : bf16_bits_to_f32(sbits);
-            const float c = -(sc * (float)(zq + 128));                         // exact: 8 bits x 11 bits
 #pragma unroll
-            for (int r = 0; r < 4; ++r) acc[r] = __builtin_fmaf(sc, P[r], __builtin_fmaf(c, X[r], acc[r]));
-            P = w8f4{0.f, 0.f, 0.f, 0.f};
-            X = w8f4{0.f, 0.f, 0.f, 0.f};
+            for (int r = 0; r < 4; ++r) acc[r] = __builtin_fmaf(sc, P0[r] + P1[r], acc[r]);
+            P0 = w8f4{0.f, 0.f, 0.f, 0.f};
+            P1 = w8f4{0.f, 0.f, 0.f, 0.f};
             in_span = 0;
             ++span_idx;
         }
@@ -383,7 +374,7 @@ bool w8a16_stream_takes(int64_t M, int64_t N, int64_t K_row, int group, size_t w
     const size_t xbytes = (size_t)M * ((size_t)K * 2 + 16);
     const int64_t cg = xbytes > 40 * 1024 ? 4 : xbytes > 12 * 1024 ? 2 : 1, nt = 256 * cg, kv = K / 8;
     const int64_t xj = (M * kv + nt - 1) / nt;
-    if (xbytes + (size_t)(K / 128) * 64 > 160 * 1024) return false;
+    if (xbytes > 160 * 1024) return false;
     if (nt % kv == 0) return xj <= 8;
     return kv == 2 * nt && cg == 1 && K / 512 == 8 && xj <= 2;
 }
@@ -408,7 +399,7 @@ int w8a16_stream_dispatch(const void* x, const void* smooth, const uint8_t* wq, 
                    (uint32_t)(0x100000000ull / (uint64_t)(K / 8)) + 1u, (int)K_row, (int)(K_row / group), part};
     const size_t xbytes = (size_t)M * ((size_t)K * 2 + 16);
     const int cg = xbytes > 40 * 1024 ? 4 : xbytes > 12 * 1024 ? 2 : 1;
-    const size_t red = (size_t)3 * cg * 64 * 16, img = xbytes + (size_t)(K / 128) * 64;
+    const size_t red = (size_t)3 * cg * 64 * 16, img = xbytes;
     const size_t lds_bytes = img > red ? img : red;
     if (lds_bytes > 160 * 1024) return AMCT_E_UNSUPPORTED;
     return dtype == AMCT_F16 ? stream16_dispatch_dt<AMCT_F16>(a, smooth != nullptr, cg, nln, lds_bytes, st)

@@ -549,8 +549,8 @@ def spin_up(dev):
 
 
 def time_case(case, steps, warmup, dev, repeats):
-    """`repeats` timed regions of exactly `steps` launches each (device time by events on the launch stream, host
-    time around the same region); returns the median host time of a region, the median device time per launch and the latter for every region."""
+    """`repeats` timed regions of exactly `steps` launches each, every region between two synchronizes (device time by
+    events on the launch stream, host time from the first launch until the closing event reads complete); returns the median host time of a region, the median device time per launch and the latter for every region."""
     import torch
     for i in range(warmup):
         case.launch(i)
@@ -560,13 +560,19 @@ def time_case(case, steps, warmup, dev, repeats):
     for _ in range(repeats):
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
-        t0 = time.perf_counter()
         e0.record()
+        t0 = time.perf_counter()
         for i in range(steps):
             case.launch(idx + i)
         e1.record()
+        # The host clock stops when the event behind the last launch reads complete (polled: a blocking wait adds the
+        # host's wake-up latency, and torch.cuda.synchronize costs 30 - 45 us on this runtime even when nothing is
+        # pending -- a tenth of a region of 20 launches); the synchronize that closes the region follows.
+        while not e1.query():
+            pass
+        t1 = time.perf_counter()
         torch.cuda.synchronize(dev)
-        walls.append(time.perf_counter() - t0)
+        walls.append(t1 - t0)
         devs.append(e0.elapsed_time(e1) / steps)
         idx += steps
     return sorted(walls)[len(walls) // 2], sorted(devs)[len(devs) // 2], devs
