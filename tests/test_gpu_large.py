@@ -21,7 +21,7 @@ from util import check_weight_only
 pytestmark = pytest.mark.gpu
 
 GUARD = 9 << 30                                      # bytes on either side of a buffer: +-2^31 elements of 4 bytes, and more
-NEED_FREE = 150 << 30
+NEED_FREE = 200 << 30
 
 
 @pytest.fixture()
@@ -233,3 +233,119 @@ def test_w8a16_weight_beyond_4gib(big, M):
     cols = col_sample(N, 1 << 20).to(dev)
     check_weight_only(out[:, cols].cpu(), x.cpu(), wq[cols].cpu().to(torch.int32), scales[cols].cpu(), None, K, None, None,
                       bool(rounded), what=M, exact_rel=2e-5)
+
+
+R4, C4 = 32768 + 8, 65536                            # fp32: row 32768 starts at element 2^31 (byte 2^33)
+ROWS4 = [0, 1, 16383, 32767, 32768, 32769, R4 - 1]
+
+
+def test_quantise_with_given_factors_and_minmax_beyond_2g_elements(big):
+    """amct_quant_with_params and amct_minmax on fp32 [32776, 65536], groups of 128 (int4 range, asymmetric), codes as
+    int32 (8.6 GB of them): the sampled rows against the call on those rows alone."""
+    dev, lib = big, _lib.load()
+    G = C4 // 128
+    w = banded((R4, C4), torch.float32, dev).normal_()
+    scale = banded((R4, G), torch.float32, dev).uniform_(0.05, 0.5)
+    offset = banded((R4, G), torch.int32, dev)
+    offset.copy_(torch.randint(-8, 8, (R4, G), device=dev, dtype=torch.int32))
+    dq = banded((R4, C4), torch.float32, dev)
+    codes = banded((R4, C4), torch.int32, dev)
+    call(lib.amct_quant_with_params, w, scale, offset, dq, codes, _lib.CODES_I32, None, _lib.COL_NONE, R4, C4, 128, -8, 7, 0,
+         _lib.STAGE_FULL, _lib.F32, stream(dev))
+    sdq, scodes = ops.quant_with_params(w[ROWS4].contiguous(), scale[ROWS4].contiguous(), offset[ROWS4].contiguous(), 128, -8, 7,
+                                        codes_kind=_lib.CODES_I32)
+    same(dq[ROWS4], sdq, "dequantised rows")
+    same(codes[ROWS4], scodes, "codes")
+    del dq, codes
+    mn = banded((R4, G), torch.float32, dev)
+    mx = banded((R4, G), torch.float32, dev)
+    call(lib.amct_minmax, w, mn, mx, R4, C4, 128, _lib.F32, stream(dev))
+    smn, smx = ops.minmax(w[ROWS4].contiguous(), 128)
+    same(mn[ROWS4], smn, "group minima")
+    same(mx[ROWS4], smx, "group maxima")
+
+
+def test_static_quantise_beyond_2g_elements(big):
+    """amct_quantize on bf16 [65552, 32768] with one scale and zero-point per column."""
+    dev, lib = big, _lib.load()
+    x = banded((R, C), torch.bfloat16, dev).normal_()
+    sc = (20.0 + 20.0 * torch.rand(C, device=dev)).to(torch.bfloat16)
+    zp = torch.randint(-20, 20, (C,), device=dev).to(torch.bfloat16)
+    q = banded((R, C), torch.int8, dev)
+    call(lib.amct_quantize, x, None, sc, zp, q, R, C, C, 0, _lib.BF16, stream(dev))
+    same(q[ROWS], ops.quantize_static(x[ROWS].contiguous(), sc, zp, False), "codes")
+
+
+def test_fp8_block_dequant_beyond_2g_elements(big):
+    """The checkpoint converter's fp8 weight with one fp32 scale per 128 x 128 block: whole block rows of the big call
+    (the first, and the ones around element 2^31) against the call on those rows alone."""
+    dev, lib = big, _lib.load()
+    rows = R - R % 128 + 128                          # 65664: whole blocks
+    w = banded((rows, C), torch.uint8, dev)
+    for i in range(0, rows, 8192):
+        w[i:i + 8192] = torch.randint(0, 256, w[i:i + 8192].shape, device=dev, dtype=torch.uint8)
+    scale = banded((rows // 128, C // 128), torch.float32, dev).uniform_(0.5, 2.0)
+    out = banded((rows, C), torch.bfloat16, dev)
+    call(lib.amct_fp8_block_dequant, w, scale, out, rows, C, 128, _lib.BF16, stream(dev))
+    small = banded((256, C), torch.bfloat16, dev)
+    for r0 in (0, 65536 - 128, rows - 256):
+        call(lib.amct_fp8_block_dequant, w[r0:r0 + 256].clone(), scale[r0 // 128:r0 // 128 + 2].clone(), small, 256, C, 128,
+             _lib.BF16, stream(dev))
+        same(out[r0:r0 + 256], small, "rows from {}".format(r0))
+
+
+def test_int4_pair_packing_beyond_2g_elements(big):
+    """pack_4bit of the converter: int8 [65552, 32768] int4 values -> two output channels per byte."""
+    dev, lib = big, _lib.load()
+    x = banded((R, C), torch.int8, dev)
+    for i in range(0, R, 8192):
+        x[i:i + 8192] = torch.randint(-8, 8, x[i:i + 8192].shape, device=dev, dtype=torch.int8)
+    y = banded((R // 2, C), torch.int8, dev)
+    call(lib.amct_pack_int4_pairs_n, x, y, R, C, stream(dev))
+    small = torch.empty(1, C, dtype=torch.int8, device=dev)
+    for r in (0, 32767, 32768, R // 2 - 1):
+        call(lib.amct_pack_int4_pairs_n, x[2 * r:2 * r + 2].clone(), small, 2, C, stream(dev))
+        same(y[r:r + 1], small, "output row {}".format(r))
+
+
+def test_int4_layout_conversions_beyond_4gib(big):
+    """The reference's operand int32 [k, n] (one int4 each, 34 GB here) -> words [k, n/8] -> the GEMM layout uint8
+    [n, k/2] (2^32 + 2^17 bytes) -> back to int32 [k, n]: column blocks at the start, around the packed row that starts
+    at byte 2^32, and at the end, against the conversions of those columns alone; and the round trip as a whole."""
+    dev, lib = big, _lib.load()
+    k, n = 4096, (1 << 21) + 64
+    codes = banded((k, n), torch.int32, dev)
+    for i in range(0, k, 64):
+        codes[i:i + 64] = torch.randint(-8, 8, (64, n), device=dev, dtype=torch.int32)
+    words = banded((k, n // 8), torch.int32, dev)
+    call(lib.amct_pack_int4_words, codes, words, k, n, stream(dev))
+    packed = banded((n, k // 2), torch.uint8, dev)
+    call(lib.amct_words_to_nibbles_nk, words, packed, k, n, stream(dev))
+    for c0 in (0, (1 << 21) - 64, 1 << 21, n - 64):
+        sub = codes[:, c0:c0 + 64].contiguous()
+        sw = ops.pack_int4_words(sub)
+        same(words[:, c0 // 8:c0 // 8 + 8].contiguous(), sw, "words of columns from {}".format(c0))
+        same(packed[c0:c0 + 64], ops.words_to_nibbles_nk(sw, k, 64), "nibbles of columns from {}".format(c0))
+    back = banded((k, n), torch.int32, dev)
+    call(lib.amct_nibbles_nk_to_codes_kn, packed, back, k, n, stream(dev))
+    for i in range(0, k, 256):
+        assert torch.equal(back[i:i + 256], codes[i:i + 256]), "round trip, rows from {}".format(i)
+
+
+def test_awq_loss_beyond_2g_elements(big):
+    """mean((y - yhat)^4) over 2^31 + 2^19 bf16 elements against torch in fp64, block by block."""
+    dev, lib = big, _lib.load()
+    n = R * C
+    y = banded((n,), torch.bfloat16, dev).normal_()
+    yhat = banded((n,), torch.bfloat16, dev).normal_()
+    yhat[n - 1] = 300.0                               # a term that only an index beyond 2^31 reaches: (300 - y)^4 / n is ~4
+    loss = banded((1,), torch.float32, dev)
+    wsb = lib.amct_awq_loss_workspace_bytes()
+    ws = banded((wsb,), torch.uint8, dev)
+    call(lib.amct_awq_loss, y, yhat, n, _lib.BF16, loss, ws, wsb, stream(dev))
+    tot = 0.0
+    for i in range(0, n, 1 << 26):
+        d = (y[i:i + (1 << 26)] - yhat[i:i + (1 << 26)]).double()
+        tot += float((d * d * d * d).sum())
+    want = tot / n
+    assert want > 10.0 and abs(float(loss[0]) - want) <= 1e-5 * want, (float(loss[0]), want)
