@@ -148,9 +148,48 @@ __global__ __launch_bounds__(kBlock) void gptq_block_quad_k(GptqArgs a) {
         sr[i] = srow[g];
         zr[i] = ASYM ? (float)zrow[g] : 0.f;
     }
+    // Software pipeline: the chain of step i (broadcast, two divisions, quantisation: about 30 dependent operations) is
+    // the critical path of the whole kernel -- a thread block takes the same 128 x chain whether the matrix has 64 rows
+    // or 14336 -- and the updates of step i - 1 are independent of it except for the one slot that holds column i.  So
+    // step i - 1 updates only that slot before step i starts (the "critical" slot: one product and one subtraction), and
+    // the other slots of step i - 1 are updated INSIDE the chain of step i, a third of them in each of its three parts,
+    // where they fill the issue slots the chain leaves empty.  Every element still receives its updates in step order:
+    // the operations and their order per element are those of the loop above.
+    float err_prev = 0.f;
+    float hprev[8][4];                                              // row i - 1 of the block of Hinv, this lane's columns
+#pragma unroll
+    for (int m = 0; m < 8; ++m)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) hprev[m][e] = 0.f;
 #pragma clang loop unroll(full)
     for (int i = 0; i < kGqMax; ++i) {
         const int mi = i >> 4, qi = (i >> 2) & 3, ei = i & 3;
+        const int mp = (i - 1) >> 4;                                // slot row of column i - 1 (i >= 1)
+        // the slots of step i - 1 that are still to be updated: (m, e) with m >= mp, except the slot of column i
+        auto pending = [&](int part) {
+            if (i == 0) return;
+#pragma unroll
+            for (int sl = 0; sl < 32; ++sl) {
+                const int m = sl >> 2, e = sl & 3;
+                if (sl % 3 != part || m < mp || (m == mi && e == ei)) continue;
+                const float p = err_prev * hprev[m][e];
+                if (m > mp) w[m][e] = w[m][e] - p;
+                else if (4 * q + e >= ((i - 1) & 15)) w[m][e] = w[m][e] - p;
+            }
+        };
+        // row i of the block of Hinv for the updates of this step: the diagonal, the critical slot, and (for the next
+        // iteration) this lane's columns at and behind slot row mi
+        const float hdiag = hs[i * kGqMax + i];
+        const int inx = i + 1 < kGqMax ? i + 1 : i;                 // column i + 1, whose slot is updated before step i + 1
+        const int mn = inx >> 4, en = inx & 3;
+        const float hcrit = hs[i * kGqMax + 16 * mn + 4 * q + en];
+        float hcur[8][4];
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            if (m < mi) continue;
+            const float4 h = *reinterpret_cast<const float4*>(&hs[i * kGqMax + 16 * m + 4 * q]);
+            hcur[m][0] = h.x; hcur[m][1] = h.y; hcur[m][2] = h.z; hcur[m][3] = h.w;
+        }
         float wi;
         if (qi == 0) wi = quad_bcast<0>(w[mi][ei]);
         else if (qi == 1) wi = quad_bcast<1>(w[mi][ei]);
@@ -163,24 +202,38 @@ __global__ __launch_bounds__(kBlock) void gptq_block_quad_k(GptqArgs a) {
             zr[i % kGqAhead] = ASYM ? (float)zrow[g] : 0.f;
         }
         float t = wi / sc;
+        pending(0);
+        __builtin_amdgcn_sched_barrier(0);
         if (ASYM) t = t + z;
         t = __builtin_rintf(t);
         t = __builtin_amdgcn_fmed3f(t, a.qmin, a.qmax);
         const float wq = (t - z) * sc;
-        const float err = (wi - wq) / hs[i * kGqMax + i];
+        const float dlt = wi - wq;
+        pending(1);
+        __builtin_amdgcn_sched_barrier(0);
+        const float err = dlt / hdiag;
+        pending(2);
+        __builtin_amdgcn_sched_barrier(0);
         if (q == qi) eo[mi][ei] = err;
+        // the critical slot: the one that holds column i + 1 (column i itself -- the reference's update runs from j = i,
+        // W[n][i] -= err * Hinv[i][i]: not read again, but what the caller gets back -- shares its slot with columns of
+        // the other lanes and is updated with them, among the pending slots of the next iteration)
+        if (i + 1 < kGqMax) {
+            const float p = err * hcrit;
+            if (mn > mi) w[mn][en] = w[mn][en] - p;
+            else if (4 * q + en >= (i & 15)) w[mn][en] = w[mn][en] - p;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        err_prev = err;
 #pragma unroll
-        for (int m = mi; m < 8; ++m) {
-            const float4 h = *reinterpret_cast<const float4*>(&hs[i * kGqMax + 16 * m + 4 * q]);
-            const float hv[4] = {h.x, h.y, h.z, h.w};
+        for (int m = 0; m < 8; ++m) {
+            if (m < mi) continue;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float p = err * hv[e];
-                if (m > mi) w[m][e] = w[m][e] - p;
-                else if (4 * q + e >= (i & 15)) w[m][e] = w[m][e] - p;
-            }
+            for (int e = 0; e < 4; ++e) hprev[m][e] = hcur[m][e];
         }
     }
+    // what step 127 leaves pending: column 127 itself (slot (7, 3) of lane 3)
+    if (q == 3) w[7][3] = w[7][3] - err_prev * hprev[7][3];
     if (n < a.rows) {
         float* wo = a.w + n * a.ld_w + 4 * q;
         float* er = a.err + n * a.ld_e + 4 * q;
